@@ -1,0 +1,286 @@
+"""ctypes front end of the CPU oracle (TEST INFRASTRUCTURE ONLY).
+
+Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may import this
+module. It loads oracle/libaion_oracle.so (built by oracle/Makefile) and wraps each
+function with numpy in/out. See aion_oracle.h for what each function restates.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libaion_oracle.so")
+
+Q4_0, Q8_0 = 3, 4
+BLOCK_BYTES = {Q4_0: 18, Q8_0: 34}
+UNBOUNDED = 0xFFFFFFFF
+
+
+def build():
+    subprocess.check_call(["make", "-C", _HERE, "-B", "libaion_oracle.so"], stdout=subprocess.DEVNULL)
+
+
+def _load():
+    if not os.path.exists(_LIB_PATH):
+        build()
+    lib = C.CDLL(_LIB_PATH)
+    sz, f, i, vp = C.c_size_t, C.c_float, C.c_int, C.c_void_p
+    lib.orc_f32_to_f16.argtypes = [f]; lib.orc_f32_to_f16.restype = C.c_uint16
+    lib.orc_f16_to_f32.argtypes = [C.c_uint16]; lib.orc_f16_to_f32.restype = f
+    lib.orc_exp_approx.argtypes = [f]; lib.orc_exp_approx.restype = f
+    lib.orc_tanh_approx.argtypes = [f]; lib.orc_tanh_approx.restype = f
+    lib.orc_quantize.argtypes = [i, vp, sz, sz, vp, vp]
+    lib.orc_dequantize.argtypes = [i, vp, sz, sz, vp, vp]
+    lib.orc_prepare_a.argtypes = [vp, sz, sz, sz, vp, vp, vp]; lib.orc_prepare_a.restype = None
+    lib.orc_matmul_nt_q8.argtypes = [sz, sz, sz, f, f, vp, sz, vp, vp, sz, i]
+    lib.orc_matmul_q8_kmajor.argtypes = [sz, sz, sz, f, f, vp, sz, vp, sz, vp, sz, i]
+    lib.orc_matmul_q_packed.argtypes = [i, sz, sz, sz, f, f, vp, sz, vp, vp, sz, sz, i]
+    lib.orc_matmul_q_f32a.argtypes = [i, i, sz, sz, sz, f, f, vp, sz, vp, vp, sz, i]
+    lib.orc_attention_blocked.argtypes = [vp, vp, vp, vp, vp, vp, vp, i]
+    lib.orc_attention_f64.argtypes = [vp, vp, vp, vp, vp, vp, vp]
+    lib.orc_rmsnorm.argtypes = [vp, vp, vp, vp, sz, sz, f, vp]; lib.orc_rmsnorm.restype = None
+    lib.orc_rope.argtypes = [vp, vp, sz, sz, sz, sz, f, f, f, vp]; lib.orc_rope.restype = None
+    lib.orc_gate_gelu.argtypes = [vp, vp, sz, vp]; lib.orc_gate_gelu.restype = None
+    lib.orc_gather_rows.argtypes = [i, vp, sz, vp, sz, vp]; lib.orc_gather_rows.restype = None
+    lib.orc_argmax.argtypes = [vp, sz, sz, vp]; lib.orc_argmax.restype = None
+    lib.orc_cast_f32_f16.argtypes = [vp, sz, vp]; lib.orc_cast_f32_f16.restype = None
+    lib.orc_decoder_create.argtypes = [vp, i]; lib.orc_decoder_create.restype = vp
+    lib.orc_decoder_destroy.argtypes = [vp]; lib.orc_decoder_destroy.restype = None
+    lib.orc_decoder_set_weight.argtypes = [vp, C.c_char_p, vp, sz]
+    lib.orc_decoder_reset.argtypes = [vp]; lib.orc_decoder_reset.restype = None
+    lib.orc_decoder_forward.argtypes = [vp, vp, sz, sz, vp]; lib.orc_decoder_forward.restype = C.c_int32
+    return lib
+
+
+_lib = _load()
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def f32_to_f16_bits(v):
+    return int(_lib.orc_f32_to_f16(float(np.float32(v))))
+
+
+def f16_bits_to_f32(b):
+    return float(_lib.orc_f16_to_f32(int(b)))
+
+
+def exp_approx(x):
+    return float(_lib.orc_exp_approx(float(np.float32(x))))
+
+
+def tanh_approx(x):
+    return float(_lib.orc_tanh_approx(float(np.float32(x))))
+
+
+def quantize(dtype, values, quant_axis):
+    """f32 array -> packed blocks (uint8), row-major over block space."""
+    v = _f32(values)
+    shape = (C.c_size_t * v.ndim)(*v.shape)
+    out = np.zeros(v.size // 32 * BLOCK_BYTES[dtype], dtype=np.uint8)
+    rc = _lib.orc_quantize(dtype, shape, v.ndim, quant_axis, _p(v), _p(out))
+    if rc != 0:
+        raise ValueError("orc_quantize: InvalidArgument")
+    return out
+
+
+def dequantize(dtype, blocks, shape, quant_axis):
+    out = np.zeros(shape, dtype=np.float32)
+    sh = (C.c_size_t * len(shape))(*shape)
+    b = np.ascontiguousarray(blocks, dtype=np.uint8)
+    rc = _lib.orc_dequantize(dtype, sh, len(shape), quant_axis, _p(b), _p(out))
+    if rc != 0:
+        raise ValueError("orc_dequantize: InvalidArgument")
+    return out
+
+
+def prepare_a(a):
+    a = _f32(a)
+    m, k = a.shape
+    aq = np.zeros((m, k), dtype=np.int8)
+    sc = np.zeros((m, k // 32), dtype=np.float32)
+    sm = np.zeros((m, k // 32), dtype=np.int32)
+    _lib.orc_prepare_a(_p(a), m, k, k, _p(aq), _p(sc), _p(sm))
+    return aq, sc, sm
+
+
+def _c_init(m, n, c, beta):
+    if c is None:
+        if beta != 0.0:
+            raise ValueError("beta != 0 needs c")
+        return np.zeros((m, n), dtype=np.float32)
+    return np.array(c, dtype=np.float32, copy=True).reshape(m, n)
+
+
+def matmul_nt_q8(a, b_blocks, n, alpha=1.0, beta=0.0, c=None, threads=1):
+    a = _f32(a); m, k = a.shape
+    b = np.ascontiguousarray(b_blocks, dtype=np.uint8)
+    out = _c_init(m, n, c, beta)
+    rc = _lib.orc_matmul_nt_q8(m, n, k, alpha, beta, _p(a), k, _p(b), _p(out), n, threads)
+    if rc != 0:
+        raise ValueError("orc_matmul_nt_q8: InvalidArgument")
+    return out
+
+
+def matmul_q8_kmajor(a, b_blocks, n, alpha=1.0, beta=0.0, c=None, threads=1):
+    a = _f32(a); m, k = a.shape
+    b = np.ascontiguousarray(b_blocks, dtype=np.uint8)
+    out = _c_init(m, n, c, beta)
+    rc = _lib.orc_matmul_q8_kmajor(m, n, k, alpha, beta, _p(a), k, _p(b), n, _p(out), n, threads)
+    if rc != 0:
+        raise ValueError("orc_matmul_q8_kmajor: InvalidArgument")
+    return out
+
+
+def matmul_q_packed(dtype, a, b_blocks, n, alpha=1.0, beta=0.0, c=None, kc=256, threads=1):
+    a = _f32(a); m, k = a.shape
+    b = np.ascontiguousarray(b_blocks, dtype=np.uint8)
+    out = _c_init(m, n, c, beta)
+    rc = _lib.orc_matmul_q_packed(dtype, m, n, k, alpha, beta, _p(a), k, _p(b), _p(out), n, kc, threads)
+    if rc != 0:
+        raise ValueError("orc_matmul_q_packed: InvalidArgument")
+    return out
+
+
+def matmul_q_f32a(dtype, nt, a, b_blocks, n, alpha=1.0, beta=0.0, c=None, threads=1):
+    a = _f32(a); m, k = a.shape
+    b = np.ascontiguousarray(b_blocks, dtype=np.uint8)
+    out = _c_init(m, n, c, beta)
+    rc = _lib.orc_matmul_q_f32a(dtype, 1 if nt else 0, m, n, k, alpha, beta, _p(a), k, _p(b), _p(out), n, threads)
+    if rc != 0:
+        raise ValueError("orc_matmul_q_f32a: InvalidArgument")
+    return out
+
+
+class _AttnShape(C.Structure):
+    _fields_ = [(n, C.c_size_t) for n in ("batch", "l_q", "t_kv", "h_q", "h_kv", "d_k", "d_v")] + [
+        ("scale", C.c_float), ("soft_cap", C.c_float),
+        ("win_left", C.c_uint32), ("win_right", C.c_uint32), ("win_chunk", C.c_uint32),
+        ("kv_dtype", C.c_int)]
+
+
+def _attn_args(q, k, v, scale, window, soft_cap, positions, kv_lengths):
+    q = _f32(q)
+    B, L, Hq, Dk = q.shape
+    if k.dtype == np.float16:
+        k = np.ascontiguousarray(k).view(np.uint16); v = np.ascontiguousarray(v).view(np.uint16); kvd = 1
+    elif k.dtype == np.uint16:
+        k = np.ascontiguousarray(k); v = np.ascontiguousarray(v); kvd = 1
+    else:
+        k = _f32(k); v = _f32(v); kvd = 0
+    _, T, Hkv, _ = k.shape
+    Dv = v.shape[3]
+    left, right, chunk = window
+    s = _AttnShape(B, L, T, Hq, Hkv, Dk, Dv, scale, soft_cap, left, right, chunk, kvd)
+    pos = None if positions is None else np.ascontiguousarray(positions, dtype=np.int32)
+    kl = None if kv_lengths is None else np.ascontiguousarray(kv_lengths, dtype=np.int32)
+    out = np.zeros((B, L, Hq, Dv), dtype=np.float32)
+    return s, q, k, v, pos, kl, out
+
+
+CAUSAL = (UNBOUNDED, 0, 0)
+FULL = (UNBOUNDED, UNBOUNDED, 0)
+
+
+def attention_blocked(q, k, v, scale, window=CAUSAL, soft_cap=0.0, positions=None, kv_lengths=None, segs=1):
+    s, q, k, v, pos, kl, out = _attn_args(q, k, v, scale, window, soft_cap, positions, kv_lengths)
+    rc = _lib.orc_attention_blocked(C.byref(s), _p(q), _p(k), _p(v), _p(pos), _p(kl), _p(out), segs)
+    if rc != 0:
+        raise ValueError("orc_attention_blocked: InvalidArgument")
+    return out
+
+
+def attention_f64(q, k, v, scale, window=CAUSAL, soft_cap=0.0, positions=None, kv_lengths=None):
+    s, q, k, v, pos, kl, out = _attn_args(q, k, v, scale, window, soft_cap, positions, kv_lengths)
+    rc = _lib.orc_attention_f64(C.byref(s), _p(q), _p(k), _p(v), _p(pos), _p(kl), _p(out))
+    if rc != 0:
+        raise ValueError("orc_attention_f64: InvalidArgument")
+    return out
+
+
+def rmsnorm(x, gamma, eps, beta=None, residual=None):
+    x = _f32(x); rows, cols = x.shape
+    g = _f32(gamma); b = None if beta is None else _f32(beta); r = None if residual is None else _f32(residual)
+    out = np.zeros_like(x)
+    _lib.orc_rmsnorm(_p(x), _p(g), _p(b), _p(r), rows, cols, eps, _p(out))
+    return out
+
+
+def rope(x, positions, base=10000.0, scale_factor=1.0, proportion=1.0):
+    x = _f32(x); B, T, H, D = x.shape
+    pos = np.ascontiguousarray(positions, dtype=np.int32)
+    out = np.zeros_like(x)
+    _lib.orc_rope(_p(x), _p(pos), B, T, H, D, base, scale_factor, proportion, _p(out))
+    return out
+
+
+def gate_gelu(a, b):
+    a = _f32(a); b = _f32(b)
+    out = np.zeros_like(a)
+    _lib.orc_gate_gelu(_p(a), _p(b), a.size, _p(out))
+    return out
+
+
+def gather_rows(table, ids, d, dtype=0):
+    ids = np.ascontiguousarray(ids, dtype=np.int32)
+    t = np.ascontiguousarray(table)
+    out = np.zeros((ids.size, d), dtype=np.float32)
+    _lib.orc_gather_rows(dtype, _p(t), d, _p(ids), ids.size, _p(out))
+    return out
+
+
+def argmax(x):
+    x = _f32(x); rows, n = x.shape
+    out = np.zeros(rows, dtype=np.int32)
+    _lib.orc_argmax(_p(x), rows, n, _p(out))
+    return out
+
+
+def cast_f32_f16(x):
+    x = _f32(x)
+    out = np.zeros(x.shape, dtype=np.uint16)
+    _lib.orc_cast_f32_f16(_p(x), x.size, _p(out))
+    return out.view(np.float16)
+
+
+class _DecCfg(C.Structure):
+    _fields_ = [(n, C.c_size_t) for n in ("layers", "hidden", "heads", "kv_heads", "head_dim", "ffn", "vocab", "max_seq")] + [
+        ("eps", C.c_float), ("rope_base", C.c_float), ("wdtype", C.c_int)]
+
+
+class Decoder:
+    """The synthetic decoder run through the oracle kernels (see orc_decoder_* in aion_oracle.h)."""
+
+    def __init__(self, layers, hidden, heads, kv_heads, head_dim, ffn, vocab, max_seq,
+                 eps=1e-6, rope_base=10000.0, wdtype=Q4_0, threads=1):
+        self.cfg = _DecCfg(layers, hidden, heads, kv_heads, head_dim, ffn, vocab, max_seq, eps, rope_base, wdtype)
+        self.vocab = vocab
+        self._h = _lib.orc_decoder_create(C.byref(self.cfg), threads)
+
+    def set_weight(self, name, data):
+        d = np.ascontiguousarray(data)
+        _lib.orc_decoder_set_weight(self._h, name.encode(), _p(d), d.nbytes)
+
+    def reset(self):
+        _lib.orc_decoder_reset(self._h)
+
+    def forward(self, tokens, pos0, want_logits=True):
+        t = np.ascontiguousarray(tokens, dtype=np.int32)
+        logits = np.zeros(self.vocab, dtype=np.float32) if want_logits else None
+        tok = _lib.orc_decoder_forward(self._h, _p(t), t.size, pos0, _p(logits))
+        if tok < 0:
+            raise ValueError("orc_decoder_forward failed")
+        return int(tok), logits
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            _lib.orc_decoder_destroy(self._h)
+            self._h = None
