@@ -1,0 +1,239 @@
+"""Host-side mirror of aion's backend vocabulary over the C ABI (numpy in, numpy out).
+
+Names follow aion: a `HipBackend` owns one device context (Backend + Session,
+backend/backend.zig:24-107), `DeviceBuffer` is a DeviceMemory allocation
+(runtime/device_memory.zig:36-108), `Weight` is a quantized rank-2 parameter after the
+backend's private re-lay, and the `step_*` methods take the operands of the matching
+ExecutableProgram step (runtime/executable.zig).
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import hip
+from .hip import (BF16, F16, F32, GEMM_BF16_MFMA, GEMM_EXACT_I8, I32, KMAJOR_KN, Q4_0, Q8_0, ROWS_NK, UNBOUNDED,  # noqa: F401
+                  AionHipError)
+
+BLOCK_BYTES = {Q4_0: 18, Q8_0: 34}
+CAUSAL = (UNBOUNDED, 0, 0)
+FULL = (UNBOUNDED, UNBOUNDED, 0)
+
+
+def quantize_blocks(dtype, values, quant_axis):
+    """storage/quantize.zig `quantizeBlocks` over the whole tensor: f32 array -> packed bytes."""
+    lib = hip.load_library()
+    v = np.ascontiguousarray(values, dtype=np.float32)
+    if v.ndim == 0:
+        raise AionHipError(hip.INVALID_ARGUMENT, "rank-0 tensor")
+    if dtype not in BLOCK_BYTES:
+        raise AionHipError(hip.UNSUPPORTED, "dtype %r is not block-quantized" % (dtype,))
+    shape = (C.c_size_t * v.ndim)(*v.shape)
+    out = np.empty(v.size // 32 * BLOCK_BYTES[dtype], dtype=np.uint8)
+    rc = lib.aionhip_quantize_blocks(dtype, shape, v.ndim, quant_axis, v.ctypes.data, v.size, 0, 0, out.ctypes.data, out.nbytes)
+    if rc != hip.OK:
+        raise AionHipError(rc, "quantize_blocks(shape=%s, axis=%d)" % (v.shape, quant_axis))
+    return out
+
+
+class DeviceBuffer:
+    def __init__(self, backend, handle, nbytes):
+        self.backend, self.handle, self.nbytes = backend, handle, nbytes
+
+    def free(self):
+        if self.handle:
+            self.backend._lib.aionhip_free(self.backend._ctx, self.handle)
+            self.handle = 0
+
+    def numpy(self, dtype, shape=None, offset=0):
+        return self.backend.download(self, dtype, shape, offset)
+
+
+class Weight:
+    def __init__(self, backend, ptr, dtype, layout, n, k):
+        self.backend, self.ptr, self.dtype, self.layout, self.n, self.k = backend, ptr, dtype, layout, n, k
+
+    @property
+    def packed_bytes(self):
+        return self.backend._lib.aionhip_weight_packed_bytes(self.ptr)
+
+    @property
+    def device_bytes(self):
+        return self.backend._lib.aionhip_weight_device_bytes(self.ptr)
+
+    def download(self):
+        out = np.empty(self.packed_bytes, dtype=np.uint8)
+        self.backend._check(self.backend._lib.aionhip_weight_download(self.backend._ctx, self.ptr, out.ctypes.data, out.nbytes))
+        return out
+
+    def free(self):
+        if self.ptr:
+            self.backend._lib.aionhip_weight_free(self.backend._ctx, self.ptr)
+            self.ptr = None
+
+
+class HipBackend:
+    def __init__(self, device=0, stream=None):
+        self._lib = hip.load_library()
+        ctx = C.c_void_p()
+        rc = self._lib.aionhip_create(device, stream, C.byref(ctx))
+        if rc != hip.OK:
+            raise AionHipError(rc, "aionhip_create(device=%d): no usable HIP device" % device)
+        self._ctx = ctx
+        self.name = self._lib.aionhip_name().decode()
+
+    # ---- context
+    def _check(self, rc):
+        if rc != hip.OK:
+            raise AionHipError(rc, self._lib.aionhip_last_error(self._ctx).decode())
+
+    def close(self):
+        if self._ctx:
+            self._lib.aionhip_destroy(self._ctx)
+            self._ctx = None
+
+    def sync(self):
+        self._check(self._lib.aionhip_sync(self._ctx))
+
+    def last_kernel(self):
+        return self._lib.aionhip_last_kernel(self._ctx).decode()
+
+    def set_gemm_mode(self, mode):
+        self._check(self._lib.aionhip_set_gemm_mode(self._ctx, mode))
+
+    def device_info(self):
+        cu, wave, hbm = C.c_int(), C.c_int(), C.c_uint64()
+        arch = C.create_string_buffer(64)
+        self._check(self._lib.aionhip_device_info(self._ctx, C.byref(cu), C.byref(wave), C.byref(hbm), arch, 64))
+        return {"cu_count": cu.value, "wave_size": wave.value, "hbm_bytes": hbm.value, "arch": arch.value.decode()}
+
+    # ---- device memory
+    def alloc(self, nbytes, alignment=256):
+        h = C.c_uint64()
+        self._check(self._lib.aionhip_alloc(self._ctx, nbytes, alignment, C.byref(h)))
+        return DeviceBuffer(self, h.value, nbytes)
+
+    def upload(self, array):
+        a = np.ascontiguousarray(array)
+        buf = self.alloc(max(a.nbytes, 1))
+        if a.nbytes:
+            self._check(self._lib.aionhip_h2d(self._ctx, buf.handle, 0, a.ctypes.data, a.nbytes))
+        return buf
+
+    def write(self, buf, array, offset=0):
+        a = np.ascontiguousarray(array)
+        self._check(self._lib.aionhip_h2d(self._ctx, buf.handle, offset, a.ctypes.data, a.nbytes))
+
+    def download(self, buf, dtype, shape=None, offset=0):
+        dt = np.dtype(dtype)
+        if shape is None:
+            shape = ((buf.nbytes - offset) // dt.itemsize,)
+        out = np.empty(shape, dtype=dt)
+        if out.nbytes:
+            self._check(self._lib.aionhip_d2h(self._ctx, out.ctypes.data, buf.handle, offset, out.nbytes))
+        return out
+
+    def zeros(self, nbytes):
+        buf = self.alloc(nbytes)
+        self._check(self._lib.aionhip_memset(self._ctx, buf.handle, 0, 0, nbytes))
+        return buf
+
+    # ---- quantize / weights
+    def quantize_device(self, dtype, src_buf, rows, cols, quant_axis):
+        out = self.alloc(rows * cols // 32 * BLOCK_BYTES[dtype])
+        self._check(self._lib.aionhip_quantize_device(self._ctx, dtype, rows, cols, quant_axis, src_buf.handle, out.handle))
+        return out
+
+    def upload_weight(self, dtype, layout, n, k, packed_blocks, ld_blocks=0):
+        b = np.ascontiguousarray(packed_blocks, dtype=np.uint8)
+        w = C.c_void_p()
+        self._check(self._lib.aionhip_weight_upload(self._ctx, dtype, layout, n, k, ld_blocks, b.ctypes.data, C.byref(w)))
+        return Weight(self, w, dtype, layout, n, k)
+
+    def weight_from_device(self, dtype, layout, n, k, blocks_buf, ld_blocks=0):
+        w = C.c_void_p()
+        self._check(self._lib.aionhip_weight_from_device(self._ctx, dtype, layout, n, k, ld_blocks, blocks_buf.handle, C.byref(w)))
+        return Weight(self, w, dtype, layout, n, k)
+
+    # ---- steps
+    def step_matmul(self, weight, a_buf, m, c_buf, lda=0, ldc=0, alpha=1.0, beta=0.0, a_offset=0, c_offset=0):
+        fn = self._lib.aionhip_step_matmul_nt if weight.layout == ROWS_NK else self._lib.aionhip_step_matmul
+        self._check(fn(self._ctx, weight.ptr, m, a_buf.handle + a_offset, lda, c_buf.handle + c_offset, ldc, alpha, beta))
+
+    def matmul(self, weight, a, alpha=1.0, beta=0.0, c=None):
+        """Convenience: numpy A [m,k] -> numpy C [m,n] through the step (uploads, runs, downloads)."""
+        a = np.ascontiguousarray(a, dtype=np.float32)
+        m = a.shape[0]
+        a_buf = self.upload(a)
+        if c is None:
+            c_buf = self.alloc(max(m * weight.n * 4, 4))
+        else:
+            c_buf = self.upload(np.ascontiguousarray(c, dtype=np.float32))
+        try:
+            self.step_matmul(weight, a_buf, m, c_buf, alpha=alpha, beta=beta)
+            return self.download(c_buf, np.float32, (m, weight.n))
+        finally:
+            a_buf.free()
+            c_buf.free()
+
+    def step_attention(self, out, q, k, v, shape, scale, q_dtype=F32, kv_dtype=F16, window=CAUSAL, soft_cap=0.0,
+                       query_positions=None, kv_lengths=None):
+        B, L, T, Hq, Hkv, Dk, Dv = shape
+        p = hip.Attention(out.handle, q.handle, k.handle, v.handle,
+                          query_positions.handle if query_positions is not None else 0,
+                          kv_lengths.handle if kv_lengths is not None else 0,
+                          B, L, T, Hq, Hkv, Dk, Dv, q_dtype, kv_dtype, scale, soft_cap, window[0], window[1], window[2])
+        self._check(self._lib.aionhip_step_attention(self._ctx, C.byref(p)))
+
+    def step_rmsnorm(self, out, x, gamma, rows, cols, eps, beta=None, residual=None):
+        self._check(self._lib.aionhip_step_rmsnorm(self._ctx, out.handle, x.handle, gamma.handle,
+                                                   beta.handle if beta is not None else 0,
+                                                   residual.handle if residual is not None else 0, rows, cols, eps))
+
+    def step_rope(self, out, x, positions, b, t, h, d, base=10000.0, scale_factor=1.0, proportion=1.0):
+        self._check(self._lib.aionhip_step_rope(self._ctx, out.handle, x.handle, positions.handle, b, t, h, d, base, scale_factor, proportion))
+
+    def step_add(self, out, a, b, n):
+        self._check(self._lib.aionhip_step_add(self._ctx, out.handle, a.handle, b.handle, n))
+
+    def step_gate_gelu(self, out, a, b, n):
+        self._check(self._lib.aionhip_step_gate_gelu(self._ctx, out.handle, a.handle, b.handle, n))
+
+    def step_gather_rows(self, table_dtype, out, table, ids, n_ids, d, vocab):
+        self._check(self._lib.aionhip_step_gather_rows(self._ctx, table_dtype, out.handle, table.handle, ids.handle, n_ids, d, vocab))
+
+    def step_append_f16(self, cache, src, write_index, b, s, t_cap, row_elems):
+        self._check(self._lib.aionhip_step_append_f16(self._ctx, cache.handle, src.handle, write_index.handle, b, s, t_cap, row_elems))
+
+    def step_cast_f32_f16(self, out, x, n):
+        self._check(self._lib.aionhip_step_cast_f32_f16(self._ctx, out.handle, x.handle, n))
+
+    def step_argmax(self, out, x, rows, n):
+        self._check(self._lib.aionhip_step_argmax(self._ctx, out.handle, x.handle, rows, n))
+
+    # ---- timing
+    def event(self):
+        e = C.c_void_p()
+        self._check(self._lib.aionhip_event_create(self._ctx, C.byref(e)))
+        return e
+
+    def record(self, e):
+        self._check(self._lib.aionhip_event_record(self._ctx, e))
+
+    def elapsed_ms(self, start, stop):
+        ms = C.c_float()
+        self._check(self._lib.aionhip_event_elapsed_ms(self._ctx, start, stop, C.byref(ms)))
+        return ms.value
+
+    def profile_start(self):
+        self._check(self._lib.aionhip_profile_start(self._ctx))
+
+    def profile_stop(self):
+        """-> list of (kernel name, milliseconds), one per timed launch, in launch order."""
+        n = C.c_size_t()
+        self._check(self._lib.aionhip_profile_stop(self._ctx, C.byref(n)))
+        out = []
+        name, ms = C.c_char_p(), C.c_float()
+        for i in range(n.value):
+            self._check(self._lib.aionhip_profile_entry(self._ctx, i, C.byref(name), C.byref(ms)))
+            out.append((name.value.decode(), ms.value))
+        return out

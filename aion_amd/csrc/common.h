@@ -1,0 +1,136 @@
+// Internal declarations shared by the HIP sources of libaion_hip.so (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+#include <vector>
+
+#include "../../include/aion_hip.h"
+
+using u32x4 = __attribute__((ext_vector_type(4))) unsigned int;   // one 16-byte global load
+using f32x4 = __attribute__((ext_vector_type(4))) float;
+
+constexpr int QK = 32;        // elements per quant block (aion backend/types.zig:40-50)
+constexpr int Q8_BYTES = 34;  // f16 scale + 32 x i8
+constexpr int Q4_BYTES = 18;  // f16 scale + 16 nibble bytes
+
+// One timed kernel launch (per-dispatch GPU timestamps, as aion's WebGPU backend collects with
+// AION_PROFILE_GPU=dispatch, backend/gpu/timestamp_profile.zig).
+struct ProfRecord {
+    const char *name;
+    hipEvent_t start, stop;
+    float ms;
+};
+
+struct aionhip_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    bool own_stream = false;
+    std::string err;
+    const char *last_kernel = "";
+    int gemm_mode = AIONHIP_GEMM_EXACT_I8;
+    int cu_count = 0;
+    // prepared-activation scratch (int8 codes, per-block f32 scale, per-block code sum)
+    void *scratch = nullptr;
+    size_t scratch_bytes = 0;
+    // second scratch for GEMM staging (dequantized weights / bf16 activations / split-K partials)
+    void *scratch2 = nullptr;
+    size_t scratch2_bytes = 0;
+    // per-launch timing, off by default
+    bool profiling = false;
+    std::vector<ProfRecord> prof;
+    std::vector<hipEvent_t> event_pool;
+};
+
+// Brackets one kernel launch with stream events while profiling is on.
+void prof_begin(aionhip_ctx *ctx, const char *name);
+void prof_end(aionhip_ctx *ctx);
+
+// Device-private weight layout: row n of the [N,K] operand is one contiguous run.
+//   q8_0: qs[n][K] int8,               sc[n][K/32] f16
+//   q4_0: qs[n][K/2] nibble bytes,     sc[n][K/32] f16
+// q4 nibble order inside each 32-bit word (8 elements e0..e7): byte i = e[i] | e[4+i] << 4, so
+// (w & 0x0F0F0F0F) is elements 0..3 and ((w >> 4) & 0x0F0F0F0F) is elements 4..7, each directly
+// usable as the byte operand of a 4-way int8 dot.
+struct aionhip_weight {
+    int dtype = 0;
+    int layout = 0;
+    size_t n = 0, k = 0;
+    uint8_t *qs = nullptr;
+    __half *sc = nullptr;
+    size_t qs_bytes = 0, sc_bytes = 0;
+};
+
+int set_err(aionhip_ctx *ctx, int status, const char *fmt, ...);
+int ensure_scratch(aionhip_ctx *ctx, size_t bytes);
+int ensure_scratch2(aionhip_ctx *ctx, size_t bytes);
+
+#define HIP_TRY(ctx, expr)                                                                          \
+    do {                                                                                            \
+        hipError_t e_ = (expr);                                                                     \
+        if (e_ != hipSuccess)                                                                       \
+            return set_err((ctx), e_ == hipErrorOutOfMemory ? AIONHIP_OUT_OF_MEMORY : AIONHIP_EXECUTION_FAILED, \
+                           "%s: %s", #expr, hipGetErrorString(e_));                                 \
+    } while (0)
+
+#define LAUNCH_CHECK(ctx, name)                                                                     \
+    do {                                                                                            \
+        (ctx)->last_kernel = (name);                                                                \
+        hipError_t e_ = hipGetLastError();                                                          \
+        if (e_ != hipSuccess) return set_err((ctx), AIONHIP_EXECUTION_FAILED, "launch %s: %s", (name), hipGetErrorString(e_)); \
+    } while (0)
+
+// ---- prepared activations (aion cpu/kernels/matmul_q_i8.zig:187-264) --------------------------
+struct PreparedAct {
+    int8_t *q;      // [m][k]
+    float *scale;   // [m][k/32]
+    int *sum;       // [m][k/32]   plain sum of the 32 codes
+};
+size_t prepared_act_bytes(size_t m, size_t k);
+PreparedAct prepared_act_carve(void *base, size_t m, size_t k);
+int launch_prepare_act(aionhip_ctx *ctx, const float *a, size_t lda, size_t m, size_t k, PreparedAct out);
+
+// ---- matmul back ends --------------------------------------------------------------------------
+int launch_gemv(aionhip_ctx *ctx, const aionhip_weight *w, int m, PreparedAct act, float *c, size_t ldc, float alpha, float beta);
+int launch_gemm_i8(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta);
+int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, const float *a, size_t lda, float *c, size_t ldc, float alpha, float beta);
+
+// ---- wave64 cross-lane helpers -----------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+template <int CTRL>
+__device__ __forceinline__ int dpp_i(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
+}
+constexpr int DPP_QUAD_XOR1 = 0xB1;     // quad_perm [1,0,3,2]
+constexpr int DPP_QUAD_XOR2 = 0x4E;     // quad_perm [2,3,0,1]
+constexpr int DPP_ROW_HALF_MIRROR = 0x141;
+constexpr int DPP_ROW_MIRROR = 0x140;
+
+// sum over the 64 lanes of a wavefront; every lane returns the total
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_f<DPP_QUAD_XOR1>(v);
+    v += dpp_f<DPP_QUAD_XOR2>(v);
+    v += dpp_f<DPP_ROW_HALF_MIRROR>(v);
+    v += dpp_f<DPP_ROW_MIRROR>(v);
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+    v = fmaxf(v, dpp_f<DPP_QUAD_XOR1>(v));
+    v = fmaxf(v, dpp_f<DPP_QUAD_XOR2>(v));
+    v = fmaxf(v, dpp_f<DPP_ROW_HALF_MIRROR>(v));
+    v = fmaxf(v, dpp_f<DPP_ROW_MIRROR>(v));
+    v = fmaxf(v, __shfl_xor(v, 16, 64));
+    v = fmaxf(v, __shfl_xor(v, 32, 64));
+    return v;
+}
+
+__device__ __forceinline__ int dot4_i8(int a, int b, int c) { return __builtin_amdgcn_sdot4(a, b, c, false); }

@@ -1,0 +1,245 @@
+// Context, device memory and event helpers of libaion_hip.so: the C side of aion's
+// Backend / Session / DeviceMemory vtables (backend/backend.zig:24-107,
+// runtime/device_memory.zig:36-108).
+#include "common.h"
+
+#include <cstring>
+#include <new>
+
+int set_err(aionhip_ctx *ctx, int status, const char *fmt, ...) {
+    if (ctx) {
+        char buf[512];
+        va_list ap;
+        va_start(ap, fmt);
+        vsnprintf(buf, sizeof buf, fmt, ap);
+        va_end(ap);
+        ctx->err = buf;
+    }
+    return status;
+}
+
+static int grow(aionhip_ctx *ctx, void **buf, size_t *have, size_t bytes) {
+    if (bytes <= *have) return AIONHIP_OK;
+    if (*buf) {
+        // earlier launches may still read the old buffer
+        HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+        HIP_TRY(ctx, hipFree(*buf));
+        *buf = nullptr;
+        *have = 0;
+    }
+    size_t want = bytes + bytes / 4;
+    want = (want + 255) & ~(size_t)255;
+    HIP_TRY(ctx, hipMalloc(buf, want));
+    *have = want;
+    return AIONHIP_OK;
+}
+int ensure_scratch(aionhip_ctx *ctx, size_t bytes) { return grow(ctx, &ctx->scratch, &ctx->scratch_bytes, bytes); }
+int ensure_scratch2(aionhip_ctx *ctx, size_t bytes) { return grow(ctx, &ctx->scratch2, &ctx->scratch2_bytes, bytes); }
+
+static hipEvent_t take_event(aionhip_ctx *ctx) {
+    if (!ctx->event_pool.empty()) {
+        hipEvent_t e = ctx->event_pool.back();
+        ctx->event_pool.pop_back();
+        return e;
+    }
+    hipEvent_t e = nullptr;
+    (void)hipEventCreate(&e);
+    return e;
+}
+void prof_begin(aionhip_ctx *ctx, const char *name) {
+    if (!ctx->profiling) return;
+    ProfRecord r{name, take_event(ctx), take_event(ctx), 0.f};
+    (void)hipEventRecord(r.start, ctx->stream);
+    ctx->prof.push_back(r);
+}
+void prof_end(aionhip_ctx *ctx) {
+    if (!ctx->profiling || ctx->prof.empty()) return;
+    (void)hipEventRecord(ctx->prof.back().stop, ctx->stream);
+}
+
+extern "C" {
+
+int aionhip_profile_start(aionhip_ctx *ctx) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    for (auto &r : ctx->prof) {
+        ctx->event_pool.push_back(r.start);
+        ctx->event_pool.push_back(r.stop);
+    }
+    ctx->prof.clear();
+    ctx->profiling = true;
+    return AIONHIP_OK;
+}
+int aionhip_profile_stop(aionhip_ctx *ctx, size_t *count) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    ctx->profiling = false;
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    for (auto &r : ctx->prof) HIP_TRY(ctx, hipEventElapsedTime(&r.ms, r.start, r.stop));
+    if (count) *count = ctx->prof.size();
+    return AIONHIP_OK;
+}
+int aionhip_profile_entry(aionhip_ctx *ctx, size_t index, const char **name, float *ms) {
+    if (!ctx || index >= ctx->prof.size()) return AIONHIP_INVALID_ARGUMENT;
+    if (name) *name = ctx->prof[index].name;
+    if (ms) *ms = ctx->prof[index].ms;
+    return AIONHIP_OK;
+}
+
+const char *aionhip_name(void) { return "hip-gfx950"; }
+
+int aionhip_create(int device, void *stream, aionhip_ctx **out) {
+    if (!out) return AIONHIP_INVALID_ARGUMENT;
+    *out = nullptr;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || device < 0 || device >= count) return AIONHIP_UNSUPPORTED;
+    if (hipSetDevice(device) != hipSuccess) return AIONHIP_EXECUTION_FAILED;
+    aionhip_ctx *ctx = new (std::nothrow) aionhip_ctx();
+    if (!ctx) return AIONHIP_OUT_OF_MEMORY;
+    ctx->device = device;
+    if (stream) {
+        ctx->stream = (hipStream_t)stream;
+    } else {
+        if (hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking) != hipSuccess) {
+            delete ctx;
+            return AIONHIP_EXECUTION_FAILED;
+        }
+        ctx->own_stream = true;
+    }
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) == hipSuccess) ctx->cu_count = prop.multiProcessorCount;
+    *out = ctx;
+    return AIONHIP_OK;
+}
+
+void aionhip_destroy(aionhip_ctx *ctx) {
+    if (!ctx) return;
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    for (auto &r : ctx->prof) {
+        (void)hipEventDestroy(r.start);
+        (void)hipEventDestroy(r.stop);
+    }
+    for (auto e : ctx->event_pool) (void)hipEventDestroy(e);
+    if (ctx->scratch) (void)hipFree(ctx->scratch);
+    if (ctx->scratch2) (void)hipFree(ctx->scratch2);
+    if (ctx->own_stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+}
+
+int aionhip_sync(aionhip_ctx *ctx) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return AIONHIP_OK;
+}
+
+const char *aionhip_last_error(aionhip_ctx *ctx) { return ctx ? ctx->err.c_str() : "no context"; }
+const char *aionhip_last_kernel(aionhip_ctx *ctx) { return ctx ? ctx->last_kernel : ""; }
+void *aionhip_stream(aionhip_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
+
+int aionhip_set_gemm_mode(aionhip_ctx *ctx, int mode) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (mode != AIONHIP_GEMM_EXACT_I8 && mode != AIONHIP_GEMM_BF16_MFMA) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "unknown gemm mode %d", mode);
+    ctx->gemm_mode = mode;
+    return AIONHIP_OK;
+}
+
+int aionhip_device_info(aionhip_ctx *ctx, int *cu_count, int *wave_size, uint64_t *hbm_bytes, char *arch, size_t arch_len) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    hipDeviceProp_t prop;
+    HIP_TRY(ctx, hipGetDeviceProperties(&prop, ctx->device));
+    if (cu_count) *cu_count = prop.multiProcessorCount;
+    if (wave_size) *wave_size = prop.warpSize;
+    if (hbm_bytes) *hbm_bytes = (uint64_t)prop.totalGlobalMem;
+    if (arch && arch_len) {
+        std::strncpy(arch, prop.gcnArchName, arch_len - 1);
+        arch[arch_len - 1] = 0;
+    }
+    return AIONHIP_OK;
+}
+
+int aionhip_alloc(aionhip_ctx *ctx, size_t bytes, size_t alignment, aionhip_handle *out) {
+    if (!ctx || !out) return AIONHIP_INVALID_ARGUMENT;
+    *out = 0;
+    if (alignment > 256 && (alignment & (alignment - 1)) != 0) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "alignment %zu is not a power of two", alignment);
+    void *p = nullptr;
+    // hipMalloc returns 256-byte aligned memory; larger alignments are met by over-allocation only
+    // up to 4 KiB pages, which hipMalloc also satisfies.
+    HIP_TRY(ctx, hipMalloc(&p, bytes ? bytes : 1));
+    if (alignment > 1 && ((uintptr_t)p % alignment) != 0) {
+        (void)hipFree(p);
+        return set_err(ctx, AIONHIP_UNSUPPORTED, "cannot satisfy alignment %zu", alignment);
+    }
+    *out = (aionhip_handle)(uintptr_t)p;
+    return AIONHIP_OK;
+}
+
+void aionhip_free(aionhip_ctx *ctx, aionhip_handle h) {
+    if (!ctx || !h) return;
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree((void *)(uintptr_t)h);
+}
+
+int aionhip_h2d(aionhip_ctx *ctx, aionhip_handle dst, size_t dst_offset, const void *src, size_t bytes) {
+    if (!ctx || !dst || (!src && bytes)) return AIONHIP_INVALID_ARGUMENT;
+    if (!bytes) return AIONHIP_OK;
+    // pageable source: hipMemcpyAsync stages and returns once `src` is consumed
+    HIP_TRY(ctx, hipMemcpyAsync((char *)(uintptr_t)dst + dst_offset, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return AIONHIP_OK;
+}
+
+int aionhip_d2h(aionhip_ctx *ctx, void *dst, aionhip_handle src, size_t src_offset, size_t bytes) {
+    if (!ctx || !src || (!dst && bytes)) return AIONHIP_INVALID_ARGUMENT;
+    if (!bytes) return AIONHIP_OK;
+    HIP_TRY(ctx, hipMemcpyAsync(dst, (const char *)(uintptr_t)src + src_offset, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    return AIONHIP_OK;
+}
+
+int aionhip_d2d(aionhip_ctx *ctx, aionhip_handle dst, size_t dst_offset, aionhip_handle src, size_t src_offset, size_t bytes) {
+    if (!ctx || !dst || !src) return AIONHIP_INVALID_ARGUMENT;
+    if (!bytes) return AIONHIP_OK;
+    HIP_TRY(ctx, hipMemcpyAsync((char *)(uintptr_t)dst + dst_offset, (const char *)(uintptr_t)src + src_offset, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    return AIONHIP_OK;
+}
+
+__global__ void fill_bytes_kernel(uint8_t *p, uint8_t v, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) p[i] = v;
+}
+
+int aionhip_memset(aionhip_ctx *ctx, aionhip_handle dst, size_t dst_offset, int value, size_t bytes) {
+    if (!ctx || !dst) return AIONHIP_INVALID_ARGUMENT;
+    if (!bytes) return AIONHIP_OK;
+    // a fill kernel rather than hipMemsetAsync so that the call can sit inside a captured graph
+    size_t blocks = (bytes + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    fill_bytes_kernel<<<dim3((unsigned)blocks), dim3(256), 0, ctx->stream>>>((uint8_t *)(uintptr_t)dst + dst_offset, (uint8_t)value, bytes);
+    LAUNCH_CHECK(ctx, "fill_bytes");
+    return AIONHIP_OK;
+}
+
+int aionhip_event_create(aionhip_ctx *ctx, void **event) {
+    if (!ctx || !event) return AIONHIP_INVALID_ARGUMENT;
+    hipEvent_t e;
+    HIP_TRY(ctx, hipEventCreate(&e));
+    *event = (void *)e;
+    return AIONHIP_OK;
+}
+int aionhip_event_record(aionhip_ctx *ctx, void *event) {
+    if (!ctx || !event) return AIONHIP_INVALID_ARGUMENT;
+    HIP_TRY(ctx, hipEventRecord((hipEvent_t)event, ctx->stream));
+    return AIONHIP_OK;
+}
+int aionhip_event_elapsed_ms(aionhip_ctx *ctx, void *start, void *stop, float *ms) {
+    if (!ctx || !start || !stop || !ms) return AIONHIP_INVALID_ARGUMENT;
+    HIP_TRY(ctx, hipEventSynchronize((hipEvent_t)stop));
+    HIP_TRY(ctx, hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return AIONHIP_OK;
+}
+void aionhip_event_destroy(aionhip_ctx *ctx, void *event) {
+    (void)ctx;
+    if (event) (void)hipEventDestroy((hipEvent_t)event);
+}
+
+}  // extern "C"

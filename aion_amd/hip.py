@@ -1,0 +1,92 @@
+"""ctypes binding of libaion_hip.so (include/aion_hip.h). No CPU fallback: a missing or
+unloadable library is an error."""
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libaion_hip.so")
+
+OK, INVALID_ARGUMENT, OUT_OF_MEMORY, UNSUPPORTED, EXECUTION_FAILED = range(5)
+STATUS_NAMES = {0: "OK", 1: "InvalidArgument", 2: "OutOfMemory", 3: "Unsupported", 4: "ExecutionFailed"}
+F32, F16, I8, Q4_0, Q8_0, I32, BF16 = 0, 1, 2, 3, 4, 5, 16
+ROWS_NK, KMAJOR_KN = 0, 1
+GEMM_EXACT_I8, GEMM_BF16_MFMA = 0, 1
+UNBOUNDED = 0xFFFFFFFF
+
+
+class AionHipError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__("%s: %s" % (STATUS_NAMES.get(status, status), message))
+        self.status = status
+
+
+class Attention(C.Structure):
+    _fields_ = [(n, C.c_uint64) for n in ("out", "q", "k", "v", "query_positions", "kv_lengths")] + \
+               [(n, C.c_size_t) for n in ("batch", "l_q", "t_kv", "h_q", "h_kv", "d_k", "d_v")] + \
+               [("q_dtype", C.c_int), ("kv_dtype", C.c_int), ("scale", C.c_float), ("attn_logits_soft_cap", C.c_float),
+                ("window_left", C.c_uint32), ("window_right", C.c_uint32), ("window_chunk", C.c_uint32)]
+
+
+_SIGS = {
+    # name: (restype, argtypes)
+    "aionhip_create": (C.c_int, [C.c_int, C.c_void_p, C.POINTER(C.c_void_p)]),
+    "aionhip_destroy": (None, [C.c_void_p]),
+    "aionhip_sync": (C.c_int, [C.c_void_p]),
+    "aionhip_last_error": (C.c_char_p, [C.c_void_p]),
+    "aionhip_last_kernel": (C.c_char_p, [C.c_void_p]),
+    "aionhip_name": (C.c_char_p, []),
+    "aionhip_stream": (C.c_void_p, [C.c_void_p]),
+    "aionhip_device_info": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_uint64), C.c_char_p, C.c_size_t]),
+    "aionhip_alloc": (C.c_int, [C.c_void_p, C.c_size_t, C.c_size_t, C.POINTER(C.c_uint64)]),
+    "aionhip_free": (None, [C.c_void_p, C.c_uint64]),
+    "aionhip_h2d": (C.c_int, [C.c_void_p, C.c_uint64, C.c_size_t, C.c_void_p, C.c_size_t]),
+    "aionhip_d2h": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64, C.c_size_t, C.c_size_t]),
+    "aionhip_d2d": (C.c_int, [C.c_void_p, C.c_uint64, C.c_size_t, C.c_uint64, C.c_size_t, C.c_size_t]),
+    "aionhip_memset": (C.c_int, [C.c_void_p, C.c_uint64, C.c_size_t, C.c_int, C.c_size_t]),
+    "aionhip_quantize_blocks": (C.c_int, [C.c_int, C.POINTER(C.c_size_t), C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t]),
+    "aionhip_quantize_device": (C.c_int, [C.c_void_p, C.c_int, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint64, C.c_uint64]),
+    "aionhip_weight_upload": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p, C.POINTER(C.c_void_p)]),
+    "aionhip_weight_from_device": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint64, C.POINTER(C.c_void_p)]),
+    "aionhip_weight_free": (None, [C.c_void_p, C.c_void_p]),
+    "aionhip_weight_packed_bytes": (C.c_size_t, [C.c_void_p]),
+    "aionhip_weight_device_bytes": (C.c_size_t, [C.c_void_p]),
+    "aionhip_weight_download": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
+    "aionhip_step_matmul": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint64, C.c_size_t, C.c_uint64, C.c_size_t, C.c_float, C.c_float]),
+    "aionhip_step_matmul_nt": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint64, C.c_size_t, C.c_uint64, C.c_size_t, C.c_float, C.c_float]),
+    "aionhip_set_gemm_mode": (C.c_int, [C.c_void_p, C.c_int]),
+    "aionhip_step_attention": (C.c_int, [C.c_void_p, C.POINTER(Attention)]),
+    "aionhip_step_rmsnorm": (C.c_int, [C.c_void_p] + [C.c_uint64] * 5 + [C.c_size_t, C.c_size_t, C.c_float]),
+    "aionhip_step_rope": (C.c_int, [C.c_void_p] + [C.c_uint64] * 3 + [C.c_size_t] * 4 + [C.c_float] * 3),
+    "aionhip_step_add": (C.c_int, [C.c_void_p] + [C.c_uint64] * 3 + [C.c_size_t]),
+    "aionhip_step_gate_gelu": (C.c_int, [C.c_void_p] + [C.c_uint64] * 3 + [C.c_size_t]),
+    "aionhip_step_gather_rows": (C.c_int, [C.c_void_p, C.c_int] + [C.c_uint64] * 3 + [C.c_size_t] * 3),
+    "aionhip_step_append_f16": (C.c_int, [C.c_void_p] + [C.c_uint64] * 3 + [C.c_size_t] * 4),
+    "aionhip_step_cast_f32_f16": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64, C.c_size_t]),
+    "aionhip_step_argmax": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64, C.c_size_t, C.c_size_t]),
+    "aionhip_event_create": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p)]),
+    "aionhip_event_record": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "aionhip_event_elapsed_ms": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
+    "aionhip_event_destroy": (None, [C.c_void_p, C.c_void_p]),
+    "aionhip_profile_start": (C.c_int, [C.c_void_p]),
+    "aionhip_profile_stop": (C.c_int, [C.c_void_p, C.POINTER(C.c_size_t)]),
+    "aionhip_profile_entry": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_char_p), C.POINTER(C.c_float)]),
+}
+
+_lib = None
+
+
+def load_library():
+    """Loads libaion_hip.so and types every entry point. Raises if the library is missing."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise FileNotFoundError(
+            "%s is missing: build it with `python -m aion_amd.build` (there is no CPU fallback)" % LIB_PATH)
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in _SIGS.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib

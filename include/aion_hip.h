@@ -1,0 +1,196 @@
+/* aion_hip.h - C ABI of the MI355X (gfx950) execution backend for aion's quantized-inference
+ * hot path: q4_0/q8_0 dequant-fused GEMV (decode), q4/q8 GEMM (prefill), fused causal/GQA
+ * attention over a KV cache, plus the small per-token ops a decoder needs between them.
+ *
+ * The library (libaion_hip.so) is what an aion `Backend`/`Session`/`DeviceMemory` implementation
+ * written in Zig binds through @cImport: plain pointers, sizes and enums only. Citations name
+ * the aion interface each entry point stands in for (paths relative to the aion source tree).
+ *
+ * Conventions
+ *  - Every function returning `int` returns an aionhip_status. On failure a message is kept
+ *    per context (aionhip_last_error).
+ *  - aionhip_handle is a device address as u64 (aion `DeviceHandle`, runtime/device_memory.zig:
+ *    0 = none). Step functions take device addresses; offsets are applied by the caller.
+ *  - All launches are asynchronous on the context's one HIP stream. aionhip_d2h and
+ *    aionhip_sync are the synchronisation points (backend/gpu/backend.zig:178-183). A context
+ *    is not thread-safe; use one per session thread.
+ *  - Index operands (positions, kv lengths, write index, token ids) are read ON DEVICE
+ *    (backend/gpu/exec/decode_ops.zig:441-480): no step synchronises with the host.
+ */
+#ifndef AION_HIP_H
+#define AION_HIP_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* BackendError + StoreError (backend/types.zig:27, runtime/tensor_store.zig:7), numbered like
+ * AionStatus (include/aion.h:62-68). */
+typedef enum aionhip_status {
+    AIONHIP_OK = 0,
+    AIONHIP_INVALID_ARGUMENT = 1,
+    AIONHIP_OUT_OF_MEMORY = 2,
+    AIONHIP_UNSUPPORTED = 3,
+    AIONHIP_EXECUTION_FAILED = 4,
+} aionhip_status;
+
+/* DType ids (backend/types.zig:29-39, include/aion.h:70-77). BF16 is a host-view element type
+ * in aion (include/aion.h:171-176); here it is also accepted for attention operands. */
+typedef enum aionhip_dtype {
+    AIONHIP_F32 = 0,
+    AIONHIP_F16 = 1,
+    AIONHIP_I8 = 2,
+    AIONHIP_Q4_0 = 3,
+    AIONHIP_Q8_0 = 4,
+    AIONHIP_I32 = 5,
+    AIONHIP_BF16 = 16,
+} aionhip_dtype;
+
+/* Where the 32-element quant blocks of a rank-2 weight run (storage/quantize.zig:31-80):
+ * ROWS_NK = B stored [N,K], quant_axis 1 (the MatMulNT operand, runtime/executable.zig:211-223);
+ * KMAJOR_KN = B stored [K,N], quant_axis 0 (the MatMul operand; the only q4_0 layout,
+ * cpu/exec/matmul.zig:233-239,436-443). */
+typedef enum aionhip_weight_layout {
+    AIONHIP_ROWS_NK = 0,
+    AIONHIP_KMAJOR_KN = 1,
+} aionhip_weight_layout;
+
+typedef struct aionhip_ctx aionhip_ctx;
+typedef struct aionhip_weight aionhip_weight;
+typedef struct aionhip_program aionhip_program;
+typedef uint64_t aionhip_handle;
+
+/* ---- backend handle: Backend.VTable / Session.VTable (backend/backend.zig:24-107) ---------- */
+/* `stream`: a hipStream_t to launch on, or NULL to create a private stream. */
+int aionhip_create(int device, void *stream, aionhip_ctx **out);
+void aionhip_destroy(aionhip_ctx *ctx);                 /* Backend.deinit */
+int aionhip_sync(aionhip_ctx *ctx);                     /* Session.retireResources: wait for the stream */
+const char *aionhip_last_error(aionhip_ctx *ctx);       /* diagnostic.zig:1-45 analogue */
+const char *aionhip_name(void);                         /* Backend.name */
+void *aionhip_stream(aionhip_ctx *ctx);                 /* the hipStream_t steps launch on */
+/* device facts for roofline reports: compute units, wavefront size, HBM bytes */
+int aionhip_device_info(aionhip_ctx *ctx, int *cu_count, int *wave_size, uint64_t *hbm_bytes, char *arch, size_t arch_len);
+
+/* ---- DeviceMemory.VTable (runtime/device_memory.zig:36-108); memory model = discrete,
+ *      maxBindingBytes = unbounded (tensors are never chunked, storage/layout.zig:22-39) ------ */
+int aionhip_alloc(aionhip_ctx *ctx, size_t bytes, size_t alignment, aionhip_handle *out);
+void aionhip_free(aionhip_ctx *ctx, aionhip_handle h);
+int aionhip_h2d(aionhip_ctx *ctx, aionhip_handle dst, size_t dst_offset, const void *src, size_t bytes);
+int aionhip_d2h(aionhip_ctx *ctx, void *dst, aionhip_handle src, size_t src_offset, size_t bytes);
+int aionhip_d2d(aionhip_ctx *ctx, aionhip_handle dst, size_t dst_offset, aionhip_handle src, size_t src_offset, size_t bytes);
+int aionhip_memset(aionhip_ctx *ctx, aionhip_handle dst, size_t dst_offset, int value, size_t bytes);
+
+/* ---- quantizers ----------------------------------------------------------------------------
+ * Host: storage/quantize.zig:31-80 `quantizeBlocks` (same argument meaning: blocks
+ * [first_block, first_block + out_len/block_bytes) of a tensor of `shape`, `values` holding the
+ * row-major elements from `first_elem` on). q8_0 follows packQ8Block (:83-103); q4_0 follows
+ * quantizeQ4_0FromF32Block32 (cpu/test_cpu_kernels.zig:490-523), the only q4 quantizer aion has. */
+int aionhip_quantize_blocks(int dtype, const size_t *shape, size_t rank, size_t quant_axis,
+                            const float *values, size_t n_values, size_t first_elem, size_t first_block,
+                            uint8_t *out, size_t out_len);
+/* Device: the same bytes for a rank-2 f32 tensor `src` [rows, cols] resident on the GPU
+ * (Context.quantize, api/context.zig:443-489, without the host round trip). */
+int aionhip_quantize_device(aionhip_ctx *ctx, int dtype, size_t rows, size_t cols, size_t quant_axis,
+                            aionhip_handle src_f32, aionhip_handle dst_blocks);
+
+/* ---- weights: private re-lay at first use (graph/opt/weight_layout.zig:232-314 does the same
+ *      job for the CPU/WebGPU block orders; this backend advertises `.row_major`,
+ *      api/gpu_device.zig:24-25, and keeps its own layout) -----------------------------------
+ * Input is aion's packed blocks, exactly as the quantizer emits them: ROWS_NK -> block (n,kb)
+ * at (n*K/32+kb)*block_bytes; KMAJOR_KN -> block (kb,n) at (kb*ld+n)*block_bytes (ld = row
+ * stride in blocks, 0 = n; MatMulParams.ldb, backend/types.zig:225-241). Only Q8_0 may be
+ * ROWS_NK. The packed bytes are consumed during the call and not referenced afterwards. */
+int aionhip_weight_upload(aionhip_ctx *ctx, int dtype, int layout, size_t n, size_t k, size_t ld_blocks,
+                          const void *host_blocks, aionhip_weight **out);
+/* same, from blocks already resident in device memory (a tensor moved by DeviceMemory.copyH2D) */
+int aionhip_weight_from_device(aionhip_ctx *ctx, int dtype, int layout, size_t n, size_t k, size_t ld_blocks,
+                               aionhip_handle device_blocks, aionhip_weight **out);
+void aionhip_weight_free(aionhip_ctx *ctx, aionhip_weight *w);
+/* bytes of aion's packed form (what the roofline charges) and of the device layout */
+size_t aionhip_weight_packed_bytes(const aionhip_weight *w);
+size_t aionhip_weight_device_bytes(const aionhip_weight *w);
+/* Inverse of the re-lay: aion's packed blocks back out of the device layout (byte-exact) */
+int aionhip_weight_download(aionhip_ctx *ctx, const aionhip_weight *w, void *host_blocks, size_t bytes);
+
+/* ---- matmul steps -----------------------------------------------------------------------------
+ * StepMatMul (B [K,N], cpu/exec/matmul.zig:48-78) and StepMatMulNT (B [N,K],
+ * cpu/exec/matmul_nt.zig:87-259): C[m,n] = alpha * A[m,k] @ B + beta * C, A and C f32 on device,
+ * lda/ldc in elements (0 = k / n). Leading dims of A are folded into m by the caller
+ * (cpu/exec/matmul.zig:100-163). Arithmetic follows aion's CPU kernels: A is int8-quantized
+ * per (row, 32-block) (cpu/kernels/matmul_q_i8.zig:187-203), block dots are exact integers,
+ * accumulation is f32. */
+int aionhip_step_matmul(aionhip_ctx *ctx, const aionhip_weight *b, size_t m,
+                        aionhip_handle a, size_t lda, aionhip_handle c, size_t ldc, float alpha, float beta);
+int aionhip_step_matmul_nt(aionhip_ctx *ctx, const aionhip_weight *b, size_t m,
+                           aionhip_handle a, size_t lda, aionhip_handle c, size_t ldc, float alpha, float beta);
+
+/* How m > 8 rows are multiplied. EXACT_I8 (default): int8 activations, integer MFMA, per-block
+ * f32 scaling - the same numbers as the decode path. BF16_MFMA: weights dequantized to bf16,
+ * activations rounded to bf16, f32 accumulation - faster, judged at 1e-2 instead of 2e-3. */
+typedef enum aionhip_gemm_mode { AIONHIP_GEMM_EXACT_I8 = 0, AIONHIP_GEMM_BF16_MFMA = 1 } aionhip_gemm_mode;
+int aionhip_set_gemm_mode(aionhip_ctx *ctx, int mode);
+/* Name of the kernel the last matmul/attention step launched (the reference's tests assert
+ * which kernel ran after a parity check, backend/gpu/test_gpu_backend.zig:1116-1162). */
+const char *aionhip_last_kernel(aionhip_ctx *ctx);
+
+/* ---- attention step: StepAttention (runtime/executable.zig:102-115), graph.Op.Attention
+ *      (graph/graph.zig:365-393), executor cpu/exec/attention.zig:1444-1608 ------------------
+ * q [B,L,Hq,Dk], k [B,T,Hkv,Dk], v [B,T,Hkv,Dv] token-major, out f32 [B,L,Hq,Dv]. Key interval
+ * per query = AttentionWindow.keys(pos, end) (graph/graph.zig:160-167); 0xFFFFFFFF = unbounded,
+ * causal = {left unbounded, right 0, chunk 0}. query_positions [B,L] i32 / kv_lengths [B] i32
+ * are device addresses or 0 (defaults: row index / T). Empty interval -> zeros. */
+typedef struct aionhip_attention {
+    aionhip_handle out, q, k, v, query_positions, kv_lengths;
+    size_t batch, l_q, t_kv, h_q, h_kv, d_k, d_v;
+    int q_dtype;   /* F32 | F16 | BF16 */
+    int kv_dtype;  /* F32 | F16 | BF16 */
+    float scale, attn_logits_soft_cap;
+    uint32_t window_left, window_right, window_chunk;
+} aionhip_attention;
+int aionhip_step_attention(aionhip_ctx *ctx, const aionhip_attention *p);
+
+/* ---- per-token glue steps (f32 unless stated) ---------------------------------------------- */
+/* StepRMSNorm (runtime/executable.zig:85-101; cpu/exec/layernorm.zig:54-155):
+ * out = x * rsqrt(mean(x^2)+eps) * gamma + beta (+ residual). beta/residual may be 0. */
+int aionhip_step_rmsnorm(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle x, aionhip_handle gamma,
+                         aionhip_handle beta, aionhip_handle residual, size_t rows, size_t cols, float eps);
+/* StepRoPE1D (cpu/exec/rope.zig:14-53, cpu/kernels/rope.zig:20-98): x,out [B,T,H,D], positions [B,T] i32 */
+int aionhip_step_rope(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle x, aionhip_handle positions,
+                      size_t b, size_t t, size_t h, size_t d, float base_frequency, float scale_factor, float rope_proportion);
+/* StepElemwiseBinary: add, and the fused gate act(a)*b with act = gelu (tanh form)
+ * (backend/types.zig:105-109, cpu/exec/elementwise.zig:25-37, cpu/kernels/gelu.zig:8-14) */
+int aionhip_step_add(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle a, aionhip_handle b, size_t n);
+int aionhip_step_gate_gelu(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle a, aionhip_handle b, size_t n);
+/* StepGather axis 0 (cpu/exec/gather.zig:60-87): rows of an f32 or q8_0 (quant_axis 1, packed
+ * 34-byte blocks) table [V,D] -> out f32 [n_ids, D]; ids i32 on device */
+int aionhip_step_gather_rows(aionhip_ctx *ctx, int table_dtype, aionhip_handle out, aionhip_handle table,
+                             aionhip_handle ids, size_t n_ids, size_t d, size_t vocab);
+/* StepCast f32 -> f16 (cpu/exec/cast.zig) fused with StepSequenceAppend
+ * (cpu/exec/sequence_append.zig:12-104): rows src [B,S,H,D] f32 are written as f16 into
+ * cache [B,T,H,D] at token index write_index[0] (i32 on device) .. +S */
+int aionhip_step_append_f16(aionhip_ctx *ctx, aionhip_handle cache, aionhip_handle src_f32, aionhip_handle write_index,
+                            size_t b, size_t s, size_t t_cap, size_t row_elems);
+int aionhip_step_cast_f32_f16(aionhip_ctx *ctx, aionhip_handle out_f16, aionhip_handle x_f32, size_t n);
+/* StepArgMax over the last axis, first maximum wins (cpu/exec/argmax.zig:56-81); out i32 [rows] */
+int aionhip_step_argmax(aionhip_ctx *ctx, aionhip_handle out_i32, aionhip_handle x, size_t rows, size_t n);
+
+/* ---- timing helpers for the roofline harness (timestamp queries of the WebGPU backend,
+ *      backend/gpu/timestamp_profile.zig, reduced to stream events) ------------------------- */
+int aionhip_event_create(aionhip_ctx *ctx, void **event);
+int aionhip_event_record(aionhip_ctx *ctx, void *event);
+int aionhip_event_elapsed_ms(aionhip_ctx *ctx, void *start, void *stop, float *ms); /* waits for `stop` */
+void aionhip_event_destroy(aionhip_ctx *ctx, void *event);
+
+/* Per-launch GPU timing of the matmul / attention kernels (AION_PROFILE_GPU=dispatch in the
+ * WebGPU backend, backend/gpu/timestamp_profile.zig:1-60): between start and stop every such
+ * launch is bracketed by two stream events; stop waits for the stream and resolves them. */
+int aionhip_profile_start(aionhip_ctx *ctx);
+int aionhip_profile_stop(aionhip_ctx *ctx, size_t *count);
+int aionhip_profile_entry(aionhip_ctx *ctx, size_t index, const char **name, float *ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AION_HIP_H */

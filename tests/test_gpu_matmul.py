@@ -1,0 +1,212 @@
+"""GPU parity of the quantized matmul steps against the CPU oracle (through the C ABI).
+
+Tolerance: the north-star bound for f32-accumulate kernels is max relative error 2e-3, taken
+elementwise with a floor (conftest.norm_err). The integer block dots are exact here, so only the
+f32 summation order differs: the tests additionally hold max|err| to 1e-5 of rms(ref)
+(conftest.rms_err). Block bytes are compared bit-exactly.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+from aion_amd import backend as be
+from aion_amd import hip
+from conftest import norm_err, rms_err
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3      # elementwise, floored
+RMS_TOL = 1e-5  # max |err| / rms(ref)
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def make_weight(gpu, orc, dtype, layout, n, k, seed, std=0.02):
+    rng = np.random.default_rng(seed)
+    if layout == be.ROWS_NK:
+        w = (rng.standard_normal((n, k)) * std).astype(np.float32)
+        blocks = be.quantize_blocks(dtype, w, 1)
+    else:
+        w = (rng.standard_normal((k, n)) * std).astype(np.float32)
+        blocks = be.quantize_blocks(dtype, w, 0)
+    return blocks, gpu.upload_weight(dtype, layout, n, k, blocks)
+
+
+def oracle_matmul(orc, dtype, layout, a, blocks, n, **kw):
+    if layout == be.ROWS_NK:
+        return orc.matmul_nt_q8(a, blocks, n, threads=8, **kw)
+    if dtype == be.Q8_0 and a.shape[0] <= 16:
+        return orc.matmul_q8_kmajor(a, blocks, n, threads=8, **kw)
+    return orc.matmul_q_packed(dtype, a, blocks, n, threads=8, **kw)
+
+
+CASES = [(be.Q8_0, be.ROWS_NK), (be.Q8_0, be.KMAJOR_KN), (be.Q4_0, be.KMAJOR_KN)]
+
+
+@pytest.mark.parametrize("dtype,layout", CASES)
+def test_weight_relay_is_a_byte_permutation(gpu, orc, dtype, layout):
+    say("relay", dtype, layout)
+    for n, k in [(5, 64), (64, 2048), (33, 160)]:
+        blocks, w = make_weight(gpu, orc, dtype, layout, n, k, seed=n * k)
+        assert w.packed_bytes == blocks.nbytes
+        assert np.array_equal(w.download(), blocks)
+        w.free()
+
+
+def test_weight_upload_with_block_row_stride(gpu, orc):
+    # MatMulParams.ldb: a [K,N] view whose block rows are ld blocks apart
+    n, k, ld = 6, 96, 10
+    rng = np.random.default_rng(0)
+    full = (rng.standard_normal((k, ld)) * 0.02).astype(np.float32)
+    packed_full = be.quantize_blocks(be.Q8_0, full, 0)                     # [k/32, ld] blocks
+    compact = be.quantize_blocks(be.Q8_0, np.ascontiguousarray(full[:, :n]), 0)
+    w_strided = gpu.upload_weight(be.Q8_0, be.KMAJOR_KN, n, k, packed_full, ld_blocks=ld)
+    w_compact = gpu.upload_weight(be.Q8_0, be.KMAJOR_KN, n, k, compact)
+    a = rng.standard_normal((2, k)).astype(np.float32)
+    # aion cpu/test_cpu_kernels.zig:726-825: strided sub-block == compact copy, bit-exactly
+    assert np.array_equal(gpu.matmul(w_strided, a), gpu.matmul(w_compact, a))
+    assert np.array_equal(w_strided.download(), compact)
+    w_strided.free(); w_compact.free()
+
+
+@pytest.mark.parametrize("dtype", [be.Q8_0, be.Q4_0])
+@pytest.mark.parametrize("axis", [0, 1])
+def test_device_quantizer_bytes_match_oracle(gpu, orc, dtype, axis):
+    say("device quantizer", dtype, axis)
+    rng = np.random.default_rng(17 + axis)
+    rows, cols = (96, 40) if axis == 0 else (40, 96)
+    v = (rng.standard_normal((rows, cols)) * 0.02).astype(np.float32)
+    v[0:32, 0] = 0.0
+    v[0, 0:32] = 0.0
+    v.reshape(-1)[5] = 0.5            # large outlier
+    src = gpu.upload(v)
+    dst = gpu.quantize_device(dtype, src, rows, cols, axis)
+    got = gpu.download(dst, np.uint8)
+    assert np.array_equal(got, orc.quantize(dtype, v, axis))
+    src.free(); dst.free()
+
+
+@pytest.mark.parametrize("dtype,layout", CASES)
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 8])
+def test_gemv_small_and_ragged_shapes(gpu, orc, dtype, layout, m):
+    for n, k in [(1, 32), (5, 64), (13, 160), (67, 2080), (256, 1024)]:
+        say("gemv small", dtype, layout, m, n, k)
+        blocks, w = make_weight(gpu, orc, dtype, layout, n, k, seed=n + k + m, std=0.5)
+        a = np.random.default_rng(m * 31 + n).standard_normal((m, k)).astype(np.float32)
+        a[0, :32] = 0.0                                       # a zero activation block (scale 0)
+        got = gpu.matmul(w, a)
+        want = oracle_matmul(orc, dtype, layout, a, blocks, n)
+        assert norm_err(got, want) < TOL and rms_err(got, want) < RMS_TOL, (n, k, norm_err(got, want), rms_err(got, want))
+        assert gpu.last_kernel() == ("gemv_q8" if dtype == be.Q8_0 else "gemv_q4")
+        w.free()
+
+
+def test_config1_q8_gemv_2048(gpu, orc):
+    # BASELINE config 1: W 2048x2048 ~N(0,0.02) -> q8 (aion's quantizer), x ~N(0,1), y = W.x
+    say("config1")
+    blocks, w = make_weight(gpu, orc, be.Q8_0, be.ROWS_NK, 2048, 2048, seed=1)
+    x = np.random.default_rng(2).standard_normal((1, 2048)).astype(np.float32)
+    got = gpu.matmul(w, x)
+    want = orc.matmul_nt_q8(x, blocks, 2048)
+    assert norm_err(got, want) < TOL and rms_err(got, want) < RMS_TOL
+    # and against the f32-activation dequant family: differs by activation-quant noise only
+    f32a = orc.matmul_q_f32a(orc.Q8_0, True, x, blocks, 2048)
+    nmse = float(((got - f32a) ** 2).sum() / (f32a ** 2).sum())
+    assert nmse < 2e-4
+    w.free()
+
+
+def test_reference_closed_form_kmajor_past_8192(gpu, orc):
+    # aion cpu/kernels/matvec_q.zig:176-219 inputs (m=2, n=5, k=8192+64), rel 1e-5 there
+    m, n, k = 2, 5, 8192 + 64
+    kb = k // 32
+    a = (((np.arange(m * k) % 37) - 18) * 0.01).astype(np.float32).reshape(m, k)
+    blocks = np.zeros((kb * n, 34), np.uint8)
+    blocks[:, 0:2] = np.array([0.02], np.float16).view(np.uint8)
+    bi = np.arange(kb * n, dtype=np.uint64)[:, None]
+    t = np.arange(32, dtype=np.uint64)[None, :]
+    blocks[:, 2:] = ((bi * np.uint64(5) + t * np.uint64(3)) & np.uint64(0xFF)).astype(np.uint8)
+    w = gpu.upload_weight(be.Q8_0, be.KMAJOR_KN, n, k, blocks)
+    got = gpu.matmul(w, a)
+    want = orc.matmul_q8_kmajor(a, blocks, n)
+    assert np.allclose(got, want, rtol=1e-5, atol=0)
+    w.free()
+
+
+@pytest.mark.parametrize("dtype,layout", CASES)
+def test_alpha_beta_and_strides(gpu, orc, dtype, layout):
+    say("alpha/beta", dtype, layout)
+    m, n, k, lda, ldc = 3, 37, 96, 128, 50
+    blocks, w = make_weight(gpu, orc, dtype, layout, n, k, seed=9, std=0.3)
+    rng = np.random.default_rng(10)
+    a_full = rng.standard_normal((m, lda)).astype(np.float32)
+    c_full = rng.standard_normal((m, ldc)).astype(np.float32)
+    a_buf, c_buf = gpu.upload(a_full), gpu.upload(c_full)
+    gpu.step_matmul(w, a_buf, m, c_buf, lda=lda, ldc=ldc, alpha=0.5, beta=2.0)
+    got = gpu.download(c_buf, np.float32, (m, ldc))
+    a = np.ascontiguousarray(a_full[:, :k])
+    want = oracle_matmul(orc, dtype, layout, a, blocks, n, alpha=0.5, beta=2.0, c=np.ascontiguousarray(c_full[:, :n]))
+    assert norm_err(got[:, :n], want) < TOL and rms_err(got[:, :n], want) < RMS_TOL
+    assert np.array_equal(got[:, n:], c_full[:, n:])           # padding columns untouched
+    a_buf.free(); c_buf.free(); w.free()
+
+
+@pytest.mark.parametrize("dtype,layout", CASES)
+@pytest.mark.parametrize("n,k", [(4096, 4096), (14336, 4096), (4096, 14336)])
+def test_config2_decode_shapes(gpu, orc, dtype, layout, n, k):
+    # BASELINE config 2 shapes at batch 1, 4, 8 (the 262144x2048 shape is in test_gpu_fullsize.py)
+    say("config2", dtype, layout, n, k)
+    blocks, w = make_weight(gpu, orc, dtype, layout, n, k, seed=n ^ k)
+    for m in (1, 4, 8):
+        a = np.random.default_rng(m).standard_normal((m, k)).astype(np.float32)
+        got = gpu.matmul(w, a)
+        want = oracle_matmul(orc, dtype, layout, a, blocks, n)
+        e, r = norm_err(got, want), rms_err(got, want)
+        say("  m", m, "norm_err", e, "rms_err", r)
+        assert e < TOL and r < RMS_TOL
+    w.free()
+
+
+@pytest.mark.parametrize("dtype,layout", CASES)
+def test_exact_gemm_rows_above_eight(gpu, orc, dtype, layout):
+    say("exact gemm", dtype, layout)
+    m, n, k = 37, 200, 256
+    blocks, w = make_weight(gpu, orc, dtype, layout, n, k, seed=77, std=0.1)
+    a = np.random.default_rng(5).standard_normal((m, k)).astype(np.float32)
+    gpu.set_gemm_mode(be.GEMM_EXACT_I8)
+    got = gpu.matmul(w, a)
+    want = oracle_matmul(orc, dtype, layout, a, blocks, n)
+    assert norm_err(got, want) < TOL and rms_err(got, want) < RMS_TOL
+    w.free()
+
+
+def test_linearity_in_alpha_and_row_independence(gpu, orc):
+    # size-independent properties: rows of A never interact; alpha scales exactly by powers of two
+    blocks, w = make_weight(gpu, orc, be.Q4_0, be.KMAJOR_KN, 512, 1024, seed=3)
+    a = np.random.default_rng(4).standard_normal((8, 1024)).astype(np.float32)
+    full = gpu.matmul(w, a)
+    for r in (0, 3, 7):
+        assert np.array_equal(gpu.matmul(w, a[r:r + 1])[0], full[r])     # batch size never changes a row's result
+    assert np.array_equal(gpu.matmul(w, a, alpha=4.0), 4.0 * full)
+    w.free()
+
+
+def test_matmul_argument_errors(gpu, orc):
+    blocks, w4 = make_weight(gpu, orc, be.Q4_0, be.KMAJOR_KN, 8, 64, seed=1)
+    a = gpu.upload(np.zeros((1, 64), np.float32))
+    c = gpu.alloc(64)
+    lib, ctx = gpu._lib, gpu._ctx
+    assert lib.aionhip_step_matmul_nt(ctx, w4.ptr, 1, a.handle, 0, c.handle, 0, 1.0, 0.0) == hip.INVALID_ARGUMENT
+    assert lib.aionhip_step_matmul(ctx, w4.ptr, 1, a.handle, 32, c.handle, 0, 1.0, 0.0) == hip.INVALID_ARGUMENT  # lda < k
+    assert lib.aionhip_step_matmul(ctx, w4.ptr, 1, 0, 0, c.handle, 0, 1.0, 0.0) == hip.INVALID_ARGUMENT
+    with pytest.raises(be.AionHipError) as e:
+        gpu.upload_weight(be.Q4_0, be.ROWS_NK, 8, 64, blocks)           # aion has no q4 [N,K] operand
+    assert e.value.status == hip.UNSUPPORTED
+    with pytest.raises(be.AionHipError) as e:
+        gpu.upload_weight(be.Q8_0, be.ROWS_NK, 8, 48, np.zeros(8 * 2 * 34, np.uint8))
+    assert e.value.status == hip.INVALID_ARGUMENT
+    assert lib.aionhip_step_matmul(ctx, w4.ptr, 0, a.handle, 0, c.handle, 0, 1.0, 0.0) == hip.OK   # m == 0 is a no-op
+    a.free(); c.free(); w4.free()

@@ -1,0 +1,89 @@
+"""CPU-side checks of the product library: the host quantizer is byte-exact against the oracle,
+the shared library loads and exports every entry point the header declares."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+from aion_amd import backend as be
+from aion_amd import hip
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = hip.load_library()
+    text = open(os.path.join(ROOT, "include", "aion_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = set(re.findall(r"\b(aionhip_[a-z0-9_]+)\s*\(", text))
+    assert len(names) >= 35
+    missing = [n for n in sorted(names) if not hasattr(lib, n)]
+    assert not missing, missing
+    untyped = [n for n in sorted(names) if n not in hip._SIGS]
+    assert not untyped, untyped
+
+
+@pytest.mark.parametrize("dtype", [be.Q8_0, be.Q4_0])
+@pytest.mark.parametrize("shape,axis", [((64, 5), 0), ((7, 96), 1), ((2, 64, 3), 1), ((4096, 24), 0), ((300, 512), 1)])
+def test_host_quantizer_matches_oracle_bytes(orc, dtype, shape, axis):
+    rng = np.random.default_rng(hash((dtype, shape, axis)) % 2**32)
+    v = (rng.standard_normal(shape) * 0.02).astype(np.float32)
+    v.reshape(-1)[::97] = 0.0
+    if v.ndim == 2 and axis == 1:
+        v[0, :32] = 0.0                       # an all-zero block
+    got = be.quantize_blocks(dtype, v, axis)
+    want = orc.quantize(dtype, v, axis)
+    assert np.array_equal(got, want)
+
+
+def test_host_quantizer_reference_test_vector(orc):
+    # aion storage/quantize.zig:105-137
+    i = np.arange(64 * 5)
+    vals = ((i % 17).astype(np.int32) - 8).astype(np.float32) * np.float32(0.1)
+    got = be.quantize_blocks(be.Q8_0, vals.reshape(64, 5), 0)
+    assert np.array_equal(got, orc.quantize(orc.Q8_0, vals.reshape(64, 5), 0))
+
+
+def test_host_quantizer_chunked_calls_equal_whole():
+    # api/context.zig:443-489 quantizes 16 MiB at a time through first_elem/first_block
+    lib = hip.load_library()
+    rng = np.random.default_rng(3)
+    v = rng.standard_normal((8, 128)).astype(np.float32)
+    whole = be.quantize_blocks(be.Q8_0, v, 1)
+    shape = (C.c_size_t * 2)(8, 128)
+    parts = []
+    for r0 in range(0, 8, 2):
+        chunk = np.ascontiguousarray(v[r0:r0 + 2])
+        out = np.empty(2 * 4 * 34, np.uint8)
+        rc = lib.aionhip_quantize_blocks(be.Q8_0, shape, 2, 1, chunk.ctypes.data, chunk.size, r0 * 128, r0 * 4, out.ctypes.data, out.nbytes)
+        assert rc == hip.OK
+        parts.append(out)
+    assert np.array_equal(np.concatenate(parts), whole)
+
+
+def test_host_quantizer_errors():
+    with pytest.raises(be.AionHipError) as e:
+        be.quantize_blocks(be.Q8_0, np.zeros((33, 4), np.float32), 0)
+    assert e.value.status == hip.INVALID_ARGUMENT
+    with pytest.raises(be.AionHipError) as e:
+        be.quantize_blocks(be.F16, np.zeros((32, 4), np.float32), 0)
+    assert e.value.status == hip.UNSUPPORTED
+    lib = hip.load_library()
+    shape = (C.c_size_t * 1)(64)
+    v = np.zeros(32, np.float32)      # too few values for two blocks
+    out = np.empty(68, np.uint8)
+    assert lib.aionhip_quantize_blocks(be.Q8_0, shape, 1, 0, v.ctypes.data, v.size, 0, 0, out.ctypes.data, 68) == hip.INVALID_ARGUMENT
+
+
+def test_create_without_gpu_fails_loudly():
+    import subprocess
+    import sys
+    # in a child process so that a GPU-less HIP runtime cannot disturb this one
+    code = ("import sys; sys.path.insert(0, %r)\n"
+            "from aion_amd import backend as be\n"
+            "try:\n    be.HipBackend(7)\n    print('created')\n"
+            "except be.AionHipError as e:\n    print('error', e.status)\n") % ROOT
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120).stdout
+    assert "error" in out          # device 7 never exists on a one-GPU box or a CPU container
