@@ -1,7 +1,496 @@
-// Attention step (placeholder until the kernels land): rejects every call loudly.
+// Attention step: grouped-query attention over token-major K/V with an interval window per query
+// (aion graph/graph.zig:130-181,365-393; CPU executor cpu/exec/attention.zig:627-815,1347-1442).
+//
+// attn_flash_kernel - d_k = d_v in {64,128,256}, K/V f16 or bf16. Flash-style online softmax with
+//   MFMA for both products, written in the transposed form so that no cross-lane shuffle of the
+//   probabilities is needed:
+//       S^T[keys x rows] = K_tile[keys x d] . Q^T[d x rows]          (A = K rows straight from HBM)
+//       O^T[dv x rows]  += V_tile^T[dv x keys] . P^T[keys x rows]    (A = V^T gathered through LDS)
+//   A wavefront owns 16 query rows (row = position-major, GQA head fastest, all sharing one K/V
+//   head); each lane's accumulators, running max and sum belong to ONE query row, so the softmax
+//   bookkeeping is per-lane scalar work. Two launch shapes:
+//     split mode (few query rows: decode) - a workgroup is one 16-row tile x one key segment, its
+//       four wavefronts interleave 32-key tiles and merge through LDS; segments merge in
+//       attn_merge_kernel (the flash-decoding split of cpu/exec/attention.zig:879-962).
+//     prefill mode - a workgroup is four 16-row tiles, each wavefront walks its own key range
+//       (whole tiles outside every row's interval are skipped: the causal triangle).
+// attn_generic_kernel - any head size / f32 K,V: one wavefront per query row, scores staged in
+//   global scratch. Slow; it exists so that every shape the op allows has a GPU path.
+//
+// Softmax uses exp2 on (s - m) * log2(e); aion's CPU path uses a 4th-order polynomial exp
+// (cpu/kernels/fast_math.zig:79-92, rel. err 4e-5), so results agree to ~1e-4, not bitwise.
 #include "common.h"
+
+#include <climits>
+
+namespace {
+
+using f16x8 = __attribute__((ext_vector_type(8))) _Float16;
+using bf16x8 = __attribute__((ext_vector_type(8))) __bf16;
+
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr int TILE_KEYS = 32;
+
+struct AttnArgs {
+    const void *q, *k, *v;
+    float *out;
+    const int *positions, *kv_lengths;
+    float *partial;
+    int B, L, T, Hq, Hkv, groups, rows_total, row_tiles, nseg;
+    int q_dtype, kv_dtype;
+    float scale, soft_cap;
+    unsigned win_left, win_right, win_chunk;
+};
+
+__device__ __forceinline__ unsigned short f32_to_bf16_bits(float x) {
+    unsigned u = __float_as_uint(x);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return (unsigned short)(u >> 16);
+}
+__device__ __forceinline__ float bf16_bits_to_f32(unsigned short b) { return __uint_as_float((unsigned)b << 16); }
+
+template <int KV>
+__device__ __forceinline__ unsigned short to_half_bits(float x) {
+    if (KV == AIONHIP_F16) return __half_as_ushort(__float2half_rn(x));
+    return f32_to_bf16_bits(x);
+}
+template <int KV>
+__device__ __forceinline__ float from_half_bits(unsigned short b) {
+    if (KV == AIONHIP_F16) return __half2float(__ushort_as_half(b));
+    return bf16_bits_to_f32(b);
+}
+template <int KV>
+__device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
+    if (KV == AIONHIP_F16)
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ float load_scalar(const void *p, int dtype, size_t i) {
+    if (dtype == AIONHIP_F32) return ((const float *)p)[i];
+    if (dtype == AIONHIP_F16) return __half2float(((const __half *)p)[i]);
+    return bf16_bits_to_f32(((const unsigned short *)p)[i]);
+}
+
+// AttentionWindow.keys (aion graph/graph.zig:160-167)
+__device__ __forceinline__ void window_keys(unsigned left, unsigned right, unsigned chunk, int pos, int kv_end, int &lo, int &hi) {
+    const long anchor = chunk > 0 ? (long)(pos / (int)chunk) * (int)chunk : pos;
+    const long span = chunk > 0 ? chunk : 1;
+    const long l = anchor - (anchor < (long)left ? anchor : (long)left);
+    long h = right == 0xFFFFFFFFu ? (long)INT_MAX : anchor + span + (long)right;
+    if (h > kv_end) h = kv_end;
+    lo = (int)l;
+    hi = (int)h;
+}
+
+__device__ __forceinline__ int wave_min_i(int v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v = min(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ int wave_max_i(int v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v = max(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+template <int D>
+struct FlashCfg {
+    static constexpr int ROW_BYTES = D * 2 + 16;                 // +16 B: the four key groups land in distinct LDS banks
+    static constexpr int WAVE_LDS = TILE_KEYS * ROW_BYTES;       // one staged V tile per wavefront
+    static constexpr int WG_LDS = 4 * WAVE_LDS;
+    static constexpr int MERGE_LDS = 4 * (16 * D + 32) * 4;      // split mode: 4 x (acc[16][D], m[16], l[16]) f32
+    static constexpr int LDS_BYTES = WG_LDS > MERGE_LDS ? WG_LDS : MERGE_LDS;
+};
+
+template <int KV, int D, bool SPLIT>
+__global__ __launch_bounds__(256) void attn_flash_kernel(AttnArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    using Cfg = FlashCfg<D>;
+    constexpr int KK = D / 32;   // MFMA k-steps over the head dim
+    constexpr int MT = D / 16;   // 16-wide dv tiles
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n = lane & 15, g = lane >> 4;
+    const int unit = blockIdx.y;
+    const int b = unit / a.Hkv, hk = unit % a.Hkv;
+    int rt, seg;
+    if (SPLIT) { rt = blockIdx.x / a.nseg; seg = blockIdx.x % a.nseg; }
+    else { rt = blockIdx.x * 4 + wave; seg = 0; }
+
+    // ---- this lane's query row
+    const int r = rt * 16 + n;
+    const bool row_ok = rt < a.row_tiles && r < a.rows_total;
+    const int li = row_ok ? r / a.groups : 0, gi = row_ok ? r % a.groups : 0;
+    const int hq = hk * a.groups + gi;
+    int kv_end = a.kv_lengths ? a.kv_lengths[b] : a.T;
+    kv_end = max(0, min(kv_end, a.T));
+    int lo = 0, hi = 0;
+    if (row_ok) {
+        const int pos = a.positions ? a.positions[(size_t)b * a.L + li] : li;
+        window_keys(a.win_left, a.win_right, a.win_chunk, max(pos, 0), kv_end, lo, hi);
+        if (hi < lo) hi = lo;
+    }
+    const int uni_lo = wave_min_i(hi > lo ? lo : INT_MAX);
+    const int uni_hi = wave_max_i(hi > lo ? hi : 0);
+
+    // ---- Q^T operand: 8 consecutive d of row n per k-step, converted to the K/V element type
+    u32x4 qf[KK];
+    {
+        const size_t qbase = (((size_t)b * a.L + li) * a.Hq + hq) * D;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            unsigned short h[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float x = row_ok ? load_scalar(a.q, a.q_dtype, qbase + kk * 32 + g * 8 + j) : 0.f;
+                h[j] = to_half_bits<KV>(x);
+            }
+            qf[kk] = u32x4{(unsigned)h[0] | ((unsigned)h[1] << 16), (unsigned)h[2] | ((unsigned)h[3] << 16),
+                           (unsigned)h[4] | ((unsigned)h[5] << 16), (unsigned)h[6] | ((unsigned)h[7] << 16)};
+        }
+    }
+
+    f32x4 acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+
+    // ---- key tiles of this wavefront
+    int t_begin = 0, t_end = 0, t_step = 1;
+    if (uni_hi > uni_lo) {
+        const int tb = uni_lo / TILE_KEYS, te = (uni_hi + TILE_KEYS - 1) / TILE_KEYS;
+        if (SPLIT) {
+            const int per = (te - tb + a.nseg - 1) / a.nseg;
+            t_begin = tb + seg * per + wave;
+            t_end = min(tb + (seg + 1) * per, te);
+            t_step = 4;
+        } else {
+            t_begin = tb;
+            t_end = te;
+        }
+    }
+
+    unsigned char *vs = lds + wave * Cfg::WAVE_LDS;
+    const unsigned short *kp = (const unsigned short *)a.k;
+    const unsigned short *vp = (const unsigned short *)a.v;
+    const size_t kv_row = (size_t)a.Hkv * D;                     // elements between consecutive tokens
+    const size_t kv_base = ((size_t)b * a.T * a.Hkv + hk) * D;
+
+    for (int t = t_begin; t < t_end; t += t_step) {
+        const int key0 = t * TILE_KEYS;
+        // -- stage V[key0 .. key0+32) into LDS (rows outside the union interval as zeros)
+        constexpr int CHUNKS_PER_KEY = D / 8;
+#pragma unroll
+        for (int i = 0; i < TILE_KEYS * CHUNKS_PER_KEY / 64; ++i) {
+            const int c = lane + 64 * i;
+            const int key = c / CHUNKS_PER_KEY, col8 = c % CHUNKS_PER_KEY;
+            const int kabs = key0 + key;
+            u32x4 val = u32x4{0u, 0u, 0u, 0u};
+            if (kabs >= uni_lo && kabs < uni_hi)
+                val = *(const u32x4 *)(vp + kv_base + (size_t)kabs * kv_row + col8 * 8);
+            *(u32x4 *)(vs + key * Cfg::ROW_BYTES + col8 * 16) = val;
+        }
+        // -- S^T = K . Q^T for two 16-key halves
+        f32x4 s[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int kabs = min(key0 + h * 16 + n, a.T - 1);
+            const unsigned short *krow = kp + kv_base + (size_t)kabs * kv_row + g * 8;
+            f32x4 c = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) {
+                const u32x4 kf = *(const u32x4 *)(krow + kk * 32);
+                c = mfma16<KV>(kf, qf[kk], c);
+            }
+            s[h] = c;
+        }
+        // -- scale, soft cap, interval mask; lane holds keys key0 + h*16 + g*4 + i of row n
+        float p[8];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = key0 + h * 16 + g * 4 + i;
+                float x = s[h][i] * a.scale;
+                if (a.soft_cap > 0.f) x = a.soft_cap * tanhf(x / a.soft_cap);
+                const bool ok = key >= lo && key < hi;
+                x = ok ? x : -INFINITY;
+                p[h * 4 + i] = x;
+                mx = fmaxf(mx, x);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);
+        float alpha = 1.f, rowsum = 0.f;
+        if (m_new > -INFINITY) {
+            alpha = m_run > -INFINITY ? exp2f((m_run - m_new) * LOG2E) : 1.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                p[j] = p[j] > -INFINITY ? exp2f((p[j] - m_new) * LOG2E) : 0.f;
+                rowsum += p[j];
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) p[j] = 0.f;
+        }
+        rowsum += __shfl_xor(rowsum, 16, 64);
+        rowsum += __shfl_xor(rowsum, 32, 64);
+        l_run = l_run * alpha + rowsum;
+        m_run = m_new;
+        u32x4 pf;
+        pf.x = (unsigned)to_half_bits<KV>(p[0]) | ((unsigned)to_half_bits<KV>(p[1]) << 16);
+        pf.y = (unsigned)to_half_bits<KV>(p[2]) | ((unsigned)to_half_bits<KV>(p[3]) << 16);
+        pf.z = (unsigned)to_half_bits<KV>(p[4]) | ((unsigned)to_half_bits<KV>(p[5]) << 16);
+        pf.w = (unsigned)to_half_bits<KV>(p[6]) | ((unsigned)to_half_bits<KV>(p[7]) << 16);
+
+        // the staged tile is written and read by this wavefront only
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+        // -- O^T += V^T . P^T ; operand slot j of lane group g is key g*4+j (j<4) / 16+g*4+j-4
+        const unsigned char *vcol = vs + n * 2;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            unsigned short e[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int key = j < 4 ? g * 4 + j : 16 + g * 4 + (j - 4);
+                e[j] = *(const unsigned short *)(vcol + key * Cfg::ROW_BYTES + mt * 32);
+            }
+            const u32x4 vf = u32x4{(unsigned)e[0] | ((unsigned)e[1] << 16), (unsigned)e[2] | ((unsigned)e[3] << 16),
+                                   (unsigned)e[4] | ((unsigned)e[5] << 16), (unsigned)e[6] | ((unsigned)e[7] << 16)};
+            f32x4 c = acc[mt];
+            c *= alpha;
+            acc[mt] = mfma16<KV>(vf, pf, c);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+
+    if (!SPLIT) {
+        if (row_ok) {
+            const float inv = l_run > 0.f ? 1.f / l_run : 0.f;      // empty interval -> zeros
+            float *o = a.out + (((size_t)b * a.L + li) * a.Hq + hq) * D + g * 4;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) *(f32x4 *)(o + mt * 16) = acc[mt] * inv;
+        }
+        return;
+    }
+
+    // ---- split mode: merge the four wavefronts through LDS
+    __syncthreads();
+    float *mg = (float *)lds;
+    constexpr int WSTRIDE = 16 * D + 32;
+    {
+        float *w = mg + wave * WSTRIDE;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) w[n * D + mt * 16 + g * 4 + i] = acc[mt][i];
+        if (g == 0) { w[16 * D + n] = m_run; w[16 * D + 16 + n] = l_run; }
+    }
+    __syncthreads();
+    const size_t pslot = ((size_t)(unit * a.row_tiles + rt) * a.nseg + seg) * WSTRIDE;
+    for (int idx = threadIdx.x; idx < 16 * D; idx += 256) {
+        const int row = idx / D;
+        float m_all = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) m_all = fmaxf(m_all, mg[w * WSTRIDE + 16 * D + row]);
+        float o = 0.f, l_all = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float mw = mg[w * WSTRIDE + 16 * D + row];
+            const float f = mw > -INFINITY ? exp2f((mw - m_all) * LOG2E) : 0.f;
+            o += mg[w * WSTRIDE + idx] * f;
+            l_all += mg[w * WSTRIDE + 16 * D + 16 + row] * f;
+        }
+        if (a.nseg == 1) {
+            const int rr = rt * 16 + row;
+            if (rr < a.rows_total) {
+                const int l2 = rr / a.groups, g2 = rr % a.groups;
+                a.out[(((size_t)b * a.L + l2) * a.Hq + hk * a.groups + g2) * D + idx % D] = l_all > 0.f ? o / l_all : 0.f;
+            }
+        } else {
+            a.partial[pslot + idx] = o;
+            if (idx % D == 0) {
+                a.partial[pslot + 16 * D + row] = m_all;
+                a.partial[pslot + 16 * D + 16 + row] = l_all;
+            }
+        }
+    }
+}
+
+// log-sum-exp merge of the key segments of one (unit, row tile)
+template <int D>
+__global__ __launch_bounds__(256) void attn_merge_kernel(AttnArgs a) {
+    constexpr int WSTRIDE = 16 * D + 32;
+    const int unit = blockIdx.y, rt = blockIdx.x;
+    const int b = unit / a.Hkv, hk = unit % a.Hkv;
+    const float *base = a.partial + (size_t)(unit * a.row_tiles + rt) * a.nseg * WSTRIDE;
+    for (int idx = threadIdx.x; idx < 16 * D; idx += 256) {
+        const int row = idx / D;
+        const int rr = rt * 16 + row;
+        if (rr >= a.rows_total) continue;
+        float m_all = -INFINITY;
+        for (int s = 0; s < a.nseg; ++s) m_all = fmaxf(m_all, base[(size_t)s * WSTRIDE + 16 * D + row]);
+        float o = 0.f, l_all = 0.f;
+        for (int s = 0; s < a.nseg; ++s) {
+            const float ms = base[(size_t)s * WSTRIDE + 16 * D + row];
+            const float f = ms > -INFINITY ? exp2f((ms - m_all) * LOG2E) : 0.f;
+            o += base[(size_t)s * WSTRIDE + idx] * f;
+            l_all += base[(size_t)s * WSTRIDE + 16 * D + 16 + row] * f;
+        }
+        const int l2 = rr / a.groups, g2 = rr % a.groups;
+        a.out[(((size_t)b * a.L + l2) * a.Hq + hk * a.groups + g2) * D + idx % D] = l_all > 0.f ? o / l_all : 0.f;
+    }
+}
+
+// One wavefront per query row; any head sizes and element types. scores: [rows][T] f32 scratch.
+__global__ __launch_bounds__(256) void attn_generic_kernel(AttnArgs a, int d_k, int d_v, float *scores) {
+    const int lane = threadIdx.x & 63;
+    const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const size_t total_rows = (size_t)a.B * a.L * a.Hq;
+    if (row >= total_rows) return;
+    const int hq = (int)(row % a.Hq);
+    const int li = (int)((row / a.Hq) % a.L);
+    const int b = (int)(row / ((size_t)a.Hq * a.L));
+    const int hk = hq / a.groups;
+    int kv_end = a.kv_lengths ? a.kv_lengths[b] : a.T;
+    kv_end = max(0, min(kv_end, a.T));
+    const int pos = a.positions ? a.positions[(size_t)b * a.L + li] : li;
+    int lo, hi;
+    window_keys(a.win_left, a.win_right, a.win_chunk, max(pos, 0), kv_end, lo, hi);
+    float *o = a.out + row * d_v;
+    if (hi <= lo) {
+        for (int j = lane; j < d_v; j += 64) o[j] = 0.f;
+        return;
+    }
+    float *sc = scores + row * a.T;
+    const size_t qb = row * d_k;
+    float mx = -INFINITY;
+    for (int t = lo + lane; t < hi; t += 64) {
+        const size_t kb = (((size_t)b * a.T + t) * a.Hkv + hk) * d_k;
+        float d = 0.f;
+        for (int j = 0; j < d_k; ++j) d += (load_scalar(a.q, a.q_dtype, qb + j) * a.scale) * load_scalar(a.k, a.kv_dtype, kb + j);
+        if (a.soft_cap > 0.f) d = a.soft_cap * tanhf(d / a.soft_cap);
+        sc[t] = d;
+        mx = fmaxf(mx, d);
+    }
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int t = lo + lane; t < hi; t += 64) {
+        const float p = exp2f((sc[t] - mx) * LOG2E);
+        sc[t] = p;
+        sum += p;
+    }
+    sum = wave_sum(sum);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    const float inv = 1.f / sum;
+    for (int j = lane; j < d_v; j += 64) {
+        float acc = 0.f;
+        for (int t = lo; t < hi; ++t) acc += sc[t] * load_scalar(a.v, a.kv_dtype, (((size_t)b * a.T + t) * a.Hkv + hk) * d_v + j);
+        o[j] = acc * inv;
+    }
+}
+
+template <int KV, int D>
+int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
+    using Cfg = FlashCfg<D>;
+    const int units = a.B * a.Hkv;
+    const bool split = a.rows_total <= 64;
+    if (split) {
+        // fill the device: ~2 workgroups per CU, at least 4 tiles (128 keys) per workgroup
+        const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
+        const int tiles = (a.T + TILE_KEYS - 1) / TILE_KEYS;
+        int nseg = (2 * cus + units * a.row_tiles - 1) / (units * a.row_tiles);
+        nseg = max(1, min(nseg, (tiles + 3) / 4));
+        nseg = min(nseg, 256);
+        a.nseg = nseg;
+        if (nseg > 1) {
+            const size_t bytes = (size_t)units * a.row_tiles * nseg * (16 * D + 32) * sizeof(float);
+            int rc = ensure_scratch2(ctx, bytes);
+            if (rc) return rc;
+            a.partial = (float *)ctx->scratch2;
+        }
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)attn_flash_kernel<KV, D, true>, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
+        prof_begin(ctx, "attn_flash_split");
+        attn_flash_kernel<KV, D, true><<<dim3((unsigned)(a.row_tiles * nseg), (unsigned)units), dim3(256), Cfg::LDS_BYTES, ctx->stream>>>(a);
+        if (nseg > 1) attn_merge_kernel<D><<<dim3((unsigned)a.row_tiles, (unsigned)units), dim3(256), 0, ctx->stream>>>(a);
+        prof_end(ctx);
+        LAUNCH_CHECK(ctx, "attn_flash_split");
+    } else {
+        a.nseg = 1;
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)attn_flash_kernel<KV, D, false>, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
+        prof_begin(ctx, "attn_flash_prefill");
+        attn_flash_kernel<KV, D, false><<<dim3((unsigned)((a.row_tiles + 3) / 4), (unsigned)units), dim3(256), Cfg::LDS_BYTES, ctx->stream>>>(a);
+        prof_end(ctx);
+        LAUNCH_CHECK(ctx, "attn_flash_prefill");
+    }
+    return AIONHIP_OK;
+}
+
+template <int KV>
+int launch_flash_d(aionhip_ctx *ctx, AttnArgs &a, int d) {
+    if (d == 64) return launch_flash<KV, 64>(ctx, a);
+    if (d == 128) return launch_flash<KV, 128>(ctx, a);
+    return launch_flash<KV, 256>(ctx, a);
+}
+
+bool dtype_ok(int d) { return d == AIONHIP_F32 || d == AIONHIP_F16 || d == AIONHIP_BF16; }
+
+}  // namespace
 
 extern "C" int aionhip_step_attention(aionhip_ctx *ctx, const aionhip_attention *p) {
     if (!ctx || !p) return AIONHIP_INVALID_ARGUMENT;
-    return set_err(ctx, AIONHIP_UNSUPPORTED, "attention is not built yet");
+    if (!p->out || !p->q || !p->k || !p->v) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "attention: null operand");
+    if (!dtype_ok(p->q_dtype) || !dtype_ok(p->kv_dtype)) return set_err(ctx, AIONHIP_UNSUPPORTED, "attention: q/kv dtype must be f32, f16 or bf16");
+    if (p->h_kv == 0 || p->h_q == 0 || p->h_q % p->h_kv != 0) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "attention: h_q %zu is not a multiple of h_kv %zu", p->h_q, p->h_kv);
+    if (p->d_k == 0 || p->d_v == 0) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "attention: zero head size");
+    if (p->batch == 0 || p->l_q == 0) return AIONHIP_OK;
+    const size_t lim = 0x7FFFFFFF;
+    if (p->batch > lim || p->l_q > lim || p->t_kv > lim || p->h_q > 65535 || p->d_k > 65535 || p->d_v > 65535 ||
+        p->batch * p->h_kv > 65535 || p->l_q * (p->h_q / p->h_kv) > lim)
+        return set_err(ctx, AIONHIP_UNSUPPORTED, "attention: dimension too large");
+
+    AttnArgs a{};
+    a.q = (const void *)(uintptr_t)p->q;
+    a.k = (const void *)(uintptr_t)p->k;
+    a.v = (const void *)(uintptr_t)p->v;
+    a.out = (float *)(uintptr_t)p->out;
+    a.positions = (const int *)(uintptr_t)p->query_positions;
+    a.kv_lengths = (const int *)(uintptr_t)p->kv_lengths;
+    a.B = (int)p->batch; a.L = (int)p->l_q; a.T = (int)p->t_kv; a.Hq = (int)p->h_q; a.Hkv = (int)p->h_kv;
+    a.groups = a.Hq / a.Hkv;
+    a.rows_total = a.L * a.groups;
+    a.row_tiles = (a.rows_total + 15) / 16;
+    a.nseg = 1;
+    a.q_dtype = p->q_dtype; a.kv_dtype = p->kv_dtype;
+    a.scale = p->scale; a.soft_cap = p->attn_logits_soft_cap;
+    a.win_left = p->window_left; a.win_right = p->window_right; a.win_chunk = p->window_chunk;
+
+    if (a.T == 0) {
+        // no keys at all: every interval is empty -> zeros (cpu/exec/attention.zig:787-815)
+        return aionhip_memset(ctx, p->out, 0, 0, p->batch * p->l_q * p->h_q * p->d_v * sizeof(float));
+    }
+
+    const bool flash = p->d_k == p->d_v && (p->d_k == 64 || p->d_k == 128 || p->d_k == 256) &&
+                       (p->kv_dtype == AIONHIP_F16 || p->kv_dtype == AIONHIP_BF16) &&
+                       ((p->k | p->v | p->out) & 15) == 0;
+    if (flash) {
+        if (p->kv_dtype == AIONHIP_F16) return launch_flash_d<AIONHIP_F16>(ctx, a, (int)p->d_k);
+        return launch_flash_d<AIONHIP_BF16>(ctx, a, (int)p->d_k);
+    }
+    const size_t rows = p->batch * p->l_q * p->h_q;
+    int rc = ensure_scratch2(ctx, rows * p->t_kv * sizeof(float));
+    if (rc) return rc;
+    prof_begin(ctx, "attn_generic");
+    attn_generic_kernel<<<dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, ctx->stream>>>(a, (int)p->d_k, (int)p->d_v, (float *)ctx->scratch2);
+    prof_end(ctx);
+    LAUNCH_CHECK(ctx, "attn_generic");
+    return AIONHIP_OK;
 }

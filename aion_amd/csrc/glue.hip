@@ -1,13 +1,269 @@
-// Per-token glue steps (placeholder until the kernels land): every call is rejected loudly.
+// Per-token glue steps between the matmuls of a decoder: RMSNorm(+residual), RoPE, add,
+// gelu-gate, row gather, f32->f16 cast + KV append, argmax. All HBM/launch-bound, one pass each.
+// Formulas follow aion's CPU executors (cited per kernel) including its polynomial tanh/exp for
+// the gelu gate, so a decoder run tracks the CPU path closely.
 #include "common.h"
 
-extern "C" {
-int aionhip_step_rmsnorm(aionhip_ctx *ctx, aionhip_handle, aionhip_handle, aionhip_handle, aionhip_handle, aionhip_handle, size_t, size_t, float) { return set_err(ctx, AIONHIP_UNSUPPORTED, "rmsnorm is not built yet"); }
-int aionhip_step_rope(aionhip_ctx *ctx, aionhip_handle, aionhip_handle, aionhip_handle, size_t, size_t, size_t, size_t, float, float, float) { return set_err(ctx, AIONHIP_UNSUPPORTED, "rope is not built yet"); }
-int aionhip_step_add(aionhip_ctx *ctx, aionhip_handle, aionhip_handle, aionhip_handle, size_t) { return set_err(ctx, AIONHIP_UNSUPPORTED, "add is not built yet"); }
-int aionhip_step_gate_gelu(aionhip_ctx *ctx, aionhip_handle, aionhip_handle, aionhip_handle, size_t) { return set_err(ctx, AIONHIP_UNSUPPORTED, "gate is not built yet"); }
-int aionhip_step_gather_rows(aionhip_ctx *ctx, int, aionhip_handle, aionhip_handle, aionhip_handle, size_t, size_t, size_t) { return set_err(ctx, AIONHIP_UNSUPPORTED, "gather is not built yet"); }
-int aionhip_step_append_f16(aionhip_ctx *ctx, aionhip_handle, aionhip_handle, aionhip_handle, size_t, size_t, size_t, size_t) { return set_err(ctx, AIONHIP_UNSUPPORTED, "append is not built yet"); }
-int aionhip_step_cast_f32_f16(aionhip_ctx *ctx, aionhip_handle, aionhip_handle, size_t) { return set_err(ctx, AIONHIP_UNSUPPORTED, "cast is not built yet"); }
-int aionhip_step_argmax(aionhip_ctx *ctx, aionhip_handle, aionhip_handle, size_t, size_t) { return set_err(ctx, AIONHIP_UNSUPPORTED, "argmax is not built yet"); }
+namespace {
+
+__device__ __forceinline__ float block_sum(float v, float *red) {
+    v = wave_sum(v);
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    if (lane == 0) red[w] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < (int)(blockDim.x >> 6); ++i) t += red[i];
+    __syncthreads();
+    return t;
 }
+
+// cpu/exec/layernorm.zig:54-155 + cpu/kernels/layernorm.zig:69-147 (rmsnorm mode):
+// inv = 1/sqrt(sum(x^2)/cols + eps); out = (x*inv)*gamma + beta; out += residual
+__global__ __launch_bounds__(256) void rmsnorm_kernel(float *__restrict__ out, const float *__restrict__ x, const float *__restrict__ gamma,
+                                                      const float *__restrict__ beta, const float *__restrict__ residual,
+                                                      size_t cols, float eps) {
+    __shared__ float red[4];
+    const size_t row = blockIdx.x;
+    const float *xr = x + row * cols;
+    float ss = 0.f;
+    for (size_t c = threadIdx.x; c < cols; c += 256) ss += xr[c] * xr[c];
+    ss = block_sum(ss, red);
+    const float inv = 1.f / sqrtf(ss * (1.f / (float)cols) + eps);
+    for (size_t c = threadIdx.x; c < cols; c += 256) {
+        float y = (xr[c] * inv) * gamma[c] + (beta ? beta[c] : 0.f);
+        if (residual) y += residual[row * cols + c];
+        out[row * cols + c] = y;
+    }
+}
+
+// cpu/exec/rope.zig:14-53 + cpu/kernels/rope.zig:20-98: pairs (i, i + D/2); the frequency is
+// multiplied up iteratively in f32, the angle pos*f is rounded to f32, sin/cos are taken in f64.
+__global__ void rope_kernel(float *__restrict__ out, const float *__restrict__ x, const int *__restrict__ positions,
+                            size_t tokens, int H, int D, int rope_pairs, float freq_step, float scale_factor) {
+    const int half = D / 2;
+    const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= tokens * (size_t)half) return;
+    const size_t tok = gid / half;
+    const int i = (int)(gid % half);
+    const float *xr = x + tok * H * D;
+    float *orow = out + tok * H * D;
+    if (i >= rope_pairs) {
+        for (int h = 0; h < H; ++h) {
+            orow[h * D + i] = xr[h * D + i];
+            orow[h * D + half + i] = xr[h * D + half + i];
+        }
+        return;
+    }
+    float f = scale_factor;
+    for (int j = 0; j < i; ++j) f *= freq_step;
+    const float ang = (float)positions[tok] * f;
+    const float cs = (float)cos((double)ang), sn = (float)sin((double)ang);
+    for (int h = 0; h < H; ++h) {
+        const float xl = xr[h * D + i], xh = xr[h * D + half + i];
+        orow[h * D + i] = xl * cs - xh * sn;
+        orow[h * D + half + i] = xl * sn + xh * cs;
+    }
+}
+
+__global__ void add_kernel(float *__restrict__ out, const float *__restrict__ a, const float *__restrict__ b, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = a[i] + b[i];
+}
+
+// cpu/kernels/fast_math.zig:53-148: exp(x) = 2^n * P4(r ln2), sigmoid, tanh = 2 sigmoid(2x) - 1
+__device__ __forceinline__ float exp_approx(float x_in) {
+    const float x = fminf(80.f, fmaxf(-80.f, x_in));
+    const float y = x * 1.4426950408889634f;
+    const float nf = floorf(y + 0.5f);
+    const float t = (y - nf) * 0.6931471805599453f;
+    const float p = 1.f + t * (1.f + t * (0.5f + t * ((1.f / 6.f) + t * (1.f / 24.f))));
+    return __uint_as_float((unsigned)((int)nf + 127) << 23) * p;
+}
+__device__ __forceinline__ float tanh_approx(float x) {
+    const float z = 2.f * x;
+    const float e = exp_approx(-fabsf(z));
+    float sg = (z >= 0.f ? 1.f : e) / (1.f + e);
+    sg = fminf(1.f, fmaxf(0.f, sg));
+    return fminf(1.f, fmaxf(-1.f, 2.f * sg - 1.f));
+}
+// cpu/exec/elementwise.zig:25-37 (gate) + cpu/kernels/gelu.zig:8-14
+__global__ void gate_gelu_kernel(float *__restrict__ out, const float *__restrict__ a, const float *__restrict__ b, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float x = a[i];
+    const float t = 0.7978845608028654f * (x + 0.044715f * (x * x * x));
+    out[i] = (0.5f * x * (1.f + tanh_approx(t))) * b[i];
+}
+
+// cpu/exec/gather.zig:60-87: one workgroup per gathered row; ids outside [0, vocab) give zeros
+__global__ __launch_bounds__(256) void gather_rows_kernel(int dtype, float *__restrict__ out, const void *__restrict__ table,
+                                                          const int *__restrict__ ids, size_t d, size_t vocab) {
+    const size_t i = blockIdx.x;
+    const long id = ids[i];
+    float *o = out + i * d;
+    if (id < 0 || (size_t)id >= vocab) {
+        for (size_t c = threadIdx.x; c < d; c += 256) o[c] = 0.f;
+        return;
+    }
+    if (dtype == AIONHIP_F32) {
+        const float *src = (const float *)table + (size_t)id * d;
+        for (size_t c = threadIdx.x; c < d; c += 256) o[c] = src[c];
+    } else {
+        const uint8_t *src = (const uint8_t *)table + (size_t)id * (d / QK) * Q8_BYTES;
+        for (size_t c = threadIdx.x; c < d; c += 256) {
+            const uint8_t *blk = src + (c / QK) * Q8_BYTES;
+            const float s = __half2float(__ushort_as_half(*reinterpret_cast<const uint16_t *>(blk)));
+            o[c] = (float)(int8_t)blk[2 + c % QK] * s;
+        }
+    }
+}
+
+// cpu/exec/cast.zig (f32 -> f16, RNE) and cpu/exec/sequence_append.zig:12-104
+__global__ void cast_f16_kernel(__half *__restrict__ out, const float *__restrict__ x, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = __float2half_rn(x[i]);
+}
+__global__ void append_f16_kernel(__half *__restrict__ cache, const float *__restrict__ src, const int *__restrict__ write_index,
+                                  size_t s_len, size_t t_cap, size_t row_elems, size_t total) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const size_t e = i % row_elems, s = (i / row_elems) % s_len, b = i / (row_elems * s_len);
+    const long t = (long)write_index[0] + (long)s;
+    if (t < 0 || (size_t)t >= t_cap) return;      // never write outside the cache
+    cache[(b * t_cap + (size_t)t) * row_elems + e] = __float2half_rn(src[i]);
+}
+
+// cpu/exec/argmax.zig:56-81: strict > keeps the first maximum
+__global__ __launch_bounds__(256) void argmax_kernel(int *__restrict__ out, const float *__restrict__ x, size_t n) {
+    __shared__ float bv[256];
+    __shared__ int bi[256];
+    const float *row = x + (size_t)blockIdx.x * n;
+    float best = -INFINITY;
+    int idx = 0x7FFFFFFF;
+    for (size_t j = threadIdx.x; j < n; j += 256) {
+        const float v = row[j];
+        if (idx == 0x7FFFFFFF || v > best) { best = v; idx = (int)j; }
+    }
+    bv[threadIdx.x] = best;
+    bi[threadIdx.x] = idx;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if ((int)threadIdx.x < s) {
+            const float ov = bv[threadIdx.x + s];
+            const int oi = bi[threadIdx.x + s];
+            if (oi != 0x7FFFFFFF && (bi[threadIdx.x] == 0x7FFFFFFF || ov > bv[threadIdx.x] || (ov == bv[threadIdx.x] && oi < bi[threadIdx.x]))) {
+                bv[threadIdx.x] = ov;
+                bi[threadIdx.x] = oi;
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[blockIdx.x] = bi[0] == 0x7FFFFFFF ? 0 : bi[0];
+}
+
+inline unsigned grid_for(size_t n, unsigned block) { return (unsigned)((n + block - 1) / block); }
+template <class T>
+inline T *dp(aionhip_handle h) { return (T *)(uintptr_t)h; }
+
+}  // namespace
+
+extern "C" {
+
+int aionhip_step_rmsnorm(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle x, aionhip_handle gamma, aionhip_handle beta,
+                         aionhip_handle residual, size_t rows, size_t cols, float eps) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (!out || !x || !gamma) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "rmsnorm: null operand");
+    if (!(eps > 0.f) || !(eps < INFINITY)) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "rmsnorm: eps must be positive and finite");
+    if (!rows || !cols) return AIONHIP_OK;
+    if (rows > 0x7FFFFFFFu) return set_err(ctx, AIONHIP_UNSUPPORTED, "rmsnorm: too many rows");
+    rmsnorm_kernel<<<dim3((unsigned)rows), dim3(256), 0, ctx->stream>>>(dp<float>(out), dp<const float>(x), dp<const float>(gamma),
+                                                                        dp<const float>(beta), dp<const float>(residual), cols, eps);
+    LAUNCH_CHECK(ctx, "rmsnorm");
+    return AIONHIP_OK;
+}
+
+int aionhip_step_rope(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle x, aionhip_handle positions, size_t b, size_t t, size_t h,
+                      size_t d, float base_frequency, float scale_factor, float rope_proportion) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (!out || !x || !positions) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "rope: null operand");
+    if (!(base_frequency > 0.f) || !(base_frequency < INFINITY) || !(scale_factor > 0.f) || !(scale_factor < INFINITY) ||
+        !(rope_proportion >= 0.f && rope_proportion <= 1.f))
+        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "rope: base/scale must be positive and finite, proportion in [0,1]");
+    if (d % 2 != 0 || d > 65534 || h > 65535) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "rope: head size must be even");
+    const size_t tokens = b * t;
+    if (!tokens || !h || !d) return AIONHIP_OK;
+    const size_t half = d / 2;
+    size_t rope_pairs = (size_t)floorf(rope_proportion * (float)half);
+    if (rope_pairs > half) rope_pairs = half;
+    const float freq_step = (float)pow((double)base_frequency, (double)(-2.0f / (float)d));
+    rope_kernel<<<dim3(grid_for(tokens * half, 128)), dim3(128), 0, ctx->stream>>>(dp<float>(out), dp<const float>(x), dp<const int>(positions),
+                                                                                   tokens, (int)h, (int)d, (int)rope_pairs, freq_step, scale_factor);
+    LAUNCH_CHECK(ctx, "rope");
+    return AIONHIP_OK;
+}
+
+int aionhip_step_add(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle a, aionhip_handle b, size_t n) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (!out || !a || !b) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "add: null operand");
+    if (!n) return AIONHIP_OK;
+    add_kernel<<<dim3(grid_for(n, 256)), dim3(256), 0, ctx->stream>>>(dp<float>(out), dp<const float>(a), dp<const float>(b), n);
+    LAUNCH_CHECK(ctx, "add");
+    return AIONHIP_OK;
+}
+
+int aionhip_step_gate_gelu(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle a, aionhip_handle b, size_t n) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (!out || !a || !b) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "gate: null operand");
+    if (!n) return AIONHIP_OK;
+    gate_gelu_kernel<<<dim3(grid_for(n, 256)), dim3(256), 0, ctx->stream>>>(dp<float>(out), dp<const float>(a), dp<const float>(b), n);
+    LAUNCH_CHECK(ctx, "gate_gelu");
+    return AIONHIP_OK;
+}
+
+int aionhip_step_gather_rows(aionhip_ctx *ctx, int table_dtype, aionhip_handle out, aionhip_handle table, aionhip_handle ids,
+                             size_t n_ids, size_t d, size_t vocab) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (table_dtype != AIONHIP_F32 && table_dtype != AIONHIP_Q8_0) return set_err(ctx, AIONHIP_UNSUPPORTED, "gather: table must be f32 or q8_0");
+    if (!out || !table || !ids) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "gather: null operand");
+    if (table_dtype == AIONHIP_Q8_0 && d % QK != 0) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "gather: q8_0 row length must be a multiple of 32");
+    if (!n_ids || !d) return AIONHIP_OK;
+    if (n_ids > 0x7FFFFFFFu) return set_err(ctx, AIONHIP_UNSUPPORTED, "gather: too many ids");
+    gather_rows_kernel<<<dim3((unsigned)n_ids), dim3(256), 0, ctx->stream>>>(table_dtype, dp<float>(out), dp<const void>(table), dp<const int>(ids), d, vocab);
+    LAUNCH_CHECK(ctx, "gather_rows");
+    return AIONHIP_OK;
+}
+
+int aionhip_step_append_f16(aionhip_ctx *ctx, aionhip_handle cache, aionhip_handle src_f32, aionhip_handle write_index, size_t b,
+                            size_t s, size_t t_cap, size_t row_elems) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (!cache || !src_f32 || !write_index) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "append: null operand");
+    if (s > t_cap) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "append: %zu new tokens exceed the cache capacity %zu", s, t_cap);
+    const size_t total = b * s * row_elems;
+    if (!total) return AIONHIP_OK;
+    append_f16_kernel<<<dim3(grid_for(total, 256)), dim3(256), 0, ctx->stream>>>(dp<__half>(cache), dp<const float>(src_f32), dp<const int>(write_index),
+                                                                                 s, t_cap, row_elems, total);
+    LAUNCH_CHECK(ctx, "append_f16");
+    return AIONHIP_OK;
+}
+
+int aionhip_step_cast_f32_f16(aionhip_ctx *ctx, aionhip_handle out_f16, aionhip_handle x_f32, size_t n) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (!out_f16 || !x_f32) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "cast: null operand");
+    if (!n) return AIONHIP_OK;
+    cast_f16_kernel<<<dim3(grid_for(n, 256)), dim3(256), 0, ctx->stream>>>(dp<__half>(out_f16), dp<const float>(x_f32), n);
+    LAUNCH_CHECK(ctx, "cast_f32_f16");
+    return AIONHIP_OK;
+}
+
+int aionhip_step_argmax(aionhip_ctx *ctx, aionhip_handle out_i32, aionhip_handle x, size_t rows, size_t n) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (!out_i32 || !x) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "argmax: null operand");
+    if (n == 0) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "argmax: empty axis");
+    if (!rows) return AIONHIP_OK;
+    if (rows > 0x7FFFFFFFu || n > 0x7FFFFFFFu) return set_err(ctx, AIONHIP_UNSUPPORTED, "argmax: dimension too large");
+    argmax_kernel<<<dim3((unsigned)rows), dim3(256), 0, ctx->stream>>>(dp<int>(out_i32), dp<const float>(x), n);
+    LAUNCH_CHECK(ctx, "argmax");
+    return AIONHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,192 @@
+"""GPU parity of the attention step against the CPU oracle (through the C ABI).
+
+Tolerances (max |err| over the output, outputs are O(1) softmax averages of N(0,1) values):
+f32 accumulate with f16 K/V: 2e-3; bf16 operands (q rounded to bf16, probabilities to bf16): 1e-2.
+The reference is the textbook f64 attention (orc.attention_f64); aion's blocked CPU algorithm
+(orc.attention_blocked, polynomial exp) is compared as well at the same bound.
+"""
+import math
+import sys
+
+import numpy as np
+import pytest
+
+from aion_amd import backend as be
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def to_bf16(x):
+    """round-to-nearest-even f32 -> bf16 bits (uint16) and the f32 value they stand for"""
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) >> 16
+    bits = u.astype(np.uint16)
+    return bits, (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+def run_attention(gpu, q, k, v, scale, q_dtype, kv_dtype, window=be.CAUSAL, soft_cap=0.0, positions=None, kv_lengths=None):
+    B, L, Hq, Dk = q.shape
+    _, T, Hkv, _ = k.shape
+    Dv = v.shape[3]
+    bufs = [gpu.upload(q), gpu.upload(k), gpu.upload(v)]
+    out = gpu.alloc(max(B * L * Hq * Dv * 4, 4))
+    pos = gpu.upload(np.ascontiguousarray(positions, np.int32)) if positions is not None else None
+    kl = gpu.upload(np.ascontiguousarray(kv_lengths, np.int32)) if kv_lengths is not None else None
+    gpu.step_attention(out, bufs[0], bufs[1], bufs[2], (B, L, T, Hq, Hkv, Dk, Dv), scale, q_dtype=q_dtype, kv_dtype=kv_dtype,
+                       window=window, soft_cap=soft_cap, query_positions=pos, kv_lengths=kl)
+    res = gpu.download(out, np.float32, (B, L, Hq, Dv))
+    for b in bufs + [out] + [x for x in (pos, kl) if x is not None]:
+        b.free()
+    return res
+
+
+def make_qkv(seed, B, L, T, Hq, Hkv, D, kind):
+    rng = np.random.default_rng(seed)
+    q = rng.standard_normal((B, L, Hq, D)).astype(np.float32)
+    k = rng.standard_normal((B, T, Hkv, D)).astype(np.float32)
+    v = rng.standard_normal((B, T, Hkv, D)).astype(np.float32)
+    if kind == "f16":      # aion's cached decode: q f32, K/V cache f16
+        k16, v16 = k.astype(np.float16), v.astype(np.float16)
+        return (q, k16, v16, be.F32, be.F16), (q, k16.astype(np.float32), v16.astype(np.float32))
+    qb, qf = to_bf16(q); kb, kf = to_bf16(k); vb, vf = to_bf16(v)   # BASELINE config 4: bf16 Q/K/V
+    return (qb, kb, vb, be.BF16, be.BF16), (qf, kf, vf)
+
+
+@pytest.mark.parametrize("kind,tol", [("f16", 2e-3), ("bf16", 1e-2)])
+@pytest.mark.parametrize("D", [64, 128, 256])
+def test_prefill_causal_gqa(gpu, orc, kind, tol, D):
+    B, L, Hq, Hkv = 2, 150, 8, 2
+    say("prefill", kind, D)
+    (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(D, B, L, L, Hq, Hkv, D, kind)
+    got = run_attention(gpu, q, k, v, 1 / math.sqrt(D), qd, kd)
+    assert gpu.last_kernel() == "attn_flash_prefill"
+    ref = orc.attention_f64(qf, kf, vf, 1 / math.sqrt(D))
+    err = float(np.abs(got - ref).max())
+    say("  max err", err)
+    assert err < tol
+    blocked = orc.attention_blocked(qf, kf, vf, 1 / math.sqrt(D))
+    assert float(np.abs(got - blocked).max()) < tol
+
+
+@pytest.mark.parametrize("kind,tol", [("f16", 2e-3), ("bf16", 1e-2)])
+@pytest.mark.parametrize("T,B", [(1024, 1), (4096, 8), (777, 3)])
+def test_decode_split_k(gpu, orc, kind, tol, T, B):
+    # BASELINE config 4b shape family: 1 query token at position T-1, 8 q heads / 1 kv head, hd 256
+    Hq, Hkv, D = 8, 1, 256
+    say("decode", kind, T, B)
+    (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(T + B, B, 1, T, Hq, Hkv, D, kind)
+    pos = np.full((B, 1), T - 1, np.int32)
+    end = np.full((B,), T, np.int32)
+    got = run_attention(gpu, q, k, v, 1 / 16.0, qd, kd, positions=pos, kv_lengths=end)
+    assert gpu.last_kernel() == "attn_flash_split"
+    ref = orc.attention_f64(qf, kf, vf, 1 / 16.0, positions=pos, kv_lengths=end)
+    err = float(np.abs(got - ref).max())
+    say("  max err", err)
+    assert err < tol
+
+
+def test_decode_ragged_lengths_and_stale_cache_tail(gpu, orc):
+    # per-batch kv lengths; the cache tail beyond each length holds NaN patterns that must not leak
+    B, T, Hq, Hkv, D = 3, 600, 8, 2, 128
+    (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(5, B, 1, T, Hq, Hkv, D, "f16")
+    lens = np.array([600, 37, 1], np.int32)
+    pos = (lens - 1).reshape(B, 1)
+    for b in range(B):
+        k[b, lens[b]:] = np.float16(np.nan)
+        v[b, lens[b]:] = np.float16(np.nan)
+        kf[b, lens[b]:] = 0
+        vf[b, lens[b]:] = 0
+    got = run_attention(gpu, q, k, v, 0.1, qd, kd, positions=pos, kv_lengths=lens)
+    ref = orc.attention_f64(qf, kf, vf, 0.1, positions=pos, kv_lengths=lens)
+    assert np.isfinite(got).all()
+    assert float(np.abs(got - ref).max()) < 2e-3
+
+
+@pytest.mark.parametrize("window", [(100, 0, 0), (16, 0, 64), (be.UNBOUNDED, be.UNBOUNDED, 0), (5, 3, 0)])
+def test_windows_prefill_and_decode(gpu, orc, window):
+    B, L, Hq, Hkv, D = 1, 200, 4, 1, 64
+    say("window", window)
+    (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(11, B, L, L, Hq, Hkv, D, "f16")
+    got = run_attention(gpu, q, k, v, 0.125, qd, kd, window=window)
+    ref = orc.attention_f64(qf, kf, vf, 0.125, window=window)
+    assert float(np.abs(got - ref).max()) < 2e-3
+    # one decode row with an explicit position inside the sequence
+    pos = np.array([[131]], np.int32)
+    end = np.array([180], np.int32)
+    got1 = run_attention(gpu, q[:, :1], k, v, 0.125, qd, kd, window=window, positions=pos, kv_lengths=end)
+    ref1 = orc.attention_f64(qf[:, :1], kf, vf, 0.125, window=window, positions=pos, kv_lengths=end)
+    assert float(np.abs(got1 - ref1).max()) < 2e-3
+
+
+def test_soft_cap(gpu, orc):
+    (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(13, 1, 40, 40, 8, 1, 64, "f16")
+    # logits of std ~24 before the cap: the flash kernel feeds q to the MFMA in the K/V element
+    # type, so the reference gets the same f16-rounded q (the cap itself is what is under test)
+    q3 = (q * 3).astype(np.float16).astype(np.float32)
+    got = run_attention(gpu, q3, k, v, 1.0, qd, kd, soft_cap=5.0)
+    ref = orc.attention_f64(q3, kf, vf, 1.0, soft_cap=5.0)
+    assert float(np.abs(got - ref).max()) < 2e-3
+
+
+def test_kat_uniform_softmax_sliding_window(gpu):
+    # aion api/test_api.zig:3256-3331 -> {4,4,40,40,5,5,50,50}, abs 1e-6 (generic kernel: d_k=2, f32 K/V)
+    q = np.zeros((1, 2, 4, 2), np.float32)
+    k = np.zeros((1, 6, 2, 2), np.float32)
+    v = np.zeros((1, 6, 2, 1), np.float32)
+    for t in range(6):
+        v[0, t, 0, 0] = t + 1
+        v[0, t, 1, 0] = 10 * (t + 1)
+    got = run_attention(gpu, q, k, v, 1.0, be.F32, be.F32, window=(2, 0, 0), positions=np.array([[4, 5]], np.int32), kv_lengths=np.array([6], np.int32))
+    assert gpu.last_kernel() == "attn_generic"
+    assert np.allclose(got.reshape(-1), [4, 4, 40, 40, 5, 5, 50, 50], atol=1e-6)
+
+
+def test_kat_three_step_decode(gpu):
+    # aion api/test_nn.zig:799-901: 2, (e^-3*2+3)/(e^-3+1), (e^-8*2+e^-4*3+4)/(e^-8+e^-4+1), abs 1e-4
+    kc = np.zeros((1, 3, 1, 1), np.float32)
+    vc = np.zeros((1, 3, 1, 1), np.float32)
+    want = [2.0, (math.exp(-3) * 2 + 3) / (math.exp(-3) + 1),
+            (math.exp(-8) * 2 + math.exp(-4) * 3 + 4) / (math.exp(-8) + math.exp(-4) + 1)]
+    for t in range(3):
+        kc[0, t, 0, 0] = vc[0, t, 0, 0] = t + 2
+        q = np.full((1, 1, 1, 1), t + 2, np.float32)
+        got = run_attention(gpu, q, kc, vc, 1.0, be.F32, be.F32, positions=np.array([[t]], np.int32), kv_lengths=np.array([t + 1], np.int32))
+        assert abs(float(got.reshape(-1)[0]) - want[t]) < 1e-4
+
+
+def test_generic_path_matches_oracle_on_odd_head_sizes(gpu, orc):
+    rng = np.random.default_rng(3)
+    q = rng.standard_normal((2, 9, 6, 40)).astype(np.float32)
+    k = rng.standard_normal((2, 70, 3, 40)).astype(np.float32)
+    v = rng.standard_normal((2, 70, 3, 24)).astype(np.float32)
+    pos = np.tile(np.arange(61, 70, dtype=np.int32), (2, 1))
+    got = run_attention(gpu, q, k, v, 0.2, be.F32, be.F32, positions=pos)
+    ref = orc.attention_f64(q, k, v, 0.2, positions=pos)
+    assert float(np.abs(got - ref).max()) < 1e-4
+
+
+def test_empty_window_and_plain_equals_cached(gpu, orc):
+    (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(17, 1, 33, 33, 8, 1, 64, "f16")
+    zero = run_attention(gpu, q, k, v, 0.1, qd, kd, kv_lengths=np.array([0], np.int32))
+    assert not zero.any()
+    # plain sequence (implied positions / lengths) == explicit controls (aion cpu/test_cpu_backend.zig:1531)
+    plain = run_attention(gpu, q, k, v, 0.1, qd, kd)
+    cached = run_attention(gpu, q, k, v, 0.1, qd, kd, positions=np.arange(33, dtype=np.int32).reshape(1, 33), kv_lengths=np.array([33], np.int32))
+    assert np.array_equal(plain, cached)
+
+
+def test_attention_argument_errors(gpu):
+    from aion_amd import hip
+    a = gpu.alloc(1024)
+    with pytest.raises(be.AionHipError) as e:
+        gpu.step_attention(a, a, a, a, (1, 1, 4, 3, 2, 64, 64), 1.0)      # 3 q heads over 2 kv heads
+    assert e.value.status == hip.INVALID_ARGUMENT
+    with pytest.raises(be.AionHipError) as e:
+        gpu.step_attention(a, a, a, a, (1, 1, 4, 2, 2, 64, 64), 1.0, kv_dtype=be.I32)
+    assert e.value.status == hip.UNSUPPORTED
+    a.free()

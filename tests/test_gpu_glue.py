@@ -1,0 +1,115 @@
+"""GPU parity of the per-token glue steps against the CPU oracle (through the C ABI)."""
+import numpy as np
+import pytest
+
+from aion_amd import backend as be
+from aion_amd import hip
+
+pytestmark = pytest.mark.gpu
+
+
+def test_rmsnorm_with_and_without_residual(gpu, orc):
+    rng = np.random.default_rng(1)
+    rows, cols = 5, 2048
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    g = rng.standard_normal(cols).astype(np.float32)
+    bt = rng.standard_normal(cols).astype(np.float32)
+    r = rng.standard_normal((rows, cols)).astype(np.float32)
+    xb, gb, bb, rb = gpu.upload(x), gpu.upload(g), gpu.upload(bt), gpu.upload(r)
+    out = gpu.alloc(x.nbytes)
+    gpu.step_rmsnorm(out, xb, gb, rows, cols, 1e-6)
+    assert np.allclose(gpu.download(out, np.float32, x.shape), orc.rmsnorm(x, g, 1e-6), rtol=1e-5, atol=1e-5)
+    gpu.step_rmsnorm(out, xb, gb, rows, cols, 1e-6, beta=bb, residual=rb)
+    assert np.allclose(gpu.download(out, np.float32, x.shape), orc.rmsnorm(x, g, 1e-6, beta=bt, residual=r), rtol=1e-5, atol=1e-5)  # three-term sum: fused multiply-add vs separate rounding
+    with pytest.raises(be.AionHipError) as e:
+        gpu.step_rmsnorm(out, xb, gb, rows, cols, 0.0)
+    assert e.value.status == hip.INVALID_ARGUMENT
+    for b in (xb, gb, bb, rb, out):
+        b.free()
+
+
+@pytest.mark.parametrize("proportion", [1.0, 0.5, 0.0])
+def test_rope_matches_oracle(gpu, orc, proportion):
+    rng = np.random.default_rng(2)
+    B, T, H, D = 2, 7, 8, 256
+    x = rng.standard_normal((B, T, H, D)).astype(np.float32)
+    pos = rng.integers(0, 5000, (B, T)).astype(np.int32)
+    pos[0, 0] = 0
+    xb, pb = gpu.upload(x), gpu.upload(pos)
+    out = gpu.alloc(x.nbytes)
+    gpu.step_rope(out, xb, pb, B, T, H, D, base=10000.0, proportion=proportion)
+    got = gpu.download(out, np.float32, x.shape)
+    want = orc.rope(x, pos, base=10000.0, proportion=proportion)
+    assert np.allclose(got, want, rtol=0, atol=2e-6)
+    assert np.array_equal(got[0, 0], x[0, 0])
+    for b in (xb, pb, out):
+        b.free()
+
+
+def test_add_gate_cast_argmax(gpu, orc):
+    rng = np.random.default_rng(3)
+    n = 8192 + 5
+    a = (rng.standard_normal(n) * 3).astype(np.float32)
+    b = rng.standard_normal(n).astype(np.float32)
+    ab, bb = gpu.upload(a), gpu.upload(b)
+    out = gpu.alloc(n * 4)
+    gpu.step_add(out, ab, bb, n)
+    assert np.array_equal(gpu.download(out, np.float32, (n,)), a + b)
+    gpu.step_gate_gelu(out, ab, bb, n)
+    assert np.allclose(gpu.download(out, np.float32, (n,)), orc.gate_gelu(a, b), rtol=1e-5, atol=1e-6)
+    h = gpu.alloc(n * 2)
+    gpu.step_cast_f32_f16(h, ab, n)
+    assert np.array_equal(gpu.download(h, np.float16, (n,)), a.astype(np.float16))
+
+    rows, m = 3, 262144
+    x = rng.standard_normal((rows, m)).astype(np.float32)
+    x[0, 1000] = x[0, 200000] = 50.0          # tie: the first maximum wins
+    x[1, 0] = 60.0
+    x[2, m - 1] = 70.0
+    xb = gpu.upload(x)
+    idx = gpu.alloc(rows * 4)
+    gpu.step_argmax(idx, xb, rows, m)
+    got = gpu.download(idx, np.int32, (rows,))
+    assert list(got) == list(orc.argmax(x)) == [1000, 0, m - 1]
+    for t in (ab, bb, out, h, xb, idx):
+        t.free()
+
+
+def test_gather_rows_f32_and_q8(gpu, orc):
+    rng = np.random.default_rng(4)
+    V, D = 50, 128
+    table = (rng.standard_normal((V, D)) * 0.3).astype(np.float32)
+    ids = np.array([49, 0, 7, 7, 13], np.int32)
+    ib = gpu.upload(ids)
+    out = gpu.alloc(ids.size * D * 4)
+    tb = gpu.upload(table)
+    gpu.step_gather_rows(be.F32, out, tb, ib, ids.size, D, V)
+    assert np.array_equal(gpu.download(out, np.float32, (ids.size, D)), table[ids])
+    blocks = be.quantize_blocks(be.Q8_0, table, 1)
+    qb = gpu.upload(blocks)
+    gpu.step_gather_rows(be.Q8_0, out, qb, ib, ids.size, D, V)
+    assert np.array_equal(gpu.download(out, np.float32, (ids.size, D)), orc.gather_rows(blocks, ids, D, dtype=orc.Q8_0))
+    for t in (ib, out, tb, qb):
+        t.free()
+
+
+def test_kv_append_f16_at_device_write_index(gpu, orc):
+    rng = np.random.default_rng(5)
+    B, S, T, H, D = 2, 3, 10, 1, 64
+    cache = np.zeros((B, T, H, D), np.float16)
+    cb = gpu.upload(cache)
+    for step, widx in enumerate([0, 3, 6]):
+        src = rng.standard_normal((B, S, H, D)).astype(np.float32)
+        sb, wb = gpu.upload(src), gpu.upload(np.array([widx], np.int32))
+        gpu.step_append_f16(cb, sb, wb, B, S, T, H * D)
+        cache[:, widx:widx + S] = orc.cast_f32_f16(src)
+        assert np.array_equal(gpu.download(cb, np.float16, cache.shape), cache)
+        sb.free(); wb.free()
+    # a write index that would run past the capacity writes only what fits
+    src = np.ones((B, S, H, D), np.float32)
+    sb, wb = gpu.upload(src), gpu.upload(np.array([8], np.int32))
+    gpu.step_append_f16(cb, sb, wb, B, S, T, H * D)
+    cache[:, 8:10] = 1.0
+    assert np.array_equal(gpu.download(cb, np.float16, cache.shape), cache)
+    for t in (cb, sb, wb):
+        t.free()
