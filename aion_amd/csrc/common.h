@@ -63,6 +63,8 @@ struct aionhip_weight {
     uint8_t *qs = nullptr;
     __half *sc = nullptr;
     size_t qs_bytes = 0, sc_bytes = 0;
+    // lazily built by the bf16 MFMA GEMM: the weight dequantized to bf16 [n][k]
+    unsigned short *bf16 = nullptr;
 };
 
 int set_err(aionhip_ctx *ctx, int status, const char *fmt, ...);

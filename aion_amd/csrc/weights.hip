@@ -182,6 +182,7 @@ void aionhip_weight_free(aionhip_ctx *ctx, aionhip_weight *w) {
     if (!w) return;
     if (ctx) (void)hipStreamSynchronize(ctx->stream);
     if (w->qs) (void)hipFree(w->qs);
+    if (w->bf16) (void)hipFree(w->bf16);
     delete w;
 }
 

@@ -171,7 +171,7 @@ def test_config2_decode_shapes(gpu, orc, dtype, layout, n, k):
 
 
 @pytest.mark.parametrize("dtype,layout", CASES)
-def test_exact_gemm_rows_above_eight(gpu, orc, dtype, layout):
+def test_exact_path_rows_above_eight(gpu, orc, dtype, layout):
     say("exact gemm", dtype, layout)
     m, n, k = 37, 200, 256
     blocks, w = make_weight(gpu, orc, dtype, layout, n, k, seed=77, std=0.1)
