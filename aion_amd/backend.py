@@ -47,6 +47,12 @@ class DeviceBuffer:
     def numpy(self, dtype, shape=None, offset=0):
         return self.backend.download(self, dtype, shape, offset)
 
+    def view(self, offset_bytes):
+        """A non-owning window starting `offset_bytes` into this allocation."""
+        v = DeviceBuffer(self.backend, self.handle + offset_bytes, self.nbytes - offset_bytes)
+        v.free = lambda: None
+        return v
+
 
 class Weight:
     def __init__(self, backend, ptr, dtype, layout, n, k):
@@ -158,6 +164,34 @@ class HipBackend:
     def step_matmul(self, weight, a_buf, m, c_buf, lda=0, ldc=0, alpha=1.0, beta=0.0, a_offset=0, c_offset=0):
         fn = self._lib.aionhip_step_matmul_nt if weight.layout == ROWS_NK else self._lib.aionhip_step_matmul
         self._check(fn(self._ctx, weight.ptr, m, a_buf.handle + a_offset, lda, c_buf.handle + c_offset, ldc, alpha, beta))
+
+    def step_matmul_batch(self, weights, a_buf, m, c_bufs, lda=0, alpha=1.0, beta=0.0, c_offsets=None):
+        n = len(weights)
+        ws = (C.c_void_p * n)(*[w.ptr.value for w in weights])
+        offs = c_offsets or [0] * n
+        cs = (C.c_uint64 * n)(*[b.handle + o for b, o in zip(c_bufs, offs)])
+        self._check(self._lib.aionhip_step_matmul_batch(self._ctx, n, ws, m, a_buf.handle, lda, cs, None, alpha, beta))
+
+    def step_add_i32(self, out, a, b, n):
+        self._check(self._lib.aionhip_step_add_i32(self._ctx, out.handle, a.handle, b.handle, n))
+
+    # ---- programs (HIP graph replay of a recorded step sequence)
+    def program_begin(self):
+        self._check(self._lib.aionhip_program_begin(self._ctx))
+
+    def program_end(self):
+        p = C.c_void_p()
+        self._check(self._lib.aionhip_program_end(self._ctx, C.byref(p)))
+        return p
+
+    def program_execute(self, prog):
+        self._check(self._lib.aionhip_program_execute(self._ctx, prog))
+
+    def program_node_count(self, prog):
+        return self._lib.aionhip_program_node_count(prog)
+
+    def program_destroy(self, prog):
+        self._lib.aionhip_program_destroy(self._ctx, prog)
 
     def matmul(self, weight, a, alpha=1.0, beta=0.0, c=None):
         """Convenience: numpy A [m,k] -> numpy C [m,n] through the step (uploads, runs, downloads)."""

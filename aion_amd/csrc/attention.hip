@@ -103,7 +103,10 @@ struct FlashCfg {
     static constexpr int LDS_BYTES = WG_LDS > MERGE_LDS ? WG_LDS : MERGE_LDS;
 };
 
-template <int KV, int D, bool SPLIT>
+// HILO: q and the probabilities are fed to the MFMAs as a high and a low half-precision part
+// (x = hi + lo, ~2x the mantissa), which keeps an f32 query path at f32-level accuracy; used when
+// q arrives as f32 (aion's cached decode: f32 q over an f16 cache). K and V are exact either way.
+template <int KV, int D, bool SPLIT, bool HILO>
 __global__ __launch_bounds__(256) void attn_flash_kernel(AttnArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     using Cfg = FlashCfg<D>;
@@ -135,19 +138,23 @@ __global__ __launch_bounds__(256) void attn_flash_kernel(AttnArgs a) {
     const int uni_hi = wave_max_i(hi > lo ? hi : 0);
 
     // ---- Q^T operand: 8 consecutive d of row n per k-step, converted to the K/V element type
-    u32x4 qf[KK];
+    u32x4 qf[KK], qf_lo[HILO ? KK : 1];
     {
         const size_t qbase = (((size_t)b * a.L + li) * a.Hq + hq) * D;
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) {
-            unsigned short h[8];
+            unsigned short h[8], lo8[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const float x = row_ok ? load_scalar(a.q, a.q_dtype, qbase + kk * 32 + g * 8 + j) : 0.f;
                 h[j] = to_half_bits<KV>(x);
+                lo8[j] = HILO ? to_half_bits<KV>(x - from_half_bits<KV>(h[j])) : (unsigned short)0;
             }
             qf[kk] = u32x4{(unsigned)h[0] | ((unsigned)h[1] << 16), (unsigned)h[2] | ((unsigned)h[3] << 16),
                            (unsigned)h[4] | ((unsigned)h[5] << 16), (unsigned)h[6] | ((unsigned)h[7] << 16)};
+            if (HILO)
+                qf_lo[kk] = u32x4{(unsigned)lo8[0] | ((unsigned)lo8[1] << 16), (unsigned)lo8[2] | ((unsigned)lo8[3] << 16),
+                                  (unsigned)lo8[4] | ((unsigned)lo8[5] << 16), (unsigned)lo8[6] | ((unsigned)lo8[7] << 16)};
         }
     }
 
@@ -202,6 +209,7 @@ __global__ __launch_bounds__(256) void attn_flash_kernel(AttnArgs a) {
             for (int kk = 0; kk < KK; ++kk) {
                 const u32x4 kf = *(const u32x4 *)(krow + kk * 32);
                 c = mfma16<KV>(kf, qf[kk], c);
+                if (HILO) c = mfma16<KV>(kf, qf_lo[kk], c);
             }
             s[h] = c;
         }
@@ -239,11 +247,16 @@ __global__ __launch_bounds__(256) void attn_flash_kernel(AttnArgs a) {
         rowsum += __shfl_xor(rowsum, 32, 64);
         l_run = l_run * alpha + rowsum;
         m_run = m_new;
-        u32x4 pf;
-        pf.x = (unsigned)to_half_bits<KV>(p[0]) | ((unsigned)to_half_bits<KV>(p[1]) << 16);
-        pf.y = (unsigned)to_half_bits<KV>(p[2]) | ((unsigned)to_half_bits<KV>(p[3]) << 16);
-        pf.z = (unsigned)to_half_bits<KV>(p[4]) | ((unsigned)to_half_bits<KV>(p[5]) << 16);
-        pf.w = (unsigned)to_half_bits<KV>(p[6]) | ((unsigned)to_half_bits<KV>(p[7]) << 16);
+        unsigned short ph[8], pl[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            ph[j] = to_half_bits<KV>(p[j]);
+            pl[j] = HILO ? to_half_bits<KV>(p[j] - from_half_bits<KV>(ph[j])) : (unsigned short)0;
+        }
+        const u32x4 pf = u32x4{(unsigned)ph[0] | ((unsigned)ph[1] << 16), (unsigned)ph[2] | ((unsigned)ph[3] << 16),
+                               (unsigned)ph[4] | ((unsigned)ph[5] << 16), (unsigned)ph[6] | ((unsigned)ph[7] << 16)};
+        const u32x4 pf_lo = u32x4{(unsigned)pl[0] | ((unsigned)pl[1] << 16), (unsigned)pl[2] | ((unsigned)pl[3] << 16),
+                                  (unsigned)pl[4] | ((unsigned)pl[5] << 16), (unsigned)pl[6] | ((unsigned)pl[7] << 16)};
 
         // the staged tile is written and read by this wavefront only
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -264,7 +277,9 @@ __global__ __launch_bounds__(256) void attn_flash_kernel(AttnArgs a) {
                                    (unsigned)e[4] | ((unsigned)e[5] << 16), (unsigned)e[6] | ((unsigned)e[7] << 16)};
             f32x4 c = acc[mt];
             c *= alpha;
-            acc[mt] = mfma16<KV>(vf, pf, c);
+            c = mfma16<KV>(vf, pf, c);
+            if (HILO) c = mfma16<KV>(vf, pf_lo, c);
+            acc[mt] = c;
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -398,7 +413,7 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(AttnArgs a, int d_k, 
     }
 }
 
-template <int KV, int D>
+template <int KV, int D, bool HILO>
 int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
     using Cfg = FlashCfg<D>;
     const int units = a.B * a.Hkv;
@@ -417,17 +432,17 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
             if (rc) return rc;
             a.partial = (float *)ctx->scratch2;
         }
-        HIP_TRY(ctx, hipFuncSetAttribute((const void *)attn_flash_kernel<KV, D, true>, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)attn_flash_kernel<KV, D, true, HILO>, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
         prof_begin(ctx, "attn_flash_split");
-        attn_flash_kernel<KV, D, true><<<dim3((unsigned)(a.row_tiles * nseg), (unsigned)units), dim3(256), Cfg::LDS_BYTES, ctx->stream>>>(a);
+        attn_flash_kernel<KV, D, true, HILO><<<dim3((unsigned)(a.row_tiles * nseg), (unsigned)units), dim3(256), Cfg::LDS_BYTES, ctx->stream>>>(a);
         if (nseg > 1) attn_merge_kernel<D><<<dim3((unsigned)a.row_tiles, (unsigned)units), dim3(256), 0, ctx->stream>>>(a);
         prof_end(ctx);
         LAUNCH_CHECK(ctx, "attn_flash_split");
     } else {
         a.nseg = 1;
-        HIP_TRY(ctx, hipFuncSetAttribute((const void *)attn_flash_kernel<KV, D, false>, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)attn_flash_kernel<KV, D, false, HILO>, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
         prof_begin(ctx, "attn_flash_prefill");
-        attn_flash_kernel<KV, D, false><<<dim3((unsigned)((a.row_tiles + 3) / 4), (unsigned)units), dim3(256), Cfg::LDS_BYTES, ctx->stream>>>(a);
+        attn_flash_kernel<KV, D, false, HILO><<<dim3((unsigned)((a.row_tiles + 3) / 4), (unsigned)units), dim3(256), Cfg::LDS_BYTES, ctx->stream>>>(a);
         prof_end(ctx);
         LAUNCH_CHECK(ctx, "attn_flash_prefill");
     }
@@ -436,9 +451,10 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
 
 template <int KV>
 int launch_flash_d(aionhip_ctx *ctx, AttnArgs &a, int d) {
-    if (d == 64) return launch_flash<KV, 64>(ctx, a);
-    if (d == 128) return launch_flash<KV, 128>(ctx, a);
-    return launch_flash<KV, 256>(ctx, a);
+    const bool hilo = a.q_dtype == AIONHIP_F32;
+    if (d == 64) return hilo ? launch_flash<KV, 64, true>(ctx, a) : launch_flash<KV, 64, false>(ctx, a);
+    if (d == 128) return hilo ? launch_flash<KV, 128, true>(ctx, a) : launch_flash<KV, 128, false>(ctx, a);
+    return hilo ? launch_flash<KV, 256, true>(ctx, a) : launch_flash<KV, 256, false>(ctx, a);
 }
 
 bool dtype_ok(int d) { return d == AIONHIP_F32 || d == AIONHIP_F16 || d == AIONHIP_BF16; }

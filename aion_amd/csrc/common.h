@@ -40,6 +40,8 @@ struct aionhip_ctx {
     // second scratch for GEMM staging (dequantized weights / bf16 activations / split-K partials)
     void *scratch2 = nullptr;
     size_t scratch2_bytes = 0;
+    // true between aionhip_program_begin/end: launches are captured, nothing may synchronise or allocate
+    bool capturing = false;
     // per-launch timing, off by default
     bool profiling = false;
     std::vector<ProfRecord> prof;
@@ -98,6 +100,8 @@ int launch_prepare_act(aionhip_ctx *ctx, const float *a, size_t lda, size_t m, s
 
 // ---- matmul back ends --------------------------------------------------------------------------
 int launch_gemv(aionhip_ctx *ctx, const aionhip_weight *w, int m, PreparedAct act, float *c, size_t ldc, float alpha, float beta);
+int launch_gemv_batch(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count, int m,
+                      PreparedAct act, float alpha, float beta);
 int launch_gemm_i8(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta);
 int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, const float *a, size_t lda, float *c, size_t ldc, float alpha, float beta);
 

@@ -20,6 +20,8 @@ int set_err(aionhip_ctx *ctx, int status, const char *fmt, ...) {
 
 static int grow(aionhip_ctx *ctx, void **buf, size_t *have, size_t bytes) {
     if (bytes <= *have) return AIONHIP_OK;
+    if (ctx->capturing)
+        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "scratch must grow to %zu bytes while a program is being recorded: run the steps once before recording", bytes);
     if (*buf) {
         // earlier launches may still read the old buffer
         HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
@@ -181,6 +183,7 @@ void aionhip_free(aionhip_ctx *ctx, aionhip_handle h) {
 int aionhip_h2d(aionhip_ctx *ctx, aionhip_handle dst, size_t dst_offset, const void *src, size_t bytes) {
     if (!ctx || !dst || (!src && bytes)) return AIONHIP_INVALID_ARGUMENT;
     if (!bytes) return AIONHIP_OK;
+    if (ctx->capturing) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "h2d synchronises and cannot be recorded into a program");
     // pageable source: hipMemcpyAsync stages and returns once `src` is consumed
     HIP_TRY(ctx, hipMemcpyAsync((char *)(uintptr_t)dst + dst_offset, src, bytes, hipMemcpyHostToDevice, ctx->stream));
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
@@ -190,6 +193,7 @@ int aionhip_h2d(aionhip_ctx *ctx, aionhip_handle dst, size_t dst_offset, const v
 int aionhip_d2h(aionhip_ctx *ctx, void *dst, aionhip_handle src, size_t src_offset, size_t bytes) {
     if (!ctx || !src || (!dst && bytes)) return AIONHIP_INVALID_ARGUMENT;
     if (!bytes) return AIONHIP_OK;
+    if (ctx->capturing) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "d2h synchronises and cannot be recorded into a program");
     HIP_TRY(ctx, hipMemcpyAsync(dst, (const char *)(uintptr_t)src + src_offset, bytes, hipMemcpyDeviceToHost, ctx->stream));
     HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
     return AIONHIP_OK;

@@ -14,15 +14,38 @@
 
 namespace {
 
+// Up to four weights that multiply the SAME activation rows (q/k/v, gate/up) run as one launch:
+// their rows are concatenated, a wavefront's row group never straddles two weights.
+struct GemvSeg {
+    const u32x4 *qs;
+    const __half *sc;
+    float *c;
+    size_t ldc;
+    int n;          // rows of this weight
+    int first_wave; // first wavefront of this segment
+};
+struct GemvBatch {
+    GemvSeg seg[4];
+    int count;
+    int total_waves;
+};
+
 template <int DT, int B, int R>
-__global__ __launch_bounds__(256) void gemv_kernel(const u32x4 *__restrict__ qs, const __half *__restrict__ sc,
-                                                   const u32x4 *__restrict__ aq, const float *__restrict__ a_scale,
-                                                   const int *__restrict__ a_sum, float *__restrict__ c,
-                                                   int N, int K, int m, size_t ldc, float alpha, float beta) {
+__global__ __launch_bounds__(256) void gemv_kernel(GemvBatch batch, const u32x4 *__restrict__ aq, const float *__restrict__ a_scale,
+                                                   const int *__restrict__ a_sum, int K, int m, float alpha, float beta) {
     const int lane = threadIdx.x & 63;
-    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int row0 = wave * R;
-    if (row0 >= N) return;
+    const int gwave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (gwave >= batch.total_waves) return;
+    int si = 0;
+#pragma unroll
+    for (int i = 1; i < 4; ++i)
+        if (i < batch.count && gwave >= batch.seg[i].first_wave) si = i;
+    const u32x4 *__restrict__ qs = batch.seg[si].qs;
+    const __half *__restrict__ sc = batch.seg[si].sc;
+    float *__restrict__ c = batch.seg[si].c;
+    const size_t ldc = batch.seg[si].ldc;
+    const int N = batch.seg[si].n;
+    const int row0 = (gwave - batch.seg[si].first_wave) * R;
     const int KB = K >> 5;
     constexpr bool Q8 = DT == AIONHIP_Q8_0;
     const int chunks = Q8 ? (K >> 4) : KB;      // 16-byte weight chunks per row
@@ -108,50 +131,56 @@ __global__ __launch_bounds__(256) void gemv_kernel(const u32x4 *__restrict__ qs,
 }
 
 template <int DT, int B>
-void launch_r(aionhip_ctx *ctx, const aionhip_weight *w, int m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
-    const int N = (int)w->n, K = (int)w->k;
+void launch_r(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count, int m,
+              PreparedAct act, float alpha, float beta) {
+    const int K = (int)ws[0]->k;
+    long n_total = 0;
+    for (int i = 0; i < count; ++i) n_total += (long)ws[i]->n;
     // rows per wavefront: enough wavefronts to give every CU ~8, then amortise activation loads
     const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
     int R = 4;
-    if ((long)N < (long)cus * 8 * 4) R = 2;
-    if ((long)N < (long)cus * 8 * 2) R = 1;
-    if (B >= 4 && R < 2 && N >= cus * 4) R = 2;   // batched rows are VALU-heavy: reuse the activation registers
-    const auto *qs = (const u32x4 *)w->qs;
+    if (n_total < (long)cus * 8 * 4) R = 2;
+    if (n_total < (long)cus * 8 * 2) R = 1;
+    if (B >= 4 && R < 2 && n_total >= cus * 4) R = 2;   // batched rows are VALU-heavy: reuse the activation registers
+    GemvBatch batch{};
+    batch.count = count;
+    int waves = 0;
+    for (int i = 0; i < count; ++i) {
+        batch.seg[i] = GemvSeg{(const u32x4 *)ws[i]->qs, ws[i]->sc, cs[i], ldcs[i], (int)ws[i]->n, waves};
+        waves += ((int)ws[i]->n + R - 1) / R;
+    }
+    batch.total_waves = waves;
     const auto *aq = (const u32x4 *)act.q;
-#define GO(RR)                                                                                          \
-    do {                                                                                                \
-        const int waves = (N + RR - 1) / RR;                                                            \
-        const dim3 grid((unsigned)((waves + 3) / 4)), block(256);                                       \
-        gemv_kernel<DT, B, RR><<<grid, block, 0, ctx->stream>>>(qs, w->sc, aq, act.scale, act.sum, c, N, K, m, ldc, alpha, beta); \
-    } while (0)
-    if (R == 4) GO(4);
-    else if (R == 2) GO(2);
-    else GO(1);
-#undef GO
+    const dim3 grid((unsigned)((waves + 3) / 4)), block(256);
+    if (R == 4) gemv_kernel<DT, B, 4><<<grid, block, 0, ctx->stream>>>(batch, aq, act.scale, act.sum, K, m, alpha, beta);
+    else if (R == 2) gemv_kernel<DT, B, 2><<<grid, block, 0, ctx->stream>>>(batch, aq, act.scale, act.sum, K, m, alpha, beta);
+    else gemv_kernel<DT, B, 1><<<grid, block, 0, ctx->stream>>>(batch, aq, act.scale, act.sum, K, m, alpha, beta);
 }
 
 template <int DT>
-void launch_b(aionhip_ctx *ctx, const aionhip_weight *w, int m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
-    if (m == 1) launch_r<DT, 1>(ctx, w, m, act, c, ldc, alpha, beta);
-    else if (m == 2) launch_r<DT, 2>(ctx, w, m, act, c, ldc, alpha, beta);
-    else if (m <= 4) launch_r<DT, 4>(ctx, w, m, act, c, ldc, alpha, beta);
-    else launch_r<DT, 8>(ctx, w, m, act, c, ldc, alpha, beta);
+void launch_b(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count, int m,
+              PreparedAct act, float alpha, float beta) {
+    if (m == 1) launch_r<DT, 1>(ctx, ws, cs, ldcs, count, m, act, alpha, beta);
+    else if (m == 2) launch_r<DT, 2>(ctx, ws, cs, ldcs, count, m, act, alpha, beta);
+    else if (m <= 4) launch_r<DT, 4>(ctx, ws, cs, ldcs, count, m, act, alpha, beta);
+    else launch_r<DT, 8>(ctx, ws, cs, ldcs, count, m, act, alpha, beta);
 }
 
 }  // namespace
 
-int launch_gemv(aionhip_ctx *ctx, const aionhip_weight *w, int m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
+int launch_gemv_batch(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count, int m,
+                      PreparedAct act, float alpha, float beta) {
     if (m < 1 || m > 8) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "gemv: m=%d outside 1..8", m);
-    if (w->dtype == AIONHIP_Q8_0) {
-        prof_begin(ctx, "gemv_q8");
-        launch_b<AIONHIP_Q8_0>(ctx, w, m, act, c, ldc, alpha, beta);
-        prof_end(ctx);
-        LAUNCH_CHECK(ctx, "gemv_q8");
-    } else {
-        prof_begin(ctx, "gemv_q4");
-        launch_b<AIONHIP_Q4_0>(ctx, w, m, act, c, ldc, alpha, beta);
-        prof_end(ctx);
-        LAUNCH_CHECK(ctx, "gemv_q4");
-    }
+    if (count < 1 || count > 4) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "gemv: %d weights in one launch (1..4)", count);
+    const char *name = ws[0]->dtype == AIONHIP_Q8_0 ? "gemv_q8" : "gemv_q4";
+    prof_begin(ctx, name);
+    if (ws[0]->dtype == AIONHIP_Q8_0) launch_b<AIONHIP_Q8_0>(ctx, ws, cs, ldcs, count, m, act, alpha, beta);
+    else launch_b<AIONHIP_Q4_0>(ctx, ws, cs, ldcs, count, m, act, alpha, beta);
+    prof_end(ctx);
+    LAUNCH_CHECK(ctx, name);
     return AIONHIP_OK;
+}
+
+int launch_gemv(aionhip_ctx *ctx, const aionhip_weight *w, int m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
+    return launch_gemv_batch(ctx, &w, &c, &ldc, 1, m, act, alpha, beta);
 }

@@ -1,0 +1,90 @@
+// Programs: a fixed sequence of steps recorded once and replayed per token.
+//
+// aion compiles a model into an ExecutableProgram (a step list, runtime/executable.zig) and its
+// WebGPU backend caches and replays the per-step dispatch state because a decode program is
+// identical every token (backend/gpu/frame.zig:77-86, backend/gpu/backend.zig:616-638). Here the
+// replayable form is a HIP graph: between aionhip_program_begin and aionhip_program_end the
+// ordinary aionhip_step_* calls are captured instead of executed. Everything that varies per token
+// (token id, positions, cache write index, kv length) lives in device buffers the steps read, so
+// the same graph is valid for every token.
+#include "common.h"
+
+#include <new>
+
+struct aionhip_program {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    size_t nodes = 0;
+};
+
+namespace {
+__global__ void add_i32_kernel(int *__restrict__ out, const int *__restrict__ a, const int *__restrict__ b, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = a[i] + b[i];
+}
+}  // namespace
+
+extern "C" {
+
+int aionhip_program_begin(aionhip_ctx *ctx) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (ctx->capturing) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "program_begin: already recording");
+    if (ctx->profiling) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "program_begin: stop profiling first (events cannot be captured)");
+    HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+    HIP_TRY(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    ctx->capturing = true;
+    return AIONHIP_OK;
+}
+
+int aionhip_program_end(aionhip_ctx *ctx, aionhip_program **out) {
+    if (!ctx || !out) return AIONHIP_INVALID_ARGUMENT;
+    *out = nullptr;
+    if (!ctx->capturing) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "program_end: not recording");
+    ctx->capturing = false;
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
+    if (e != hipSuccess || !graph) return set_err(ctx, AIONHIP_EXECUTION_FAILED, "hipStreamEndCapture: %s", hipGetErrorString(e));
+    aionhip_program *p = new (std::nothrow) aionhip_program();
+    if (!p) {
+        (void)hipGraphDestroy(graph);
+        return set_err(ctx, AIONHIP_OUT_OF_MEMORY, "host allocation failed");
+    }
+    p->graph = graph;
+    (void)hipGraphGetNodes(graph, nullptr, &p->nodes);
+    e = hipGraphInstantiate(&p->exec, graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(graph);
+        delete p;
+        return set_err(ctx, AIONHIP_EXECUTION_FAILED, "hipGraphInstantiate: %s", hipGetErrorString(e));
+    }
+    *out = p;
+    return AIONHIP_OK;
+}
+
+int aionhip_program_execute(aionhip_ctx *ctx, aionhip_program *prog) {
+    if (!ctx || !prog || !prog->exec) return AIONHIP_INVALID_ARGUMENT;
+    if (ctx->capturing) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "program_execute: a recording is open");
+    HIP_TRY(ctx, hipGraphLaunch(prog->exec, ctx->stream));
+    return AIONHIP_OK;
+}
+
+size_t aionhip_program_node_count(const aionhip_program *prog) { return prog ? prog->nodes : 0; }
+
+void aionhip_program_destroy(aionhip_ctx *ctx, aionhip_program *prog) {
+    if (!prog) return;
+    if (ctx) (void)hipStreamSynchronize(ctx->stream);
+    if (prog->exec) (void)hipGraphExecDestroy(prog->exec);
+    if (prog->graph) (void)hipGraphDestroy(prog->graph);
+    delete prog;
+}
+
+int aionhip_step_add_i32(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle a, aionhip_handle b, size_t n) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (!out || !a || !b) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "add_i32: null operand");
+    if (!n) return AIONHIP_OK;
+    add_i32_kernel<<<dim3((unsigned)((n + 63) / 64)), dim3(64), 0, ctx->stream>>>((int *)(uintptr_t)out, (const int *)(uintptr_t)a, (const int *)(uintptr_t)b, n);
+    LAUNCH_CHECK(ctx, "add_i32");
+    return AIONHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,249 @@
+"""Synthetic decoder-only transformer assembled from the backend's steps (BASELINE config 5).
+
+The step sequence is the one aion's graph compiler emits for a decoder (pattern of
+src/bench/models.zig:433-536, trimmed to a plain pre-norm block): Gather -> per layer
+[RMSNorm -> MatMul q,k,v -> RoPE1D(q,k) -> Cast f16 + SequenceAppend(k,v) -> Attention ->
+MatMul o -> add -> RMSNorm -> MatMul gate,up -> gate(gelu) -> MatMul down -> add] ->
+RMSNorm -> MatMul lm_head -> ArgMax. q4_0 weights are [K,N] quant_axis 0 MatMul operands (the
+only q4 layout aion has), q8_0 weights are [N,K] quant_axis 1 MatMulNT operands.
+
+Prefill runs the steps eagerly; the single-token decode step is recorded once into a program
+(HIP graph) and replayed per token. Token id, position, cache write index and kv length stay in
+device buffers: the argmax of one replay is the gather index of the next.
+"""
+import math
+from dataclasses import dataclass
+
+import numpy as np
+
+from . import backend as be
+
+
+@dataclass
+class DecoderConfig:
+    layers: int = 26
+    hidden: int = 2048
+    heads: int = 8
+    kv_heads: int = 1
+    head_dim: int = 256
+    ffn: int = 8192
+    vocab: int = 262144
+    max_seq: int = 256
+    eps: float = 1e-6
+    rope_base: float = 10000.0
+    wdtype: int = be.Q4_0
+
+    @property
+    def q_dim(self):
+        return self.heads * self.head_dim
+
+    @property
+    def kv_dim(self):
+        return self.kv_heads * self.head_dim
+
+
+def weight_shapes(cfg):
+    """name -> (n, k) of every quantized matmul weight (C[.., n] = A[.., k] @ W)."""
+    shapes = {}
+    for l in range(cfg.layers):
+        shapes["l%d.wq" % l] = (cfg.q_dim, cfg.hidden)
+        shapes["l%d.wk" % l] = (cfg.kv_dim, cfg.hidden)
+        shapes["l%d.wv" % l] = (cfg.kv_dim, cfg.hidden)
+        shapes["l%d.wo" % l] = (cfg.hidden, cfg.q_dim)
+        shapes["l%d.wgate" % l] = (cfg.ffn, cfg.hidden)
+        shapes["l%d.wup" % l] = (cfg.ffn, cfg.hidden)
+        shapes["l%d.wdown" % l] = (cfg.hidden, cfg.ffn)
+    shapes["lm_head"] = (cfg.vocab, cfg.hidden)
+    return shapes
+
+
+class SyntheticWeights:
+    """Seeded ~N(0,0.02) weights through the aion quantizers. A 2^22-sample normal pool is read at a
+    per-tensor offset and tiled, which keeps a 2-billion-parameter model's set-up to seconds; the
+    per-block statistics are those of N(0,0.02)."""
+
+    def __init__(self, cfg, seed=0):
+        self.cfg = cfg
+        rng = np.random.default_rng(seed)
+        self.pool = (rng.standard_normal(1 << 22) * 0.02).astype(np.float32)
+        self.seed = seed
+
+    def _values(self, name, count):
+        off = (hash_name(name) * 2654435761 + self.seed) % (self.pool.size - 1)
+        reps = -(-(count + off) // self.pool.size)
+        return np.tile(self.pool, reps)[off:off + count]
+
+    def blocks(self, name):
+        n, k = weight_shapes(self.cfg)[name]
+        v = self._values(name, n * k)
+        if self.cfg.wdtype == be.Q8_0:
+            return be.quantize_blocks(be.Q8_0, v.reshape(n, k), 1)       # [N,K] axis 1
+        return be.quantize_blocks(be.Q4_0, v.reshape(k, n), 0)           # [K,N] axis 0
+
+    def embed(self):
+        return self._values("embed", self.cfg.vocab * self.cfg.hidden).reshape(self.cfg.vocab, self.cfg.hidden).copy()
+
+
+def hash_name(name):
+    h = 2166136261
+    for ch in name.encode():
+        h = ((h ^ ch) * 16777619) & 0xFFFFFFFF
+    return h
+
+
+class Decoder:
+    def __init__(self, gpu, cfg, weights, on_weight=None):
+        """on_weight(name, host_array) is called for every tensor (the tests feed the oracle with it)."""
+        self.gpu, self.cfg = gpu, cfg
+        layout = be.ROWS_NK if cfg.wdtype == be.Q8_0 else be.KMAJOR_KN
+        self.w = {}
+        for name, (n, k) in weight_shapes(cfg).items():
+            blocks = weights.blocks(name)
+            self.w[name] = gpu.upload_weight(cfg.wdtype, layout, n, k, blocks)
+            if on_weight:
+                on_weight(name, blocks)
+        emb = weights.embed()
+        self.embed = gpu.upload(emb)
+        if on_weight:
+            on_weight("embed", emb)
+        ones = np.ones(cfg.hidden, np.float32)
+        self.gamma = gpu.upload(ones)          # every RMSNorm uses gamma = 1 (config 5)
+        if on_weight:
+            for l in range(cfg.layers):
+                on_weight("l%d.norm1" % l, ones)
+                on_weight("l%d.norm2" % l, ones)
+            on_weight("norm_f", ones)
+        kv_bytes = cfg.max_seq * cfg.kv_dim * 2
+        self.kc = [gpu.zeros(kv_bytes) for _ in range(cfg.layers)]
+        self.vc = [gpu.zeros(kv_bytes) for _ in range(cfg.layers)]
+        self.one = gpu.upload(np.ones(1, np.int32))
+        self.logits = gpu.alloc(cfg.vocab * 4)
+        self.token = gpu.alloc(4)
+        self.state = {}        # S -> activation buffers
+        self.program = None
+        self.pos = 0
+
+    def _buffers(self, s):
+        if s in self.state:
+            return self.state[s]
+        c, g = self.cfg, self.gpu
+        f = 4 * s
+        b = {
+            "ids": g.alloc(4 * s), "positions": g.alloc(4 * s), "write_index": g.alloc(4), "kv_len": g.alloc(4),
+            "x": g.alloc(f * c.hidden), "h": g.alloc(f * c.hidden), "o": g.alloc(f * c.hidden),
+            "q": g.alloc(f * c.q_dim), "qr": g.alloc(f * c.q_dim), "att": g.alloc(f * c.q_dim),
+            "k": g.alloc(f * c.kv_dim), "kr": g.alloc(f * c.kv_dim), "v": g.alloc(f * c.kv_dim),
+            "gate": g.alloc(f * c.ffn), "up": g.alloc(f * c.ffn), "act": g.alloc(f * c.ffn),
+            "hl": g.alloc(4 * c.hidden),
+        }
+        self.state[s] = b
+        return b
+
+    def _forward(self, s, b):
+        """Launches every step of one forward pass over `s` tokens (eagerly, or into an open recording)."""
+        c, g = self.cfg, self.gpu
+        g.step_gather_rows(be.F32, b["x"], self.embed, b["ids"], s, c.hidden, c.vocab)
+        scale = 1.0 / math.sqrt(c.head_dim)
+        for l in range(c.layers):
+            p = "l%d." % l
+            g.step_rmsnorm(b["h"], b["x"], self.gamma, s, c.hidden, c.eps)
+            g.step_matmul_batch([self.w[p + "wq"], self.w[p + "wk"], self.w[p + "wv"]], b["h"], s, [b["q"], b["k"], b["v"]])
+            g.step_rope(b["qr"], b["q"], b["positions"], 1, s, c.heads, c.head_dim, base=c.rope_base)
+            g.step_rope(b["kr"], b["k"], b["positions"], 1, s, c.kv_heads, c.head_dim, base=c.rope_base)
+            g.step_append_f16(self.kc[l], b["kr"], b["write_index"], 1, s, c.max_seq, c.kv_dim)
+            g.step_append_f16(self.vc[l], b["v"], b["write_index"], 1, s, c.max_seq, c.kv_dim)
+            g.step_attention(b["att"], b["qr"], self.kc[l], self.vc[l], (1, s, c.max_seq, c.heads, c.kv_heads, c.head_dim, c.head_dim),
+                             scale, q_dtype=be.F32, kv_dtype=be.F16, window=be.CAUSAL,
+                             query_positions=b["positions"], kv_lengths=b["kv_len"])
+            g.step_matmul(self.w[p + "wo"], b["att"], s, b["o"])
+            g.step_add(b["x"], b["x"], b["o"], s * c.hidden)
+            g.step_rmsnorm(b["h"], b["x"], self.gamma, s, c.hidden, c.eps)
+            g.step_matmul_batch([self.w[p + "wgate"], self.w[p + "wup"]], b["h"], s, [b["gate"], b["up"]])
+            g.step_gate_gelu(b["act"], b["gate"], b["up"], s * c.ffn)
+            g.step_matmul(self.w[p + "wdown"], b["act"], s, b["o"])
+            g.step_add(b["x"], b["x"], b["o"], s * c.hidden)
+        last = b["x"].view((s - 1) * c.hidden * 4)
+        g.step_rmsnorm(b["hl"], last, self.gamma, 1, c.hidden, c.eps)
+        g.step_matmul(self.w["lm_head"], b["hl"], 1, self.logits)
+        g.step_argmax(self.token, self.logits, 1, c.vocab)
+
+    def reset(self):
+        self.pos = 0
+
+    def prefill(self, tokens):
+        """Runs the prompt (positions pos .. pos+len-1); returns the greedy next token."""
+        t = np.ascontiguousarray(tokens, np.int32)
+        s = t.size
+        if self.pos + s > self.cfg.max_seq:
+            raise ValueError("prompt exceeds the cache capacity")
+        b = self._buffers(s)
+        g = self.gpu
+        g.write(b["ids"], t)
+        g.write(b["positions"], np.arange(self.pos, self.pos + s, dtype=np.int32))
+        g.write(b["write_index"], np.array([self.pos], np.int32))
+        g.write(b["kv_len"], np.array([self.pos + s], np.int32))
+        self._forward(s, b)
+        self.pos += s
+        return int(g.download(self.token, np.int32, (1,))[0])
+
+    def logits_host(self):
+        return self.gpu.download(self.logits, np.float32, (self.cfg.vocab,))
+
+    def begin_decode(self, first_token):
+        """Prepares the single-token state and records the decode program (one warm-up step runs
+        eagerly first so that every scratch buffer has its final size; it is then rolled back)."""
+        g = self.gpu
+        b = self._buffers(1)
+        self._set_decode_state(b, first_token, self.pos)
+        if self.program is None:
+            self._forward(1, b)                      # eager warm-up at the current position
+            g.sync()
+            self._set_decode_state(b, first_token, self.pos)
+            g.program_begin()
+            self._forward(1, b)
+            # advance the device-resident loop state: next id = argmax, positions/write index/kv length += 1
+            g._check(g._lib.aionhip_d2d(g._ctx, b["ids"].handle, 0, self.token.handle, 0, 4))
+            g.step_add_i32(b["positions"], b["positions"], self.one, 1)
+            g.step_add_i32(b["write_index"], b["write_index"], self.one, 1)
+            g.step_add_i32(b["kv_len"], b["kv_len"], self.one, 1)
+            self.program = g.program_end()
+
+    def _set_decode_state(self, b, token, pos):
+        g = self.gpu
+        g.write(b["ids"], np.array([token], np.int32))
+        g.write(b["positions"], np.array([pos], np.int32))
+        g.write(b["write_index"], np.array([pos], np.int32))
+        g.write(b["kv_len"], np.array([pos + 1], np.int32))
+
+    def decode_step(self, read_token=True):
+        """Replays the decode program once; returns the token it produced (a 4-byte read-back)."""
+        if self.pos + 1 > self.cfg.max_seq:
+            raise ValueError("cache capacity exhausted")
+        self.gpu.program_execute(self.program)
+        self.pos += 1
+        if read_token:
+            return int(self.gpu.download(self.token, np.int32, (1,))[0])
+        return None
+
+    def decode_step_eager(self, token):
+        """The same step without a program (used by tests to check the replayed graph)."""
+        b = self._buffers(1)
+        self._set_decode_state(b, token, self.pos)
+        self._forward(1, b)
+        self.pos += 1
+        return int(self.gpu.download(self.token, np.int32, (1,))[0])
+
+    def close(self):
+        if self.program is not None:
+            self.gpu.program_destroy(self.program)
+            self.program = None
+        for w in self.w.values():
+            w.free()
+        for lst in (self.kc, self.vc):
+            for t in lst:
+                t.free()
+        for bufs in self.state.values():
+            for t in bufs.values():
+                t.free()
+        for t in (self.embed, self.gamma, self.one, self.logits, self.token):
+            t.free()

@@ -53,6 +53,13 @@ _SIGS = {
     "aionhip_weight_download": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
     "aionhip_step_matmul": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint64, C.c_size_t, C.c_uint64, C.c_size_t, C.c_float, C.c_float]),
     "aionhip_step_matmul_nt": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint64, C.c_size_t, C.c_uint64, C.c_size_t, C.c_float, C.c_float]),
+    "aionhip_step_matmul_batch": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_void_p), C.c_size_t, C.c_uint64, C.c_size_t, C.POINTER(C.c_uint64), C.POINTER(C.c_size_t), C.c_float, C.c_float]),
+    "aionhip_step_add_i32": (C.c_int, [C.c_void_p] + [C.c_uint64] * 3 + [C.c_size_t]),
+    "aionhip_program_begin": (C.c_int, [C.c_void_p]),
+    "aionhip_program_end": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p)]),
+    "aionhip_program_execute": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "aionhip_program_node_count": (C.c_size_t, [C.c_void_p]),
+    "aionhip_program_destroy": (None, [C.c_void_p, C.c_void_p]),
     "aionhip_set_gemm_mode": (C.c_int, [C.c_void_p, C.c_int]),
     "aionhip_step_attention": (C.c_int, [C.c_void_p, C.POINTER(Attention)]),
     "aionhip_step_rmsnorm": (C.c_int, [C.c_void_p] + [C.c_uint64] * 5 + [C.c_size_t, C.c_size_t, C.c_float]),

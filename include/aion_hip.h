@@ -126,6 +126,15 @@ int aionhip_step_matmul(aionhip_ctx *ctx, const aionhip_weight *b, size_t m,
 int aionhip_step_matmul_nt(aionhip_ctx *ctx, const aionhip_weight *b, size_t m,
                            aionhip_handle a, size_t lda, aionhip_handle c, size_t ldc, float alpha, float beta);
 
+/* Several matmul steps that read the SAME activation (q/k/v, gate/up) as one call: the activation
+ * is prepared once and, for m <= 8, all weights stream through one launch. aion keeps such
+ * siblings as separate MatMul/MatMulNT steps (graph/opt/weight_layout.zig:72-115 re-lays but never
+ * concatenates); every C[i] is what the separate step would have produced. count <= 4; weights
+ * share k and dtype; ldc may be NULL (each n). */
+int aionhip_step_matmul_batch(aionhip_ctx *ctx, size_t count, const aionhip_weight *const *b, size_t m,
+                              aionhip_handle a, size_t lda, const aionhip_handle *c, const size_t *ldc,
+                              float alpha, float beta);
+
 /* How m > 8 rows are multiplied. EXACT_I8 (default): int8 activations, integer MFMA, per-block
  * f32 scaling - the same numbers as the decode path. BF16_MFMA: weights dequantized to bf16,
  * activations rounded to bf16, f32 accumulation - faster, judged at 1e-2 instead of 2e-3. */
@@ -175,6 +184,23 @@ int aionhip_step_append_f16(aionhip_ctx *ctx, aionhip_handle cache, aionhip_hand
 int aionhip_step_cast_f32_f16(aionhip_ctx *ctx, aionhip_handle out_f16, aionhip_handle x_f32, size_t n);
 /* StepArgMax over the last axis, first maximum wins (cpu/exec/argmax.zig:56-81); out i32 [rows] */
 int aionhip_step_argmax(aionhip_ctx *ctx, aionhip_handle out_i32, aionhip_handle x, size_t rows, size_t n);
+
+/* i32 elementwise add (StepElemwiseBinary on i32, cpu/exec/elementwise.zig): advances positions,
+ * the cache write index and kv lengths on the device between replays of a decode program */
+int aionhip_step_add_i32(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle a, aionhip_handle b, size_t n);
+
+/* ---- programs: record a fixed step sequence once, replay it per token ----------------------
+ * Session.execute(prog) (backend/backend.zig:42-44) runs aion's ExecutableProgram step list; the
+ * WebGPU backend replays cached dispatch state because a decode program is identical every token
+ * (backend/gpu/frame.zig:77-86). Between program_begin and program_end the aionhip_step_* calls
+ * are recorded into a HIP graph instead of executed; program_execute replays it (asynchronous).
+ * While recording: no h2d/d2h/free/sync, no profiling, and scratch cannot grow - run the same
+ * steps once eagerly first. Per-token inputs must live in device buffers the steps read. */
+int aionhip_program_begin(aionhip_ctx *ctx);
+int aionhip_program_end(aionhip_ctx *ctx, aionhip_program **out);
+int aionhip_program_execute(aionhip_ctx *ctx, aionhip_program *prog);
+size_t aionhip_program_node_count(const aionhip_program *prog);
+void aionhip_program_destroy(aionhip_ctx *ctx, aionhip_program *prog);
 
 /* ---- timing helpers for the roofline harness (timestamp queries of the WebGPU backend,
  *      backend/gpu/timestamp_profile.zig, reduced to stream events) ------------------------- */

@@ -705,7 +705,11 @@ int32_t orc_decoder_forward(orc_decoder *d, const int32_t *tokens, size_t s, siz
         as.scale = 1.0f / std::sqrt((float)c.head_dim); as.soft_cap = 0.0f;
         as.win_left = 0xFFFFFFFFu; as.win_right = 0; as.win_chunk = 0; as.kv_dtype = 1;
         const int32_t end = (int32_t)(pos0 + s);
-        if (orc_attention_blocked(&as, qr.data(), d->kc[l].data(), d->vc[l].data(), pos.data(), &end, att.data(), 1)) return -1;
+        if (c.attn_exact) {
+            if (orc_attention_f64(&as, qr.data(), d->kc[l].data(), d->vc[l].data(), pos.data(), &end, att.data())) return -1;
+        } else if (orc_attention_blocked(&as, qr.data(), d->kc[l].data(), d->vc[l].data(), pos.data(), &end, att.data(), 1)) {
+            return -1;
+        }
         if (d->matmul(wname(l, "wo"), s, H, QD, att.data(), o.data())) return -1;
         for (size_t i = 0; i < s * H; ++i) x[i] += o[i];
         orc_rmsnorm(x.data(), (const float *)g2->data(), nullptr, nullptr, s, H, c.eps, h.data());

@@ -124,6 +124,8 @@ typedef struct {
     size_t layers, hidden, heads, kv_heads, head_dim, ffn, vocab, max_seq;
     float eps, rope_base;
     int wdtype;
+    int attn_exact; /* 0: blocked attention with the polynomial exp (aion's CPU path); 1: textbook f64
+                       softmax - used to measure how far the CPU path itself moves under a 4e-5 change */
 } orc_decoder_cfg;
 typedef struct orc_decoder orc_decoder;
 orc_decoder *orc_decoder_create(const orc_decoder_cfg *cfg, int threads);

@@ -253,15 +253,15 @@ def cast_f32_f16(x):
 
 class _DecCfg(C.Structure):
     _fields_ = [(n, C.c_size_t) for n in ("layers", "hidden", "heads", "kv_heads", "head_dim", "ffn", "vocab", "max_seq")] + [
-        ("eps", C.c_float), ("rope_base", C.c_float), ("wdtype", C.c_int)]
+        ("eps", C.c_float), ("rope_base", C.c_float), ("wdtype", C.c_int), ("attn_exact", C.c_int)]
 
 
 class Decoder:
     """The synthetic decoder run through the oracle kernels (see orc_decoder_* in aion_oracle.h)."""
 
     def __init__(self, layers, hidden, heads, kv_heads, head_dim, ffn, vocab, max_seq,
-                 eps=1e-6, rope_base=10000.0, wdtype=Q4_0, threads=1):
-        self.cfg = _DecCfg(layers, hidden, heads, kv_heads, head_dim, ffn, vocab, max_seq, eps, rope_base, wdtype)
+                 eps=1e-6, rope_base=10000.0, wdtype=Q4_0, threads=1, attn_exact=False):
+        self.cfg = _DecCfg(layers, hidden, heads, kv_heads, head_dim, ffn, vocab, max_seq, eps, rope_base, wdtype, 1 if attn_exact else 0)
         self.vocab = vocab
         self._h = _lib.orc_decoder_create(C.byref(self.cfg), threads)
 
