@@ -15,6 +15,9 @@ cpu_baseline = the oracle's restatement of the aion CPU kernel for this op (pack
 M=1, aion cpu/exec/matmul.zig) timed on this host's cores on a bounded sample.
 
 `--sweep` adds the q8 legs and batch 4 / 8 (per-shape kernel GB/s) in a "sweep" object.
+`--extras gemm,attention,decoder` adds the other BASELINE configs (prefill GEMM TFLOP/s, attention
+TFLOP/s and GB/s, end-to-end decode tokens/s of the synthetic 26-layer decoder) in an "extras"
+object of the same JSON line.
 """
 import argparse
 import json
@@ -54,6 +57,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--sweep", action="store_true", help="also time q8 and batch 4/8 per shape")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--extras", default="", help="comma list of gemm,attention,decoder")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend is single-GPU (aion runs one program on one device); --gpus %d is not supported" % args.gpus)
@@ -134,6 +138,19 @@ def main():
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(host_blocks, batch)
 
+    extras = [e for e in args.extras.split(",") if e]
+    if extras:
+        for ws in sets:
+            for w in ws:
+                w.free()
+        out["extras"] = {}
+        if "gemm" in extras:
+            out["extras"]["prefill_gemm"] = run_gemm(gpu, be)
+        if "attention" in extras:
+            out["extras"]["attention"] = run_attention(gpu, be)
+        if "decoder" in extras:
+            out["extras"]["decoder"] = run_decoder(gpu, be, with_cpu=not args.no_cpu)
+
     out["config"]["setup_s"] = round(setup_s, 1)
     print(json.dumps(out))
     gpu.close()
@@ -169,6 +186,185 @@ def run_sweep(gpu, be, q4_blocks):
                 x.free(); y.free()
             for w in ws:
                 w.free()
+    return res
+
+
+MFMA_PEAK = {"bf16": 2500.0, "int8": 5000.0}   # dense TFLOP/s (TOP/s)
+
+
+def run_gemm(gpu, be):
+    """BASELINE config 3: M in {512, 2048}, K = 4096, N in {4096, 14336}; kernel time from per-launch events."""
+    res = {}
+    rng = np.random.default_rng(3)
+    k = 4096
+    for dtype, layout, tag in ((be.Q4_0, be.KMAJOR_KN, "q4"), (be.Q8_0, be.ROWS_NK, "q8")):
+        for n in (4096, 14336):
+            w = gpu.upload_weight(dtype, layout, n, k, synth_blocks(be, dtype, layout, n, k, seed=n))
+            for m in (512, 2048):
+                x = gpu.upload(rng.standard_normal((m, k)).astype(np.float32))
+                y = gpu.alloc(m * n * 4)
+                for mode, kname, peak in ((be.GEMM_BF16_MFMA, "gemm_bf16", "bf16"), (be.GEMM_EXACT_I8, "gemm_i8_" + tag, "int8")):
+                    gpu.set_gemm_mode(mode)
+                    for _ in range(2):
+                        gpu.step_matmul(w, x, m, y)
+                    gpu.sync()
+                    gpu.profile_start()
+                    t0 = time.perf_counter()
+                    for _ in range(10):
+                        gpu.step_matmul(w, x, m, y)
+                    prof = [ms for (nm, ms) in gpu.profile_stop() if nm == kname]
+                    wall = (time.perf_counter() - t0) / 10
+                    ms = sum(prof) / len(prof)
+                    tf = 2.0 * m * n * k / (ms * 1e-3) / 1e12
+                    res["%s M%d N%d %s" % (tag, m, n, "bf16" if mode == be.GEMM_BF16_MFMA else "exact_i8")] = {
+                        "kernel_ms": round(ms, 4), "step_wall_ms": round(wall * 1e3, 4), "TFLOPs": round(tf, 1),
+                        "frac_mfma_peak": round(tf / MFMA_PEAK[peak], 4), "peak": peak}
+                x.free(); y.free()
+            w.free()
+    gpu.set_gemm_mode(be.GEMM_EXACT_I8)
+    return res
+
+
+def _bf16_bits(x):
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def run_attention(gpu, be):
+    """BASELINE config 4: 8 q heads / 1 kv head, head_dim 256, bf16 Q/K/V, scale 1/16, causal."""
+    res = {}
+    rng = np.random.default_rng(4)
+    Hq, Hkv, D = 8, 1, 256
+
+    def timed(name, shape, bufs, pos=None, kl=None, iters=10):
+        for _ in range(2):
+            gpu.step_attention(bufs[3], bufs[0], bufs[1], bufs[2], shape, 1 / 16.0, q_dtype=be.BF16, kv_dtype=be.BF16,
+                               query_positions=pos, kv_lengths=kl)
+        gpu.sync()
+        gpu.profile_start()
+        for _ in range(iters):
+            gpu.step_attention(bufs[3], bufs[0], bufs[1], bufs[2], shape, 1 / 16.0, q_dtype=be.BF16, kv_dtype=be.BF16,
+                               query_positions=pos, kv_lengths=kl)
+        prof = [ms for (nm, ms) in gpu.profile_stop() if nm == name]
+        return sum(prof) / len(prof)
+
+    for L in (1024, 4096):
+        q = gpu.upload(_bf16_bits(rng.standard_normal((1, L, Hq, D))))
+        k = gpu.upload(_bf16_bits(rng.standard_normal((1, L, Hkv, D))))
+        v = gpu.upload(_bf16_bits(rng.standard_normal((1, L, Hkv, D))))
+        o = gpu.alloc(L * Hq * D * 4)
+        ms = timed("attn_flash_prefill", (1, L, L, Hq, Hkv, D, D), (q, k, v, o))
+        flops = 4.0 * Hq * D * L * (L + 1) / 2
+        tf = flops / (ms * 1e-3) / 1e12
+        res["prefill L%d" % L] = {"kernel_ms": round(ms, 4), "TFLOPs": round(tf, 1), "frac_mfma_peak": round(tf / MFMA_PEAK["bf16"], 4)}
+        for t in (q, k, v, o):
+            t.free()
+    for T in (1024, 4096, 16384):
+        for B in (1, 8):
+            q = gpu.upload(_bf16_bits(rng.standard_normal((B, 1, Hq, D))))
+            k = gpu.upload(_bf16_bits(rng.standard_normal((B, T, Hkv, D))))
+            v = gpu.upload(_bf16_bits(rng.standard_normal((B, T, Hkv, D))))
+            o = gpu.alloc(B * Hq * D * 4)
+            pos = gpu.upload(np.full((B, 1), T - 1, np.int32))
+            kl = gpu.upload(np.full((B,), T, np.int32))
+            ms = timed("attn_flash_split", (B, 1, T, Hq, Hkv, D, D), (q, k, v, o), pos, kl, iters=20)
+            by = B * 2 * T * Hkv * D * 2 + B * Hq * D * (2 + 4)
+            res["decode T%d B%d" % (T, B)] = {"kernel_us": round(ms * 1e3, 2), "GBps": round(by / (ms * 1e-3) / 1e9, 1),
+                                              "frac_hbm_peak": round(by / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+            for t in (q, k, v, o, pos, kl):
+                t.free()
+    return res
+
+
+def run_decoder(gpu, be, with_cpu=True):
+    """BASELINE config 5: 26 layers, hidden 2048, 8 heads / 1 kv head, head_dim 256, GeGLU 8192, vocab 262144,
+    q4 weights; 128-token prompt, greedy decode of 128 tokens at batch 1."""
+    from aion_amd.decoder import Decoder, DecoderConfig, SyntheticWeights, weight_shapes
+    cfg = DecoderConfig()
+    t0 = time.time()
+    oracle = None
+    if with_cpu:
+        from oracle import oracle as orc
+        threads = min(16, os.cpu_count() or 1)
+        oracle = orc.Decoder(cfg.layers, cfg.hidden, cfg.heads, cfg.kv_heads, cfg.head_dim, cfg.ffn, cfg.vocab, cfg.max_seq,
+                             eps=cfg.eps, rope_base=cfg.rope_base, wdtype=cfg.wdtype, threads=threads)
+    dec = Decoder(gpu, cfg, SyntheticWeights(cfg, 0), on_weight=oracle.set_weight if oracle else None)
+    setup_s = time.time() - t0
+    prompt = np.random.default_rng(5).integers(0, cfg.vocab, 128).astype(np.int32)
+    weight_bytes = sum(n * k // 32 * 18 for (n, k) in weight_shapes(cfg).values())
+
+    gpu.set_gemm_mode(be.GEMM_BF16_MFMA)
+    dec.prefill(prompt); dec.reset()             # warm-up (builds the bf16 weight copies, sizes scratch)
+    gpu.sync()
+    t = time.perf_counter()
+    tok = dec.prefill(prompt)
+    prefill_ms = (time.perf_counter() - t) * 1e3
+    gpu.set_gemm_mode(be.GEMM_EXACT_I8)
+    dec.reset()
+    tok_exact = dec.prefill(prompt)              # the decode continues from the exact-arithmetic prefill
+    first = tok_exact
+    dec.begin_decode(first)
+    gpu.sync()
+    tokens = []
+    t = time.perf_counter()
+    for _ in range(128):
+        tokens.append(dec.decode_step())
+    gpu.sync()
+    decode_s = time.perf_counter() - t
+    # the same 128 steps without reading the token back each step (device-resident greedy loop)
+    dec.pos = 128
+    dec.begin_decode(first)
+    gpu.sync()
+    t = time.perf_counter()
+    for _ in range(128):
+        dec.decode_step(read_token=False)
+    gpu.sync()
+    decode_nosync_s = time.perf_counter() - t
+    res = {
+        "config": "26 layers, hidden 2048, 8q/1kv heads x 256, ffn 8192 (GeGLU), vocab 262144, q4_0 weights, f16 KV cache, prompt 128, greedy 128, batch 1",
+        "setup_s": round(setup_s, 1),
+        "prefill_128_ms_bf16_mfma": round(prefill_ms, 3),
+        "prefill_tokens_per_s": round(128 / (prefill_ms * 1e-3), 1),
+        "prefill_next_token_bf16_vs_exact": [int(tok), int(tok_exact)],
+        "decode_tokens_per_s": round(128 / decode_s, 1),
+        "decode_ms_per_token": round(decode_s / 128 * 1e3, 4),
+        "decode_tokens_per_s_no_readback": round(128 / decode_nosync_s, 1),
+        "decode_weight_GBps": round(weight_bytes / (decode_nosync_s / 128) / 1e9, 1),
+        "weight_bytes_per_token": weight_bytes,
+        "program_nodes": int(gpu.program_node_count(dec.program)),
+    }
+    if oracle is not None:
+        # CPU reference-algorithm baseline + parity on a bounded sample: the prompt and 4 decode steps
+        t = time.perf_counter()
+        otok, ologits = oracle.forward(prompt, 0)
+        cpu_prefill_s = time.perf_counter() - t
+        dec.reset()
+        gtok = dec.prefill(prompt)
+        glogits = dec.logits_host()
+        rms = float(np.sqrt((ologits.astype(np.float64) ** 2).mean()))
+        agree = [int(gtok == otok)]
+        errs = [float(np.abs(glogits - ologits).max()) / rms]
+        dec.begin_decode(gtok)
+        fed = gtok
+        t = time.perf_counter()
+        n_cpu = 4
+        cpu_decode_s = 0.0
+        for i in range(n_cpu):
+            g_next = dec.decode_step()
+            glogits = dec.logits_host()
+            t = time.perf_counter()
+            o_next, ologits = oracle.forward(np.array([fed], np.int32), 128 + i)
+            cpu_decode_s += time.perf_counter() - t
+            rms = float(np.sqrt((ologits.astype(np.float64) ** 2).mean()))
+            errs.append(float(np.abs(glogits - ologits).max()) / rms)
+            agree.append(int(g_next == o_next))
+            fed = g_next
+        res["cpu_reference"] = {"kind": "port", "cores": min(16, os.cpu_count() or 1),
+                                "prefill_128_s": round(cpu_prefill_s, 2), "decode_tokens_per_s": round(n_cpu / cpu_decode_s, 3),
+                                "sample": "prompt + %d teacher-forced decode steps" % n_cpu,
+                                "gpu_vs_cpu_logits_max_err_over_rms": [round(e, 4) for e in errs],
+                                "greedy_token_agreement": agree}
+    dec.close()
     return res
 
 
