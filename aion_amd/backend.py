@@ -172,6 +172,21 @@ class HipBackend:
         cs = (C.c_uint64 * n)(*[b.handle + o for b, o in zip(c_bufs, offs)])
         self._check(self._lib.aionhip_step_matmul_batch(self._ctx, n, ws, m, a_buf.handle, lda, cs, None, alpha, beta))
 
+    def step_rmsnorm_matmul(self, weights, x, gamma, rows, c_bufs, eps, beta_norm=None, alpha=1.0, beta=0.0):
+        n = len(weights)
+        ws = (C.c_void_p * n)(*[w.ptr.value for w in weights])
+        cs = (C.c_uint64 * n)(*[b.handle for b in c_bufs])
+        self._check(self._lib.aionhip_step_rmsnorm_matmul(self._ctx, n, ws, rows, x.handle, gamma.handle,
+                                                          beta_norm.handle if beta_norm is not None else 0, eps, cs, None, alpha, beta))
+
+    def step_gate_matmul(self, weight, gate, up, rows, c_buf, alpha=1.0, beta=0.0):
+        self._check(self._lib.aionhip_step_gate_matmul(self._ctx, weight.ptr, rows, gate.handle, up.handle, c_buf.handle, 0, alpha, beta))
+
+    def step_rope_append(self, q_out, q, k, v, k_cache, v_cache, positions, write_index, b, s, t_cap, h_q, h_kv, d,
+                         base=10000.0, scale_factor=1.0, proportion=1.0):
+        self._check(self._lib.aionhip_step_rope_append(self._ctx, q_out.handle, q.handle, k.handle, v.handle, k_cache.handle, v_cache.handle,
+                                                       positions.handle, write_index.handle, b, s, t_cap, h_q, h_kv, d, base, scale_factor, proportion))
+
     def step_add_i32(self, out, a, b, n):
         self._check(self._lib.aionhip_step_add_i32(self._ctx, out.handle, a.handle, b.handle, n))
 

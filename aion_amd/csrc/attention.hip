@@ -141,14 +141,29 @@ __global__ __launch_bounds__(256) void attn_flash_kernel(AttnArgs a) {
     u32x4 qf[KK], qf_lo[HILO ? KK : 1];
     {
         const size_t qbase = (((size_t)b * a.L + li) * a.Hq + hq) * D;
+        const bool q_f32_vec = a.q_dtype == AIONHIP_F32 && (((uintptr_t)a.q) & 15) == 0;
+        const bool q_same = a.q_dtype == KV && (((uintptr_t)a.q) & 15) == 0;
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) {
+            if (q_same) {            // already in the MFMA element type: one 16-byte load
+                qf[kk] = row_ok ? *(const u32x4 *)((const unsigned short *)a.q + qbase + kk * 32 + g * 8) : u32x4{0u, 0u, 0u, 0u};
+                if (HILO) qf_lo[kk] = u32x4{0u, 0u, 0u, 0u};
+                continue;
+            }
+            float x[8];
+            if (q_f32_vec) {
+                const f32x4 *qp = (const f32x4 *)((const float *)a.q + qbase + kk * 32 + g * 8);
+                const f32x4 x0 = row_ok ? qp[0] : f32x4{0.f, 0.f, 0.f, 0.f}, x1 = row_ok ? qp[1] : f32x4{0.f, 0.f, 0.f, 0.f};
+                x[0] = x0.x; x[1] = x0.y; x[2] = x0.z; x[3] = x0.w; x[4] = x1.x; x[5] = x1.y; x[6] = x1.z; x[7] = x1.w;
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) x[j] = row_ok ? load_scalar(a.q, a.q_dtype, qbase + kk * 32 + g * 8 + j) : 0.f;
+            }
             unsigned short h[8], lo8[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                const float x = row_ok ? load_scalar(a.q, a.q_dtype, qbase + kk * 32 + g * 8 + j) : 0.f;
-                h[j] = to_half_bits<KV>(x);
-                lo8[j] = HILO ? to_half_bits<KV>(x - from_half_bits<KV>(h[j])) : (unsigned short)0;
+                h[j] = to_half_bits<KV>(x[j]);
+                lo8[j] = HILO ? to_half_bits<KV>(x[j] - from_half_bits<KV>(h[j])) : (unsigned short)0;
             }
             qf[kk] = u32x4{(unsigned)h[0] | ((unsigned)h[1] << 16), (unsigned)h[2] | ((unsigned)h[3] << 16),
                            (unsigned)h[4] | ((unsigned)h[5] << 16), (unsigned)h[6] | ((unsigned)h[7] << 16)};
@@ -338,15 +353,16 @@ __global__ __launch_bounds__(256) void attn_flash_kernel(AttnArgs a) {
     }
 }
 
-// log-sum-exp merge of the key segments of one (unit, row tile)
+// log-sum-exp merge of the key segments: one workgroup per (row tile, 64-wide dv slice, unit)
 template <int D>
 __global__ __launch_bounds__(256) void attn_merge_kernel(AttnArgs a) {
     constexpr int WSTRIDE = 16 * D + 32;
-    const int unit = blockIdx.y, rt = blockIdx.x;
+    constexpr int SLICES = D / 64;
+    const int unit = blockIdx.y, rt = blockIdx.x / SLICES, slice = blockIdx.x % SLICES;
     const int b = unit / a.Hkv, hk = unit % a.Hkv;
     const float *base = a.partial + (size_t)(unit * a.row_tiles + rt) * a.nseg * WSTRIDE;
-    for (int idx = threadIdx.x; idx < 16 * D; idx += 256) {
-        const int row = idx / D;
+    for (int e = threadIdx.x; e < 16 * 64; e += 256) {
+        const int row = e >> 6, dv = slice * 64 + (e & 63);
         const int rr = rt * 16 + row;
         if (rr >= a.rows_total) continue;
         float m_all = -INFINITY;
@@ -355,11 +371,11 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnArgs a) {
         for (int s = 0; s < a.nseg; ++s) {
             const float ms = base[(size_t)s * WSTRIDE + 16 * D + row];
             const float f = ms > -INFINITY ? exp2f((ms - m_all) * LOG2E) : 0.f;
-            o += base[(size_t)s * WSTRIDE + idx] * f;
+            o += base[(size_t)s * WSTRIDE + row * D + dv] * f;
             l_all += base[(size_t)s * WSTRIDE + 16 * D + 16 + row] * f;
         }
         const int l2 = rr / a.groups, g2 = rr % a.groups;
-        a.out[(((size_t)b * a.L + l2) * a.Hq + hk * a.groups + g2) * D + idx % D] = l_all > 0.f ? o / l_all : 0.f;
+        a.out[(((size_t)b * a.L + l2) * a.Hq + hk * a.groups + g2) * D + dv] = l_all > 0.f ? o / l_all : 0.f;
     }
 }
 
@@ -419,11 +435,11 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
     const int units = a.B * a.Hkv;
     const bool split = a.rows_total <= 64;
     if (split) {
-        // fill the device: ~2 workgroups per CU, at least 4 tiles (128 keys) per workgroup
+        // key segments: at least 8 tiles (two per wavefront) each, at most ~2 workgroups per CU
         const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
         const int tiles = (a.T + TILE_KEYS - 1) / TILE_KEYS;
         int nseg = (2 * cus + units * a.row_tiles - 1) / (units * a.row_tiles);
-        nseg = max(1, min(nseg, (tiles + 3) / 4));
+        nseg = max(1, min(nseg, tiles / 8));
         nseg = min(nseg, 256);
         a.nseg = nseg;
         if (nseg > 1) {
@@ -432,15 +448,23 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
             if (rc) return rc;
             a.partial = (float *)ctx->scratch2;
         }
-        HIP_TRY(ctx, hipFuncSetAttribute((const void *)attn_flash_kernel<KV, D, true, HILO>, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
+        static bool attr_split = false;   // per kernel instantiation
+        if (!attr_split) {
+            HIP_TRY(ctx, hipFuncSetAttribute((const void *)attn_flash_kernel<KV, D, true, HILO>, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
+            attr_split = true;
+        }
         prof_begin(ctx, "attn_flash_split");
         attn_flash_kernel<KV, D, true, HILO><<<dim3((unsigned)(a.row_tiles * nseg), (unsigned)units), dim3(256), Cfg::LDS_BYTES, ctx->stream>>>(a);
-        if (nseg > 1) attn_merge_kernel<D><<<dim3((unsigned)a.row_tiles, (unsigned)units), dim3(256), 0, ctx->stream>>>(a);
+        if (nseg > 1) attn_merge_kernel<D><<<dim3((unsigned)(a.row_tiles * (D / 64)), (unsigned)units), dim3(256), 0, ctx->stream>>>(a);
         prof_end(ctx);
         LAUNCH_CHECK(ctx, "attn_flash_split");
     } else {
         a.nseg = 1;
-        HIP_TRY(ctx, hipFuncSetAttribute((const void *)attn_flash_kernel<KV, D, false, HILO>, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
+        static bool attr_prefill = false;
+        if (!attr_prefill) {
+            HIP_TRY(ctx, hipFuncSetAttribute((const void *)attn_flash_kernel<KV, D, false, HILO>, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
+            attr_prefill = true;
+        }
         prof_begin(ctx, "attn_flash_prefill");
         attn_flash_kernel<KV, D, false, HILO><<<dim3((unsigned)((a.row_tiles + 3) / 4), (unsigned)units), dim3(256), Cfg::LDS_BYTES, ctx->stream>>>(a);
         prof_end(ctx);

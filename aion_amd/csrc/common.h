@@ -99,6 +99,37 @@ PreparedAct prepared_act_carve(void *base, size_t m, size_t k);
 int launch_prepare_act(aionhip_ctx *ctx, const float *a, size_t lda, size_t m, size_t k, PreparedAct out);
 
 // ---- matmul back ends --------------------------------------------------------------------------
+// Up to four weights that multiply the SAME activation rows (q/k/v, gate/up) run as one launch:
+// their rows are concatenated, a wavefront's row group never straddles two weights.
+struct GemvSeg {
+    const u32x4 *qs;
+    const __half *sc;
+    float *c;
+    size_t ldc;
+    int n;          // rows of this weight
+    int first_wave; // first wavefront of this segment
+};
+struct GemvBatch {
+    GemvSeg seg[4];
+    int count;
+    int total_waves;
+};
+// What the single-row GEMV computes its activation from, inside the kernel (no separate launch):
+//   PRO_QUANT   a = x
+//   PRO_RMSNORM a = x * rsqrt(mean(x^2)+eps) * gamma + beta
+//   PRO_GATE    a = gelu_tanh(x) * y
+enum { PRO_QUANT = 0, PRO_RMSNORM = 1, PRO_GATE = 2 };
+struct FusedIn {
+    const float *x, *y, *gamma, *beta;
+    float eps;
+};
+constexpr size_t FUSED_MAX_K = 8192;
+int launch_gemv_fused(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count,
+                      int prologue, FusedIn in, float alpha, float beta);
+int launch_rmsnorm(aionhip_ctx *ctx, float *out, const float *x, const float *gamma, const float *beta, const float *residual,
+                   size_t rows, size_t cols, float eps);
+int launch_gate_gelu(aionhip_ctx *ctx, float *out, const float *a, const float *b, size_t n);
+
 int launch_gemv(aionhip_ctx *ctx, const aionhip_weight *w, int m, PreparedAct act, float *c, size_t ldc, float alpha, float beta);
 int launch_gemv_batch(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count, int m,
                       PreparedAct act, float alpha, float beta);
@@ -140,3 +171,34 @@ __device__ __forceinline__ float wave_max(float v) {
 }
 
 __device__ __forceinline__ int dot4_i8(int a, int b, int c) { return __builtin_amdgcn_sdot4(a, b, c, false); }
+
+// aion cpu/kernels/fast_math.zig:53-148: exp(x) = 2^n * P4(r ln2), sigmoid, tanh = 2 sigmoid(2x) - 1
+__device__ __forceinline__ float aion_exp_approx(float x_in) {
+    const float x = fminf(80.f, fmaxf(-80.f, x_in));
+    const float y = x * 1.4426950408889634f;
+    const float nf = floorf(y + 0.5f);
+    const float t = (y - nf) * 0.6931471805599453f;
+    const float p = 1.f + t * (1.f + t * (0.5f + t * ((1.f / 6.f) + t * (1.f / 24.f))));
+    return __uint_as_float((unsigned)((int)nf + 127) << 23) * p;
+}
+__device__ __forceinline__ float aion_tanh_approx(float x) {
+    const float z = 2.f * x;
+    const float e = aion_exp_approx(-fabsf(z));
+    float sg = (z >= 0.f ? 1.f : e) / (1.f + e);
+    sg = fminf(1.f, fmaxf(0.f, sg));
+    return fminf(1.f, fmaxf(-1.f, 2.f * sg - 1.f));
+}
+// aion cpu/exec/elementwise.zig:25-37 (gate) + cpu/kernels/gelu.zig:8-14: gelu_tanh(x) * up
+__device__ __forceinline__ float aion_gate_gelu(float x, float up) {
+    const float t = 0.7978845608028654f * (x + 0.044715f * (x * x * x));
+    return (0.5f * x * (1.f + aion_tanh_approx(t))) * up;
+}
+// sum over a 256-thread workgroup; red: 4 floats of LDS. Every thread returns the total.
+__device__ __forceinline__ float block_sum_256(float v, float *red) {
+    v = wave_sum(v);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    const float t = (red[0] + red[1]) + (red[2] + red[3]);
+    __syncthreads();
+    return t;
+}

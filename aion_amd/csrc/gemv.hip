@@ -14,22 +14,6 @@
 
 namespace {
 
-// Up to four weights that multiply the SAME activation rows (q/k/v, gate/up) run as one launch:
-// their rows are concatenated, a wavefront's row group never straddles two weights.
-struct GemvSeg {
-    const u32x4 *qs;
-    const __half *sc;
-    float *c;
-    size_t ldc;
-    int n;          // rows of this weight
-    int first_wave; // first wavefront of this segment
-};
-struct GemvBatch {
-    GemvSeg seg[4];
-    int count;
-    int total_waves;
-};
-
 template <int DT, int B, int R>
 __global__ __launch_bounds__(256) void gemv_kernel(GemvBatch batch, const u32x4 *__restrict__ aq, const float *__restrict__ a_scale,
                                                    const int *__restrict__ a_sum, int K, int m, float alpha, float beta) {

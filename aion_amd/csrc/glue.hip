@@ -6,17 +6,6 @@
 
 namespace {
 
-__device__ __forceinline__ float block_sum(float v, float *red) {
-    v = wave_sum(v);
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    if (lane == 0) red[w] = v;
-    __syncthreads();
-    float t = 0.f;
-    for (int i = 0; i < (int)(blockDim.x >> 6); ++i) t += red[i];
-    __syncthreads();
-    return t;
-}
-
 // cpu/exec/layernorm.zig:54-155 + cpu/kernels/layernorm.zig:69-147 (rmsnorm mode):
 // inv = 1/sqrt(sum(x^2)/cols + eps); out = (x*inv)*gamma + beta; out += residual
 __global__ __launch_bounds__(256) void rmsnorm_kernel(float *__restrict__ out, const float *__restrict__ x, const float *__restrict__ gamma,
@@ -27,7 +16,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(float *__restrict__ out, c
     const float *xr = x + row * cols;
     float ss = 0.f;
     for (size_t c = threadIdx.x; c < cols; c += 256) ss += xr[c] * xr[c];
-    ss = block_sum(ss, red);
+    ss = block_sum_256(ss, red);
     const float inv = 1.f / sqrtf(ss * (1.f / (float)cols) + eps);
     for (size_t c = threadIdx.x; c < cols; c += 256) {
         float y = (xr[c] * inv) * gamma[c] + (beta ? beta[c] : 0.f);
@@ -37,7 +26,13 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(float *__restrict__ out, c
 }
 
 // cpu/exec/rope.zig:14-53 + cpu/kernels/rope.zig:20-98: pairs (i, i + D/2); the frequency is
-// multiplied up iteratively in f32, the angle pos*f is rounded to f32, sin/cos are taken in f64.
+// multiplied up iteratively in f32 and the angle pos*f is rounded to f32, as on the CPU. aion
+// takes sin/cos of that f32 angle in f64 and rounds; here sincosf (full range reduction, <= 2 ulp).
+__device__ __forceinline__ float rope_freq(int i, float freq_step, float scale_factor) {
+    float f = scale_factor;
+    for (int j = 0; j < i; ++j) f *= freq_step;
+    return f;
+}
 __global__ void rope_kernel(float *__restrict__ out, const float *__restrict__ x, const int *__restrict__ positions,
                             size_t tokens, int H, int D, int rope_pairs, float freq_step, float scale_factor) {
     const int half = D / 2;
@@ -54,14 +49,48 @@ __global__ void rope_kernel(float *__restrict__ out, const float *__restrict__ x
         }
         return;
     }
-    float f = scale_factor;
-    for (int j = 0; j < i; ++j) f *= freq_step;
-    const float ang = (float)positions[tok] * f;
-    const float cs = (float)cos((double)ang), sn = (float)sin((double)ang);
+    const float ang = (float)positions[tok] * rope_freq(i, freq_step, scale_factor);
+    float sn, cs;
+    sincosf(ang, &sn, &cs);
     for (int h = 0; h < H; ++h) {
         const float xl = xr[h * D + i], xh = xr[h * D + half + i];
         orow[h * D + i] = xl * cs - xh * sn;
         orow[h * D + half + i] = xl * sn + xh * cs;
+    }
+}
+
+// RoPE1D(q), RoPE1D(k) -> f16 -> SequenceAppend(k cache), Cast f16 + SequenceAppend(v cache) for the
+// tokens of one step, as one launch: thread (token, pair i) rotates pair i of every q head and
+// k head and copies the matching v elements. Same arithmetic as the four separate steps.
+__global__ void rope_append_kernel(float *__restrict__ q_out, const float *__restrict__ q, const float *__restrict__ k, const float *__restrict__ v,
+                                   __half *__restrict__ kcache, __half *__restrict__ vcache, const int *__restrict__ positions,
+                                   const int *__restrict__ write_index, size_t batch, size_t s_len, size_t t_cap, int Hq, int Hkv, int D,
+                                   int rope_pairs, float freq_step, float scale_factor) {
+    const int half = D / 2;
+    const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= batch * s_len * (size_t)half) return;
+    const size_t tok = gid / half;                 // b * s_len + s
+    const int i = (int)(gid % half);
+    const size_t b = tok / s_len, s = tok % s_len;
+    float sn = 0.f, cs = 1.f;
+    if (i < rope_pairs) sincosf((float)positions[tok] * rope_freq(i, freq_step, scale_factor), &sn, &cs);
+    const float *qr = q + tok * Hq * D;
+    float *qo = q_out + tok * Hq * D;
+    for (int h = 0; h < Hq; ++h) {
+        const float xl = qr[h * D + i], xh = qr[h * D + half + i];
+        qo[h * D + i] = i < rope_pairs ? xl * cs - xh * sn : xl;
+        qo[h * D + half + i] = i < rope_pairs ? xl * sn + xh * cs : xh;
+    }
+    const long t = (long)write_index[0] + (long)s;
+    if (t < 0 || (size_t)t >= t_cap) return;       // never write outside the cache
+    const float *kr = k + tok * Hkv * D, *vr = v + tok * Hkv * D;
+    __half *kc = kcache + (b * t_cap + (size_t)t) * Hkv * D, *vc = vcache + (b * t_cap + (size_t)t) * Hkv * D;
+    for (int h = 0; h < Hkv; ++h) {
+        const float xl = kr[h * D + i], xh = kr[h * D + half + i];
+        kc[h * D + i] = __float2half_rn(i < rope_pairs ? xl * cs - xh * sn : xl);
+        kc[h * D + half + i] = __float2half_rn(i < rope_pairs ? xl * sn + xh * cs : xh);
+        vc[h * D + i] = __float2half_rn(vr[h * D + i]);
+        vc[h * D + half + i] = __float2half_rn(vr[h * D + half + i]);
     }
 }
 
@@ -70,29 +99,11 @@ __global__ void add_kernel(float *__restrict__ out, const float *__restrict__ a,
     if (i < n) out[i] = a[i] + b[i];
 }
 
-// cpu/kernels/fast_math.zig:53-148: exp(x) = 2^n * P4(r ln2), sigmoid, tanh = 2 sigmoid(2x) - 1
-__device__ __forceinline__ float exp_approx(float x_in) {
-    const float x = fminf(80.f, fmaxf(-80.f, x_in));
-    const float y = x * 1.4426950408889634f;
-    const float nf = floorf(y + 0.5f);
-    const float t = (y - nf) * 0.6931471805599453f;
-    const float p = 1.f + t * (1.f + t * (0.5f + t * ((1.f / 6.f) + t * (1.f / 24.f))));
-    return __uint_as_float((unsigned)((int)nf + 127) << 23) * p;
-}
-__device__ __forceinline__ float tanh_approx(float x) {
-    const float z = 2.f * x;
-    const float e = exp_approx(-fabsf(z));
-    float sg = (z >= 0.f ? 1.f : e) / (1.f + e);
-    sg = fminf(1.f, fmaxf(0.f, sg));
-    return fminf(1.f, fmaxf(-1.f, 2.f * sg - 1.f));
-}
 // cpu/exec/elementwise.zig:25-37 (gate) + cpu/kernels/gelu.zig:8-14
 __global__ void gate_gelu_kernel(float *__restrict__ out, const float *__restrict__ a, const float *__restrict__ b, size_t n) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    const float x = a[i];
-    const float t = 0.7978845608028654f * (x + 0.044715f * (x * x * x));
-    out[i] = (0.5f * x * (1.f + tanh_approx(t))) * b[i];
+    out[i] = aion_gate_gelu(a[i], b[i]);
 }
 
 // cpu/exec/gather.zig:60-87: one workgroup per gathered row; ids outside [0, vocab) give zeros
@@ -133,17 +144,11 @@ __global__ void append_f16_kernel(__half *__restrict__ cache, const float *__res
     cache[(b * t_cap + (size_t)t) * row_elems + e] = __float2half_rn(src[i]);
 }
 
-// cpu/exec/argmax.zig:56-81: strict > keeps the first maximum
-__global__ __launch_bounds__(256) void argmax_kernel(int *__restrict__ out, const float *__restrict__ x, size_t n) {
-    __shared__ float bv[256];
-    __shared__ int bi[256];
-    const float *row = x + (size_t)blockIdx.x * n;
-    float best = -INFINITY;
-    int idx = 0x7FFFFFFF;
-    for (size_t j = threadIdx.x; j < n; j += 256) {
-        const float v = row[j];
-        if (idx == 0x7FFFFFFF || v > best) { best = v; idx = (int)j; }
-    }
+// cpu/exec/argmax.zig:56-81: strict > keeps the first maximum. Two stages: ARGMAX_PARTS workgroups
+// per row each reduce a contiguous slice to (value, index), then one workgroup picks among them
+// (ties -> the smaller index, which is the first maximum).
+constexpr int ARGMAX_PARTS = 64;
+__device__ __forceinline__ void argmax_reduce_256(float &best, int &idx, float *bv, int *bi) {
     bv[threadIdx.x] = best;
     bi[threadIdx.x] = idx;
     __syncthreads();
@@ -158,7 +163,39 @@ __global__ __launch_bounds__(256) void argmax_kernel(int *__restrict__ out, cons
         }
         __syncthreads();
     }
-    if (threadIdx.x == 0) out[blockIdx.x] = bi[0] == 0x7FFFFFFF ? 0 : bi[0];
+    best = bv[0];
+    idx = bi[0];
+}
+__global__ __launch_bounds__(256) void argmax_part_kernel(float *__restrict__ pv, int *__restrict__ pi, const float *__restrict__ x, size_t n) {
+    __shared__ float bv[256];
+    __shared__ int bi[256];
+    const size_t row = blockIdx.y;
+    const size_t per = (n + ARGMAX_PARTS - 1) / ARGMAX_PARTS;
+    const size_t lo = blockIdx.x * per, hi = lo + per < n ? lo + per : n;
+    const float *r = x + row * n;
+    float best = -INFINITY;
+    int idx = 0x7FFFFFFF;
+    for (size_t j = lo + threadIdx.x; j < hi; j += 256) {
+        const float v = r[j];
+        if (idx == 0x7FFFFFFF || v > best) { best = v; idx = (int)j; }
+    }
+    argmax_reduce_256(best, idx, bv, bi);
+    if (threadIdx.x == 0) {
+        pv[row * ARGMAX_PARTS + blockIdx.x] = best;
+        pi[row * ARGMAX_PARTS + blockIdx.x] = idx;
+    }
+}
+__global__ __launch_bounds__(256) void argmax_final_kernel(int *__restrict__ out, const float *__restrict__ pv, const int *__restrict__ pi) {
+    __shared__ float bv[256];
+    __shared__ int bi[256];
+    float best = -INFINITY;
+    int idx = 0x7FFFFFFF;
+    if (threadIdx.x < ARGMAX_PARTS) {
+        best = pv[blockIdx.x * ARGMAX_PARTS + threadIdx.x];
+        idx = pi[blockIdx.x * ARGMAX_PARTS + threadIdx.x];
+    }
+    argmax_reduce_256(best, idx, bv, bi);
+    if (threadIdx.x == 0) out[blockIdx.x] = idx == 0x7FFFFFFF ? 0 : idx;
 }
 
 inline unsigned grid_for(size_t n, unsigned block) { return (unsigned)((n + block - 1) / block); }
@@ -166,6 +203,18 @@ template <class T>
 inline T *dp(aionhip_handle h) { return (T *)(uintptr_t)h; }
 
 }  // namespace
+
+int launch_rmsnorm(aionhip_ctx *ctx, float *out, const float *x, const float *gamma, const float *beta, const float *residual,
+                   size_t rows, size_t cols, float eps) {
+    rmsnorm_kernel<<<dim3((unsigned)rows), dim3(256), 0, ctx->stream>>>(out, x, gamma, beta, residual, cols, eps);
+    LAUNCH_CHECK(ctx, "rmsnorm");
+    return AIONHIP_OK;
+}
+int launch_gate_gelu(aionhip_ctx *ctx, float *out, const float *a, const float *b, size_t n) {
+    gate_gelu_kernel<<<dim3(grid_for(n, 256)), dim3(256), 0, ctx->stream>>>(out, a, b, n);
+    LAUNCH_CHECK(ctx, "gate_gelu");
+    return AIONHIP_OK;
+}
 
 extern "C" {
 
@@ -176,10 +225,7 @@ int aionhip_step_rmsnorm(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle x,
     if (!(eps > 0.f) || !(eps < INFINITY)) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "rmsnorm: eps must be positive and finite");
     if (!rows || !cols) return AIONHIP_OK;
     if (rows > 0x7FFFFFFFu) return set_err(ctx, AIONHIP_UNSUPPORTED, "rmsnorm: too many rows");
-    rmsnorm_kernel<<<dim3((unsigned)rows), dim3(256), 0, ctx->stream>>>(dp<float>(out), dp<const float>(x), dp<const float>(gamma),
-                                                                        dp<const float>(beta), dp<const float>(residual), cols, eps);
-    LAUNCH_CHECK(ctx, "rmsnorm");
-    return AIONHIP_OK;
+    return launch_rmsnorm(ctx, dp<float>(out), dp<const float>(x), dp<const float>(gamma), dp<const float>(beta), dp<const float>(residual), rows, cols, eps);
 }
 
 int aionhip_step_rope(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle x, aionhip_handle positions, size_t b, size_t t, size_t h,
@@ -202,6 +248,29 @@ int aionhip_step_rope(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle x, ai
     return AIONHIP_OK;
 }
 
+int aionhip_step_rope_append(aionhip_ctx *ctx, aionhip_handle q_out, aionhip_handle q, aionhip_handle k, aionhip_handle v,
+                             aionhip_handle k_cache, aionhip_handle v_cache, aionhip_handle positions, aionhip_handle write_index,
+                             size_t b, size_t s, size_t t_cap, size_t h_q, size_t h_kv, size_t d, float base_frequency,
+                             float scale_factor, float rope_proportion) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (!q_out || !q || !k || !v || !k_cache || !v_cache || !positions || !write_index) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "rope_append: null operand");
+    if (!(base_frequency > 0.f) || !(base_frequency < INFINITY) || !(scale_factor > 0.f) || !(scale_factor < INFINITY) ||
+        !(rope_proportion >= 0.f && rope_proportion <= 1.f))
+        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "rope_append: base/scale must be positive and finite, proportion in [0,1]");
+    if (d % 2 != 0 || d > 65534 || h_q > 65535 || h_kv > 65535) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "rope_append: head size must be even");
+    if (s > t_cap) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "rope_append: %zu new tokens exceed the cache capacity %zu", s, t_cap);
+    const size_t half = d / 2, total = b * s * half;
+    if (!total || !h_q || !h_kv) return AIONHIP_OK;
+    size_t rope_pairs = (size_t)floorf(rope_proportion * (float)half);
+    if (rope_pairs > half) rope_pairs = half;
+    const float freq_step = (float)pow((double)base_frequency, (double)(-2.0f / (float)d));
+    rope_append_kernel<<<dim3(grid_for(total, 128)), dim3(128), 0, ctx->stream>>>(
+        dp<float>(q_out), dp<const float>(q), dp<const float>(k), dp<const float>(v), dp<__half>(k_cache), dp<__half>(v_cache),
+        dp<const int>(positions), dp<const int>(write_index), b, s, t_cap, (int)h_q, (int)h_kv, (int)d, (int)rope_pairs, freq_step, scale_factor);
+    LAUNCH_CHECK(ctx, "rope_append");
+    return AIONHIP_OK;
+}
+
 int aionhip_step_add(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle a, aionhip_handle b, size_t n) {
     if (!ctx) return AIONHIP_INVALID_ARGUMENT;
     if (!out || !a || !b) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "add: null operand");
@@ -215,9 +284,7 @@ int aionhip_step_gate_gelu(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle 
     if (!ctx) return AIONHIP_INVALID_ARGUMENT;
     if (!out || !a || !b) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "gate: null operand");
     if (!n) return AIONHIP_OK;
-    gate_gelu_kernel<<<dim3(grid_for(n, 256)), dim3(256), 0, ctx->stream>>>(dp<float>(out), dp<const float>(a), dp<const float>(b), n);
-    LAUNCH_CHECK(ctx, "gate_gelu");
-    return AIONHIP_OK;
+    return launch_gate_gelu(ctx, dp<float>(out), dp<const float>(a), dp<const float>(b), n);
 }
 
 int aionhip_step_gather_rows(aionhip_ctx *ctx, int table_dtype, aionhip_handle out, aionhip_handle table, aionhip_handle ids,
@@ -261,7 +328,13 @@ int aionhip_step_argmax(aionhip_ctx *ctx, aionhip_handle out_i32, aionhip_handle
     if (n == 0) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "argmax: empty axis");
     if (!rows) return AIONHIP_OK;
     if (rows > 0x7FFFFFFFu || n > 0x7FFFFFFFu) return set_err(ctx, AIONHIP_UNSUPPORTED, "argmax: dimension too large");
-    argmax_kernel<<<dim3((unsigned)rows), dim3(256), 0, ctx->stream>>>(dp<int>(out_i32), dp<const float>(x), n);
+    if (rows > 65535) return set_err(ctx, AIONHIP_UNSUPPORTED, "argmax: more than 65535 rows");
+    int rc = ensure_scratch2(ctx, rows * ARGMAX_PARTS * 8);
+    if (rc) return rc;
+    float *pv = (float *)ctx->scratch2;
+    int *pi = (int *)(pv + rows * ARGMAX_PARTS);
+    argmax_part_kernel<<<dim3(ARGMAX_PARTS, (unsigned)rows), dim3(256), 0, ctx->stream>>>(pv, pi, dp<const float>(x), n);
+    argmax_final_kernel<<<dim3((unsigned)rows), dim3(256), 0, ctx->stream>>>(dp<int>(out_i32), pv, pi);
     LAUNCH_CHECK(ctx, "argmax");
     return AIONHIP_OK;
 }

@@ -1,77 +1,93 @@
 // StepMatMul / StepMatMulNT entry points: argument checks (the aion compiler's validation,
 // graph/program/compiler.zig:189-239,337-357), activation preparation, kernel routing
-// (the counterpart of cpu/exec/matmul.zig:233-296 `matvecRoute` / `gemm2D`).
+// (the counterpart of cpu/exec/matmul.zig:233-296 `matvecRoute` / `gemm2D`):
+//   m == 1, k <= 8192, 16-byte aligned A  -> gemv_fused_kernel (activation prepared in the kernel)
+//   m <= 8                                -> prepare_act_kernel + gemv_kernel
+//   m  > 8                                -> gemm_i8_kernel (exact) or gemm_bf16_kernel
 #include "common.h"
 
 namespace {
 
 constexpr size_t GEMV_MAX_M = 8;
 
-int run_matmul(aionhip_ctx *ctx, const aionhip_weight *b, size_t m, aionhip_handle a_h, size_t lda,
-               aionhip_handle c_h, size_t ldc, float alpha, float beta) {
-    if (m == 0) return AIONHIP_OK;
-    if (!a_h || !c_h) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "matmul: null A or C");
-    if (lda == 0) lda = b->k;
-    if (ldc == 0) ldc = b->n;
-    if (lda < b->k || ldc < b->n) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "matmul: lda=%zu < k=%zu or ldc=%zu < n=%zu", lda, b->k, ldc, b->n);
-    if ((a_h & 3) || (c_h & 3)) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "matmul: A and C must be 4-byte aligned");
-    if (m > 0x7FFFFFFFu) return set_err(ctx, AIONHIP_UNSUPPORTED, "matmul: m exceeds 2^31-1");
-    const float *a = (const float *)(uintptr_t)a_h;
-    float *c = (float *)(uintptr_t)c_h;
+struct Batch {
+    size_t count = 0, k = 0;
+    const aionhip_weight *w[4];
+    float *c[4];
+    size_t ldc[4];
+    aionhip_handle c_h[4];
+};
 
-    if (m > GEMV_MAX_M && ctx->gemm_mode == AIONHIP_GEMM_BF16_MFMA)
-        return launch_gemm_bf16(ctx, b, m, a, lda, c, ldc, alpha, beta);
-
-    int rc = ensure_scratch(ctx, prepared_act_bytes(m, b->k));
-    if (rc) return rc;
-    PreparedAct act = prepared_act_carve(ctx->scratch, m, b->k);
-    rc = launch_prepare_act(ctx, a, lda, m, b->k, act);
-    if (rc) return rc;
-    if (m <= GEMV_MAX_M) return launch_gemv(ctx, b, (int)m, act, c, ldc, alpha, beta);
-    return launch_gemm_i8(ctx, b, m, act, c, ldc, alpha, beta);
+int check_batch(aionhip_ctx *ctx, const char *what, size_t count, const aionhip_weight *const *bs, const aionhip_handle *c_hs,
+                const size_t *ldcs_in, Batch &out) {
+    if (count == 0 || count > 4) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "%s: 1..4 weights per call", what);
+    if (!bs || !c_hs) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "%s: null argument", what);
+    out.count = count;
+    out.k = bs[0] ? bs[0]->k : 0;
+    for (size_t i = 0; i < count; ++i) {
+        if (!bs[i] || !c_hs[i]) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "%s: null weight or C", what);
+        if (bs[i]->k != out.k || bs[i]->dtype != bs[0]->dtype) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "%s: weights must share k and dtype", what);
+        out.ldc[i] = ldcs_in && ldcs_in[i] ? ldcs_in[i] : bs[i]->n;
+        if (out.ldc[i] < bs[i]->n || (c_hs[i] & 3)) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "%s: ldc below n, or C not 4-byte aligned", what);
+        out.w[i] = bs[i];
+        out.c[i] = (float *)(uintptr_t)c_hs[i];
+        out.c_h[i] = c_hs[i];
+    }
+    return AIONHIP_OK;
 }
 
-int run_matmul_batch(aionhip_ctx *ctx, size_t count, const aionhip_weight *const *bs, size_t m, aionhip_handle a_h, size_t lda,
-                     const aionhip_handle *c_hs, const size_t *ldcs_in, float alpha, float beta) {
-    if (count == 0 || m == 0) return AIONHIP_OK;
-    if (count > 4) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "matmul_batch: at most 4 weights per call");
-    if (!bs || !c_hs || !a_h) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "matmul_batch: null argument");
-    const size_t k = bs[0] ? bs[0]->k : 0;
-    float *cs[4];
-    size_t ldcs[4];
-    for (size_t i = 0; i < count; ++i) {
-        if (!bs[i] || !c_hs[i]) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "matmul_batch: null weight or C");
-        if (bs[i]->k != k || bs[i]->dtype != bs[0]->dtype) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "matmul_batch: weights must share k and dtype");
-        ldcs[i] = ldcs_in && ldcs_in[i] ? ldcs_in[i] : bs[i]->n;
-        if (ldcs[i] < bs[i]->n || (c_hs[i] & 3)) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "matmul_batch: bad ldc or C alignment");
-        cs[i] = (float *)(uintptr_t)c_hs[i];
-    }
-    if (lda == 0) lda = k;
-    if (lda < k || (a_h & 3)) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "matmul_batch: bad lda or A alignment");
-    if (m > GEMV_MAX_M) {
-        // prefill: the weights run one after the other (each is MFMA-bound on its own)
-        for (size_t i = 0; i < count; ++i) {
-            int rc = run_matmul(ctx, bs[i], m, a_h, lda, c_hs[i], ldcs[i], alpha, beta);
+// every weight of `b` against the f32 rows at `a` (already materialised)
+int run_rows(aionhip_ctx *ctx, const Batch &b, size_t m, const float *a, size_t lda, float alpha, float beta) {
+    if (m > 0x7FFFFFFFu) return set_err(ctx, AIONHIP_UNSUPPORTED, "matmul: m exceeds 2^31-1");
+    if (m == 1 && b.k <= FUSED_MAX_K && ((uintptr_t)a & 15) == 0)
+        return launch_gemv_fused(ctx, b.w, b.c, b.ldc, (int)b.count, PRO_QUANT, FusedIn{a, nullptr, nullptr, nullptr, 0.f}, alpha, beta);
+    if (m > GEMV_MAX_M && ctx->gemm_mode == AIONHIP_GEMM_BF16_MFMA) {
+        for (size_t i = 0; i < b.count; ++i) {
+            int rc = launch_gemm_bf16(ctx, b.w[i], m, a, lda, b.c[i], b.ldc[i], alpha, beta);
             if (rc) return rc;
         }
         return AIONHIP_OK;
     }
-    int rc = ensure_scratch(ctx, prepared_act_bytes(m, k));
+    int rc = ensure_scratch(ctx, prepared_act_bytes(m, b.k));
     if (rc) return rc;
-    PreparedAct act = prepared_act_carve(ctx->scratch, m, k);
-    rc = launch_prepare_act(ctx, (const float *)(uintptr_t)a_h, lda, m, k, act);
+    PreparedAct act = prepared_act_carve(ctx->scratch, m, b.k);
+    rc = launch_prepare_act(ctx, a, lda, m, b.k, act);
     if (rc) return rc;
-    return launch_gemv_batch(ctx, bs, cs, ldcs, (int)count, (int)m, act, alpha, beta);
+    if (m <= GEMV_MAX_M) return launch_gemv_batch(ctx, b.w, b.c, b.ldc, (int)b.count, (int)m, act, alpha, beta);
+    for (size_t i = 0; i < b.count; ++i) {
+        rc = launch_gemm_i8(ctx, b.w[i], m, act, b.c[i], b.ldc[i], alpha, beta);
+        if (rc) return rc;
+    }
+    return AIONHIP_OK;
+}
+
+int run_matmul(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, aionhip_handle a_h, size_t lda, aionhip_handle c_h, size_t ldc,
+               float alpha, float beta) {
+    if (m == 0) return AIONHIP_OK;
+    if (!a_h || !c_h) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "matmul: null A or C");
+    if (lda == 0) lda = w->k;
+    if (lda < w->k || (a_h & 3)) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "matmul: lda=%zu below k=%zu, or A not 4-byte aligned", lda, w->k);
+    Batch b;
+    int rc = check_batch(ctx, "matmul", 1, &w, &c_h, &ldc, b);
+    if (rc) return rc;
+    return run_rows(ctx, b, m, (const float *)(uintptr_t)a_h, lda, alpha, beta);
 }
 
 }  // namespace
 
 extern "C" {
 
-int aionhip_step_matmul_batch(aionhip_ctx *ctx, size_t count, const aionhip_weight *const *b, size_t m, aionhip_handle a, size_t lda,
+int aionhip_step_matmul_batch(aionhip_ctx *ctx, size_t count, const aionhip_weight *const *bs, size_t m, aionhip_handle a, size_t lda,
                               const aionhip_handle *c, const size_t *ldc, float alpha, float beta) {
     if (!ctx) return AIONHIP_INVALID_ARGUMENT;
-    return run_matmul_batch(ctx, count, b, m, a, lda, c, ldc, alpha, beta);
+    if (count == 0 || m == 0) return AIONHIP_OK;
+    Batch b;
+    int rc = check_batch(ctx, "matmul_batch", count, bs, c, ldc, b);
+    if (rc) return rc;
+    if (!a) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "matmul_batch: null A");
+    if (lda == 0) lda = b.k;
+    if (lda < b.k || (a & 3)) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "matmul_batch: lda below k, or A not 4-byte aligned");
+    return run_rows(ctx, b, m, (const float *)(uintptr_t)a, lda, alpha, beta);
 }
 
 int aionhip_step_matmul(aionhip_ctx *ctx, const aionhip_weight *b, size_t m, aionhip_handle a, size_t lda,
@@ -87,6 +103,49 @@ int aionhip_step_matmul_nt(aionhip_ctx *ctx, const aionhip_weight *b, size_t m, 
     // StepMatMulNT: B is q8_0 [N,K] with quant_axis 1 (runtime/executable.zig:211-223)
     if (b->layout != AIONHIP_ROWS_NK || b->dtype != AIONHIP_Q8_0) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "MatMulNT needs a q8_0 [N,K] weight (quant_axis 1)");
     return run_matmul(ctx, b, m, a, lda, c, ldc, alpha, beta);
+}
+
+int aionhip_step_rmsnorm_matmul(aionhip_ctx *ctx, size_t count, const aionhip_weight *const *bs, size_t rows, aionhip_handle x,
+                                aionhip_handle gamma, aionhip_handle beta_norm, float eps, const aionhip_handle *c, const size_t *ldc,
+                                float alpha, float beta) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (count == 0 || rows == 0) return AIONHIP_OK;
+    Batch b;
+    int rc = check_batch(ctx, "rmsnorm_matmul", count, bs, c, ldc, b);
+    if (rc) return rc;
+    if (!x || !gamma) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "rmsnorm_matmul: null x or gamma");
+    if (!(eps > 0.f) || !(eps < INFINITY)) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "rmsnorm_matmul: eps must be positive and finite");
+    const float *xp = (const float *)(uintptr_t)x, *gp = (const float *)(uintptr_t)gamma, *bp = (const float *)(uintptr_t)beta_norm;
+    if (rows == 1 && b.k <= FUSED_MAX_K && ((x | gamma | beta_norm) & 15) == 0)
+        return launch_gemv_fused(ctx, b.w, b.c, b.ldc, (int)b.count, PRO_RMSNORM, FusedIn{xp, nullptr, gp, bp, eps}, alpha, beta);
+    // several rows: the norm runs as its own kernel into scratch, then the ordinary routing
+    const size_t act_bytes = (prepared_act_bytes(rows, b.k) + 255) & ~(size_t)255;
+    rc = ensure_scratch(ctx, act_bytes + rows * b.k * sizeof(float));
+    if (rc) return rc;
+    float *h = (float *)((char *)ctx->scratch + act_bytes);
+    rc = launch_rmsnorm(ctx, h, xp, gp, bp, nullptr, rows, b.k, eps);
+    if (rc) return rc;
+    return run_rows(ctx, b, rows, h, b.k, alpha, beta);
+}
+
+int aionhip_step_gate_matmul(aionhip_ctx *ctx, const aionhip_weight *w, size_t rows, aionhip_handle gate, aionhip_handle up,
+                             aionhip_handle c, size_t ldc, float alpha, float beta) {
+    if (!ctx || !w) return AIONHIP_INVALID_ARGUMENT;
+    if (rows == 0) return AIONHIP_OK;
+    Batch b;
+    int rc = check_batch(ctx, "gate_matmul", 1, &w, &c, &ldc, b);
+    if (rc) return rc;
+    if (!gate || !up || ((gate | up) & 3)) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "gate_matmul: null or misaligned gate/up");
+    const float *gp = (const float *)(uintptr_t)gate, *up_p = (const float *)(uintptr_t)up;
+    if (rows == 1 && b.k <= FUSED_MAX_K && ((gate | up) & 15) == 0)
+        return launch_gemv_fused(ctx, b.w, b.c, b.ldc, 1, PRO_GATE, FusedIn{gp, up_p, nullptr, nullptr, 0.f}, alpha, beta);
+    const size_t act_bytes = (prepared_act_bytes(rows, b.k) + 255) & ~(size_t)255;
+    rc = ensure_scratch(ctx, act_bytes + rows * b.k * sizeof(float));
+    if (rc) return rc;
+    float *h = (float *)((char *)ctx->scratch + act_bytes);
+    rc = launch_gate_gelu(ctx, h, gp, up_p, rows * b.k);
+    if (rc) return rc;
+    return run_rows(ctx, b, rows, h, b.k, alpha, beta);
 }
 
 }  // extern "C"

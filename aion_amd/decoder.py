@@ -146,25 +146,22 @@ class Decoder:
         scale = 1.0 / math.sqrt(c.head_dim)
         for l in range(c.layers):
             p = "l%d." % l
-            g.step_rmsnorm(b["h"], b["x"], self.gamma, s, c.hidden, c.eps)
-            g.step_matmul_batch([self.w[p + "wq"], self.w[p + "wk"], self.w[p + "wv"]], b["h"], s, [b["q"], b["k"], b["v"]])
-            g.step_rope(b["qr"], b["q"], b["positions"], 1, s, c.heads, c.head_dim, base=c.rope_base)
-            g.step_rope(b["kr"], b["k"], b["positions"], 1, s, c.kv_heads, c.head_dim, base=c.rope_base)
-            g.step_append_f16(self.kc[l], b["kr"], b["write_index"], 1, s, c.max_seq, c.kv_dim)
-            g.step_append_f16(self.vc[l], b["v"], b["write_index"], 1, s, c.max_seq, c.kv_dim)
+            # RMSNorm -> MatMul q, k, v (one call: the norm is not materialised)
+            g.step_rmsnorm_matmul([self.w[p + "wq"], self.w[p + "wk"], self.w[p + "wv"]], b["x"], self.gamma, s,
+                                  [b["q"], b["k"], b["v"]], c.eps)
+            # RoPE1D(q), RoPE1D(k) -> f16 -> append, v -> f16 -> append
+            g.step_rope_append(b["qr"], b["q"], b["k"], b["v"], self.kc[l], self.vc[l], b["positions"], b["write_index"],
+                               1, s, c.max_seq, c.heads, c.kv_heads, c.head_dim, base=c.rope_base)
             g.step_attention(b["att"], b["qr"], self.kc[l], self.vc[l], (1, s, c.max_seq, c.heads, c.kv_heads, c.head_dim, c.head_dim),
                              scale, q_dtype=be.F32, kv_dtype=be.F16, window=be.CAUSAL,
                              query_positions=b["positions"], kv_lengths=b["kv_len"])
-            g.step_matmul(self.w[p + "wo"], b["att"], s, b["o"])
-            g.step_add(b["x"], b["x"], b["o"], s * c.hidden)
-            g.step_rmsnorm(b["h"], b["x"], self.gamma, s, c.hidden, c.eps)
-            g.step_matmul_batch([self.w[p + "wgate"], self.w[p + "wup"]], b["h"], s, [b["gate"], b["up"]])
-            g.step_gate_gelu(b["act"], b["gate"], b["up"], s * c.ffn)
-            g.step_matmul(self.w[p + "wdown"], b["act"], s, b["o"])
-            g.step_add(b["x"], b["x"], b["o"], s * c.hidden)
+            # MatMul o with beta = 1: x = x + att @ Wo (the residual add rides on the matmul's beta)
+            g.step_matmul(self.w[p + "wo"], b["att"], s, b["x"], beta=1.0)
+            g.step_rmsnorm_matmul([self.w[p + "wgate"], self.w[p + "wup"]], b["x"], self.gamma, s, [b["gate"], b["up"]], c.eps)
+            # gate(gelu) -> MatMul down, beta = 1
+            g.step_gate_matmul(self.w[p + "wdown"], b["gate"], b["up"], s, b["x"], beta=1.0)
         last = b["x"].view((s - 1) * c.hidden * 4)
-        g.step_rmsnorm(b["hl"], last, self.gamma, 1, c.hidden, c.eps)
-        g.step_matmul(self.w["lm_head"], b["hl"], 1, self.logits)
+        g.step_rmsnorm_matmul([self.w["lm_head"]], last, self.gamma, 1, [self.logits], c.eps)
         g.step_argmax(self.token, self.logits, 1, c.vocab)
 
     def reset(self):

@@ -135,6 +135,18 @@ int aionhip_step_matmul_batch(aionhip_ctx *ctx, size_t count, const aionhip_weig
                               aionhip_handle a, size_t lda, const aionhip_handle *c, const size_t *ldc,
                               float alpha, float beta);
 
+/* StepRMSNorm feeding MatMul steps, and the fused gate feeding a MatMul step, as one call each:
+ * the normalised (or gated) activation is not written out; for one row it is built inside the GEMV
+ * kernel. Same arithmetic as aionhip_step_rmsnorm / aionhip_step_gate_gelu followed by the matmul
+ * step(s). aion fuses at step level the same way (RMSNorm.residual, ElemwiseBinary.gate:
+ * graph/opt/fuse_steps.zig:19-88); these two go one step further because a decode step on this
+ * GPU is bound by launch count, not bandwidth. */
+int aionhip_step_rmsnorm_matmul(aionhip_ctx *ctx, size_t count, const aionhip_weight *const *b, size_t rows,
+                                aionhip_handle x, aionhip_handle gamma, aionhip_handle beta_norm, float eps,
+                                const aionhip_handle *c, const size_t *ldc, float alpha, float beta);
+int aionhip_step_gate_matmul(aionhip_ctx *ctx, const aionhip_weight *b, size_t rows, aionhip_handle gate, aionhip_handle up,
+                             aionhip_handle c, size_t ldc, float alpha, float beta);
+
 /* How m > 8 rows are multiplied. EXACT_I8 (default): int8 activations, integer MFMA, per-block
  * f32 scaling - the same numbers as the decode path. BF16_MFMA: weights dequantized to bf16,
  * activations rounded to bf16, f32 accumulation - faster, judged at 1e-2 instead of 2e-3. */
@@ -168,6 +180,13 @@ int aionhip_step_rmsnorm(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle x,
 /* StepRoPE1D (cpu/exec/rope.zig:14-53, cpu/kernels/rope.zig:20-98): x,out [B,T,H,D], positions [B,T] i32 */
 int aionhip_step_rope(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle x, aionhip_handle positions,
                       size_t b, size_t t, size_t h, size_t d, float base_frequency, float scale_factor, float rope_proportion);
+/* RoPE1D(q) + RoPE1D(k) + Cast f16 + SequenceAppend(k cache) + Cast f16 + SequenceAppend(v cache)
+ * of one step as a single launch (same arithmetic as the separate steps): q,q_out [B,S,Hq,D] f32,
+ * k,v [B,S,Hkv,D] f32, caches [B,T,Hkv,D] f16, positions [B,S] i32, write_index [1] i32 on device */
+int aionhip_step_rope_append(aionhip_ctx *ctx, aionhip_handle q_out, aionhip_handle q, aionhip_handle k, aionhip_handle v,
+                             aionhip_handle k_cache, aionhip_handle v_cache, aionhip_handle positions, aionhip_handle write_index,
+                             size_t b, size_t s, size_t t_cap, size_t h_q, size_t h_kv, size_t d,
+                             float base_frequency, float scale_factor, float rope_proportion);
 /* StepElemwiseBinary: add, and the fused gate act(a)*b with act = gelu (tanh form)
  * (backend/types.zig:105-109, cpu/exec/elementwise.zig:25-37, cpu/kernels/gelu.zig:8-14) */
 int aionhip_step_add(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle a, aionhip_handle b, size_t n);

@@ -113,3 +113,35 @@ def test_kv_append_f16_at_device_write_index(gpu, orc):
     assert np.array_equal(gpu.download(cb, np.float16, cache.shape), cache)
     for t in (cb, sb, wb):
         t.free()
+
+
+def test_rope_append_equals_the_separate_steps(gpu, orc):
+    rng = np.random.default_rng(6)
+    B, S, T, Hq, Hkv, D = 2, 3, 12, 8, 1, 64
+    q = rng.standard_normal((B, S, Hq, D)).astype(np.float32)
+    k = rng.standard_normal((B, S, Hkv, D)).astype(np.float32)
+    v = rng.standard_normal((B, S, Hkv, D)).astype(np.float32)
+    pos = np.array([[4, 5, 6], [4, 5, 6]], np.int32)
+    qb, kb, vb, pb, wb = gpu.upload(q), gpu.upload(k), gpu.upload(v), gpu.upload(pos), gpu.upload(np.array([4], np.int32))
+    qo = gpu.alloc(q.nbytes)
+    kc, vc = gpu.zeros(B * T * Hkv * D * 2), gpu.zeros(B * T * Hkv * D * 2)
+    gpu.step_rope_append(qo, qb, kb, vb, kc, vc, pb, wb, B, S, T, Hq, Hkv, D)
+    assert np.allclose(gpu.download(qo, np.float32, q.shape), orc.rope(q, pos), atol=2e-6)
+    want_k = np.zeros((B, T, Hkv, D), np.float16)
+    want_v = np.zeros((B, T, Hkv, D), np.float16)
+    want_k[:, 4:7] = orc.cast_f32_f16(orc.rope(k, pos))
+    want_v[:, 4:7] = orc.cast_f32_f16(v)
+    got_k = gpu.download(kc, np.float16, want_k.shape)
+    assert np.allclose(got_k.astype(np.float32), want_k.astype(np.float32), atol=2e-3)   # f16 ulp at |x| < 4
+    assert np.array_equal(gpu.download(vc, np.float16, want_v.shape), want_v)
+    assert not got_k[:, :4].any() and not got_k[:, 7:].any()
+    # and against this backend's own separate steps: identical arithmetic, identical bits
+    qo2, kr = gpu.alloc(q.nbytes), gpu.alloc(k.nbytes)
+    kc2 = gpu.zeros(B * T * Hkv * D * 2)
+    gpu.step_rope(qo2, qb, pb, B, S, Hq, D)
+    gpu.step_rope(kr, kb, pb, B, S, Hkv, D)
+    gpu.step_append_f16(kc2, kr, wb, B, S, T, Hkv * D)
+    assert np.array_equal(gpu.download(qo2, np.float32, q.shape), gpu.download(qo, np.float32, q.shape))
+    assert np.array_equal(gpu.download(kc2, np.float16, want_k.shape), got_k)
+    for t in (qb, kb, vb, pb, wb, qo, kc, vc, qo2, kr, kc2):
+        t.free()

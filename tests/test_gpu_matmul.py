@@ -100,7 +100,8 @@ def test_gemv_small_and_ragged_shapes(gpu, orc, dtype, layout, m):
         got = gpu.matmul(w, a)
         want = oracle_matmul(orc, dtype, layout, a, blocks, n)
         assert norm_err(got, want) < TOL and rms_err(got, want) < RMS_TOL, (n, k, norm_err(got, want), rms_err(got, want))
-        assert gpu.last_kernel() == ("gemv_q8" if dtype == be.Q8_0 else "gemv_q4")
+        want_kernel = "gemv_q8" if dtype == be.Q8_0 else "gemv_q4"
+        assert gpu.last_kernel() == (want_kernel + "_fused" if m == 1 else want_kernel)
         w.free()
 
 
@@ -210,3 +211,56 @@ def test_matmul_argument_errors(gpu, orc):
     assert e.value.status == hip.INVALID_ARGUMENT
     assert lib.aionhip_step_matmul(ctx, w4.ptr, 0, a.handle, 0, c.handle, 0, 1.0, 0.0) == hip.OK   # m == 0 is a no-op
     a.free(); c.free(); w4.free()
+
+
+@pytest.mark.parametrize("dtype,layout", CASES)
+def test_single_row_fused_kernel_equals_prepared_path(gpu, orc, dtype, layout):
+    # m == 1 builds the int8 activation inside the GEMV; a 2-row call goes through prepare_act + gemv.
+    # Same codes, same scales, same per-lane order: the shared row must agree bit for bit.
+    for n, k in [(67, 2080), (2048, 2048), (300, 8192)]:
+        blocks, w = make_weight(gpu, orc, dtype, layout, n, k, seed=n + k)
+        a = np.random.default_rng(n).standard_normal((2, k)).astype(np.float32)
+        one = gpu.matmul(w, a[:1])
+        assert gpu.last_kernel().endswith("_fused")
+        two = gpu.matmul(w, a)
+        assert not gpu.last_kernel().endswith("_fused")
+        assert np.array_equal(one[0], two[0])
+        w.free()
+
+
+@pytest.mark.parametrize("dtype,layout", CASES)
+@pytest.mark.parametrize("rows", [1, 3])
+def test_rmsnorm_matmul_and_gate_matmul_match_the_separate_steps(gpu, orc, dtype, layout, rows):
+    say("fused steps", dtype, layout, rows)
+    rng = np.random.default_rng(rows + dtype)
+    k, n1, n2 = 2048, 512, 96
+    b1, w1 = make_weight(gpu, orc, dtype, layout, n1, k, seed=1)
+    b2, w2 = make_weight(gpu, orc, dtype, layout, n2, k, seed=2)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    gamma = (1 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    xb, gb = gpu.upload(x), gpu.upload(gamma)
+    c1, c2 = gpu.alloc(rows * n1 * 4), gpu.alloc(rows * n2 * 4)
+    gpu.step_rmsnorm_matmul([w1, w2], xb, gb, rows, [c1, c2], 1e-6)
+    if rows == 1:
+        assert gpu.last_kernel().endswith("_rmsnorm")
+    got1, got2 = gpu.download(c1, np.float32, (rows, n1)), gpu.download(c2, np.float32, (rows, n2))
+    h = orc.rmsnorm(x, gamma, 1e-6)
+    want1, want2 = oracle_matmul(orc, dtype, layout, h, b1, n1), oracle_matmul(orc, dtype, layout, h, b2, n2)
+    # the norm's sum of squares is reduced in a different order than on the CPU: an activation on a
+    # rounding boundary may take the neighbouring int8 code, worth up to ~1e-3 of rms per flipped code
+    assert rms_err(got1, want1) < 3e-3 and rms_err(got2, want2) < 3e-3
+    # gate: act = gelu(gate) * up, K = ffn
+    gate = (rng.standard_normal((rows, k)) * 2).astype(np.float32)
+    up = rng.standard_normal((rows, k)).astype(np.float32)
+    gtb, upb = gpu.upload(gate), gpu.upload(up)
+    res0 = rng.standard_normal((rows, n1)).astype(np.float32)
+    cres = gpu.upload(res0)
+    gpu.step_gate_matmul(w1, gtb, upb, rows, cres, beta=1.0)          # accumulates into C: a fused residual add
+    if rows == 1:
+        assert gpu.last_kernel().endswith("_gate")
+    act = orc.gate_gelu(gate, up).reshape(rows, k)
+    want = oracle_matmul(orc, dtype, layout, act, b1, n1, beta=1.0, c=res0)
+    assert rms_err(gpu.download(cres, np.float32, (rows, n1)), want) < 3e-3
+    for t in (xb, gb, c1, c2, gtb, upb, cres):
+        t.free()
+    w1.free(); w2.free()
