@@ -106,6 +106,9 @@ class HipBackend:
     def set_gemm_mode(self, mode):
         self._check(self._lib.aionhip_set_gemm_mode(self._ctx, mode))
 
+    def set_attention_precise(self, on):
+        self._check(self._lib.aionhip_set_attention_precise(self._ctx, 1 if on else 0))
+
     def device_info(self):
         cu, wave, hbm = C.c_int(), C.c_int(), C.c_uint64()
         arch = C.create_string_buffer(64)

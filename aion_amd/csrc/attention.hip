@@ -59,6 +59,15 @@ __device__ __forceinline__ float from_half_bits(unsigned short b) {
     if (KV == AIONHIP_F16) return __half2float(__ushort_as_half(b));
     return bf16_bits_to_f32(b);
 }
+// two f32 -> one 32-bit word of two halves (RNE), low half first
+template <int KV>
+__device__ __forceinline__ unsigned pack2(float a, float b) {
+    if (KV == AIONHIP_F16) {
+        const __half2 h = __floats2half2_rn(a, b);
+        return *reinterpret_cast<const unsigned *>(&h);
+    }
+    return (unsigned)f32_to_bf16_bits(a) | ((unsigned)f32_to_bf16_bits(b) << 16);
+}
 template <int KV>
 __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
     if (KV == AIONHIP_F16)
@@ -94,22 +103,26 @@ __device__ __forceinline__ int wave_max_i(int v) {
     return v;
 }
 
-template <int D>
+// NW = wavefronts per workgroup: 4 in prefill mode, 8 in split mode (a decode over a short cache
+// is one workgroup whose eight wavefronts take one 32-key tile each)
+template <int D, int NW>
 struct FlashCfg {
     static constexpr int ROW_BYTES = D * 2 + 16;                 // +16 B: the four key groups land in distinct LDS banks
     static constexpr int WAVE_LDS = TILE_KEYS * ROW_BYTES;       // one staged V tile per wavefront
-    static constexpr int WG_LDS = 4 * WAVE_LDS;
-    static constexpr int MERGE_LDS = 4 * (16 * D + 32) * 4;      // split mode: 4 x (acc[16][D], m[16], l[16]) f32
+    static constexpr int WG_LDS = NW * WAVE_LDS;
+    static constexpr int MERGE_LDS = (NW * (16 * (D + 4) + 32) + 16 * NW + 32) * 4;   // split mode: NW x (acc[16][D+4], m[16], l[16]) f32 + merge factors
     static constexpr int LDS_BYTES = WG_LDS > MERGE_LDS ? WG_LDS : MERGE_LDS;
 };
+constexpr int SPLIT_NW = 8;
 
 // HILO: q and the probabilities are fed to the MFMAs as a high and a low half-precision part
 // (x = hi + lo, ~2x the mantissa), which keeps an f32 query path at f32-level accuracy; used when
 // q arrives as f32 (aion's cached decode: f32 q over an f16 cache). K and V are exact either way.
 template <int KV, int D, bool SPLIT, bool HILO>
-__global__ __launch_bounds__(256) void attn_flash_kernel(AttnArgs a) {
+__global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel(AttnArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    using Cfg = FlashCfg<D>;
+    constexpr int NW = SPLIT ? SPLIT_NW : 4;
+    using Cfg = FlashCfg<D, NW>;
     constexpr int KK = D / 32;   // MFMA k-steps over the head dim
     constexpr int MT = D / 16;   // 16-wide dv tiles
 
@@ -121,56 +134,76 @@ __global__ __launch_bounds__(256) void attn_flash_kernel(AttnArgs a) {
     if (SPLIT) { rt = blockIdx.x / a.nseg; seg = blockIdx.x % a.nseg; }
     else { rt = blockIdx.x * 4 + wave; seg = 0; }
 
-    // ---- this lane's query row
+    // ---- this lane's query row. Loads are requested in dependency order and consumed late: the index
+    // operands first, then q (its address needs no loaded value), so one memory round trip covers both.
     const int r = rt * 16 + n;
     const bool row_ok = rt < a.row_tiles && r < a.rows_total;
     const int li = row_ok ? r / a.groups : 0, gi = row_ok ? r % a.groups : 0;
     const int hq = hk * a.groups + gi;
-    int kv_end = a.kv_lengths ? a.kv_lengths[b] : a.T;
-    kv_end = max(0, min(kv_end, a.T));
+    const int kv_end_raw = a.kv_lengths ? a.kv_lengths[b] : a.T;
+    const int pos_raw = (row_ok && a.positions) ? a.positions[(size_t)b * a.L + li] : li;
+
+    const size_t qbase = (((size_t)b * a.L + li) * a.Hq + hq) * D;
+    const bool q_f32_vec = a.q_dtype == AIONHIP_F32 && (((uintptr_t)a.q) & 15) == 0;
+    const bool q_same = a.q_dtype == KV && (((uintptr_t)a.q) & 15) == 0;
+    u32x4 qf[KK], qf_lo[HILO ? KK : 1];
+    f32x4 qx0[KK], qx1[KK];
+    if (q_same) {                    // already in the MFMA element type: one 16-byte load per k-step
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk)
+            qf[kk] = *(const u32x4 *)((const unsigned short *)a.q + qbase + kk * 32 + g * 8);
+    } else if (q_f32_vec) {
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            const f32x4 *qp = (const f32x4 *)((const float *)a.q + qbase + kk * 32 + g * 8);
+            qx0[kk] = qp[0];
+            qx1[kk] = qp[1];
+        }
+    }
+
+    int kv_end = max(0, min(kv_end_raw, a.T));
     int lo = 0, hi = 0;
     if (row_ok) {
-        const int pos = a.positions ? a.positions[(size_t)b * a.L + li] : li;
-        window_keys(a.win_left, a.win_right, a.win_chunk, max(pos, 0), kv_end, lo, hi);
+        window_keys(a.win_left, a.win_right, a.win_chunk, max(pos_raw, 0), kv_end, lo, hi);
         if (hi < lo) hi = lo;
     }
     const int uni_lo = wave_min_i(hi > lo ? lo : INT_MAX);
     const int uni_hi = wave_max_i(hi > lo ? hi : 0);
 
     // ---- Q^T operand: 8 consecutive d of row n per k-step, converted to the K/V element type
-    u32x4 qf[KK], qf_lo[HILO ? KK : 1];
-    {
-        const size_t qbase = (((size_t)b * a.L + li) * a.Hq + hq) * D;
-        const bool q_f32_vec = a.q_dtype == AIONHIP_F32 && (((uintptr_t)a.q) & 15) == 0;
-        const bool q_same = a.q_dtype == KV && (((uintptr_t)a.q) & 15) == 0;
 #pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-            if (q_same) {            // already in the MFMA element type: one 16-byte load
-                qf[kk] = row_ok ? *(const u32x4 *)((const unsigned short *)a.q + qbase + kk * 32 + g * 8) : u32x4{0u, 0u, 0u, 0u};
-                if (HILO) qf_lo[kk] = u32x4{0u, 0u, 0u, 0u};
-                continue;
-            }
-            float x[8];
-            if (q_f32_vec) {
-                const f32x4 *qp = (const f32x4 *)((const float *)a.q + qbase + kk * 32 + g * 8);
-                const f32x4 x0 = row_ok ? qp[0] : f32x4{0.f, 0.f, 0.f, 0.f}, x1 = row_ok ? qp[1] : f32x4{0.f, 0.f, 0.f, 0.f};
-                x[0] = x0.x; x[1] = x0.y; x[2] = x0.z; x[3] = x0.w; x[4] = x1.x; x[5] = x1.y; x[6] = x1.z; x[7] = x1.w;
-            } else {
-#pragma unroll
-                for (int j = 0; j < 8; ++j) x[j] = row_ok ? load_scalar(a.q, a.q_dtype, qbase + kk * 32 + g * 8 + j) : 0.f;
-            }
-            unsigned short h[8], lo8[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                h[j] = to_half_bits<KV>(x[j]);
-                lo8[j] = HILO ? to_half_bits<KV>(x[j] - from_half_bits<KV>(h[j])) : (unsigned short)0;
-            }
-            qf[kk] = u32x4{(unsigned)h[0] | ((unsigned)h[1] << 16), (unsigned)h[2] | ((unsigned)h[3] << 16),
-                           (unsigned)h[4] | ((unsigned)h[5] << 16), (unsigned)h[6] | ((unsigned)h[7] << 16)};
-            if (HILO)
-                qf_lo[kk] = u32x4{(unsigned)lo8[0] | ((unsigned)lo8[1] << 16), (unsigned)lo8[2] | ((unsigned)lo8[3] << 16),
-                                  (unsigned)lo8[4] | ((unsigned)lo8[5] << 16), (unsigned)lo8[6] | ((unsigned)lo8[7] << 16)};
+    for (int kk = 0; kk < KK; ++kk) {
+        if (q_same) {
+            if (!row_ok) qf[kk] = u32x4{0u, 0u, 0u, 0u};
+            if (HILO) qf_lo[kk] = u32x4{0u, 0u, 0u, 0u};
+            continue;
         }
+        float x[8];
+        if (q_f32_vec) {
+            x[0] = qx0[kk].x; x[1] = qx0[kk].y; x[2] = qx0[kk].z; x[3] = qx0[kk].w;
+            x[4] = qx1[kk].x; x[5] = qx1[kk].y; x[6] = qx1[kk].z; x[7] = qx1[kk].w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) x[j] = load_scalar(a.q, a.q_dtype, qbase + kk * 32 + g * 8 + j);
+        }
+        if (!HILO) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) x[j] = row_ok ? x[j] : 0.f;
+            qf[kk] = u32x4{pack2<KV>(x[0], x[1]), pack2<KV>(x[2], x[3]), pack2<KV>(x[4], x[5]), pack2<KV>(x[6], x[7])};
+            continue;
+        }
+        unsigned short h[8], lo8[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float xv = row_ok ? x[j] : 0.f;
+            h[j] = to_half_bits<KV>(xv);
+            lo8[j] = HILO ? to_half_bits<KV>(xv - from_half_bits<KV>(h[j])) : (unsigned short)0;
+        }
+        qf[kk] = u32x4{(unsigned)h[0] | ((unsigned)h[1] << 16), (unsigned)h[2] | ((unsigned)h[3] << 16),
+                       (unsigned)h[4] | ((unsigned)h[5] << 16), (unsigned)h[6] | ((unsigned)h[7] << 16)};
+        if (HILO)
+            qf_lo[kk] = u32x4{(unsigned)lo8[0] | ((unsigned)lo8[1] << 16), (unsigned)lo8[2] | ((unsigned)lo8[3] << 16),
+                              (unsigned)lo8[4] | ((unsigned)lo8[5] << 16), (unsigned)lo8[6] | ((unsigned)lo8[7] << 16)};
     }
 
     f32x4 acc[MT];
@@ -186,7 +219,7 @@ __global__ __launch_bounds__(256) void attn_flash_kernel(AttnArgs a) {
             const int per = (te - tb + a.nseg - 1) / a.nseg;
             t_begin = tb + seg * per + wave;
             t_end = min(tb + (seg + 1) * per, te);
-            t_step = 4;
+            t_step = NW;
         } else {
             t_begin = tb;
             t_end = te;
@@ -201,30 +234,33 @@ __global__ __launch_bounds__(256) void attn_flash_kernel(AttnArgs a) {
 
     for (int t = t_begin; t < t_end; t += t_step) {
         const int key0 = t * TILE_KEYS;
-        // -- stage V[key0 .. key0+32) into LDS (rows outside the union interval as zeros)
+        // -- request this tile's K (MFMA operand layout) and then V (staging layout); loads return in
+        //    order, so the S MFMAs wait for K only while V is still in flight
         constexpr int CHUNKS_PER_KEY = D / 8;
+        constexpr int NV = TILE_KEYS * CHUNKS_PER_KEY / 64;
+        u32x4 kf[2][KK], vreg[NV];
 #pragma unroll
-        for (int i = 0; i < TILE_KEYS * CHUNKS_PER_KEY / 64; ++i) {
+        for (int h = 0; h < 2; ++h) {
+            const int kabs = min(key0 + h * 16 + n, a.T - 1);
+            const unsigned short *krow = kp + kv_base + (size_t)kabs * kv_row + g * 8;
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) kf[h][kk] = *(const u32x4 *)(krow + kk * 32);
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
             const int c = lane + 64 * i;
-            const int key = c / CHUNKS_PER_KEY, col8 = c % CHUNKS_PER_KEY;
-            const int kabs = key0 + key;
-            u32x4 val = u32x4{0u, 0u, 0u, 0u};
-            if (kabs >= uni_lo && kabs < uni_hi)
-                val = *(const u32x4 *)(vp + kv_base + (size_t)kabs * kv_row + col8 * 8);
-            *(u32x4 *)(vs + key * Cfg::ROW_BYTES + col8 * 16) = val;
+            const int kabs = min(key0 + c / CHUNKS_PER_KEY, a.T - 1);
+            vreg[i] = *(const u32x4 *)(vp + kv_base + (size_t)kabs * kv_row + (c % CHUNKS_PER_KEY) * 8);
         }
         // -- S^T = K . Q^T for two 16-key halves
         f32x4 s[2];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const int kabs = min(key0 + h * 16 + n, a.T - 1);
-            const unsigned short *krow = kp + kv_base + (size_t)kabs * kv_row + g * 8;
             f32x4 c = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int kk = 0; kk < KK; ++kk) {
-                const u32x4 kf = *(const u32x4 *)(krow + kk * 32);
-                c = mfma16<KV>(kf, qf[kk], c);
-                if (HILO) c = mfma16<KV>(kf, qf_lo[kk], c);
+                c = mfma16<KV>(kf[h][kk], qf[kk], c);
+                if (HILO) c = mfma16<KV>(kf[h][kk], qf_lo[kk], c);
             }
             s[h] = c;
         }
@@ -273,12 +309,22 @@ __global__ __launch_bounds__(256) void attn_flash_kernel(AttnArgs a) {
         const u32x4 pf_lo = u32x4{(unsigned)pl[0] | ((unsigned)pl[1] << 16), (unsigned)pl[2] | ((unsigned)pl[3] << 16),
                                   (unsigned)pl[4] | ((unsigned)pl[5] << 16), (unsigned)pl[6] | ((unsigned)pl[7] << 16)};
 
-        // the staged tile is written and read by this wavefront only
+        // -- stage V into this wavefront's LDS tile (keys outside the union interval as zeros: the cache
+        //    tail may hold anything) ; the tile is written and read by this wavefront only
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = lane + 64 * i;
+            const int key = c / CHUNKS_PER_KEY, col8 = c % CHUNKS_PER_KEY;
+            const int kabs = key0 + key;
+            const bool inside = kabs >= uni_lo && kabs < uni_hi;
+            *(u32x4 *)(vs + key * Cfg::ROW_BYTES + col8 * 16) = inside ? vreg[i] : u32x4{0u, 0u, 0u, 0u};
+        }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
         // -- O^T += V^T . P^T ; operand slot j of lane group g is key g*4+j (j<4) / 16+g*4+j-4
+        const bool rescale = __any(alpha != 1.f);     // wavefront-uniform: skip 4*MT multiplies when no row's max moved
         const unsigned char *vcol = vs + n * 2;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
@@ -291,7 +337,7 @@ __global__ __launch_bounds__(256) void attn_flash_kernel(AttnArgs a) {
             const u32x4 vf = u32x4{(unsigned)e[0] | ((unsigned)e[1] << 16), (unsigned)e[2] | ((unsigned)e[3] << 16),
                                    (unsigned)e[4] | ((unsigned)e[5] << 16), (unsigned)e[6] | ((unsigned)e[7] << 16)};
             f32x4 c = acc[mt];
-            c *= alpha;
+            if (rescale) c *= alpha;
             c = mfma16<KV>(vf, pf, c);
             if (HILO) c = mfma16<KV>(vf, pf_lo, c);
             acc[mt] = c;
@@ -310,43 +356,58 @@ __global__ __launch_bounds__(256) void attn_flash_kernel(AttnArgs a) {
         return;
     }
 
-    // ---- split mode: merge the four wavefronts through LDS
+    // ---- split mode: merge the wavefronts through LDS. Rows are D+4 floats apart so that the sixteen
+    // lanes of a row group write their 16-byte pieces to distinct banks.
     __syncthreads();
     float *mg = (float *)lds;
-    constexpr int WSTRIDE = 16 * D + 32;
+    constexpr int RS = D + 4;                 // padded row stride (floats)
+    constexpr int WSTRIDE = 16 * RS + 32;     // one wavefront's slot: acc[16][RS], m[16], l[16]
     {
         float *w = mg + wave * WSTRIDE;
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) w[n * D + mt * 16 + g * 4 + i] = acc[mt][i];
-        if (g == 0) { w[16 * D + n] = m_run; w[16 * D + 16 + n] = l_run; }
+        for (int mt = 0; mt < MT; ++mt) *(f32x4 *)(w + n * RS + mt * 16 + g * 4) = acc[mt];
+        if (g == 0) { w[16 * RS + n] = m_run; w[16 * RS + 16 + n] = l_run; }
     }
     __syncthreads();
-    const size_t pslot = ((size_t)(unit * a.row_tiles + rt) * a.nseg + seg) * WSTRIDE;
-    for (int idx = threadIdx.x; idx < 16 * D; idx += 256) {
-        const int row = idx / D;
+    // per (row, wavefront) weights exp2(m_w - m_all), once; kept behind the NW slots
+    float *fac = mg + NW * WSTRIDE;           // [16][NW] factors, then [16] m_all, [16] l_all
+    if (threadIdx.x < 16) {
+        const int row = threadIdx.x;
         float m_all = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) m_all = fmaxf(m_all, mg[w * WSTRIDE + 16 * D + row]);
-        float o = 0.f, l_all = 0.f;
+        for (int w = 0; w < NW; ++w) m_all = fmaxf(m_all, mg[w * WSTRIDE + 16 * RS + row]);
+        float l_all = 0.f;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const float mw = mg[w * WSTRIDE + 16 * D + row];
+        for (int w = 0; w < NW; ++w) {
+            const float mw = mg[w * WSTRIDE + 16 * RS + row];
             const float f = mw > -INFINITY ? exp2f((mw - m_all) * LOG2E) : 0.f;
-            o += mg[w * WSTRIDE + idx] * f;
-            l_all += mg[w * WSTRIDE + 16 * D + 16 + row] * f;
+            fac[row * NW + w] = f;
+            l_all += mg[w * WSTRIDE + 16 * RS + 16 + row] * f;
         }
+        fac[16 * NW + row] = m_all;
+        fac[16 * NW + 16 + row] = l_all;
+    }
+    __syncthreads();
+    // partial slot layout in global memory (read by attn_merge_kernel): [16][D] o, [16] m, [16] l
+    constexpr int PSTRIDE = 16 * D + 32;
+    const size_t pslot = ((size_t)(unit * a.row_tiles + rt) * a.nseg + seg) * PSTRIDE;
+    for (int e = threadIdx.x; e < 16 * D / 4; e += NW * 64) {
+        const int row = e / (D / 4), col = (e % (D / 4)) * 4;
+        f32x4 o = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < NW; ++w) o += *(const f32x4 *)(mg + w * WSTRIDE + row * RS + col) * fac[row * NW + w];
+        const float l_all = fac[16 * NW + 16 + row];
         if (a.nseg == 1) {
             const int rr = rt * 16 + row;
             if (rr < a.rows_total) {
                 const int l2 = rr / a.groups, g2 = rr % a.groups;
-                a.out[(((size_t)b * a.L + l2) * a.Hq + hk * a.groups + g2) * D + idx % D] = l_all > 0.f ? o / l_all : 0.f;
+                const float inv = l_all > 0.f ? 1.f / l_all : 0.f;
+                *(f32x4 *)(a.out + (((size_t)b * a.L + l2) * a.Hq + hk * a.groups + g2) * D + col) = o * inv;
             }
         } else {
-            a.partial[pslot + idx] = o;
-            if (idx % D == 0) {
-                a.partial[pslot + 16 * D + row] = m_all;
+            *(f32x4 *)(a.partial + pslot + row * D + col) = o;
+            if (col == 0) {
+                a.partial[pslot + 16 * D + row] = fac[16 * NW + row];
                 a.partial[pslot + 16 * D + 16 + row] = l_all;
             }
         }
@@ -431,15 +492,17 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(AttnArgs a, int d_k, 
 
 template <int KV, int D, bool HILO>
 int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
-    using Cfg = FlashCfg<D>;
+    using Cfg = FlashCfg<D, 4>;
+    using SplitCfg = FlashCfg<D, SPLIT_NW>;
     const int units = a.B * a.Hkv;
     const bool split = a.rows_total <= 64;
     if (split) {
-        // key segments: at least 8 tiles (two per wavefront) each, at most ~2 workgroups per CU
+        // key segments: one 32-key tile per wavefront while that leaves the device under-filled,
+        // more tiles per wavefront beyond ~2 workgroups per CU
         const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
         const int tiles = (a.T + TILE_KEYS - 1) / TILE_KEYS;
         int nseg = (2 * cus + units * a.row_tiles - 1) / (units * a.row_tiles);
-        nseg = max(1, min(nseg, tiles / 8));
+        nseg = max(1, min(nseg, (tiles + SPLIT_NW - 1) / SPLIT_NW));
         nseg = min(nseg, 256);
         a.nseg = nseg;
         if (nseg > 1) {
@@ -450,11 +513,11 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
         }
         static bool attr_split = false;   // per kernel instantiation
         if (!attr_split) {
-            HIP_TRY(ctx, hipFuncSetAttribute((const void *)attn_flash_kernel<KV, D, true, HILO>, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
+            HIP_TRY(ctx, hipFuncSetAttribute((const void *)attn_flash_kernel<KV, D, true, HILO>, hipFuncAttributeMaxDynamicSharedMemorySize, SplitCfg::LDS_BYTES));
             attr_split = true;
         }
         prof_begin(ctx, "attn_flash_split");
-        attn_flash_kernel<KV, D, true, HILO><<<dim3((unsigned)(a.row_tiles * nseg), (unsigned)units), dim3(256), Cfg::LDS_BYTES, ctx->stream>>>(a);
+        attn_flash_kernel<KV, D, true, HILO><<<dim3((unsigned)(a.row_tiles * nseg), (unsigned)units), dim3(SPLIT_NW * 64), SplitCfg::LDS_BYTES, ctx->stream>>>(a);
         if (nseg > 1) attn_merge_kernel<D><<<dim3((unsigned)(a.row_tiles * (D / 64)), (unsigned)units), dim3(256), 0, ctx->stream>>>(a);
         prof_end(ctx);
         LAUNCH_CHECK(ctx, "attn_flash_split");
@@ -475,7 +538,7 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
 
 template <int KV>
 int launch_flash_d(aionhip_ctx *ctx, AttnArgs &a, int d) {
-    const bool hilo = a.q_dtype == AIONHIP_F32;
+    const bool hilo = a.q_dtype == AIONHIP_F32 && ctx->attn_precise;
     if (d == 64) return hilo ? launch_flash<KV, 64, true>(ctx, a) : launch_flash<KV, 64, false>(ctx, a);
     if (d == 128) return hilo ? launch_flash<KV, 128, true>(ctx, a) : launch_flash<KV, 128, false>(ctx, a);
     return hilo ? launch_flash<KV, 256, true>(ctx, a) : launch_flash<KV, 256, false>(ctx, a);

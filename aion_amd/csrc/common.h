@@ -40,6 +40,16 @@ struct aionhip_ctx {
     // second scratch for GEMM staging (dequantized weights / bf16 activations / split-K partials)
     void *scratch2 = nullptr;
     size_t scratch2_bytes = 0;
+    // attention with f32 queries: false = one MFMA pass on q rounded to the K/V element type (2e-3 class),
+    // true = q and the probabilities as hi+lo parts (f32-level accuracy, about 1.4x the instructions)
+    bool attn_precise = false;
+    // RoPE frequency tables (f32, multiplied up iteratively as on the CPU), one per (pairs, base, d, scale)
+    struct RopeTable {
+        int pairs;
+        float freq_step, scale_factor;
+        float *freq;
+    };
+    std::vector<RopeTable> rope_tables;
     // true between aionhip_program_begin/end: launches are captured, nothing may synchronise or allocate
     bool capturing = false;
     // per-launch timing, off by default
@@ -97,6 +107,7 @@ struct PreparedAct {
 size_t prepared_act_bytes(size_t m, size_t k);
 PreparedAct prepared_act_carve(void *base, size_t m, size_t k);
 int launch_prepare_act(aionhip_ctx *ctx, const float *a, size_t lda, size_t m, size_t k, PreparedAct out);
+int launch_prepare_gate(aionhip_ctx *ctx, const float *gate, const float *up, size_t m, size_t k, PreparedAct out);
 
 // ---- matmul back ends --------------------------------------------------------------------------
 // Up to four weights that multiply the SAME activation rows (q/k/v, gate/up) run as one launch:
@@ -124,11 +135,15 @@ struct FusedIn {
     float eps;
 };
 constexpr size_t FUSED_MAX_K = 8192;
+// above this K the per-workgroup prologue costs more than a separate preparation launch
+constexpr size_t FUSED_PAYS_K = 4096;
 int launch_gemv_fused(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count,
                       int prologue, FusedIn in, float alpha, float beta);
 int launch_rmsnorm(aionhip_ctx *ctx, float *out, const float *x, const float *gamma, const float *beta, const float *residual,
                    size_t rows, size_t cols, float eps);
 int launch_gate_gelu(aionhip_ctx *ctx, float *out, const float *a, const float *b, size_t n);
+// device table f[i] = scale_factor * freq_step^i built with f32 multiplies in sequence (aion cpu/kernels/rope.zig:22-30)
+int rope_table(aionhip_ctx *ctx, int pairs, float freq_step, float scale_factor, const float **out);
 
 int launch_gemv(aionhip_ctx *ctx, const aionhip_weight *w, int m, PreparedAct act, float *c, size_t ldc, float alpha, float beta);
 int launch_gemv_batch(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count, int m,

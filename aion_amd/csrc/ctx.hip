@@ -59,7 +59,40 @@ void prof_end(aionhip_ctx *ctx) {
     (void)hipEventRecord(ctx->prof.back().stop, ctx->stream);
 }
 
+int rope_table(aionhip_ctx *ctx, int pairs, float freq_step, float scale_factor, const float **out) {
+    for (const auto &t : ctx->rope_tables)
+        if (t.pairs == pairs && t.freq_step == freq_step && t.scale_factor == scale_factor) {
+            *out = t.freq;
+            return AIONHIP_OK;
+        }
+    if (ctx->capturing)
+        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "a RoPE table must be built while a program is being recorded: run the steps once before recording");
+    std::vector<float> host((size_t)(pairs > 0 ? pairs : 1));
+    float f = scale_factor;
+    for (int i = 0; i < pairs; ++i) {
+        host[(size_t)i] = f;
+        f *= freq_step;
+    }
+    void *dev = nullptr;
+    HIP_TRY(ctx, hipMalloc(&dev, host.size() * sizeof(float)));
+    hipError_t e = hipMemcpyAsync(dev, host.data(), host.size() * sizeof(float), hipMemcpyHostToDevice, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) {
+        (void)hipFree(dev);
+        return set_err(ctx, AIONHIP_EXECUTION_FAILED, "rope table upload: %s", hipGetErrorString(e));
+    }
+    ctx->rope_tables.push_back({pairs, freq_step, scale_factor, (float *)dev});
+    *out = (const float *)dev;
+    return AIONHIP_OK;
+}
+
 extern "C" {
+
+int aionhip_set_attention_precise(aionhip_ctx *ctx, int on) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    ctx->attn_precise = on != 0;
+    return AIONHIP_OK;
+}
 
 int aionhip_profile_start(aionhip_ctx *ctx) {
     if (!ctx) return AIONHIP_INVALID_ARGUMENT;
@@ -121,6 +154,7 @@ void aionhip_destroy(aionhip_ctx *ctx) {
         (void)hipEventDestroy(r.stop);
     }
     for (auto e : ctx->event_pool) (void)hipEventDestroy(e);
+    for (auto &t : ctx->rope_tables) (void)hipFree(t.freq);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
     if (ctx->scratch2) (void)hipFree(ctx->scratch2);
     if (ctx->own_stream) (void)hipStreamDestroy(ctx->stream);

@@ -6,65 +6,96 @@
 // produces the activation - runs as a prologue of the GEMV instead of as launches of their own.
 // Every workgroup recomputes the (small) activation into LDS with the same arithmetic as the
 // stand-alone kernels (same codes, same scales), then streams its weight rows exactly like
-// gemv_kernel: one wavefront per R rows, 16-byte chunks per lane, v_dot4_i32_i8, DPP fold.
+// gemv_kernel: one wavefront per R rows, 16-byte chunks per lane, v_dot4_i32_i8, DPP fold. The
+// grid is capped at a few workgroups per CU and wavefronts stride over the row groups, so the
+// prologue is paid a bounded number of times however many rows the weight has.
 // K <= 8192 (10 KB of LDS); larger K keeps the separate preparation launch.
 #include "common.h"
 
+#include <cstdlib>
+
 namespace {
 
-constexpr int MAX_CH4 = (int)(FUSED_MAX_K / 4 / 256);   // float4 chunks per thread
-
-template <int DT, int R, int PRO>
+// NCH = float4 activation chunks per thread (K <= 1024 * NCH). LDS is sized per launch:
+// K bytes of codes, K/32 scales, K/32 code sums, 4 reduction slots.
+template <int DT, int R, int PRO, int NCH>
 __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedIn in, int K, float alpha, float beta) {
-    __shared__ __attribute__((aligned(16))) int s_aq[FUSED_MAX_K / 4];
-    __shared__ float s_scale[FUSED_MAX_K / QK];
-    __shared__ int s_sum[FUSED_MAX_K / QK];
-    __shared__ float s_red[4];
+    extern __shared__ __attribute__((aligned(16))) unsigned char s_mem[];
+    int *s_aq = (int *)s_mem;
+    float *s_scale = (float *)(s_mem + K);
+    int *s_sum = (int *)(s_mem + K + (K >> 5) * 4);
+    float *s_red = (float *)(s_mem + K + (K >> 5) * 8);
+    constexpr int MAX_CH4 = NCH;
 
     const int tid = threadIdx.x, lane = tid & 63;
-    const int gwave = blockIdx.x * 4 + (tid >> 6);
-    const bool active = gwave < batch.total_waves;
-    int si = 0;
-#pragma unroll
-    for (int i = 1; i < 4; ++i)
-        if (i < batch.count && gwave >= batch.seg[i].first_wave) si = i;
-    const u32x4 *__restrict__ qs = batch.seg[si].qs;
-    const __half *__restrict__ sc = batch.seg[si].sc;
-    const int N = batch.seg[si].n;
-    const int row0 = active ? (gwave - batch.seg[si].first_wave) * R : 0;
+    const int wave_stride = gridDim.x * 4;
+    int gwave = blockIdx.x * 4 + (tid >> 6);
     const int KB = K >> 5;
     constexpr bool Q8 = DT == AIONHIP_Q8_0;
     const int chunks = Q8 ? (K >> 4) : KB;
 
-    size_t rowq[R], rows[R];
+    // the row group of wavefront index `gw`: segment, first row, row offsets
+    struct Group {
+        const u32x4 *qs;
+        const __half *sc;
+        float *c;
+        int n, row0;
+        size_t rowq[R], rows[R];
+    };
+    auto locate = [&](int gw) {
+        Group gr;
+        int si = 0;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const int row = min(row0 + r, N - 1);
-        rowq[r] = (size_t)row * chunks;
-        rows[r] = (size_t)row * KB;
-    }
-    // first weight chunk of every row: issued before the prologue so that its latency overlaps it
-    u32x4 w0[R];
-    float ws0[R];
-    const bool have0 = active && lane < chunks;
+        for (int i = 1; i < 4; ++i)
+            if (i < batch.count && gw >= batch.seg[i].first_wave) si = i;
+        gr.qs = batch.seg[si].qs;
+        gr.sc = batch.seg[si].sc;
+        gr.c = batch.seg[si].c;
+        gr.n = batch.seg[si].n;
+        gr.row0 = (gw - batch.seg[si].first_wave) * R;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        w0[r] = have0 ? __builtin_nontemporal_load(qs + rowq[r] + lane) : u32x4{0u, 0u, 0u, 0u};
-        ws0[r] = have0 ? __half2float(sc[rows[r] + (Q8 ? (lane >> 1) : lane)]) : 0.f;
-    }
-
+        for (int r = 0; r < R; ++r) {
+            const int row = min(gr.row0 + r, gr.n - 1);
+            gr.rowq[r] = (size_t)row * chunks;
+            gr.rows[r] = (size_t)row * KB;
+        }
+        return gr;
+    };
+    bool active = gwave < batch.total_waves;
+    Group cur = locate(active ? gwave : 0);
     // ---- prologue: activation -> int8 codes, per-block scale and code sum in LDS
     const int n4 = K >> 2;
-    f32x4 v[MAX_CH4];
-    float ss = 0.f;
+    f32x4 v[MAX_CH4], aux[PRO == PRO_QUANT ? 1 : MAX_CH4], aux2[PRO == PRO_RMSNORM ? MAX_CH4 : 1];
+    // every global operand of the prologue is requested up front: one memory latency, not three
 #pragma unroll
     for (int i = 0; i < MAX_CH4; ++i) {
         const int c4 = tid + 256 * i;
-        v[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (c4 < n4) {
-            v[i] = *(const f32x4 *)(in.x + (size_t)c4 * 4);
-            if (PRO == PRO_RMSNORM) ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+        const bool live = c4 < n4;
+        v[i] = live ? *(const f32x4 *)(in.x + (size_t)c4 * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+        if (PRO == PRO_RMSNORM) {
+            aux[i] = live ? *(const f32x4 *)(in.gamma + (size_t)c4 * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+            aux2[i] = (live && in.beta) ? *(const f32x4 *)(in.beta + (size_t)c4 * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+        } else if (PRO == PRO_GATE) {
+            aux[i] = live ? *(const f32x4 *)(in.y + (size_t)c4 * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
         }
+    }
+    // first weight chunk of every row: requested right behind the activation operands (loads return
+    // in order, so the prologue waits for the activation only while these stay in flight)
+    // (unconditional loads at clamped addresses: predicated loads would be waited for one by one)
+    u32x4 w0[R];
+    __half hs0[R];
+    const bool lane_has0 = lane < chunks;
+    const int l0 = min(lane, chunks - 1);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        w0[r] = __builtin_nontemporal_load(cur.qs + cur.rowq[r] + l0);
+        hs0[r] = cur.sc[cur.rows[r] + (Q8 ? (l0 >> 1) : l0)];
+    }
+
+    float ss = 0.f;
+    if (PRO == PRO_RMSNORM) {
+#pragma unroll
+        for (int i = 0; i < MAX_CH4; ++i) ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
     }
     float inv_rms = 1.f;
     if (PRO == PRO_RMSNORM) {
@@ -78,15 +109,13 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedI
         f32x4 a = v[i];
         if (live) {
             if (PRO == PRO_RMSNORM) {
-                const f32x4 gm = *(const f32x4 *)(in.gamma + (size_t)c4 * 4);
-                f32x4 bt = f32x4{0.f, 0.f, 0.f, 0.f};
-                if (in.beta) bt = *(const f32x4 *)(in.beta + (size_t)c4 * 4);
+                const f32x4 gm = aux[i], bt = aux2[i];
                 a.x = (a.x * inv_rms) * gm.x + bt.x;
                 a.y = (a.y * inv_rms) * gm.y + bt.y;
                 a.z = (a.z * inv_rms) * gm.z + bt.z;
                 a.w = (a.w * inv_rms) * gm.w + bt.w;
             } else if (PRO == PRO_GATE) {
-                const f32x4 up = *(const f32x4 *)(in.y + (size_t)c4 * 4);
+                const f32x4 up = aux[i];
                 a.x = aion_gate_gelu(a.x, up.x);
                 a.y = aion_gate_gelu(a.y, up.y);
                 a.z = aion_gate_gelu(a.z, up.z);
@@ -122,73 +151,102 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedI
         }
     }
     __syncthreads();
-    if (!active) return;
 
-    // ---- stream the rows
+    // ---- stream the row groups
     const u32x4 *aq = (const u32x4 *)s_aq;
-    float acc[R];
+    while (active) {
+        float acc[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] = 0.f;
+        for (int r = 0; r < R; ++r) acc[r] = 0.f;
 
-    auto consume = [&](int ch, const u32x4 (&w)[R], const float (&ws)[R]) {
-        const int blk = Q8 ? (ch >> 1) : ch;
-        const float as = s_scale[blk];
-        if (Q8) {
-            const u32x4 a = aq[ch];
+        auto consume = [&](int ch, const u32x4 (&w)[R], const float (&ws)[R]) {
+            const int blk = Q8 ? (ch >> 1) : ch;
+            const float as = s_scale[blk];
+            if (Q8) {
+                const u32x4 a = aq[ch];
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                int d = dot4_i8((int)a.x, (int)w[r].x, 0);
-                d = dot4_i8((int)a.y, (int)w[r].y, d);
-                d = dot4_i8((int)a.z, (int)w[r].z, d);
-                d = dot4_i8((int)a.w, (int)w[r].w, d);
-                acc[r] += (float)d * (as * ws[r]);
+                for (int r = 0; r < R; ++r) {
+                    int d = dot4_i8((int)a.x, (int)w[r].x, 0);
+                    d = dot4_i8((int)a.y, (int)w[r].y, d);
+                    d = dot4_i8((int)a.z, (int)w[r].z, d);
+                    d = dot4_i8((int)a.w, (int)w[r].w, d);
+                    acc[r] += (float)d * (as * ws[r]);
+                }
+            } else {
+                const u32x4 a0 = aq[2 * ch], a1 = aq[2 * ch + 1];
+                const int bias = 8 * s_sum[blk];
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    constexpr unsigned M = 0x0F0F0F0Fu;
+                    int d = dot4_i8((int)a0.x, (int)(w[r].x & M), -bias);
+                    d = dot4_i8((int)a0.y, (int)((w[r].x >> 4) & M), d);
+                    d = dot4_i8((int)a0.z, (int)(w[r].y & M), d);
+                    d = dot4_i8((int)a0.w, (int)((w[r].y >> 4) & M), d);
+                    d = dot4_i8((int)a1.x, (int)(w[r].z & M), d);
+                    d = dot4_i8((int)a1.y, (int)((w[r].z >> 4) & M), d);
+                    d = dot4_i8((int)a1.z, (int)(w[r].w & M), d);
+                    d = dot4_i8((int)a1.w, (int)((w[r].w >> 4) & M), d);
+                    acc[r] += (float)d * (as * ws[r]);
+                }
             }
-        } else {
-            const u32x4 a0 = aq[2 * ch], a1 = aq[2 * ch + 1];
-            const int bias = 8 * s_sum[blk];
+        };
+
+        if (lane_has0) {
+            float ws0[R];
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                constexpr unsigned M = 0x0F0F0F0Fu;
-                int d = dot4_i8((int)a0.x, (int)(w[r].x & M), -bias);
-                d = dot4_i8((int)a0.y, (int)((w[r].x >> 4) & M), d);
-                d = dot4_i8((int)a0.z, (int)(w[r].y & M), d);
-                d = dot4_i8((int)a0.w, (int)((w[r].y >> 4) & M), d);
-                d = dot4_i8((int)a1.x, (int)(w[r].z & M), d);
-                d = dot4_i8((int)a1.y, (int)((w[r].z >> 4) & M), d);
-                d = dot4_i8((int)a1.z, (int)(w[r].w & M), d);
-                d = dot4_i8((int)a1.w, (int)((w[r].w >> 4) & M), d);
-                acc[r] += (float)d * (as * ws[r]);
+            for (int r = 0; r < R; ++r) ws0[r] = __half2float(hs0[r]);
+            consume(lane, w0, ws0);
+        }
+        // the remaining chunks, U at a time with all U*R loads in flight before the first is consumed
+        constexpr int U = R == 1 ? 4 : (R == 2 ? 2 : 1);
+#pragma unroll 1
+        for (int ch0 = lane + 64; ch0 < chunks; ch0 += 64 * U) {
+            u32x4 w[U][R];
+            __half hs[U][R];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int ch = min(ch0 + 64 * u, chunks - 1);
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    w[u][r] = __builtin_nontemporal_load(cur.qs + cur.rowq[r] + ch);
+                    hs[u][r] = cur.sc[cur.rows[r] + (Q8 ? (ch >> 1) : ch)];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (ch0 + 64 * u < chunks) {
+                    float ws[R];
+#pragma unroll
+                    for (int r = 0; r < R; ++r) ws[r] = __half2float(hs[u][r]);
+                    consume(ch0 + 64 * u, w[u], ws);
+                }
             }
         }
-    };
 
-    if (have0) consume(lane, w0, ws0);
-#pragma unroll 2
-    for (int ch = lane + 64; ch < chunks; ch += 64) {
-        u32x4 w[R];
-        float ws[R];
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            w[r] = __builtin_nontemporal_load(qs + rowq[r] + ch);
-            ws[r] = __half2float(sc[rows[r] + (Q8 ? (ch >> 1) : ch)]);
+        for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
+        if (lane == 0) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                if (cur.row0 + r >= cur.n) break;
+                const float val = alpha * acc[r];
+                cur.c[cur.row0 + r] = beta == 0.f ? val : val + beta * cur.c[cur.row0 + r];
+            }
         }
-        consume(ch, w, ws);
-    }
-
+        gwave += wave_stride;
+        active = gwave < batch.total_waves;
+        if (active) {
+            cur = locate(gwave);
 #pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
-    if (lane == 0) {
-        float *c = batch.seg[si].c;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            if (row0 + r >= N) break;
-            const float val = alpha * acc[r];
-            c[row0 + r] = beta == 0.f ? val : val + beta * c[row0 + r];
+            for (int r = 0; r < R; ++r) {
+                w0[r] = __builtin_nontemporal_load(cur.qs + cur.rowq[r] + l0);
+                hs0[r] = cur.sc[cur.rows[r] + (Q8 ? (l0 >> 1) : l0)];
+            }
         }
     }
 }
 
-template <int DT, int PRO>
+template <int DT, int PRO, int NCH>
 void launch_r(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count, FusedIn in,
               float alpha, float beta) {
     const int K = (int)ws[0]->k;
@@ -206,18 +264,31 @@ void launch_r(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *c
         waves += ((int)ws[i]->n + R - 1) / R;
     }
     batch.total_waves = waves;
-    const dim3 grid((unsigned)((waves + 3) / 4)), block(256);
-    if (R == 4) gemv_fused_kernel<DT, 4, PRO><<<grid, block, 0, ctx->stream>>>(batch, in, K, alpha, beta);
-    else if (R == 2) gemv_fused_kernel<DT, 2, PRO><<<grid, block, 0, ctx->stream>>>(batch, in, K, alpha, beta);
-    else gemv_fused_kernel<DT, 1, PRO><<<grid, block, 0, ctx->stream>>>(batch, in, K, alpha, beta);
+    // at most 8 workgroups per CU: beyond that the wavefronts stride over the row groups
+    const int wgs = (waves + 3) / 4;
+    static const int cap_mult = getenv("AIONHIP_FUSED_CAP") ? atoi(getenv("AIONHIP_FUSED_CAP")) : 8;
+    const dim3 grid((unsigned)(wgs < cus * cap_mult ? wgs : cus * cap_mult)), block(256);
+    const size_t lds = (size_t)K + (size_t)(K >> 5) * 8 + 16;
+    if (R == 4) gemv_fused_kernel<DT, 4, PRO, NCH><<<grid, block, lds, ctx->stream>>>(batch, in, K, alpha, beta);
+    else if (R == 2) gemv_fused_kernel<DT, 2, PRO, NCH><<<grid, block, lds, ctx->stream>>>(batch, in, K, alpha, beta);
+    else gemv_fused_kernel<DT, 1, PRO, NCH><<<grid, block, lds, ctx->stream>>>(batch, in, K, alpha, beta);
+}
+
+template <int DT, int PRO>
+void launch_n(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count, FusedIn in,
+              float alpha, float beta) {
+    const size_t k = ws[0]->k;
+    if (k <= 2048) launch_r<DT, PRO, 2>(ctx, ws, cs, ldcs, count, in, alpha, beta);
+    else if (k <= 4096) launch_r<DT, PRO, 4>(ctx, ws, cs, ldcs, count, in, alpha, beta);
+    else launch_r<DT, PRO, 8>(ctx, ws, cs, ldcs, count, in, alpha, beta);
 }
 
 template <int DT>
 void launch_p(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count, int pro, FusedIn in,
               float alpha, float beta) {
-    if (pro == PRO_RMSNORM) launch_r<DT, PRO_RMSNORM>(ctx, ws, cs, ldcs, count, in, alpha, beta);
-    else if (pro == PRO_GATE) launch_r<DT, PRO_GATE>(ctx, ws, cs, ldcs, count, in, alpha, beta);
-    else launch_r<DT, PRO_QUANT>(ctx, ws, cs, ldcs, count, in, alpha, beta);
+    if (pro == PRO_RMSNORM) launch_n<DT, PRO_RMSNORM>(ctx, ws, cs, ldcs, count, in, alpha, beta);
+    else if (pro == PRO_GATE) launch_n<DT, PRO_GATE>(ctx, ws, cs, ldcs, count, in, alpha, beta);
+    else launch_n<DT, PRO_QUANT>(ctx, ws, cs, ldcs, count, in, alpha, beta);
 }
 
 }  // namespace

@@ -26,15 +26,12 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(float *__restrict__ out, c
 }
 
 // cpu/exec/rope.zig:14-53 + cpu/kernels/rope.zig:20-98: pairs (i, i + D/2); the frequency is
-// multiplied up iteratively in f32 and the angle pos*f is rounded to f32, as on the CPU. aion
-// takes sin/cos of that f32 angle in f64 and rounds; here sincosf (full range reduction, <= 2 ulp).
-__device__ __forceinline__ float rope_freq(int i, float freq_step, float scale_factor) {
-    float f = scale_factor;
-    for (int j = 0; j < i; ++j) f *= freq_step;
-    return f;
-}
+// multiplied up iteratively in f32 (a per-context table built on the host) and the angle pos*f is
+// rounded to f32, as on the CPU. aion takes sin/cos of that f32 angle in f64 and rounds; here
+// sincosf (full range reduction, <= 2 ulp).
+
 __global__ void rope_kernel(float *__restrict__ out, const float *__restrict__ x, const int *__restrict__ positions,
-                            size_t tokens, int H, int D, int rope_pairs, float freq_step, float scale_factor) {
+                            size_t tokens, int H, int D, int rope_pairs, const float *__restrict__ freq) {
     const int half = D / 2;
     const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (gid >= tokens * (size_t)half) return;
@@ -49,7 +46,7 @@ __global__ void rope_kernel(float *__restrict__ out, const float *__restrict__ x
         }
         return;
     }
-    const float ang = (float)positions[tok] * rope_freq(i, freq_step, scale_factor);
+    const float ang = (float)positions[tok] * freq[i];
     float sn, cs;
     sincosf(ang, &sn, &cs);
     for (int h = 0; h < H; ++h) {
@@ -60,38 +57,47 @@ __global__ void rope_kernel(float *__restrict__ out, const float *__restrict__ x
 }
 
 // RoPE1D(q), RoPE1D(k) -> f16 -> SequenceAppend(k cache), Cast f16 + SequenceAppend(v cache) for the
-// tokens of one step, as one launch: thread (token, pair i) rotates pair i of every q head and
-// k head and copies the matching v elements. Same arithmetic as the four separate steps.
+// tokens of one step, as one launch: thread (token, head slot, pair i) rotates pair i of one q head,
+// or of one k head (and copies the matching v elements). Same arithmetic as the four separate steps.
 __global__ void rope_append_kernel(float *__restrict__ q_out, const float *__restrict__ q, const float *__restrict__ k, const float *__restrict__ v,
                                    __half *__restrict__ kcache, __half *__restrict__ vcache, const int *__restrict__ positions,
                                    const int *__restrict__ write_index, size_t batch, size_t s_len, size_t t_cap, int Hq, int Hkv, int D,
-                                   int rope_pairs, float freq_step, float scale_factor) {
+                                   int rope_pairs, const float *__restrict__ freq) {
     const int half = D / 2;
+    const int slots = Hq + Hkv;
     const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (gid >= batch * s_len * (size_t)half) return;
-    const size_t tok = gid / half;                 // b * s_len + s
+    if (gid >= batch * s_len * (size_t)slots * half) return;
     const int i = (int)(gid % half);
-    const size_t b = tok / s_len, s = tok % s_len;
+    const int slot = (int)((gid / half) % slots);
+    const size_t tok = gid / ((size_t)half * slots);          // b * s_len + s
+    // every global operand is requested before the first use: one memory round trip
+    const bool rot = i < rope_pairs;
+    const bool is_q = slot < Hq;
+    const int h = is_q ? slot : slot - Hq;
+    const size_t src = is_q ? (tok * Hq + h) * D : (tok * Hkv + h) * D;
+    const float *xp = is_q ? q : k;
+    const int pos = positions[tok];
+    const int widx = write_index[0];
+    const float fr = i < rope_pairs ? freq[i] : 0.f;
+    const float xl = xp[src + i], xh = xp[src + half + i];
+    float vl = 0.f, vh = 0.f;
+    if (!is_q) { vl = v[src + i]; vh = v[src + half + i]; }
     float sn = 0.f, cs = 1.f;
-    if (i < rope_pairs) sincosf((float)positions[tok] * rope_freq(i, freq_step, scale_factor), &sn, &cs);
-    const float *qr = q + tok * Hq * D;
-    float *qo = q_out + tok * Hq * D;
-    for (int h = 0; h < Hq; ++h) {
-        const float xl = qr[h * D + i], xh = qr[h * D + half + i];
-        qo[h * D + i] = i < rope_pairs ? xl * cs - xh * sn : xl;
-        qo[h * D + half + i] = i < rope_pairs ? xl * sn + xh * cs : xh;
+    if (rot) sincosf((float)pos * fr, &sn, &cs);
+    const float yl = rot ? xl * cs - xh * sn : xl, yh = rot ? xl * sn + xh * cs : xh;
+    if (is_q) {
+        q_out[src + i] = yl;
+        q_out[src + half + i] = yh;
+        return;
     }
-    const long t = (long)write_index[0] + (long)s;
-    if (t < 0 || (size_t)t >= t_cap) return;       // never write outside the cache
-    const float *kr = k + tok * Hkv * D, *vr = v + tok * Hkv * D;
-    __half *kc = kcache + (b * t_cap + (size_t)t) * Hkv * D, *vc = vcache + (b * t_cap + (size_t)t) * Hkv * D;
-    for (int h = 0; h < Hkv; ++h) {
-        const float xl = kr[h * D + i], xh = kr[h * D + half + i];
-        kc[h * D + i] = __float2half_rn(i < rope_pairs ? xl * cs - xh * sn : xl);
-        kc[h * D + half + i] = __float2half_rn(i < rope_pairs ? xl * sn + xh * cs : xh);
-        vc[h * D + i] = __float2half_rn(vr[h * D + i]);
-        vc[h * D + half + i] = __float2half_rn(vr[h * D + half + i]);
-    }
+    const size_t b = tok / s_len, s = tok % s_len;
+    const long t = (long)widx + (long)s;
+    if (t < 0 || (size_t)t >= t_cap) return;                   // never write outside the cache
+    const size_t dst = ((b * t_cap + (size_t)t) * Hkv + h) * D;
+    kcache[dst + i] = __float2half_rn(yl);
+    kcache[dst + half + i] = __float2half_rn(yh);
+    vcache[dst + i] = __float2half_rn(vl);
+    vcache[dst + half + i] = __float2half_rn(vh);
 }
 
 __global__ void add_kernel(float *__restrict__ out, const float *__restrict__ a, const float *__restrict__ b, size_t n) {
@@ -242,8 +248,11 @@ int aionhip_step_rope(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle x, ai
     size_t rope_pairs = (size_t)floorf(rope_proportion * (float)half);
     if (rope_pairs > half) rope_pairs = half;
     const float freq_step = (float)pow((double)base_frequency, (double)(-2.0f / (float)d));
+    const float *freq = nullptr;
+    int rc = rope_table(ctx, (int)rope_pairs, freq_step, scale_factor, &freq);
+    if (rc) return rc;
     rope_kernel<<<dim3(grid_for(tokens * half, 128)), dim3(128), 0, ctx->stream>>>(dp<float>(out), dp<const float>(x), dp<const int>(positions),
-                                                                                   tokens, (int)h, (int)d, (int)rope_pairs, freq_step, scale_factor);
+                                                                                   tokens, (int)h, (int)d, (int)rope_pairs, freq);
     LAUNCH_CHECK(ctx, "rope");
     return AIONHIP_OK;
 }
@@ -259,14 +268,17 @@ int aionhip_step_rope_append(aionhip_ctx *ctx, aionhip_handle q_out, aionhip_han
         return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "rope_append: base/scale must be positive and finite, proportion in [0,1]");
     if (d % 2 != 0 || d > 65534 || h_q > 65535 || h_kv > 65535) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "rope_append: head size must be even");
     if (s > t_cap) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "rope_append: %zu new tokens exceed the cache capacity %zu", s, t_cap);
-    const size_t half = d / 2, total = b * s * half;
+    const size_t half = d / 2, total = b * s * half * (h_q + h_kv);
     if (!total || !h_q || !h_kv) return AIONHIP_OK;
     size_t rope_pairs = (size_t)floorf(rope_proportion * (float)half);
     if (rope_pairs > half) rope_pairs = half;
     const float freq_step = (float)pow((double)base_frequency, (double)(-2.0f / (float)d));
+    const float *freq = nullptr;
+    int rc = rope_table(ctx, (int)rope_pairs, freq_step, scale_factor, &freq);
+    if (rc) return rc;
     rope_append_kernel<<<dim3(grid_for(total, 128)), dim3(128), 0, ctx->stream>>>(
         dp<float>(q_out), dp<const float>(q), dp<const float>(k), dp<const float>(v), dp<__half>(k_cache), dp<__half>(v_cache),
-        dp<const int>(positions), dp<const int>(write_index), b, s, t_cap, (int)h_q, (int)h_kv, (int)d, (int)rope_pairs, freq_step, scale_factor);
+        dp<const int>(positions), dp<const int>(write_index), b, s, t_cap, (int)h_q, (int)h_kv, (int)d, (int)rope_pairs, freq);
     LAUNCH_CHECK(ctx, "rope_append");
     return AIONHIP_OK;
 }

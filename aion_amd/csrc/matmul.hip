@@ -39,7 +39,7 @@ int check_batch(aionhip_ctx *ctx, const char *what, size_t count, const aionhip_
 // every weight of `b` against the f32 rows at `a` (already materialised)
 int run_rows(aionhip_ctx *ctx, const Batch &b, size_t m, const float *a, size_t lda, float alpha, float beta) {
     if (m > 0x7FFFFFFFu) return set_err(ctx, AIONHIP_UNSUPPORTED, "matmul: m exceeds 2^31-1");
-    if (m == 1 && b.k <= FUSED_MAX_K && ((uintptr_t)a & 15) == 0)
+    if (m == 1 && b.k <= FUSED_PAYS_K && ((uintptr_t)a & 15) == 0)
         return launch_gemv_fused(ctx, b.w, b.c, b.ldc, (int)b.count, PRO_QUANT, FusedIn{a, nullptr, nullptr, nullptr, 0.f}, alpha, beta);
     if (m > GEMV_MAX_M && ctx->gemm_mode == AIONHIP_GEMM_BF16_MFMA) {
         for (size_t i = 0; i < b.count; ++i) {
@@ -116,7 +116,7 @@ int aionhip_step_rmsnorm_matmul(aionhip_ctx *ctx, size_t count, const aionhip_we
     if (!x || !gamma) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "rmsnorm_matmul: null x or gamma");
     if (!(eps > 0.f) || !(eps < INFINITY)) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "rmsnorm_matmul: eps must be positive and finite");
     const float *xp = (const float *)(uintptr_t)x, *gp = (const float *)(uintptr_t)gamma, *bp = (const float *)(uintptr_t)beta_norm;
-    if (rows == 1 && b.k <= FUSED_MAX_K && ((x | gamma | beta_norm) & 15) == 0)
+    if (rows == 1 && b.k <= FUSED_PAYS_K && ((x | gamma | beta_norm) & 15) == 0)
         return launch_gemv_fused(ctx, b.w, b.c, b.ldc, (int)b.count, PRO_RMSNORM, FusedIn{xp, nullptr, gp, bp, eps}, alpha, beta);
     // several rows: the norm runs as its own kernel into scratch, then the ordinary routing
     const size_t act_bytes = (prepared_act_bytes(rows, b.k) + 255) & ~(size_t)255;
@@ -137,8 +137,17 @@ int aionhip_step_gate_matmul(aionhip_ctx *ctx, const aionhip_weight *w, size_t r
     if (rc) return rc;
     if (!gate || !up || ((gate | up) & 3)) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "gate_matmul: null or misaligned gate/up");
     const float *gp = (const float *)(uintptr_t)gate, *up_p = (const float *)(uintptr_t)up;
-    if (rows == 1 && b.k <= FUSED_MAX_K && ((gate | up) & 15) == 0)
+    if (rows == 1 && b.k <= FUSED_PAYS_K && ((gate | up) & 15) == 0)
         return launch_gemv_fused(ctx, b.w, b.c, b.ldc, 1, PRO_GATE, FusedIn{gp, up_p, nullptr, nullptr, 0.f}, alpha, beta);
+    if (rows <= GEMV_MAX_M) {
+        // gate and activation preparation in one small launch, then the GEMV on the prepared rows
+        rc = ensure_scratch(ctx, prepared_act_bytes(rows, b.k));
+        if (rc) return rc;
+        PreparedAct act = prepared_act_carve(ctx->scratch, rows, b.k);
+        rc = launch_prepare_gate(ctx, gp, up_p, rows, b.k, act);
+        if (rc) return rc;
+        return launch_gemv_batch(ctx, b.w, b.c, b.ldc, 1, (int)rows, act, alpha, beta);
+    }
     const size_t act_bytes = (prepared_act_bytes(rows, b.k) + 255) & ~(size_t)255;
     rc = ensure_scratch(ctx, act_bytes + rows * b.k * sizeof(float));
     if (rc) return rc;

@@ -111,7 +111,9 @@ __global__ void quantize_rank2_kernel(const float *__restrict__ src, uint8_t *__
 }
 
 // Activation preparation (aion matmul_q_i8.zig:187-203): 8 lanes share one 32-element block.
-__global__ __launch_bounds__(256) void prepare_act_kernel(const float *__restrict__ a, size_t lda, size_t m, size_t k,
+// GATE: the activation is gelu_tanh(a) * up (aion cpu/exec/elementwise.zig:25-37), not written out.
+template <bool GATE>
+__global__ __launch_bounds__(256) void prepare_act_kernel(const float *__restrict__ a, const float *__restrict__ up, size_t lda, size_t m, size_t k,
                                                           int *__restrict__ aq, float *__restrict__ a_scale, int *__restrict__ a_sum) {
     const size_t kb_per_row = k / QK;
     const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -122,6 +124,13 @@ __global__ __launch_bounds__(256) void prepare_act_kernel(const float *__restric
     const float *p = a + row * lda + kb * QK + sub * 4;
     float v0 = 0.f, v1 = 0.f, v2 = 0.f, v3 = 0.f;
     if (live) { v0 = p[0]; v1 = p[1]; v2 = p[2]; v3 = p[3]; }
+    if (GATE && live) {
+        const float *u = up + row * lda + kb * QK + sub * 4;
+        v0 = aion_gate_gelu(v0, u[0]);
+        v1 = aion_gate_gelu(v1, u[1]);
+        v2 = aion_gate_gelu(v2, u[2]);
+        v3 = aion_gate_gelu(v3, u[3]);
+    }
     float amax = fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3)));
     amax = fmaxf(amax, dpp_f<DPP_QUAD_XOR1>(amax));
     amax = fmaxf(amax, dpp_f<DPP_QUAD_XOR2>(amax));
@@ -170,8 +179,16 @@ int launch_prepare_act(aionhip_ctx *ctx, const float *a, size_t lda, size_t m, s
     const size_t threads = m * (k / QK) * 8;
     if (!threads) return AIONHIP_OK;
     const size_t blocks = (threads + 255) / 256;
-    prepare_act_kernel<<<dim3((unsigned)blocks), dim3(256), 0, ctx->stream>>>(a, lda, m, k, (int *)out.q, out.scale, out.sum);
+    prepare_act_kernel<false><<<dim3((unsigned)blocks), dim3(256), 0, ctx->stream>>>(a, nullptr, lda, m, k, (int *)out.q, out.scale, out.sum);
     LAUNCH_CHECK(ctx, "prepare_act");
+    return AIONHIP_OK;
+}
+int launch_prepare_gate(aionhip_ctx *ctx, const float *gate, const float *up, size_t m, size_t k, PreparedAct out) {
+    const size_t threads = m * (k / QK) * 8;
+    if (!threads) return AIONHIP_OK;
+    const size_t blocks = (threads + 255) / 256;
+    prepare_act_kernel<true><<<dim3((unsigned)blocks), dim3(256), 0, ctx->stream>>>(gate, up, k, m, k, (int *)out.q, out.scale, out.sum);
+    LAUNCH_CHECK(ctx, "prepare_gate");
     return AIONHIP_OK;
 }
 

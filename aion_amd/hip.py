@@ -63,6 +63,7 @@ _SIGS = {
     "aionhip_program_execute": (C.c_int, [C.c_void_p, C.c_void_p]),
     "aionhip_program_node_count": (C.c_size_t, [C.c_void_p]),
     "aionhip_program_destroy": (None, [C.c_void_p, C.c_void_p]),
+    "aionhip_set_attention_precise": (C.c_int, [C.c_void_p, C.c_int]),
     "aionhip_set_gemm_mode": (C.c_int, [C.c_void_p, C.c_int]),
     "aionhip_step_attention": (C.c_int, [C.c_void_p, C.POINTER(Attention)]),
     "aionhip_step_rmsnorm": (C.c_int, [C.c_void_p] + [C.c_uint64] * 5 + [C.c_size_t, C.c_size_t, C.c_float]),

@@ -107,7 +107,7 @@ def main():
     ms_per_step = total_ms / args.steps
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
-    gemv = [ms for (name, ms) in prof if name == "gemv_q4"]
+    gemv = [ms for (name, ms) in prof if name.startswith("gemv_q4")]
     assert len(gemv) == args.steps * len(SHAPES), (len(gemv), args.steps)
     avg_launch_ms = sum(gemv) / len(gemv)
     bytes_per_launch = step_bytes / len(SHAPES)
@@ -128,7 +128,7 @@ def main():
                    "step_algorithmic_bytes": step_bytes, "wall_ms_per_step": round(wall_ms / args.steps, 5)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "gemv_q4", "avg_launch_us": round(avg_launch_ms * 1e3, 3),
+                     "kernel": "gemv_q4 (gemv_fused_kernel for K <= 8192, prepare_act + gemv_kernel above)", "avg_launch_us": round(avg_launch_ms * 1e3, 3),
                      "algorithmic_bytes_per_launch": bytes_per_launch, "per_shape": per_shape},
     }
 
@@ -163,7 +163,7 @@ def time_kernel(gpu, ws, x, y, m, name, iters=20):
     gpu.profile_start()
     for i in range(iters):
         gpu.step_matmul(ws[i % len(ws)], x, m, y)
-    prof = [ms for (nm, ms) in gpu.profile_stop() if nm == name]
+    prof = [ms for (nm, ms) in gpu.profile_stop() if nm.startswith(name)]
     return sum(prof) / len(prof)
 
 

@@ -171,6 +171,10 @@ typedef struct aionhip_attention {
     uint32_t window_left, window_right, window_chunk;
 } aionhip_attention;
 int aionhip_step_attention(aionhip_ctx *ctx, const aionhip_attention *p);
+/* f32 queries over an f16/bf16 cache: off (default) = q rounded to the cache element type, one MFMA
+ * pass (2e-3 tolerance class); on = q and the probabilities fed as hi+lo parts (agrees with an f64
+ * reference to ~1e-6, about 1.4x the kernel time at decode). */
+int aionhip_set_attention_precise(aionhip_ctx *ctx, int on);
 
 /* ---- per-token glue steps (f32 unless stated) ---------------------------------------------- */
 /* StepRMSNorm (runtime/executable.zig:85-101; cpu/exec/layernorm.zig:54-155):

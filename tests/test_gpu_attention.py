@@ -190,3 +190,18 @@ def test_attention_argument_errors(gpu):
         gpu.step_attention(a, a, a, a, (1, 1, 4, 2, 2, 64, 64), 1.0, kv_dtype=be.I32)
     assert e.value.status == hip.UNSUPPORTED
     a.free()
+
+
+def test_precise_mode_brings_f32_queries_to_f32_accuracy(gpu, orc):
+    (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(23, 2, 1, 900, 8, 1, 256, "f16")
+    pos = np.full((2, 1), 899, np.int32)
+    ref = orc.attention_f64(qf, kf, vf, 1 / 16.0, positions=pos)
+    fast = run_attention(gpu, q, k, v, 1 / 16.0, qd, kd, positions=pos)
+    gpu.set_attention_precise(True)
+    try:
+        precise = run_attention(gpu, q, k, v, 1 / 16.0, qd, kd, positions=pos)
+    finally:
+        gpu.set_attention_precise(False)
+    e_fast, e_prec = float(np.abs(fast - ref).max()), float(np.abs(precise - ref).max())
+    say("  fast", e_fast, "precise", e_prec)
+    assert e_fast < 2e-3 and e_prec < 1e-5

@@ -217,7 +217,7 @@ def test_matmul_argument_errors(gpu, orc):
 def test_single_row_fused_kernel_equals_prepared_path(gpu, orc, dtype, layout):
     # m == 1 builds the int8 activation inside the GEMV; a 2-row call goes through prepare_act + gemv.
     # Same codes, same scales, same per-lane order: the shared row must agree bit for bit.
-    for n, k in [(67, 2080), (2048, 2048), (300, 8192)]:
+    for n, k in [(67, 2080), (2048, 2048), (300, 4096)]:
         blocks, w = make_weight(gpu, orc, dtype, layout, n, k, seed=n + k)
         a = np.random.default_rng(n).standard_normal((2, k)).astype(np.float32)
         one = gpu.matmul(w, a[:1])
@@ -261,6 +261,14 @@ def test_rmsnorm_matmul_and_gate_matmul_match_the_separate_steps(gpu, orc, dtype
     act = orc.gate_gelu(gate, up).reshape(rows, k)
     want = oracle_matmul(orc, dtype, layout, act, b1, n1, beta=1.0, c=res0)
     assert rms_err(gpu.download(cres, np.float32, (rows, n1)), want) < 3e-3
-    for t in (xb, gb, c1, c2, gtb, upb, cres):
+    # a long reduction axis (K = 8192) takes the gate + preparation launch, then the GEMV
+    b3, w3 = make_weight(gpu, orc, dtype, layout, 160, 8192, seed=3)
+    gate8 = (rng.standard_normal((rows, 8192)) * 2).astype(np.float32)
+    up8 = rng.standard_normal((rows, 8192)).astype(np.float32)
+    g8, u8, c8 = gpu.upload(gate8), gpu.upload(up8), gpu.alloc(rows * 160 * 4)
+    gpu.step_gate_matmul(w3, g8, u8, rows, c8)
+    want8 = oracle_matmul(orc, dtype, layout, orc.gate_gelu(gate8, up8).reshape(rows, 8192), b3, 160)
+    assert rms_err(gpu.download(c8, np.float32, (rows, 160)), want8) < 3e-3
+    for t in (xb, gb, c1, c2, gtb, upb, cres, g8, u8, c8):
         t.free()
-    w1.free(); w2.free()
+    w1.free(); w2.free(); w3.free()
