@@ -126,7 +126,7 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
     constexpr int KK = D / 32;   // MFMA k-steps over the head dim
     constexpr int MT = D / 16;   // 16-wide dv tiles
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n = lane & 15, g = lane >> 4;
     const int unit = blockIdx.y;
     const int b = unit / a.Hkv, hk = unit % a.Hkv;
@@ -516,10 +516,14 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
             HIP_TRY(ctx, hipFuncSetAttribute((const void *)attn_flash_kernel<KV, D, true, HILO>, hipFuncAttributeMaxDynamicSharedMemorySize, SplitCfg::LDS_BYTES));
             attr_split = true;
         }
-        prof_begin(ctx, "attn_flash_split");
-        attn_flash_kernel<KV, D, true, HILO><<<dim3((unsigned)(a.row_tiles * nseg), (unsigned)units), dim3(SPLIT_NW * 64), SplitCfg::LDS_BYTES, ctx->stream>>>(a);
-        if (nseg > 1) attn_merge_kernel<D><<<dim3((unsigned)(a.row_tiles * (D / 64)), (unsigned)units), dim3(256), 0, ctx->stream>>>(a);
-        prof_end(ctx);
+        {
+            ProfScope scope(ctx, "attn_flash_split");
+            launch_k(ctx, attn_flash_kernel<KV, D, true, HILO>, dim3((unsigned)(a.row_tiles * nseg), (unsigned)units), dim3(SPLIT_NW * 64), SplitCfg::LDS_BYTES, a);
+        }
+        if (nseg > 1) {
+            ProfScope scope(ctx, "attn_merge");
+            launch_k(ctx, attn_merge_kernel<D>, dim3((unsigned)(a.row_tiles * (D / 64)), (unsigned)units), dim3(256), 0, a);
+        }
         LAUNCH_CHECK(ctx, "attn_flash_split");
     } else {
         a.nseg = 1;
@@ -528,9 +532,8 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
             HIP_TRY(ctx, hipFuncSetAttribute((const void *)attn_flash_kernel<KV, D, false, HILO>, hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES));
             attr_prefill = true;
         }
-        prof_begin(ctx, "attn_flash_prefill");
-        attn_flash_kernel<KV, D, false, HILO><<<dim3((unsigned)((a.row_tiles + 3) / 4), (unsigned)units), dim3(256), Cfg::LDS_BYTES, ctx->stream>>>(a);
-        prof_end(ctx);
+        ProfScope scope(ctx, "attn_flash_prefill");
+        launch_k(ctx, attn_flash_kernel<KV, D, false, HILO>, dim3((unsigned)((a.row_tiles + 3) / 4), (unsigned)units), dim3(256), Cfg::LDS_BYTES, a);
         LAUNCH_CHECK(ctx, "attn_flash_prefill");
     }
     return AIONHIP_OK;
@@ -591,9 +594,8 @@ extern "C" int aionhip_step_attention(aionhip_ctx *ctx, const aionhip_attention 
     const size_t rows = p->batch * p->l_q * p->h_q;
     int rc = ensure_scratch2(ctx, rows * p->t_kv * sizeof(float));
     if (rc) return rc;
-    prof_begin(ctx, "attn_generic");
-    attn_generic_kernel<<<dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, ctx->stream>>>(a, (int)p->d_k, (int)p->d_v, (float *)ctx->scratch2);
-    prof_end(ctx);
+    ProfScope scope(ctx, "attn_generic");
+    launch_k(ctx, attn_generic_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, a, (int)p->d_k, (int)p->d_v, (float *)ctx->scratch2);
     LAUNCH_CHECK(ctx, "attn_generic");
     return AIONHIP_OK;
 }

@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
+#include <hip/hip_ext.h>
 
 #include <cstdarg>
 #include <cstdint>
@@ -54,13 +55,34 @@ struct aionhip_ctx {
     bool capturing = false;
     // per-launch timing, off by default
     bool profiling = false;
+    const char *prof_name = nullptr;   // set by ProfScope: launches made through launch_k are timed under it
     std::vector<ProfRecord> prof;
     std::vector<hipEvent_t> event_pool;
 };
 
-// Brackets one kernel launch with stream events while profiling is on.
-void prof_begin(aionhip_ctx *ctx, const char *name);
-void prof_end(aionhip_ctx *ctx);
+// Names the launches made through launch_k while it is alive (and profiling is on).
+struct ProfScope {
+    aionhip_ctx *ctx;
+    const char *prev;
+    ProfScope(aionhip_ctx *c, const char *name) : ctx(c), prev(c->prof_name) { c->prof_name = name; }
+    ~ProfScope() { ctx->prof_name = prev; }
+};
+// A new profile record under the scope's name; its two events go to the launch.
+void prof_open(aionhip_ctx *ctx, hipEvent_t *start, hipEvent_t *stop);
+
+// Kernel launch on the context's stream. While profiling inside a ProfScope the launch carries its
+// own start/stop events (hipExtLaunchKernelGGL: the timestamps of the dispatch itself, so the
+// elapsed time is the kernel's duration with no barrier or launch gap in it).
+template <typename... KArgs, typename... Args>
+inline void launch_k(aionhip_ctx *ctx, void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t lds, Args... args) {
+    if (ctx->profiling && ctx->prof_name) {
+        hipEvent_t e0 = nullptr, e1 = nullptr;
+        prof_open(ctx, &e0, &e1);
+        hipExtLaunchKernelGGL(kernel, grid, block, (uint32_t)lds, ctx->stream, e0, e1, 0u, static_cast<KArgs>(args)...);
+    } else {
+        kernel<<<grid, block, lds, ctx->stream>>>(static_cast<KArgs>(args)...);
+    }
+}
 
 // Device-private weight layout: row n of the [N,K] operand is one contiguous run.
 //   q8_0: qs[n][K] int8,               sc[n][K/32] f16

@@ -2,6 +2,7 @@
 // Backend / Session / DeviceMemory vtables (backend/backend.zig:24-107,
 // runtime/device_memory.zig:36-108).
 #include "common.h"
+#include <algorithm>
 
 #include <cstring>
 #include <new>
@@ -48,15 +49,11 @@ static hipEvent_t take_event(aionhip_ctx *ctx) {
     (void)hipEventCreate(&e);
     return e;
 }
-void prof_begin(aionhip_ctx *ctx, const char *name) {
-    if (!ctx->profiling) return;
-    ProfRecord r{name, take_event(ctx), take_event(ctx), 0.f};
-    (void)hipEventRecord(r.start, ctx->stream);
+void prof_open(aionhip_ctx *ctx, hipEvent_t *start, hipEvent_t *stop) {
+    ProfRecord r{ctx->prof_name, take_event(ctx), take_event(ctx), 0.f};
     ctx->prof.push_back(r);
-}
-void prof_end(aionhip_ctx *ctx) {
-    if (!ctx->profiling || ctx->prof.empty()) return;
-    (void)hipEventRecord(ctx->prof.back().stop, ctx->stream);
+    *start = r.start;
+    *stop = r.stop;
 }
 
 int rope_table(aionhip_ctx *ctx, int pairs, float freq_step, float scale_factor, const float **out) {

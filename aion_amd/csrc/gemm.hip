@@ -27,7 +27,7 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(const uint8_t *__restrict_
                                                       int M, int N, int K, size_t ldc, float alpha, float beta) {
     constexpr int TN = 4;
     constexpr bool Q8 = DT == AIONHIP_Q8_0;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r = lane & 15, g = lane >> 4;
     const int n0 = (blockIdx.x * 4 + wave) * (TN * 16);
     const int m0 = blockIdx.y * (TM * 16);
@@ -159,7 +159,7 @@ constexpr int A_TILE = BM * LDS_ROW, B_TILE = BN * LDS_ROW;
 __global__ __launch_bounds__(256) void gemm_bf16_kernel(const unsigned short *__restrict__ A, const unsigned short *__restrict__ W,
                                                         float *__restrict__ c, int M, int N, int K, size_t ldc, float alpha, float beta) {
     __shared__ __attribute__((aligned(16))) unsigned char lds[2 * (A_TILE + B_TILE)];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, g = lane >> 4;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 64;   // 2 x 2 wavefronts, each 128 x 64
@@ -252,11 +252,11 @@ void launch_i8(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct 
     const int M = (int)m, N = (int)w->n, K = (int)w->k;
     const unsigned gx = (unsigned)((N + 255) / 256);
     if (M > 32) {
-        gemm_i8_kernel<DT, 4><<<dim3(gx, (unsigned)((M + 63) / 64)), dim3(256), 0, ctx->stream>>>(w->qs, w->sc, act.q, act.scale, act.sum, c, M, N, K, ldc, alpha, beta);
+        launch_k(ctx, gemm_i8_kernel<DT, 4>, dim3(gx, (unsigned)((M + 63) / 64)), dim3(256), 0, w->qs, w->sc, act.q, act.scale, act.sum, c, M, N, K, ldc, alpha, beta);
     } else if (M > 16) {
-        gemm_i8_kernel<DT, 2><<<dim3(gx, (unsigned)((M + 31) / 32)), dim3(256), 0, ctx->stream>>>(w->qs, w->sc, act.q, act.scale, act.sum, c, M, N, K, ldc, alpha, beta);
+        launch_k(ctx, gemm_i8_kernel<DT, 2>, dim3(gx, (unsigned)((M + 31) / 32)), dim3(256), 0, w->qs, w->sc, act.q, act.scale, act.sum, c, M, N, K, ldc, alpha, beta);
     } else {
-        gemm_i8_kernel<DT, 1><<<dim3(gx, (unsigned)((M + 15) / 16)), dim3(256), 0, ctx->stream>>>(w->qs, w->sc, act.q, act.scale, act.sum, c, M, N, K, ldc, alpha, beta);
+        launch_k(ctx, gemm_i8_kernel<DT, 1>, dim3(gx, (unsigned)((M + 15) / 16)), dim3(256), 0, w->qs, w->sc, act.q, act.scale, act.sum, c, M, N, K, ldc, alpha, beta);
     }
 }
 
@@ -264,10 +264,9 @@ void launch_i8(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct 
 
 int launch_gemm_i8(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
     const char *name = w->dtype == AIONHIP_Q8_0 ? "gemm_i8_q8" : "gemm_i8_q4";
-    prof_begin(ctx, name);
+    ProfScope scope(ctx, name);
     if (w->dtype == AIONHIP_Q8_0) launch_i8<AIONHIP_Q8_0>(ctx, w, m, act, c, ldc, alpha, beta);
     else launch_i8<AIONHIP_Q4_0>(ctx, w, m, act, c, ldc, alpha, beta);
-    prof_end(ctx);
     LAUNCH_CHECK(ctx, name);
     return AIONHIP_OK;
 }
@@ -291,13 +290,13 @@ int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *cw, size_t m, const
     unsigned short *abf = (unsigned short *)ctx->scratch2;
     {
         const size_t threads = m * (K / 8);
-        act_bf16_kernel<<<dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, ctx->stream>>>(a, lda, abf, m, K);
+        ProfScope scope(ctx, "act_bf16");
+        launch_k(ctx, act_bf16_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, a, lda, abf, m, K);
         LAUNCH_CHECK(ctx, "act_bf16");
     }
     const dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((m + BM - 1) / BM));
-    prof_begin(ctx, "gemm_bf16");
-    gemm_bf16_kernel<<<grid, dim3(256), 0, ctx->stream>>>(abf, w->bf16, c, (int)m, (int)N, (int)K, ldc, alpha, beta);
-    prof_end(ctx);
+    ProfScope scope(ctx, "gemm_bf16");
+    launch_k(ctx, gemm_bf16_kernel, grid, dim3(256), 0, abf, w->bf16, c, (int)m, (int)N, (int)K, ldc, alpha, beta);
     LAUNCH_CHECK(ctx, "gemm_bf16");
     return AIONHIP_OK;
 }

@@ -18,7 +18,7 @@ template <int DT, int B, int R>
 __global__ __launch_bounds__(256) void gemv_kernel(GemvBatch batch, const u32x4 *__restrict__ aq, const float *__restrict__ a_scale,
                                                    const int *__restrict__ a_sum, int K, int m, float alpha, float beta) {
     const int lane = threadIdx.x & 63;
-    const int gwave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int gwave = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: keep it scalar
     if (gwave >= batch.total_waves) return;
     int si = 0;
 #pragma unroll
@@ -136,9 +136,9 @@ void launch_r(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *c
     batch.total_waves = waves;
     const auto *aq = (const u32x4 *)act.q;
     const dim3 grid((unsigned)((waves + 3) / 4)), block(256);
-    if (R == 4) gemv_kernel<DT, B, 4><<<grid, block, 0, ctx->stream>>>(batch, aq, act.scale, act.sum, K, m, alpha, beta);
-    else if (R == 2) gemv_kernel<DT, B, 2><<<grid, block, 0, ctx->stream>>>(batch, aq, act.scale, act.sum, K, m, alpha, beta);
-    else gemv_kernel<DT, B, 1><<<grid, block, 0, ctx->stream>>>(batch, aq, act.scale, act.sum, K, m, alpha, beta);
+    if (R == 4) launch_k(ctx, gemv_kernel<DT, B, 4>, grid, block, 0, batch, aq, act.scale, act.sum, K, m, alpha, beta);
+    else if (R == 2) launch_k(ctx, gemv_kernel<DT, B, 2>, grid, block, 0, batch, aq, act.scale, act.sum, K, m, alpha, beta);
+    else launch_k(ctx, gemv_kernel<DT, B, 1>, grid, block, 0, batch, aq, act.scale, act.sum, K, m, alpha, beta);
 }
 
 template <int DT>
@@ -157,10 +157,9 @@ int launch_gemv_batch(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *
     if (m < 1 || m > 8) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "gemv: m=%d outside 1..8", m);
     if (count < 1 || count > 4) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "gemv: %d weights in one launch (1..4)", count);
     const char *name = ws[0]->dtype == AIONHIP_Q8_0 ? "gemv_q8" : "gemv_q4";
-    prof_begin(ctx, name);
+    ProfScope scope(ctx, name);
     if (ws[0]->dtype == AIONHIP_Q8_0) launch_b<AIONHIP_Q8_0>(ctx, ws, cs, ldcs, count, m, act, alpha, beta);
     else launch_b<AIONHIP_Q4_0>(ctx, ws, cs, ldcs, count, m, act, alpha, beta);
-    prof_end(ctx);
     LAUNCH_CHECK(ctx, name);
     return AIONHIP_OK;
 }

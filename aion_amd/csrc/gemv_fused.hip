@@ -29,7 +29,9 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedI
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave_stride = gridDim.x * 4;
-    int gwave = blockIdx.x * 4 + (tid >> 6);
+    // the wavefront index is uniform: read through a scalar, the row-group bookkeeping and the
+    // base addresses then stay in scalar registers
+    int gwave = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(tid >> 6);
     const int KB = K >> 5;
     constexpr bool Q8 = DT == AIONHIP_Q8_0;
     const int chunks = Q8 ? (K >> 4) : KB;
@@ -266,12 +268,11 @@ void launch_r(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *c
     batch.total_waves = waves;
     // at most 8 workgroups per CU: beyond that the wavefronts stride over the row groups
     const int wgs = (waves + 3) / 4;
-    static const int cap_mult = getenv("AIONHIP_FUSED_CAP") ? atoi(getenv("AIONHIP_FUSED_CAP")) : 8;
-    const dim3 grid((unsigned)(wgs < cus * cap_mult ? wgs : cus * cap_mult)), block(256);
+    const dim3 grid((unsigned)(wgs < cus * 8 ? wgs : cus * 8)), block(256);
     const size_t lds = (size_t)K + (size_t)(K >> 5) * 8 + 16;
-    if (R == 4) gemv_fused_kernel<DT, 4, PRO, NCH><<<grid, block, lds, ctx->stream>>>(batch, in, K, alpha, beta);
-    else if (R == 2) gemv_fused_kernel<DT, 2, PRO, NCH><<<grid, block, lds, ctx->stream>>>(batch, in, K, alpha, beta);
-    else gemv_fused_kernel<DT, 1, PRO, NCH><<<grid, block, lds, ctx->stream>>>(batch, in, K, alpha, beta);
+    if (R == 4) launch_k(ctx, gemv_fused_kernel<DT, 4, PRO, NCH>, grid, block, lds, batch, in, K, alpha, beta);
+    else if (R == 2) launch_k(ctx, gemv_fused_kernel<DT, 2, PRO, NCH>, grid, block, lds, batch, in, K, alpha, beta);
+    else launch_k(ctx, gemv_fused_kernel<DT, 1, PRO, NCH>, grid, block, lds, batch, in, K, alpha, beta);
 }
 
 template <int DT, int PRO>
@@ -302,10 +303,9 @@ int launch_gemv_fused(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *
     static const char *names[2][3] = {{"gemv_q4_fused", "gemv_q4_rmsnorm", "gemv_q4_gate"}, {"gemv_q8_fused", "gemv_q8_rmsnorm", "gemv_q8_gate"}};
     const bool q8 = ws[0]->dtype == AIONHIP_Q8_0;
     const char *name = names[q8 ? 1 : 0][prologue];
-    prof_begin(ctx, name);
+    ProfScope scope(ctx, name);
     if (q8) launch_p<AIONHIP_Q8_0>(ctx, ws, cs, ldcs, count, prologue, in, alpha, beta);
     else launch_p<AIONHIP_Q4_0>(ctx, ws, cs, ldcs, count, prologue, in, alpha, beta);
-    prof_end(ctx);
     LAUNCH_CHECK(ctx, name);
     return AIONHIP_OK;
 }

@@ -179,7 +179,8 @@ int launch_prepare_act(aionhip_ctx *ctx, const float *a, size_t lda, size_t m, s
     const size_t threads = m * (k / QK) * 8;
     if (!threads) return AIONHIP_OK;
     const size_t blocks = (threads + 255) / 256;
-    prepare_act_kernel<false><<<dim3((unsigned)blocks), dim3(256), 0, ctx->stream>>>(a, nullptr, lda, m, k, (int *)out.q, out.scale, out.sum);
+    ProfScope scope(ctx, "prepare_act");
+    launch_k(ctx, prepare_act_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, a, nullptr, lda, m, k, (int *)out.q, out.scale, out.sum);
     LAUNCH_CHECK(ctx, "prepare_act");
     return AIONHIP_OK;
 }
@@ -187,7 +188,8 @@ int launch_prepare_gate(aionhip_ctx *ctx, const float *gate, const float *up, si
     const size_t threads = m * (k / QK) * 8;
     if (!threads) return AIONHIP_OK;
     const size_t blocks = (threads + 255) / 256;
-    prepare_act_kernel<true><<<dim3((unsigned)blocks), dim3(256), 0, ctx->stream>>>(gate, up, k, m, k, (int *)out.q, out.scale, out.sum);
+    ProfScope scope(ctx, "prepare_gate");
+    launch_k(ctx, prepare_act_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, gate, up, k, m, k, (int *)out.q, out.scale, out.sum);
     LAUNCH_CHECK(ctx, "prepare_gate");
     return AIONHIP_OK;
 }

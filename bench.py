@@ -32,6 +32,7 @@ sys.path.insert(0, ROOT)
 
 SHAPES = [(4096, 4096), (14336, 4096), (4096, 14336), (262144, 2048)]   # N x K
 HBM_PEAK_GBPS = 8000.0
+CAL_ELEMS = 1 << 26   # the counter-calibration cast: 256 MiB read, 128 MiB written
 
 
 def algorithmic_bytes(dtype_bytes, n, k, batch):
@@ -91,8 +92,8 @@ def main():
     for i in range(args.warmup):
         step(i)
     gpu.sync()
+    # pass 1: exactly K steps between two stream events -> value
     ev0, ev1 = gpu.event(), gpu.event()
-    gpu.profile_start()
     gpu.record(ev0)
     t_wall = time.perf_counter()
     for i in range(args.steps):
@@ -101,12 +102,27 @@ def main():
     gpu.sync()
     wall_ms = (time.perf_counter() - t_wall) * 1e3
     total_ms = gpu.elapsed_ms(ev0, ev1)
+    # pass 2: the same K steps again, every dispatch carrying its own start/stop events -> roofline
+    # (kept apart from pass 1 because timed dispatches cannot be queued back to back)
+    gpu.profile_start()
+    for i in range(args.steps):
+        step(args.warmup + i)
     prof = gpu.profile_stop()
+    # counter calibration: a plain streaming kernel of known size (f32 -> f16 cast: 4 B read and
+    # 2 B written per element) so that a FETCH_SIZE / WRITE_SIZE counter run of this same command
+    # holds its own scale factor
+    cal_n = CAL_ELEMS
+    cal_src, cal_dst = gpu.alloc(cal_n * 4), gpu.alloc(cal_n * 2)
+    for _ in range(3):
+        gpu.step_cast_f32_f16(cal_dst, cal_src, cal_n)
+    gpu.sync()
+    cal_src.free(); cal_dst.free()
 
     step_bytes = sum(algorithmic_bytes(18, n, k, batch) for (n, k) in SHAPES)
     ms_per_step = total_ms / args.steps
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
+    # every profile entry is one dispatch's own start/stop timestamps (what a kernel trace reports)
     gemv = [ms for (name, ms) in prof if name.startswith("gemv_q4")]
     assert len(gemv) == args.steps * len(SHAPES), (len(gemv), args.steps)
     avg_launch_ms = sum(gemv) / len(gemv)
@@ -245,15 +261,15 @@ def run_attention(gpu, be):
         for _ in range(iters):
             gpu.step_attention(bufs[3], bufs[0], bufs[1], bufs[2], shape, 1 / 16.0, q_dtype=be.BF16, kv_dtype=be.BF16,
                                query_positions=pos, kv_lengths=kl)
-        prof = [ms for (nm, ms) in gpu.profile_stop() if nm == name]
-        return sum(prof) / len(prof)
+        prof = [ms for (nm, ms) in gpu.profile_stop() if nm in name]
+        return sum(prof) / iters
 
     for L in (1024, 4096):
         q = gpu.upload(_bf16_bits(rng.standard_normal((1, L, Hq, D))))
         k = gpu.upload(_bf16_bits(rng.standard_normal((1, L, Hkv, D))))
         v = gpu.upload(_bf16_bits(rng.standard_normal((1, L, Hkv, D))))
         o = gpu.alloc(L * Hq * D * 4)
-        ms = timed("attn_flash_prefill", (1, L, L, Hq, Hkv, D, D), (q, k, v, o))
+        ms = timed(("attn_flash_prefill",), (1, L, L, Hq, Hkv, D, D), (q, k, v, o))
         flops = 4.0 * Hq * D * L * (L + 1) / 2
         tf = flops / (ms * 1e-3) / 1e12
         res["prefill L%d" % L] = {"kernel_ms": round(ms, 4), "TFLOPs": round(tf, 1), "frac_mfma_peak": round(tf / MFMA_PEAK["bf16"], 4)}
@@ -267,7 +283,7 @@ def run_attention(gpu, be):
             o = gpu.alloc(B * Hq * D * 4)
             pos = gpu.upload(np.full((B, 1), T - 1, np.int32))
             kl = gpu.upload(np.full((B,), T, np.int32))
-            ms = timed("attn_flash_split", (B, 1, T, Hq, Hkv, D, D), (q, k, v, o), pos, kl, iters=20)
+            ms = timed(("attn_flash_split", "attn_merge"), (B, 1, T, Hq, Hkv, D, D), (q, k, v, o), pos, kl, iters=20)
             by = B * 2 * T * Hkv * D * 2 + B * Hq * D * (2 + 4)
             res["decode T%d B%d" % (T, B)] = {"kernel_us": round(ms * 1e3, 2), "GBps": round(by / (ms * 1e-3) / 1e9, 1),
                                               "frac_hbm_peak": round(by / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}

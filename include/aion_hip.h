@@ -234,7 +234,8 @@ void aionhip_event_destroy(aionhip_ctx *ctx, void *event);
 
 /* Per-launch GPU timing of the matmul / attention kernels (AION_PROFILE_GPU=dispatch in the
  * WebGPU backend, backend/gpu/timestamp_profile.zig:1-60): between start and stop every such
- * launch is bracketed by two stream events; stop waits for the stream and resolves them. */
+ * launch carries its own start and stop event (the dispatch's timestamps, as a kernel trace
+ * reports them); stop waits for the stream and resolves them. */
 int aionhip_profile_start(aionhip_ctx *ctx);
 int aionhip_profile_stop(aionhip_ctx *ctx, size_t *count);
 int aionhip_profile_entry(aionhip_ctx *ctx, size_t index, const char **name, float *ms);
