@@ -33,6 +33,11 @@ sys.path.insert(0, ROOT)
 SHAPES = [(4096, 4096), (14336, 4096), (4096, 14336), (262144, 2048)]   # N x K
 HBM_PEAK_GBPS = 8000.0
 CAL_ELEMS = 1 << 26   # the counter-calibration cast: 256 MiB read, 128 MiB written
+# HBM bytes per launch (read + written) of the GEMV kernel of each shape, from FETCH_SIZE / WRITE_SIZE
+# counter runs of this same command scaled by what the same counters read for the calibration cast
+# (factors 1.9998 and 1.0000); the summary with the commands is profiles/gemv_q4_decode_bench_kernel_stats_and_traffic.md.
+# Counters cannot be read from inside the process, so the figures are carried here.
+MEASURED_TRAFFIC = {(4096, 4096): 9.682e6, (14336, 4096): 33.332e6, (4096, 14336): 33.243e6, (262144, 2048): 303.171e6}
 
 
 def algorithmic_bytes(dtype_bytes, n, k, batch):
@@ -143,8 +148,10 @@ def main():
                    "device": info["arch"], "cu_count": info["cu_count"], "weight_sets_rotated": n_sets,
                    "step_algorithmic_bytes": step_bytes, "wall_ms_per_step": round(wall_ms / args.steps, 5)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "gemv_q4 (gemv_fused_kernel for K <= 8192, prepare_act + gemv_kernel above)", "avg_launch_us": round(avg_launch_ms * 1e3, 3),
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": round(sum(MEASURED_TRAFFIC[sh] for sh in SHAPES) / len(SHAPES)),
+                     "kernel": "gemv_q4 (gemv_fused_kernel for K <= 4096, gemv_kernel after prepare_act above)",
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, profiles/gemv_q4_decode_bench_kernel_stats_and_traffic.md", "avg_launch_us": round(avg_launch_ms * 1e3, 3),
                      "algorithmic_bytes_per_launch": bytes_per_launch, "per_shape": per_shape},
     }
 
