@@ -152,6 +152,157 @@ __global__ void act_bf16_kernel(const float *__restrict__ a, size_t lda, unsigne
     *(u32x4 *)(out + m * K + k0) = o;
 }
 
+// ---- wide-tile kernel: workgroup tile (WM*64) x 256, K step 64, v_mfma_f32_32x32x16_bf16.
+// 2 x 2 wavefronts, each (WM*32) x 128 outputs = WM x 4 tiles of 32x32 (accumulators: WM*64
+// registers). Operands go global -> registers -> LDS (row stride 144 B: 16 consecutive rows land
+// in 16 distinct 16-byte bank groups) -> 16-byte fragment reads; the next K step's global loads
+// are in flight during the MFMAs of the current one, one barrier per K step.
+// Tile order: workgroup ids go round-robin over the 8 XCDs, so id -> (xcd, slot) -> a contiguous
+// run of tiles per XCD, M fastest: the workgroups that share a weight column tile run on one L2.
+constexpr int G2_BK = 64, G2_STRIDE = 144, G2_BN = 256;
+using f32x16 = __attribute__((ext_vector_type(16))) float;
+
+template <int WM>
+__global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const unsigned short *__restrict__ A, const unsigned short *__restrict__ W,
+                                                             float *__restrict__ c, int M, int N, int K, size_t ldc, float alpha,
+                                                             float beta, int tiles_m, int tiles) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds2[];
+    constexpr int BM2 = WM * 64;
+    constexpr int A_BYTES = BM2 * G2_STRIDE, B_BYTES = G2_BN * G2_STRIDE, STAGE = A_BYTES + B_BYTES;
+    constexpr int NA = WM * 2, NB = 8;                       // 16-byte chunks per thread per stage
+    const int per_xcd = (int)gridDim.x >> 3;
+    const int t = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
+    if (t >= tiles) return;
+    const int m0 = (t % tiles_m) * BM2, n0 = (t / tiles_m) * G2_BN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l31 = lane & 31, lh = lane >> 5;
+    const int wrow = (wave >> 1) * (WM * 32), wcol = (wave & 1) * 128;
+
+    f32x16 acc[WM][4];
+#pragma unroll
+    for (int mi = 0; mi < WM; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[mi][ni][i] = 0.f;
+
+    const unsigned short *ga[NA], *gb[NB];
+    int la[NA], lb[NB];
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+        const int ch = tid + 256 * i, row = ch >> 3, part = ch & 7;
+        ga[i] = A + (size_t)min(m0 + row, M - 1) * K + part * 8;
+        la[i] = row * G2_STRIDE + part * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+        const int ch = tid + 256 * i, row = ch >> 3, part = ch & 7;
+        gb[i] = W + (size_t)min(n0 + row, N - 1) * K + part * 8;
+        lb[i] = A_BYTES + row * G2_STRIDE + part * 16;
+    }
+    const int fa = (wrow + l31) * G2_STRIDE + lh * 16;              // + mi * 32 rows + ks * 32 bytes
+    const int fb = A_BYTES + (wcol + l31) * G2_STRIDE + lh * 16;
+
+    const int KT = K / G2_BK;
+    u32x4 ra[NA], rb[NB];
+#pragma unroll
+    for (int i = 0; i < NA; ++i) ra[i] = *(const u32x4 *)(ga[i]);
+#pragma unroll
+    for (int i = 0; i < NB; ++i) rb[i] = *(const u32x4 *)(gb[i]);
+#pragma unroll
+    for (int i = 0; i < NA; ++i) *(u32x4 *)(lds2 + la[i]) = ra[i];
+#pragma unroll
+    for (int i = 0; i < NB; ++i) *(u32x4 *)(lds2 + lb[i]) = rb[i];
+    __syncthreads();
+
+    // Software pipeline, one basic block per K step so that the instruction groups can be pinned:
+    //   sub-step 0: global loads of the next K step + MFMAs(0) while the fragments of sub-step 1 are read
+    //   sub-step 1: MFMAs(1) while fragments 2 are read;  sub-step 2: MFMAs(2) while fragments 3 are read
+    //   staged registers -> the other LDS buffer, barrier
+    //   sub-step 3: MFMAs(3) while fragments 0 of the next K step are read from the other buffer
+    // The last K step repeats its own loads into the idle buffer instead of branching.
+    struct Frag {
+        u32x4 a[WM], b[4];
+    };
+    auto read_frag = [&](Frag &f, const unsigned char *st, int ks) {
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni) f.b[ni] = *(const u32x4 *)(st + fb + ni * 32 * G2_STRIDE + ks * 32);
+#pragma unroll
+        for (int mi = 0; mi < WM; ++mi) f.a[mi] = *(const u32x4 *)(st + fa + mi * 32 * G2_STRIDE + ks * 32);
+    };
+    auto mma = [&](const Frag &f) {
+#pragma unroll
+        for (int mi = 0; mi < WM; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 4; ++ni)
+                acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, f.a[mi]), __builtin_bit_cast(bf16x8, f.b[ni]), acc[mi][ni], 0, 0, 0);
+    };
+    constexpr int NMMA = WM * 4, NFR = WM + 4;
+    Frag f0, f1;
+    read_frag(f0, lds2, 0);
+    for (int kt = 0; kt < KT; ++kt) {
+        const unsigned char *st = lds2 + (kt & 1) * STAGE;
+        unsigned char *nx = lds2 + ((kt + 1) & 1) * STAGE;
+        const size_t knext = (size_t)min(kt + 1, KT - 1) * G2_BK;
+#pragma unroll
+        for (int i = 0; i < NA; ++i) ra[i] = *(const u32x4 *)(ga[i] + knext);
+#pragma unroll
+        for (int i = 0; i < NB; ++i) rb[i] = *(const u32x4 *)(gb[i] + knext);
+        read_frag(f1, st, 1);
+        mma(f0);
+        // one global load then one MFMA, NA + NB times; the fragment reads spread over the MFMAs
+#pragma unroll
+        for (int i = 0; i < NFR; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x020, (NA + NB) / NFR, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, NMMA / NFR, 0);
+        }
+        read_frag(f0, st, 2);
+        mma(f1);
+#pragma unroll
+        for (int i = 0; i < NFR; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, NMMA / NFR, 0);
+        }
+        read_frag(f1, st, 3);
+        mma(f0);
+#pragma unroll
+        for (int i = 0; i < NFR; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, NMMA / NFR, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < NA; ++i) *(u32x4 *)(nx + la[i]) = ra[i];
+#pragma unroll
+        for (int i = 0; i < NB; ++i) *(u32x4 *)(nx + lb[i]) = rb[i];
+        __syncthreads();
+        read_frag(f0, nx, 0);
+        mma(f1);
+#pragma unroll
+        for (int i = 0; i < NFR; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, NMMA / NFR, 0);
+        }
+    }
+
+    // 32x32 accumulator layout: element i of lane l is row (i / 4) * 8 + (l / 32) * 4 + i % 4, column l % 32
+#pragma unroll
+    for (int mi = 0; mi < WM; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni) {
+            const int col = n0 + wcol + ni * 32 + l31;
+            if (col >= N) continue;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int row = m0 + wrow + mi * 32 + (i >> 2) * 8 + lh * 4 + (i & 3);
+                if (row >= M) continue;
+                float *dst = c + (size_t)row * ldc + col;
+                const float v = alpha * acc[mi][ni][i];
+                *dst = beta == 0.f ? v : v + beta * *dst;
+            }
+        }
+}
+
 constexpr int BM = 256, BN = 128, BK = 32;
 constexpr int LDS_ROW = 80;                       // 64 B of bf16 + 16 B pad
 constexpr int A_TILE = BM * LDS_ROW, B_TILE = BN * LDS_ROW;
@@ -294,9 +445,35 @@ int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *cw, size_t m, const
         launch_k(ctx, act_bf16_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, a, lda, abf, m, K);
         LAUNCH_CHECK(ctx, "act_bf16");
     }
-    const dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((m + BM - 1) / BM));
     ProfScope scope(ctx, "gemm_bf16");
-    launch_k(ctx, gemm_bf16_kernel, grid, dim3(256), 0, abf, w->bf16, c, (int)m, (int)N, (int)K, ldc, alpha, beta);
+    if (K % G2_BK == 0) {
+        // 256-row tiles when they still give every CU a workgroup, else 128-row tiles
+        const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
+        const int tn = (int)((N + G2_BN - 1) / G2_BN);
+        const int tm4 = (int)((m + 255) / 256), tm2 = (int)((m + 127) / 128);
+        const bool big = (long)tm4 * tn >= cus;
+        const int tm = big ? tm4 : tm2, tiles = tm * tn;
+        const dim3 grid((unsigned)((tiles + 7) / 8 * 8));
+        static bool attr4 = false, attr2 = false;
+        if (big) {
+            constexpr int LDS = 2 * (256 + G2_BN) * G2_STRIDE;
+            if (!attr4) {
+                HIP_TRY(ctx, hipFuncSetAttribute((const void *)gemm_bf16_wide_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+                attr4 = true;
+            }
+            launch_k(ctx, gemm_bf16_wide_kernel<4>, grid, dim3(256), LDS, abf, w->bf16, c, (int)m, (int)N, (int)K, ldc, alpha, beta, tm, tiles);
+        } else {
+            constexpr int LDS = 2 * (128 + G2_BN) * G2_STRIDE;
+            if (!attr2) {
+                HIP_TRY(ctx, hipFuncSetAttribute((const void *)gemm_bf16_wide_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+                attr2 = true;
+            }
+            launch_k(ctx, gemm_bf16_wide_kernel<2>, grid, dim3(256), LDS, abf, w->bf16, c, (int)m, (int)N, (int)K, ldc, alpha, beta, tm, tiles);
+        }
+    } else {
+        const dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((m + BM - 1) / BM));
+        launch_k(ctx, gemm_bf16_kernel, grid, dim3(256), 0, abf, w->bf16, c, (int)m, (int)N, (int)K, ldc, alpha, beta);
+    }
     LAUNCH_CHECK(ctx, "gemm_bf16");
     return AIONHIP_OK;
 }
