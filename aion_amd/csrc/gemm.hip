@@ -7,11 +7,9 @@
 //   memory in MFMA layout (8 bytes per lane per tile). The per-block rescale (3 VALU ops per
 //   output element per block) is what bounds it, not the MFMA pipe.
 //
-// gemm_bf16_kernel (AIONHIP_GEMM_BF16_MFMA) - weights dequantized once to bf16 [N,K] (kept per
-//   weight: 288 GB of HBM makes the 2 B/weight copy affordable), activations rounded to bf16,
-//   v_mfma_f32_16x16x32_bf16 with f32 accumulation. Workgroup tile 256x128, K step 32, operands
-//   staged through double-buffered LDS (row stride 80 B: conflict-free 16-byte operand reads),
-//   global loads of the next K step in flight during the MFMAs of the current one.
+// gemm_bf16_wide_kernel (AIONHIP_GEMM_BF16_MFMA) - weights dequantized once to bf16 [N,K] (kept
+//   per weight: 288 GB of HBM makes the 2 B/weight copy affordable), activations rounded to bf16,
+//   v_mfma_f32_32x32x16_bf16 with f32 accumulation; described at the kernel.
 #include "common.h"
 
 namespace {
@@ -152,24 +150,34 @@ __global__ void act_bf16_kernel(const float *__restrict__ a, size_t lda, unsigne
     *(u32x4 *)(out + m * K + k0) = o;
 }
 
-// ---- wide-tile kernel: workgroup tile (WM*64) x 256, K step 64, v_mfma_f32_32x32x16_bf16.
+// ---- wide-tile kernel: workgroup tile (WM*64) x 256, K step 32, v_mfma_f32_32x32x16_bf16.
 // 2 x 2 wavefronts, each (WM*32) x 128 outputs = WM x 4 tiles of 32x32 (accumulators: WM*64
-// registers). Operands go global -> registers -> LDS (row stride 144 B: 16 consecutive rows land
-// in 16 distinct 16-byte bank groups) -> 16-byte fragment reads; the next K step's global loads
-// are in flight during the MFMAs of the current one, one barrier per K step.
+// registers). Operands go global -> LDS directly (global_load_lds_dwordx4: each wavefront load
+// fills 1 KiB = 16 rows of 64 B, no staging registers, no LDS store instructions). Rows are not
+// padded; the 16-byte chunk c of row r sits at slot c ^ ((r >> 2) & 3), chosen on the global side
+// of the load, so that the 16 consecutive rows of a fragment read hit 16 distinct bank groups.
+// Four LDS stages: the loads of K steps kt+1..kt+3 are in flight during the MFMAs of step kt - a
+// load round trip through L2 under this traffic takes about as long as two K steps of MFMAs.
+// The wavefront waits on its own loads by count (s_waitcnt vmcnt) and the stages are handed over
+// with a bare s_barrier: a fence would drain the younger stages' loads as well.
 // Tile order: workgroup ids go round-robin over the 8 XCDs, so id -> (xcd, slot) -> a contiguous
 // run of tiles per XCD, M fastest: the workgroups that share a weight column tile run on one L2.
-constexpr int G2_BK = 64, G2_STRIDE = 144, G2_BN = 256;
+constexpr int G2_BK = 32, G2_ROW = 64, G2_BN = 256;
 using f32x16 = __attribute__((ext_vector_type(16))) float;
+typedef __attribute__((address_space(3))) void lds_void;
 
-template <int WM>
-__global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const unsigned short *__restrict__ A, const unsigned short *__restrict__ W,
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14)
+constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
+
+template <int WM, int NST, int WGS_PER_CU>
+__global__ __launch_bounds__(256, WGS_PER_CU) void gemm_bf16_wide_kernel(const unsigned short *__restrict__ A, const unsigned short *__restrict__ W,
                                                              float *__restrict__ c, int M, int N, int K, size_t ldc, float alpha,
                                                              float beta, int tiles_m, int tiles) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds2[];
+    extern __shared__ __attribute__((aligned(1024))) unsigned char lds2[];
     constexpr int BM2 = WM * 64;
-    constexpr int A_BYTES = BM2 * G2_STRIDE, B_BYTES = G2_BN * G2_STRIDE, STAGE = A_BYTES + B_BYTES;
-    constexpr int NA = WM * 2, NB = 8;                       // 16-byte chunks per thread per stage
+    constexpr int A_BYTES = BM2 * G2_ROW, B_BYTES = G2_BN * G2_ROW, STAGE = A_BYTES + B_BYTES;
+    constexpr int NA = WM, NB = 4;                           // wavefront loads (16 rows each) per stage
+    constexpr int NL = NA + NB;
     const int per_xcd = (int)gridDim.x >> 3;
     const int t = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
     if (t >= tiles) return;
@@ -186,49 +194,45 @@ __global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const unsigned shor
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[mi][ni][i] = 0.f;
 
+    // load i of this wavefront covers tile rows i*64 + wave*16 .. +16; lane -> (row lane>>2, slot lane&3)
+    const int lrow = wave * 16 + (lane >> 2);
+    const int lchunk = (lane & 3) ^ ((lrow >> 2) & 3);
     const unsigned short *ga[NA], *gb[NB];
-    int la[NA], lb[NB];
 #pragma unroll
-    for (int i = 0; i < NA; ++i) {
-        const int ch = tid + 256 * i, row = ch >> 3, part = ch & 7;
-        ga[i] = A + (size_t)min(m0 + row, M - 1) * K + part * 8;
-        la[i] = row * G2_STRIDE + part * 16;
-    }
+    for (int i = 0; i < NA; ++i) ga[i] = A + (size_t)min(m0 + i * 64 + lrow, M - 1) * K + lchunk * 8;
 #pragma unroll
-    for (int i = 0; i < NB; ++i) {
-        const int ch = tid + 256 * i, row = ch >> 3, part = ch & 7;
-        gb[i] = W + (size_t)min(n0 + row, N - 1) * K + part * 8;
-        lb[i] = A_BYTES + row * G2_STRIDE + part * 16;
-    }
-    const int fa = (wrow + l31) * G2_STRIDE + lh * 16;              // + mi * 32 rows + ks * 32 bytes
-    const int fb = A_BYTES + (wcol + l31) * G2_STRIDE + lh * 16;
-
+    for (int i = 0; i < NB; ++i) gb[i] = W + (size_t)min(n0 + i * 64 + lrow, N - 1) * K + lchunk * 8;
     const int KT = K / G2_BK;
-    u32x4 ra[NA], rb[NB];
-#pragma unroll
-    for (int i = 0; i < NA; ++i) ra[i] = *(const u32x4 *)(ga[i]);
-#pragma unroll
-    for (int i = 0; i < NB; ++i) rb[i] = *(const u32x4 *)(gb[i]);
-#pragma unroll
-    for (int i = 0; i < NA; ++i) *(u32x4 *)(lds2 + la[i]) = ra[i];
-#pragma unroll
-    for (int i = 0; i < NB; ++i) *(u32x4 *)(lds2 + lb[i]) = rb[i];
-    __syncthreads();
 
-    // Software pipeline, one basic block per K step so that the instruction groups can be pinned:
-    //   sub-step 0: global loads of the next K step + MFMAs(0) while the fragments of sub-step 1 are read
-    //   sub-step 1: MFMAs(1) while fragments 2 are read;  sub-step 2: MFMAs(2) while fragments 3 are read
-    //   staged registers -> the other LDS buffer, barrier
-    //   sub-step 3: MFMAs(3) while fragments 0 of the next K step are read from the other buffer
-    // The last K step repeats its own loads into the idle buffer instead of branching.
+    auto issue_loads = [&](int kt) {
+#if defined(__HIP_DEVICE_COMPILE__)   // the builtin exists in the device pass only
+        unsigned char *stage = lds2 + (kt % NST) * STAGE + wave * 16 * G2_ROW;
+        const size_t k = (size_t)min(kt, KT - 1) * G2_BK;   // past the end: a harmless repeat into a dead stage
+#pragma unroll
+        for (int i = 0; i < NA; ++i)
+            __builtin_amdgcn_global_load_lds(ga[i] + k, (lds_void *)(stage + i * 64 * G2_ROW), 16, 0, 0);
+#pragma unroll
+        for (int i = 0; i < NB; ++i)
+            __builtin_amdgcn_global_load_lds(gb[i] + k, (lds_void *)(stage + A_BYTES + i * 64 * G2_ROW), 16, 0, 0);
+#endif
+    };
+
+    // fragment of sub-step ks: row (base + l31), chunk ks*2 + lh, at slot chunk ^ ((l31 >> 2) & 3)
+    const int swz = (l31 >> 2) & 3;
+    int foff[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) foff[ks] = l31 * G2_ROW + (((ks * 2 + lh) ^ swz) * 16);
+    const int fa = wrow * G2_ROW, fb = A_BYTES + wcol * G2_ROW;
+
     struct Frag {
         u32x4 a[WM], b[4];
     };
-    auto read_frag = [&](Frag &f, const unsigned char *st, int ks) {
+    auto read_frag = [&](Frag &f, int kt, int ks) {
+        const unsigned char *st = lds2 + (kt % NST) * STAGE;
 #pragma unroll
-        for (int ni = 0; ni < 4; ++ni) f.b[ni] = *(const u32x4 *)(st + fb + ni * 32 * G2_STRIDE + ks * 32);
+        for (int ni = 0; ni < 4; ++ni) f.b[ni] = *(const u32x4 *)(st + fb + ni * 32 * G2_ROW + foff[ks]);
 #pragma unroll
-        for (int mi = 0; mi < WM; ++mi) f.a[mi] = *(const u32x4 *)(st + fa + mi * 32 * G2_STRIDE + ks * 32);
+        for (int mi = 0; mi < WM; ++mi) f.a[mi] = *(const u32x4 *)(st + fa + mi * 32 * G2_ROW + foff[ks]);
     };
     auto mma = [&](const Frag &f) {
 #pragma unroll
@@ -238,52 +242,60 @@ __global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const unsigned shor
                 acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, f.a[mi]), __builtin_bit_cast(bf16x8, f.b[ni]), acc[mi][ni], 0, 0, 0);
     };
     constexpr int NMMA = WM * 4, NFR = WM + 4;
+
+#pragma unroll
+    for (int i = 0; i < NST - 1; ++i) issue_loads(i);
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm((NST - 2) * NL));   // stage 0 of this wavefront has landed
+    __builtin_amdgcn_s_barrier();                            // ... and everybody else's
     Frag f0, f1;
-    read_frag(f0, lds2, 0);
+    read_frag(f0, 0, 0);
     for (int kt = 0; kt < KT; ++kt) {
-        const unsigned char *st = lds2 + (kt & 1) * STAGE;
-        unsigned char *nx = lds2 + ((kt + 1) & 1) * STAGE;
-        const size_t knext = (size_t)min(kt + 1, KT - 1) * G2_BK;
-#pragma unroll
-        for (int i = 0; i < NA; ++i) ra[i] = *(const u32x4 *)(ga[i] + knext);
-#pragma unroll
-        for (int i = 0; i < NB; ++i) rb[i] = *(const u32x4 *)(gb[i] + knext);
-        read_frag(f1, st, 1);
+        // sub-step 0 while the fragments of sub-step 1 are read
+        read_frag(f1, kt, 1);
         mma(f0);
-        // one global load then one MFMA, NA + NB times; the fragment reads spread over the MFMAs
+        // two MFMAs first: the wait in front of them then covers only reads issued long ago; all
+        // reads of the next fragment follow early, so that they are back when the next sub-step starts
+        if constexpr (WM >= 2) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
 #pragma unroll
-        for (int i = 0; i < NFR; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x020, (NA + NB) / NFR, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, NMMA / NFR, 0);
+            for (int i = 0; i < NFR; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, NMMA - 2 - NFR, 0);
         }
-        read_frag(f0, st, 2);
+        // stage kt+1 landed (stage kt+2 may still be in flight); past this barrier nobody reads stage kt-1
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((NST - 3) * NL));
+        __builtin_amdgcn_s_barrier();
+        // sub-step 1 while fragments 0 of the next K step are read, then the loads of stage kt+3
+        // (an LDS-writing load may not move above an LDS read: reads first)
+        read_frag(f0, kt + 1, 0);
+        issue_loads(kt + NST - 1);
         mma(f1);
+        if constexpr (WM == 4) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
 #pragma unroll
-        for (int i = 0; i < NFR; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, NMMA / NFR, 0);
-        }
-        read_frag(f1, st, 3);
-        mma(f0);
+            for (int i = 0; i < NFR; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            }
 #pragma unroll
-        for (int i = 0; i < NFR; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, NMMA / NFR, 0);
-        }
+            for (int i = 0; i < NL / 2; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, NMMA - 2 - NFR - NL / 2, 0);
+        } else if constexpr (WM == 2) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
 #pragma unroll
-        for (int i = 0; i < NA; ++i) *(u32x4 *)(nx + la[i]) = ra[i];
-#pragma unroll
-        for (int i = 0; i < NB; ++i) *(u32x4 *)(nx + lb[i]) = rb[i];
-        __syncthreads();
-        read_frag(f0, nx, 0);
-        mma(f1);
-#pragma unroll
-        for (int i = 0; i < NFR; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, NMMA / NFR, 0);
+            for (int i = 0; i < NFR; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            }
         }
     }
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));                // no LDS-writing load may outlive the workgroup
 
     // 32x32 accumulator layout: element i of lane l is row (i / 4) * 8 + (l / 32) * 4 + i % 4, column l % 32
 #pragma unroll
@@ -296,101 +308,6 @@ __global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const unsigned shor
             for (int i = 0; i < 16; ++i) {
                 const int row = m0 + wrow + mi * 32 + (i >> 2) * 8 + lh * 4 + (i & 3);
                 if (row >= M) continue;
-                float *dst = c + (size_t)row * ldc + col;
-                const float v = alpha * acc[mi][ni][i];
-                *dst = beta == 0.f ? v : v + beta * *dst;
-            }
-        }
-}
-
-constexpr int BM = 256, BN = 128, BK = 32;
-constexpr int LDS_ROW = 80;                       // 64 B of bf16 + 16 B pad
-constexpr int A_TILE = BM * LDS_ROW, B_TILE = BN * LDS_ROW;
-
-__global__ __launch_bounds__(256) void gemm_bf16_kernel(const unsigned short *__restrict__ A, const unsigned short *__restrict__ W,
-                                                        float *__restrict__ c, int M, int N, int K, size_t ldc, float alpha, float beta) {
-    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * (A_TILE + B_TILE)];
-    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int r = lane & 15, g = lane >> 4;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-    const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 64;   // 2 x 2 wavefronts, each 128 x 64
-    constexpr int TM = 8, TN = 4;
-
-    f32x4 acc[TM][TN];
-#pragma unroll
-    for (int mi = 0; mi < TM; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < TN; ++ni) acc[mi][ni] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    // global -> LDS assignment: 16-byte chunks; A tile 1024 chunks (4 per thread), B tile 512 (2 per thread)
-    const unsigned short *ga[4];
-    const unsigned short *gb[2];
-    int la[4], lb[2];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int ch = tid + 256 * i, row = ch >> 2, part = ch & 3;
-        ga[i] = A + (size_t)min(m0 + row, M - 1) * K + part * 8;
-        la[i] = row * LDS_ROW + part * 16;
-    }
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int ch = tid + 256 * i, row = ch >> 2, part = ch & 3;
-        gb[i] = W + (size_t)min(n0 + row, N - 1) * K + part * 8;
-        lb[i] = row * LDS_ROW + part * 16;
-    }
-
-    const int KT = K / BK;
-    u32x4 ra[4], rb[2];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) ra[i] = *(const u32x4 *)(ga[i]);
-#pragma unroll
-    for (int i = 0; i < 2; ++i) rb[i] = *(const u32x4 *)(gb[i]);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) *(u32x4 *)(lds + la[i]) = ra[i];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) *(u32x4 *)(lds + A_TILE + lb[i]) = rb[i];
-    __syncthreads();
-
-    for (int kt = 0; kt < KT; ++kt) {
-        const unsigned char *sa = lds + (kt & 1) * (A_TILE + B_TILE);
-        const unsigned char *sb = sa + A_TILE;
-        const bool more = kt + 1 < KT;
-        if (more) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) ra[i] = *(const u32x4 *)(ga[i] + (size_t)(kt + 1) * BK);
-#pragma unroll
-            for (int i = 0; i < 2; ++i) rb[i] = *(const u32x4 *)(gb[i] + (size_t)(kt + 1) * BK);
-        }
-        u32x4 bf[TN];
-#pragma unroll
-        for (int ni = 0; ni < TN; ++ni) bf[ni] = *(const u32x4 *)(sb + (wn0 + ni * 16 + r) * LDS_ROW + g * 16);
-#pragma unroll
-        for (int mi = 0; mi < TM; ++mi) {
-            const u32x4 af = *(const u32x4 *)(sa + (wm0 + mi * 16 + r) * LDS_ROW + g * 16);
-#pragma unroll
-            for (int ni = 0; ni < TN; ++ni)
-                acc[mi][ni] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, af), __builtin_bit_cast(bf16x8, bf[ni]), acc[mi][ni], 0, 0, 0);
-        }
-        if (more) {
-            unsigned char *da = lds + ((kt + 1) & 1) * (A_TILE + B_TILE);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) *(u32x4 *)(da + la[i]) = ra[i];
-#pragma unroll
-            for (int i = 0; i < 2; ++i) *(u32x4 *)(da + A_TILE + lb[i]) = rb[i];
-        }
-        __syncthreads();
-    }
-
-#pragma unroll
-    for (int mi = 0; mi < TM; ++mi)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int row = m0 + wm0 + mi * 16 + g * 4 + i;
-            if (row >= M) continue;
-#pragma unroll
-            for (int ni = 0; ni < TN; ++ni) {
-                const int col = n0 + wn0 + ni * 16 + r;
-                if (col >= N) continue;
                 float *dst = c + (size_t)row * ldc + col;
                 const float v = alpha * acc[mi][ni][i];
                 *dst = beta == 0.f ? v : v + beta * *dst;
@@ -446,33 +363,38 @@ int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *cw, size_t m, const
         LAUNCH_CHECK(ctx, "act_bf16");
     }
     ProfScope scope(ctx, "gemm_bf16");
-    if (K % G2_BK == 0) {
+    {
         // 256-row tiles when they still give every CU a workgroup, else 128-row tiles
         const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
         const int tn = (int)((N + G2_BN - 1) / G2_BN);
-        const int tm4 = (int)((m + 255) / 256), tm2 = (int)((m + 127) / 128);
-        const bool big = (long)tm4 * tn >= cus;
-        const int tm = big ? tm4 : tm2, tiles = tm * tn;
+        // tallest tile that still gives every CU a workgroup; 64-row tiles when even 128-row ones leave half idle
+        const int tm4 = (int)((m + 255) / 256), tm2 = (int)((m + 127) / 128), tm1 = (int)((m + 63) / 64);
+        const int wm = (long)tm4 * tn >= cus ? 4 : ((long)tm2 * tn * 2 > cus ? 2 : 1);
+        const int tm = wm == 4 ? tm4 : (wm == 2 ? tm2 : tm1), tiles = tm * tn;
         const dim3 grid((unsigned)((tiles + 7) / 8 * 8));
-        static bool attr4 = false, attr2 = false;
-        if (big) {
-            constexpr int LDS = 2 * (256 + G2_BN) * G2_STRIDE;
-            if (!attr4) {
-                HIP_TRY(ctx, hipFuncSetAttribute((const void *)gemm_bf16_wide_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
-                attr4 = true;
+        static bool attr[3] = {false, false, false};
+        if (wm == 4) {
+            constexpr int LDS = 4 * (256 + G2_BN) * G2_ROW;
+            if (!attr[0]) {
+                HIP_TRY(ctx, hipFuncSetAttribute((const void *)gemm_bf16_wide_kernel<4, 4, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+                attr[0] = true;
             }
-            launch_k(ctx, gemm_bf16_wide_kernel<4>, grid, dim3(256), LDS, abf, w->bf16, c, (int)m, (int)N, (int)K, ldc, alpha, beta, tm, tiles);
+            launch_k(ctx, gemm_bf16_wide_kernel<4, 4, 1>, grid, dim3(256), LDS, abf, w->bf16, c, (int)m, (int)N, (int)K, ldc, alpha, beta, tm, tiles);
+        } else if (wm == 2) {
+            constexpr int LDS = 4 * (128 + G2_BN) * G2_ROW;
+            if (!attr[1]) {
+                HIP_TRY(ctx, hipFuncSetAttribute((const void *)gemm_bf16_wide_kernel<2, 4, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+                attr[1] = true;
+            }
+            launch_k(ctx, gemm_bf16_wide_kernel<2, 4, 1>, grid, dim3(256), LDS, abf, w->bf16, c, (int)m, (int)N, (int)K, ldc, alpha, beta, tm, tiles);
         } else {
-            constexpr int LDS = 2 * (128 + G2_BN) * G2_STRIDE;
-            if (!attr2) {
-                HIP_TRY(ctx, hipFuncSetAttribute((const void *)gemm_bf16_wide_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
-                attr2 = true;
+            constexpr int LDS = 4 * (64 + G2_BN) * G2_ROW;
+            if (!attr[2]) {
+                HIP_TRY(ctx, hipFuncSetAttribute((const void *)gemm_bf16_wide_kernel<1, 4, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+                attr[2] = true;
             }
-            launch_k(ctx, gemm_bf16_wide_kernel<2>, grid, dim3(256), LDS, abf, w->bf16, c, (int)m, (int)N, (int)K, ldc, alpha, beta, tm, tiles);
+            launch_k(ctx, gemm_bf16_wide_kernel<1, 4, 1>, grid, dim3(256), LDS, abf, w->bf16, c, (int)m, (int)N, (int)K, ldc, alpha, beta, tm, tiles);
         }
-    } else {
-        const dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((m + BM - 1) / BM));
-        launch_k(ctx, gemm_bf16_kernel, grid, dim3(256), 0, abf, w->bf16, c, (int)m, (int)N, (int)K, ldc, alpha, beta);
     }
     LAUNCH_CHECK(ctx, "gemm_bf16");
     return AIONHIP_OK;
