@@ -107,8 +107,8 @@ __device__ __forceinline__ int wave_max_i(int v) {
 // is one workgroup whose eight wavefronts take one 32-key tile each)
 template <int D, int NW>
 struct FlashCfg {
-    static constexpr int ROW_BYTES = D * 2 + 16;                 // +16 B: the four key groups land in distinct LDS banks
-    static constexpr int WAVE_LDS = TILE_KEYS * ROW_BYTES;       // one staged V tile per wavefront
+    static constexpr int ROW_BYTES = D * 2;                      // unpadded: the tile is filled by LDS-writing loads
+    static constexpr int WAVE_LDS = TILE_KEYS * ROW_BYTES;       // one V tile per wavefront
     static constexpr int WG_LDS = NW * WAVE_LDS;
     static constexpr int MERGE_LDS = (NW * (16 * (D + 4) + 32) + 16 * NW + 32) * 4;   // split mode: NW x (acc[16][D+4], m[16], l[16]) f32 + merge factors
     static constexpr int LDS_BYTES = WG_LDS > MERGE_LDS ? WG_LDS : MERGE_LDS;
@@ -232,13 +232,18 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
     const size_t kv_row = (size_t)a.Hkv * D;                     // elements between consecutive tokens
     const size_t kv_base = ((size_t)b * a.T * a.Hkv + hk) * D;
 
-    for (int t = t_begin; t < t_end; t += t_step) {
+    // K (MFMA operand layout, registers) of a tile is requested one tile ahead, right after the S MFMAs
+    // have released the registers. V goes global -> LDS directly (global_load_lds_dwordx4, 1 KiB per
+    // instruction) into this wavefront's tile, requested as soon as the previous tile's gathers are done.
+    // Tile layout: key row of D*2 bytes, 16-byte chunk c of key k at slot c ^ (2 * ((k >> 2) & 3)): the
+    // four key groups of a gather then read distinct banks. Keys outside the union interval are read from
+    // a clamped in-range key instead (their probabilities are exact zeros, and the cache tail may hold
+    // anything, so the value must only be finite).
+    constexpr int NVI = TILE_KEYS * D * 2 / 1024;
+    constexpr int KEYS_PER_VI = 1024 / (D * 2);
+    u32x4 kf[2][KK];
+    auto load_k = [&](int t) {
         const int key0 = t * TILE_KEYS;
-        // -- request this tile's K (MFMA operand layout) and then V (staging layout); loads return in
-        //    order, so the S MFMAs wait for K only while V is still in flight
-        constexpr int CHUNKS_PER_KEY = D / 8;
-        constexpr int NV = TILE_KEYS * CHUNKS_PER_KEY / 64;
-        u32x4 kf[2][KK], vreg[NV];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int kabs = min(key0 + h * 16 + n, a.T - 1);
@@ -246,12 +251,29 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
 #pragma unroll
             for (int kk = 0; kk < KK; ++kk) kf[h][kk] = *(const u32x4 *)(krow + kk * 32);
         }
+    };
+    const int v_key_in = (lane * 16) / (D * 2);                      // key of this lane within one V load
+    const int v_slot = ((lane * 16) % (D * 2)) / 16;                 // its 16-byte slot within the key row
+    const int v_hi_key = max(uni_hi - 1, 0);
+    auto load_v = [&](int t) {
+#if defined(__HIP_DEVICE_COMPILE__)   // the builtin exists in the device pass only
+        const int key0 = t * TILE_KEYS;
 #pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            const int c = lane + 64 * i;
-            const int kabs = min(key0 + c / CHUNKS_PER_KEY, a.T - 1);
-            vreg[i] = *(const u32x4 *)(vp + kv_base + (size_t)kabs * kv_row + (c % CHUNKS_PER_KEY) * 8);
+        for (int i = 0; i < NVI; ++i) {
+            const int key = i * KEYS_PER_VI + v_key_in;
+            const int chunk = v_slot ^ (2 * ((key >> 2) & 3));
+            const int kabs = min(max(key0 + key, uni_lo), v_hi_key);
+            __builtin_amdgcn_global_load_lds(vp + kv_base + (size_t)kabs * kv_row + chunk * 8, (lds_void *)(vs + i * 1024), 16, 0, 0);
         }
+#endif
+    };
+    if (t_begin < t_end) {
+        load_k(t_begin);
+        load_v(t_begin);
+    }
+    for (int t = t_begin; t < t_end; t += t_step) {
+        const int key0 = t * TILE_KEYS;
+        const bool more = t + t_step < t_end;      // wavefront-uniform
         // -- S^T = K . Q^T for two 16-key halves
         f32x4 s[2];
 #pragma unroll
@@ -264,6 +286,7 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
             }
             s[h] = c;
         }
+        if (more) load_k(t + t_step);
         // -- scale, soft cap, interval mask; lane holds keys key0 + h*16 + g*4 + i of row n
         float p[8];
         float mx = -INFINITY;
@@ -309,30 +332,23 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
         const u32x4 pf_lo = u32x4{(unsigned)pl[0] | ((unsigned)pl[1] << 16), (unsigned)pl[2] | ((unsigned)pl[3] << 16),
                                   (unsigned)pl[4] | ((unsigned)pl[5] << 16), (unsigned)pl[6] | ((unsigned)pl[7] << 16)};
 
-        // -- stage V into this wavefront's LDS tile (keys outside the union interval as zeros: the cache
-        //    tail may hold anything) ; the tile is written and read by this wavefront only
-#pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            const int c = lane + 64 * i;
-            const int key = c / CHUNKS_PER_KEY, col8 = c % CHUNKS_PER_KEY;
-            const int kabs = key0 + key;
-            const bool inside = kabs >= uni_lo && kabs < uni_hi;
-            *(u32x4 *)(vs + key * Cfg::ROW_BYTES + col8 * 16) = inside ? vreg[i] : u32x4{0u, 0u, 0u, 0u};
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // -- this tile's V has landed in the wavefront's LDS tile once only the younger K loads are
+        //    outstanding (loads complete in order); the tile is written and read by this wavefront only
+        if (more) __builtin_amdgcn_s_waitcnt(vmcnt_imm(2 * KK));
+        else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
 
         // -- O^T += V^T . P^T ; operand slot j of lane group g is key g*4+j (j<4) / 16+g*4+j-4
         const bool rescale = __any(alpha != 1.f);     // wavefront-uniform: skip 4*MT multiplies when no row's max moved
-        const unsigned char *vcol = vs + n * 2;
+        // element (key, dv) sits at key*ROW + ((dv/8) ^ 2g)*16 + (dv%8)*2; (key >> 2) & 3 == g for all 8 keys of a lane
+        const unsigned char *vcol = vs + (n & 7) * 2;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             unsigned short e[8];
+            const int coff = ((mt * 2 + (n >> 3)) ^ (2 * g)) * 16;
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const int key = j < 4 ? g * 4 + j : 16 + g * 4 + (j - 4);
-                e[j] = *(const unsigned short *)(vcol + key * Cfg::ROW_BYTES + mt * 32);
+                e[j] = *(const unsigned short *)(vcol + key * Cfg::ROW_BYTES + coff);
             }
             const u32x4 vf = u32x4{(unsigned)e[0] | ((unsigned)e[1] << 16), (unsigned)e[2] | ((unsigned)e[3] << 16),
                                    (unsigned)e[4] | ((unsigned)e[5] << 16), (unsigned)e[6] | ((unsigned)e[7] << 16)};
@@ -342,8 +358,7 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
             if (HILO) c = mfma16<KV>(vf, pf_lo, c);
             acc[mt] = c;
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
+        if (more) load_v(t + t_step);      // the gathers above are complete: their values fed the MFMAs
     }
 
     if (!SPLIT) {
@@ -414,29 +429,75 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
     }
 }
 
-// log-sum-exp merge of the key segments: one workgroup per (row tile, 64-wide dv slice, unit)
+// log-sum-exp merge of the key segments: one workgroup per (row tile, 16-wide dv slice, unit).
+// Thread = (segment group of 4, row of 16, 4 consecutive dv): it folds every fourth segment with all
+// of a round's loads in flight at once, then the four groups fold through LDS.
+constexpr int MERGE_DV = 16, MERGE_SG = 4, MERGE_UNROLL = 8;
 template <int D>
 __global__ __launch_bounds__(256) void attn_merge_kernel(AttnArgs a) {
     constexpr int WSTRIDE = 16 * D + 32;
-    constexpr int SLICES = D / 64;
+    constexpr int SLICES = D / MERGE_DV;
+    __shared__ float s_m[MERGE_SG][16][4], s_l[MERGE_SG][16][4];
+    __shared__ __attribute__((aligned(16))) float s_o[MERGE_SG][16][MERGE_DV];
     const int unit = blockIdx.y, rt = blockIdx.x / SLICES, slice = blockIdx.x % SLICES;
     const int b = unit / a.Hkv, hk = unit % a.Hkv;
+    const int tid = threadIdx.x, q4 = tid & 3, row = (tid >> 2) & 15, sg = tid >> 6;
     const float *base = a.partial + (size_t)(unit * a.row_tiles + rt) * a.nseg * WSTRIDE;
-    for (int e = threadIdx.x; e < 16 * 64; e += 256) {
-        const int row = e >> 6, dv = slice * 64 + (e & 63);
-        const int rr = rt * 16 + row;
-        if (rr >= a.rows_total) continue;
-        float m_all = -INFINITY;
-        for (int s = 0; s < a.nseg; ++s) m_all = fmaxf(m_all, base[(size_t)s * WSTRIDE + 16 * D + row]);
-        float o = 0.f, l_all = 0.f;
-        for (int s = 0; s < a.nseg; ++s) {
-            const float ms = base[(size_t)s * WSTRIDE + 16 * D + row];
-            const float f = ms > -INFINITY ? exp2f((ms - m_all) * LOG2E) : 0.f;
-            o += base[(size_t)s * WSTRIDE + row * D + dv] * f;
-            l_all += base[(size_t)s * WSTRIDE + 16 * D + 16 + row] * f;
+    const int dv = slice * MERGE_DV + q4 * 4;
+    float m_loc = -INFINITY, l_loc = 0.f;
+    f32x4 o_loc = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int s0 = sg; s0 < a.nseg; s0 += MERGE_SG * MERGE_UNROLL) {
+        float ms[MERGE_UNROLL], ls[MERGE_UNROLL];
+        f32x4 os[MERGE_UNROLL];
+#pragma unroll
+        for (int u = 0; u < MERGE_UNROLL; ++u) {
+            const int sidx = min(s0 + u * MERGE_SG, a.nseg - 1);      // clamped: every load is unconditional
+            const float *p = base + (size_t)sidx * WSTRIDE;
+            ms[u] = p[16 * D + row];
+            ls[u] = p[16 * D + 16 + row];
+            os[u] = *(const f32x4 *)(p + row * D + dv);
         }
-        const int l2 = rr / a.groups, g2 = rr % a.groups;
-        a.out[(((size_t)b * a.L + l2) * a.Hq + hk * a.groups + g2) * D + dv] = l_all > 0.f ? o / l_all : 0.f;
+        float m_new = m_loc;
+#pragma unroll
+        for (int u = 0; u < MERGE_UNROLL; ++u)
+            if (s0 + u * MERGE_SG < a.nseg) m_new = fmaxf(m_new, ms[u]);
+        if (m_new > -INFINITY) {
+            const float f0 = m_loc > -INFINITY ? exp2f((m_loc - m_new) * LOG2E) : 0.f;
+            o_loc *= f0;
+            l_loc *= f0;
+#pragma unroll
+            for (int u = 0; u < MERGE_UNROLL; ++u) {
+                const bool live = s0 + u * MERGE_SG < a.nseg && ms[u] > -INFINITY;
+                const float f = live ? exp2f((ms[u] - m_new) * LOG2E) : 0.f;
+                o_loc += os[u] * f;
+                l_loc += ls[u] * f;
+            }
+            m_loc = m_new;
+        }
+    }
+    s_m[sg][row][q4] = m_loc;
+    s_l[sg][row][q4] = l_loc;
+    *(f32x4 *)&s_o[sg][row][q4 * 4] = o_loc;
+    __syncthreads();
+    if (sg == 0) {
+        float m_all = -INFINITY;
+#pragma unroll
+        for (int g2 = 0; g2 < MERGE_SG; ++g2) m_all = fmaxf(m_all, s_m[g2][row][q4]);
+        f32x4 o = f32x4{0.f, 0.f, 0.f, 0.f};
+        float l_all = 0.f;
+#pragma unroll
+        for (int g2 = 0; g2 < MERGE_SG; ++g2) {
+            const float mg = s_m[g2][row][q4];
+            const float f = mg > -INFINITY ? exp2f((mg - m_all) * LOG2E) : 0.f;
+            o += *(const f32x4 *)&s_o[g2][row][q4 * 4] * f;
+            l_all += s_l[g2][row][q4] * f;
+        }
+        const int rr = rt * 16 + row;
+        if (rr < a.rows_total) {
+            const int l2 = rr / a.groups, g3 = rr % a.groups;
+            const float inv = l_all > 0.f ? 1.f / l_all : 0.f;
+            *(f32x4 *)(a.out + (((size_t)b * a.L + l2) * a.Hq + hk * a.groups + g3) * D + dv) = o * inv;
+        }
     }
 }
 
@@ -522,7 +583,7 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
         }
         if (nseg > 1) {
             ProfScope scope(ctx, "attn_merge");
-            launch_k(ctx, attn_merge_kernel<D>, dim3((unsigned)(a.row_tiles * (D / 64)), (unsigned)units), dim3(256), 0, a);
+            launch_k(ctx, attn_merge_kernel<D>, dim3((unsigned)(a.row_tiles * (D / MERGE_DV)), (unsigned)units), dim3(256), 0, a);
         }
         LAUNCH_CHECK(ctx, "attn_flash_split");
     } else {

@@ -60,6 +60,11 @@ struct aionhip_ctx {
     std::vector<hipEvent_t> event_pool;
 };
 
+// LDS-writing global loads (global_load_lds_dwordx4) take an address-space-3 destination and are
+// waited for by count: s_waitcnt immediate for "vmcnt <= n" only (gfx9 encoding: bits 3:0 and 15:14).
+typedef __attribute__((address_space(3))) void lds_void;
+constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
+
 // Names the launches made through launch_k while it is alive (and profiling is on).
 struct ProfScope {
     aionhip_ctx *ctx;

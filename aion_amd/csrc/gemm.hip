@@ -164,10 +164,7 @@ __global__ void act_bf16_kernel(const float *__restrict__ a, size_t lda, unsigne
 // run of tiles per XCD, M fastest: the workgroups that share a weight column tile run on one L2.
 constexpr int G2_BK = 32, G2_ROW = 64, G2_BN = 256;
 using f32x16 = __attribute__((ext_vector_type(16))) float;
-typedef __attribute__((address_space(3))) void lds_void;
 
-// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and 15:14)
-constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
 
 template <int WM, int NST, int WGS_PER_CU>
 __global__ __launch_bounds__(256, WGS_PER_CU) void gemm_bf16_wide_kernel(const unsigned short *__restrict__ A, const unsigned short *__restrict__ W,
