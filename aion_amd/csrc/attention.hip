@@ -429,6 +429,272 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// attn_prefill_kernel - many query rows (prefill), q already in the K/V element type or f32 (rounded).
+//   A workgroup owns 128 query rows of one (batch, kv head) - position-major, GQA head fastest - and
+//   walks the 32-key tiles of the union of their intervals once; K and V tiles are loaded by the whole
+//   workgroup and shared through LDS (double-buffered, one barrier per tile), so a K/V byte fetched
+//   from L2 feeds 128 rows instead of 16. Each wavefront owns 32 rows and works in the transposed
+//   form on v_mfma_f32_32x32x16:
+//       S^T[32 keys x 32 rows]  = K_tile[32 x D] . Q^T[D x 32]       A = K rows from LDS (16 B reads)
+//       O^T[D x 32 rows]       += V^T[D x 32 keys] . P^T[32 x 32]    A = V^T rows from LDS (8 B reads)
+//   so every accumulator, the running max and the running sum of a lane belong to ONE query row.
+//   V is transposed once per tile by the loading threads (two keys packed per 32-bit store into
+//   V^T[dv][key], row stride 72 B: stores and operand reads are bank-conflict-free); the k index of
+//   the second product is permuted (slot s of lane half h <-> key (s/4)*8 + 4h + s%4 of a 16-key step)
+//   so that the probabilities feed the MFMA straight from the S accumulators without a shuffle.
+constexpr int PF_ROWS = 128, PF_VROW = 72;
+constexpr float PF_LAZY = 8.f;
+using f32x16 = __attribute__((ext_vector_type(16))) float;
+using u32x2 = __attribute__((ext_vector_type(2))) unsigned int;
+
+template <int D>
+struct PrefillCfg {
+    static constexpr int KROW = D * 2 + 16;                         // K tile row: 16 consecutive rows -> 16 distinct 16-byte bank groups
+    static constexpr int K_BYTES = TILE_KEYS * KROW;
+    static constexpr int V_BYTES = D * PF_VROW;
+    static constexpr int STAGE = K_BYTES + V_BYTES;
+    static constexpr int LDS_BYTES = 2 * STAGE + 64;
+};
+
+template <int KV>
+__device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+    if (KV == AIONHIP_F16)
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+template <int KV, int D, bool CAP>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    using Cfg = PrefillCfg<D>;
+    constexpr int KK = D / 16;          // k-steps of the first product
+    constexpr int NJ = D / 32;          // 32-wide dv tiles of the second product
+    constexpr int CPK = D / 8;          // 16-byte chunks per key row
+    constexpr int NKL = TILE_KEYS * CPK / 256;   // K chunks per thread per tile
+    constexpr int V_ITEMS = 16 * CPK;            // V (key pair, chunk) items per tile
+    constexpr int NVL = V_ITEMS >= 256 ? V_ITEMS / 256 : 1;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l31 = lane & 31, lh = lane >> 5;
+    const int unit = blockIdx.y, b = unit / a.Hkv, hk = unit % a.Hkv;
+
+    // ---- this lane's query row (lanes l and l+32 share it)
+    const int r = blockIdx.x * PF_ROWS + wave * 32 + l31;
+    const bool row_ok = r < a.rows_total;
+    const int li = row_ok ? r / a.groups : 0, gi = row_ok ? r % a.groups : 0;
+    const int hq = hk * a.groups + gi;
+    const int kv_end_raw = a.kv_lengths ? a.kv_lengths[b] : a.T;
+    const int pos_raw = (row_ok && a.positions) ? a.positions[(size_t)b * a.L + li] : li;
+    const size_t qbase = (((size_t)b * a.L + li) * a.Hq + hq) * D;
+
+    // Q^T operand: lane (row l31, half lh) holds d = 16*kk + 8*lh .. +7 for every kk
+    u32x4 qf[KK];
+    if (a.q_dtype == KV) {
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const u32x4 *)((const unsigned short *)a.q + qbase + kk * 16 + lh * 8);
+    } else {
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            float x[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) x[j] = load_scalar(a.q, a.q_dtype, qbase + kk * 16 + lh * 8 + j);
+            qf[kk] = u32x4{pack2<KV>(x[0], x[1]), pack2<KV>(x[2], x[3]), pack2<KV>(x[4], x[5]), pack2<KV>(x[6], x[7])};
+        }
+    }
+    if (!row_ok) {
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) qf[kk] = u32x4{0u, 0u, 0u, 0u};
+    }
+
+    const int kv_end = max(0, min(kv_end_raw, a.T));
+    int lo = 0, hi = 0;
+    if (row_ok) {
+        window_keys(a.win_left, a.win_right, a.win_chunk, max(pos_raw, 0), kv_end, lo, hi);
+        if (hi < lo) hi = lo;
+    }
+    const bool live = hi > lo;
+    // wavefront: union (which tiles it computes) and intersection (which tiles need no mask)
+    const int w_lo = wave_min_i(live ? lo : INT_MAX), w_hi = wave_max_i(live ? hi : 0);
+    const int w_lo_max = wave_max_i(live ? lo : INT_MAX), w_hi_min = wave_min_i(live ? hi : 0);
+    // workgroup union through LDS
+    int *s_rng = (int *)(lds + 2 * Cfg::STAGE);
+    if (lane == 0) { s_rng[wave] = w_lo; s_rng[4 + wave] = w_hi; }
+    __syncthreads();
+    const int g_lo = min(min(s_rng[0], s_rng[1]), min(s_rng[2], s_rng[3]));
+    const int g_hi = max(max(s_rng[4], s_rng[5]), max(s_rng[6], s_rng[7]));
+    if (g_hi <= g_lo) {                                 // nothing visible to any row: zeros
+        if (row_ok) {
+            float *o = a.out + qbase;
+            for (int d = lh * (D / 2); d < (lh + 1) * (D / 2); d += 4) *(f32x4 *)(o + d) = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+        return;
+    }
+    const int t_begin = g_lo / TILE_KEYS, t_end = (g_hi + TILE_KEYS - 1) / TILE_KEYS;
+
+    const unsigned short *kp = (const unsigned short *)a.k;
+    const unsigned short *vp = (const unsigned short *)a.v;
+    const size_t kv_row = (size_t)a.Hkv * D;
+    const size_t kv_base = ((size_t)b * a.T * a.Hkv + hk) * D;
+    const int key_clamp_hi = g_hi - 1;
+
+    // ---- cooperative tile loads: registers now, LDS after the current tile's MFMAs
+    u32x4 kreg[NKL], vreg[NVL][2];
+    auto load_tile = [&](int t) {
+        const int key0 = t * TILE_KEYS;
+#pragma unroll
+        for (int i = 0; i < NKL; ++i) {
+            const int id = tid + 256 * i, key = id / CPK, c = id % CPK;
+            const int kabs = min(max(key0 + key, g_lo), key_clamp_hi);
+            kreg[i] = *(const u32x4 *)(kp + kv_base + (size_t)kabs * kv_row + c * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < NVL; ++i) {
+            const int id = min(tid + 256 * i, V_ITEMS - 1), pair = id & 15, c = id >> 4;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                // keys outside the union are read from a clamped in-range key: their probabilities are exact zeros
+                const int kabs = min(max(key0 + pair * 2 + h, g_lo), key_clamp_hi);
+                vreg[i][h] = *(const u32x4 *)(vp + kv_base + (size_t)kabs * kv_row + c * 8);
+            }
+        }
+    };
+    auto store_tile = [&](unsigned char *st) {
+#pragma unroll
+        for (int i = 0; i < NKL; ++i) {
+            const int id = tid + 256 * i, key = id / CPK, c = id % CPK;
+            *(u32x4 *)(st + key * Cfg::KROW + c * 16) = kreg[i];
+        }
+#pragma unroll
+        for (int i = 0; i < NVL; ++i) {
+            const int id = tid + 256 * i, pair = id & 15, c = id >> 4;
+            if (V_ITEMS < 256 && id >= V_ITEMS) continue;
+            unsigned char *vt = st + Cfg::K_BYTES + (c * 8) * PF_VROW + pair * 4;
+            const u32x4 x = vreg[i][0], y = vreg[i][1];
+            const unsigned xs[4] = {x.x, x.y, x.z, x.w}, ys[4] = {y.x, y.y, y.z, y.w};
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                *(unsigned *)(vt + (2 * w) * PF_VROW) = (xs[w] & 0xFFFFu) | (ys[w] << 16);
+                *(unsigned *)(vt + (2 * w + 1) * PF_VROW) = (xs[w] >> 16) | (ys[w] & 0xFFFF0000u);
+            }
+        }
+    };
+
+    f32x16 acc[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[j][i] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+    const float cap_inv = CAP ? 1.f / a.soft_cap : 0.f;
+
+    load_tile(t_begin);
+    store_tile(lds);
+    __syncthreads();
+
+    const int k_off = l31 * Cfg::KROW + lh * 16;                    // + kk * 32
+    const int v_off = Cfg::K_BYTES + l31 * PF_VROW + lh * 8;        // + j * 32 rows + step * 32 bytes (+16 for the second 4 keys)
+    for (int t = t_begin; t < t_end; ++t) {
+        const unsigned char *st = lds + ((t - t_begin) & 1) * Cfg::STAGE;
+        unsigned char *nx = lds + ((t - t_begin + 1) & 1) * Cfg::STAGE;
+        const bool more = t + 1 < t_end;
+        if (more) load_tile(t + 1);
+        const int key0 = t * TILE_KEYS;
+        const bool mine = key0 < w_hi && key0 + TILE_KEYS > w_lo;       // wavefront-uniform
+        if (mine) {
+            // -- S^T = K . Q^T, two accumulation chains
+            f32x16 s0, s1;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { s0[i] = 0.f; s1[i] = 0.f; }
+#pragma unroll
+            for (int kk = 0; kk < KK; kk += 2) {
+                const u32x4 k0 = *(const u32x4 *)(st + k_off + kk * 32);
+                const u32x4 k1 = *(const u32x4 *)(st + k_off + (kk + 1) * 32);
+                s0 = mfma32<KV>(k0, qf[kk], s0);
+                s1 = mfma32<KV>(k1, qf[kk + 1], s1);
+            }
+            // -- lane holds keys key0 + (i/4)*8 + lh*4 + i%4 of row l31
+            float x[16];
+            const bool full = key0 >= w_lo_max && key0 + TILE_KEYS <= w_hi_min;   // every key visible to every row
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                float v = (s0[i] + s1[i]) * a.scale;
+                if (CAP) v = a.soft_cap * tanhf(v * cap_inv);
+                x[i] = v;
+            }
+            if (!full) {                                                          // wavefront-uniform
+                const int kb = key0 + lh * 4;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int key = kb + (i >> 2) * 8 + (i & 3);
+                    x[i] = (key >= lo && key < hi) ? x[i] : -INFINITY;
+                }
+            }
+            float mx = x[0];
+#pragma unroll
+            for (int i = 1; i < 16; ++i) mx = fmaxf(mx, x[i]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            // the reference maximum only moves when the tile's maximum exceeds it by more than PF_LAZY:
+            // probabilities stay below e^PF_LAZY (exact in the f32 sums, fine in the 16-bit operand) and the
+            // 2*D-register rescale of the accumulators becomes rare after the first tiles
+            const float m_new = mx > m_run + PF_LAZY ? mx : m_run;
+            float alpha = 1.f, rowsum = 0.f;
+            if (m_new > -INFINITY) {
+                alpha = m_run > -INFINITY ? __builtin_amdgcn_exp2f((m_run - m_new) * LOG2E) : 1.f;
+                const float mneg = -m_new * LOG2E;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    x[i] = __builtin_amdgcn_exp2f(fmaf(x[i], LOG2E, mneg));      // exp2(-inf) = 0 for masked keys
+                    rowsum += x[i];
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) x[i] = 0.f;
+            }
+            rowsum += __shfl_xor(rowsum, 32, 64);
+            l_run = l_run * alpha + rowsum;
+            m_run = m_new;
+            // P^T operand of 16-key step s2: slots 0..7 <- accumulator elements 8*s2 .. 8*s2+7
+            u32x4 pf[2];
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2)
+                pf[s2] = u32x4{pack2<KV>(x[8 * s2], x[8 * s2 + 1]), pack2<KV>(x[8 * s2 + 2], x[8 * s2 + 3]),
+                               pack2<KV>(x[8 * s2 + 4], x[8 * s2 + 5]), pack2<KV>(x[8 * s2 + 6], x[8 * s2 + 7])};
+            // -- O^T += V^T . P^T
+            if (__any(alpha != 1.f)) {              // wavefront-uniform and rare: must stay a branch, not a select
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) acc[j] *= alpha;
+            }
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                f32x16 c = acc[j];
+#pragma unroll
+                for (int s2 = 0; s2 < 2; ++s2) {
+                    const unsigned char *vrow = st + v_off + j * 32 * PF_VROW + s2 * 32;
+                    const u32x2 va = *(const u32x2 *)(vrow), vb = *(const u32x2 *)(vrow + 16);
+                    c = mfma32<KV>(u32x4{va.x, va.y, vb.x, vb.y}, pf[s2], c);
+                }
+                acc[j] = c;
+            }
+        }
+        if (more) store_tile(nx);
+        __syncthreads();
+    }
+
+    if (row_ok) {
+        const float inv = l_run > 0.f ? 1.f / l_run : 0.f;          // empty interval -> zeros
+        float *o = a.out + qbase;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                const f32x4 v = f32x4{acc[j][q4 * 4], acc[j][q4 * 4 + 1], acc[j][q4 * 4 + 2], acc[j][q4 * 4 + 3]} * inv;
+                *(f32x4 *)(o + j * 32 + q4 * 8 + lh * 4) = v;
+            }
+    }
+}
+
 // log-sum-exp merge of the key segments: one workgroup per (row tile, 16-wide dv slice, unit).
 // Thread = (segment group of 4, row of 16, 4 consecutive dv): it folds every fourth segment with all
 // of a round's loads in flight at once, then the four groups fold through LDS.
@@ -559,10 +825,10 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
     const bool split = a.rows_total <= 64;
     if (split) {
         // key segments: one 32-key tile per wavefront while that leaves the device under-filled,
-        // more tiles per wavefront beyond ~2 workgroups per CU
+        // more tiles per wavefront beyond one workgroup per CU (its LDS tiles fill a CU)
         const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
         const int tiles = (a.T + TILE_KEYS - 1) / TILE_KEYS;
-        int nseg = (2 * cus + units * a.row_tiles - 1) / (units * a.row_tiles);
+        int nseg = (cus + units * a.row_tiles - 1) / (units * a.row_tiles);
         nseg = max(1, min(nseg, (tiles + SPLIT_NW - 1) / SPLIT_NW));
         nseg = min(nseg, 256);
         a.nseg = nseg;
@@ -586,6 +852,21 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
             launch_k(ctx, attn_merge_kernel<D>, dim3((unsigned)(a.row_tiles * (D / MERGE_DV)), (unsigned)units), dim3(256), 0, a);
         }
         LAUNCH_CHECK(ctx, "attn_flash_split");
+    } else if (!HILO) {
+        using PCfg = PrefillCfg<D>;
+        a.nseg = 1;
+        static bool attr_pf[2] = {false, false};
+        const bool cap = a.soft_cap > 0.f;
+        const void *fn = cap ? (const void *)attn_prefill_kernel<KV, D, true> : (const void *)attn_prefill_kernel<KV, D, false>;
+        if (!attr_pf[cap]) {
+            HIP_TRY(ctx, hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, PCfg::LDS_BYTES));
+            attr_pf[cap] = true;
+        }
+        ProfScope scope(ctx, "attn_prefill");
+        const dim3 grid((unsigned)((a.rows_total + PF_ROWS - 1) / PF_ROWS), (unsigned)units);
+        if (cap) launch_k(ctx, attn_prefill_kernel<KV, D, true>, grid, dim3(256), PCfg::LDS_BYTES, a);
+        else launch_k(ctx, attn_prefill_kernel<KV, D, false>, grid, dim3(256), PCfg::LDS_BYTES, a);
+        LAUNCH_CHECK(ctx, "attn_prefill");
     } else {
         a.nseg = 1;
         static bool attr_prefill = false;

@@ -268,7 +268,10 @@ void launch_r(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *c
     batch.total_waves = waves;
     // at most 8 workgroups per CU: beyond that the wavefronts stride over the row groups
     const int wgs = (waves + 3) / 4;
-    const dim3 grid((unsigned)(wgs < cus * 8 ? wgs : cus * 8)), block(256);
+#ifndef FUSED_CAP
+#define FUSED_CAP 8
+#endif
+    const dim3 grid((unsigned)(wgs < cus * FUSED_CAP ? wgs : cus * FUSED_CAP)), block(256);
     const size_t lds = (size_t)K + (size_t)(K >> 5) * 8 + 16;
     if (R == 4) launch_k(ctx, gemv_fused_kernel<DT, 4, PRO, NCH>, grid, block, lds, batch, in, K, alpha, beta);
     else if (R == 2) launch_k(ctx, gemv_fused_kernel<DT, 2, PRO, NCH>, grid, block, lds, batch, in, K, alpha, beta);

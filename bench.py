@@ -276,7 +276,7 @@ def run_attention(gpu, be):
         k = gpu.upload(_bf16_bits(rng.standard_normal((1, L, Hkv, D))))
         v = gpu.upload(_bf16_bits(rng.standard_normal((1, L, Hkv, D))))
         o = gpu.alloc(L * Hq * D * 4)
-        ms = timed(("attn_flash_prefill",), (1, L, L, Hq, Hkv, D, D), (q, k, v, o))
+        ms = timed(("attn_prefill",), (1, L, L, Hq, Hkv, D, D), (q, k, v, o))
         flops = 4.0 * Hq * D * L * (L + 1) / 2
         tf = flops / (ms * 1e-3) / 1e12
         res["prefill L%d" % L] = {"kernel_ms": round(ms, 4), "TFLOPs": round(tf, 1), "frac_mfma_peak": round(tf / MFMA_PEAK["bf16"], 4)}
