@@ -190,6 +190,14 @@ class HipBackend:
         self._check(self._lib.aionhip_step_rope_append(self._ctx, q_out.handle, q.handle, k.handle, v.handle, k_cache.handle, v_cache.handle,
                                                        positions.handle, write_index.handle, b, s, t_cap, h_q, h_kv, d, base, scale_factor, proportion))
 
+    def step_rmsnorm_qkv_rope_append(self, wq, wk, wv, x, gamma, eps, q_out, k_cache, v_cache, positions, write_index,
+                                     t_cap, h_q, h_kv, d, base=10000.0, scale_factor=1.0, proportion=1.0, beta_norm=None):
+        """One new token of one sequence: RMSNorm -> q/k/v matmuls -> RoPE -> f16 cache append, one launch."""
+        self._check(self._lib.aionhip_step_rmsnorm_qkv_rope_append(
+            self._ctx, wq.ptr, wk.ptr, wv.ptr, x.handle, gamma.handle, beta_norm.handle if beta_norm is not None else 0, eps,
+            q_out.handle, k_cache.handle, v_cache.handle, positions.handle, write_index.handle, t_cap, h_q, h_kv, d,
+            base, scale_factor, proportion))
+
     def step_add_i32(self, out, a, b, n):
         self._check(self._lib.aionhip_step_add_i32(self._ctx, out.handle, a.handle, b.handle, n))
 

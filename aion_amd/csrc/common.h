@@ -161,11 +161,23 @@ struct FusedIn {
     const float *x, *y, *gamma, *beta;
     float eps;
 };
+// Optional epilogue of the single-row GEMV. EPI_ROPE_APPEND: the three weights are Wq, Wk, Wv of one
+// attention block; a wavefront owns the rows e..e+3 and e+D/2..e+D/2+3 of one head, i.e. both halves
+// of four RoPE pairs, rotates them (q, k) and writes q as f32 and k, v as f16 rows of the KV cache at
+// the device-resident write index: the q/k/v GEMV, RoPE, the f16 cast and the cache append in one launch.
+enum { EPI_NONE = 0, EPI_ROPE_APPEND = 1 };
+struct FusedEpi {
+    const int *positions, *write_index;
+    const float *freq;
+    __half *k_cache, *v_cache;
+    int t_cap, h_kv, d, rope_pairs;
+};
 constexpr size_t FUSED_MAX_K = 8192;
 // above this K the per-workgroup prologue costs more than a separate preparation launch
 constexpr size_t FUSED_PAYS_K = 4096;
 int launch_gemv_fused(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count,
                       int prologue, FusedIn in, float alpha, float beta);
+int launch_gemv_fused_rope(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *q_out, FusedIn in, FusedEpi epi);
 int launch_rmsnorm(aionhip_ctx *ctx, float *out, const float *x, const float *gamma, const float *beta, const float *residual,
                    size_t rows, size_t cols, float eps);
 int launch_gate_gelu(aionhip_ctx *ctx, float *out, const float *a, const float *b, size_t n);

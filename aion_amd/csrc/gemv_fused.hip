@@ -18,8 +18,9 @@ namespace {
 
 // NCH = float4 activation chunks per thread (K <= 1024 * NCH). LDS is sized per launch:
 // K bytes of codes, K/32 scales, K/32 code sums, 4 reduction slots.
-template <int DT, int R, int PRO, int NCH>
-__global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedIn in, int K, float alpha, float beta) {
+template <int DT, int R, int PRO, int NCH, int EPI>
+__global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedIn in, int K, float alpha, float beta, FusedEpi epi) {
+    static_assert(EPI == EPI_NONE || R == 8, "the RoPE epilogue owns 4 + 4 rows per wavefront");
     extern __shared__ __attribute__((aligned(16))) unsigned char s_mem[];
     int *s_aq = (int *)s_mem;
     float *s_scale = (float *)(s_mem + K);
@@ -41,7 +42,7 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedI
         const u32x4 *qs;
         const __half *sc;
         float *c;
-        int n, row0;
+        int n, row0, seg;
         size_t rowq[R], rows[R];
     };
     auto locate = [&](int gw) {
@@ -54,10 +55,16 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedI
         gr.sc = batch.seg[si].sc;
         gr.c = batch.seg[si].c;
         gr.n = batch.seg[si].n;
+        gr.seg = si;
         gr.row0 = (gw - batch.seg[si].first_wave) * R;
+        if (EPI == EPI_ROPE_APPEND) {
+            // task -> (head, first of four pairs): rows head*D + e0 + {0..3} and head*D + D/2 + e0 + {0..3}
+            const int per_head = epi.d >> 3, task = gw - batch.seg[si].first_wave;
+            gr.row0 = (task / per_head) * epi.d + (task % per_head) * 4;
+        }
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int row = min(gr.row0 + r, gr.n - 1);
+            const int row = EPI == EPI_ROPE_APPEND ? gr.row0 + (r & 3) + (r >> 2) * (epi.d >> 1) : min(gr.row0 + r, gr.n - 1);
             gr.rowq[r] = (size_t)row * chunks;
             gr.rows[r] = (size_t)row * KB;
         }
@@ -227,7 +234,31 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedI
 
 #pragma unroll
         for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
-        if (lane == 0) {
+        if (EPI == EPI_ROPE_APPEND) {
+            // every lane holds all eight sums; lane p < 4 finishes pair p (aion cpu/kernels/rope.zig:20-98,
+            // cpu/exec/cast.zig, cpu/exec/sequence_append.zig:12-104 - the arithmetic of rope_append_kernel)
+            if (lane < 4) {
+                const float xl = alpha * (lane == 0 ? acc[0] : lane == 1 ? acc[1] : lane == 2 ? acc[2] : acc[3 % R]);
+                const float xh = alpha * (lane == 0 ? acc[4 % R] : lane == 1 ? acc[5 % R] : lane == 2 ? acc[6 % R] : acc[7 % R]);
+                const int half = epi.d >> 1;
+                const int head = cur.row0 / epi.d, i = cur.row0 % epi.d + lane;      // i < D/2
+                const bool rot = cur.seg < 2 && i < epi.rope_pairs;
+                float sn = 0.f, cs = 1.f;
+                if (rot) sincosf((float)epi.positions[0] * epi.freq[i], &sn, &cs);
+                const float yl = rot ? xl * cs - xh * sn : xl, yh = rot ? xl * sn + xh * cs : xh;
+                if (cur.seg == 0) {
+                    cur.c[head * epi.d + i] = yl;
+                    cur.c[head * epi.d + half + i] = yh;
+                } else {
+                    const long t = (long)epi.write_index[0];
+                    if (t >= 0 && t < (long)epi.t_cap) {                               // never write outside the cache
+                        __half *dst = (cur.seg == 1 ? epi.k_cache : epi.v_cache) + ((size_t)t * epi.h_kv + head) * epi.d;
+                        dst[i] = __float2half_rn(yl);
+                        dst[half + i] = __float2half_rn(yh);
+                    }
+                }
+            }
+        } else if (lane == 0) {
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 if (cur.row0 + r >= cur.n) break;
@@ -273,9 +304,9 @@ void launch_r(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *c
 #endif
     const dim3 grid((unsigned)(wgs < cus * FUSED_CAP ? wgs : cus * FUSED_CAP)), block(256);
     const size_t lds = (size_t)K + (size_t)(K >> 5) * 8 + 16;
-    if (R == 4) launch_k(ctx, gemv_fused_kernel<DT, 4, PRO, NCH>, grid, block, lds, batch, in, K, alpha, beta);
-    else if (R == 2) launch_k(ctx, gemv_fused_kernel<DT, 2, PRO, NCH>, grid, block, lds, batch, in, K, alpha, beta);
-    else launch_k(ctx, gemv_fused_kernel<DT, 1, PRO, NCH>, grid, block, lds, batch, in, K, alpha, beta);
+    if (R == 4) launch_k(ctx, gemv_fused_kernel<DT, 4, PRO, NCH, EPI_NONE>, grid, block, lds, batch, in, K, alpha, beta, FusedEpi{});
+    else if (R == 2) launch_k(ctx, gemv_fused_kernel<DT, 2, PRO, NCH, EPI_NONE>, grid, block, lds, batch, in, K, alpha, beta, FusedEpi{});
+    else launch_k(ctx, gemv_fused_kernel<DT, 1, PRO, NCH, EPI_NONE>, grid, block, lds, batch, in, K, alpha, beta, FusedEpi{});
 }
 
 template <int DT, int PRO>
@@ -295,7 +326,39 @@ void launch_p(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *c
     else launch_n<DT, PRO_QUANT>(ctx, ws, cs, ldcs, count, in, alpha, beta);
 }
 
+template <int DT, int NCH>
+void launch_rope(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *q_out, FusedIn in, FusedEpi epi) {
+    const int K = (int)ws[0]->k;
+    GemvBatch batch{};
+    batch.count = 3;
+    int waves = 0;
+    for (int i = 0; i < 3; ++i) {
+        batch.seg[i] = GemvSeg{(const u32x4 *)ws[i]->qs, ws[i]->sc, i == 0 ? q_out : nullptr, ws[i]->n, (int)ws[i]->n, waves};
+        waves += (int)ws[i]->n / 8;
+    }
+    batch.total_waves = waves;
+    const dim3 grid((unsigned)((waves + 3) / 4)), block(256);
+    const size_t lds = (size_t)K + (size_t)(K >> 5) * 8 + 16;
+    launch_k(ctx, gemv_fused_kernel<DT, 8, PRO_RMSNORM, NCH, EPI_ROPE_APPEND>, grid, block, lds, batch, in, K, 1.f, 0.f, epi);
+}
+
 }  // namespace
+
+int launch_gemv_fused_rope(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *q_out, FusedIn in, FusedEpi epi) {
+    const bool q8 = ws[0]->dtype == AIONHIP_Q8_0;
+    const char *name = q8 ? "gemv_q8_rmsnorm_rope" : "gemv_q4_rmsnorm_rope";
+    ProfScope scope(ctx, name);
+    const size_t k = ws[0]->k;
+    if (q8) {
+        if (k <= 2048) launch_rope<AIONHIP_Q8_0, 2>(ctx, ws, q_out, in, epi);
+        else launch_rope<AIONHIP_Q8_0, 4>(ctx, ws, q_out, in, epi);
+    } else {
+        if (k <= 2048) launch_rope<AIONHIP_Q4_0, 2>(ctx, ws, q_out, in, epi);
+        else launch_rope<AIONHIP_Q4_0, 4>(ctx, ws, q_out, in, epi);
+    }
+    LAUNCH_CHECK(ctx, name);
+    return AIONHIP_OK;
+}
 
 int launch_gemv_fused(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count, int prologue,
                       FusedIn in, float alpha, float beta) {

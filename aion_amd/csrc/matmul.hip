@@ -6,6 +6,8 @@
 //   m  > 8                                -> gemm_i8_kernel (exact) or gemm_bf16_kernel
 #include "common.h"
 
+#include <cmath>
+
 namespace {
 
 constexpr size_t GEMV_MAX_M = 8;
@@ -126,6 +128,39 @@ int aionhip_step_rmsnorm_matmul(aionhip_ctx *ctx, size_t count, const aionhip_we
     rc = launch_rmsnorm(ctx, h, xp, gp, bp, nullptr, rows, b.k, eps);
     if (rc) return rc;
     return run_rows(ctx, b, rows, h, b.k, alpha, beta);
+}
+
+int aionhip_step_rmsnorm_qkv_rope_append(aionhip_ctx *ctx, const aionhip_weight *wq, const aionhip_weight *wk, const aionhip_weight *wv,
+                                         aionhip_handle x, aionhip_handle gamma, aionhip_handle beta_norm, float eps,
+                                         aionhip_handle q_out, aionhip_handle k_cache, aionhip_handle v_cache,
+                                         aionhip_handle positions, aionhip_handle write_index, size_t t_cap, size_t h_q, size_t h_kv,
+                                         size_t d, float base_frequency, float scale_factor, float rope_proportion) {
+    if (!ctx || !wq || !wk || !wv) return AIONHIP_INVALID_ARGUMENT;
+    if (!x || !gamma || !q_out || !k_cache || !v_cache || !positions || !write_index)
+        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "qkv_rope_append: null operand");
+    if (!(eps > 0.f) || !(eps < INFINITY)) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "qkv_rope_append: eps must be positive and finite");
+    if (!(base_frequency > 0.f) || !(base_frequency < INFINITY) || !(scale_factor > 0.f) || !(scale_factor < INFINITY) ||
+        !(rope_proportion >= 0.f && rope_proportion <= 1.f))
+        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "qkv_rope_append: base/scale must be positive and finite, proportion in [0,1]");
+    const aionhip_weight *ws[3] = {wq, wk, wv};
+    for (const aionhip_weight *w : ws)
+        if (w->k != wq->k || w->dtype != wq->dtype) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "qkv_rope_append: weights must share k and dtype");
+    if (d == 0 || d % 8 != 0 || d > 65528 || h_q == 0 || h_kv == 0 || wq->n != h_q * d || wk->n != h_kv * d || wv->n != h_kv * d)
+        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "qkv_rope_append: weight rows must be heads x head size, head size a multiple of 8");
+    // one token of one sequence, short enough K for the in-kernel prologue: anything else takes the separate steps
+    if (wq->k > FUSED_PAYS_K || ((x | gamma | beta_norm) & 15) || (q_out & 3) || ((k_cache | v_cache) & 1) || t_cap == 0 || t_cap > 0x7FFFFFFFu)
+        return set_err(ctx, AIONHIP_UNSUPPORTED, "qkv_rope_append: needs k <= %zu, 16-byte aligned x/gamma/beta and a cache of 1..2^31-1 tokens", FUSED_PAYS_K);
+    const size_t half = d / 2;
+    size_t rope_pairs = (size_t)floorf(rope_proportion * (float)half);
+    if (rope_pairs > half) rope_pairs = half;
+    const float freq_step = (float)pow((double)base_frequency, (double)(-2.0f / (float)d));
+    const float *freq = nullptr;
+    int rc = rope_table(ctx, (int)rope_pairs, freq_step, scale_factor, &freq);
+    if (rc) return rc;
+    FusedEpi epi{(const int *)(uintptr_t)positions, (const int *)(uintptr_t)write_index, freq, (__half *)(uintptr_t)k_cache,
+                 (__half *)(uintptr_t)v_cache, (int)t_cap, (int)h_kv, (int)d, (int)rope_pairs};
+    FusedIn in{(const float *)(uintptr_t)x, nullptr, (const float *)(uintptr_t)gamma, (const float *)(uintptr_t)beta_norm, eps};
+    return launch_gemv_fused_rope(ctx, ws, (float *)(uintptr_t)q_out, in, epi);
 }
 
 int aionhip_step_gate_matmul(aionhip_ctx *ctx, const aionhip_weight *w, size_t rows, aionhip_handle gate, aionhip_handle up,

@@ -146,12 +146,18 @@ class Decoder:
         scale = 1.0 / math.sqrt(c.head_dim)
         for l in range(c.layers):
             p = "l%d." % l
-            # RMSNorm -> MatMul q, k, v (one call: the norm is not materialised)
-            g.step_rmsnorm_matmul([self.w[p + "wq"], self.w[p + "wk"], self.w[p + "wv"]], b["x"], self.gamma, s,
-                                  [b["q"], b["k"], b["v"]], c.eps)
-            # RoPE1D(q), RoPE1D(k) -> f16 -> append, v -> f16 -> append
-            g.step_rope_append(b["qr"], b["q"], b["k"], b["v"], self.kc[l], self.vc[l], b["positions"], b["write_index"],
-                               1, s, c.max_seq, c.heads, c.kv_heads, c.head_dim, base=c.rope_base)
+            if s == 1 and c.hidden <= 4096 and c.head_dim % 8 == 0:
+                # one new token: RMSNorm -> MatMul q, k, v -> RoPE1D(q), RoPE1D(k) -> f16 -> append, one launch
+                g.step_rmsnorm_qkv_rope_append(self.w[p + "wq"], self.w[p + "wk"], self.w[p + "wv"], b["x"], self.gamma, c.eps,
+                                               b["qr"], self.kc[l], self.vc[l], b["positions"], b["write_index"],
+                                               c.max_seq, c.heads, c.kv_heads, c.head_dim, base=c.rope_base)
+            else:
+                # RMSNorm -> MatMul q, k, v (one call: the norm is not materialised)
+                g.step_rmsnorm_matmul([self.w[p + "wq"], self.w[p + "wk"], self.w[p + "wv"]], b["x"], self.gamma, s,
+                                      [b["q"], b["k"], b["v"]], c.eps)
+                # RoPE1D(q), RoPE1D(k) -> f16 -> append, v -> f16 -> append
+                g.step_rope_append(b["qr"], b["q"], b["k"], b["v"], self.kc[l], self.vc[l], b["positions"], b["write_index"],
+                                   1, s, c.max_seq, c.heads, c.kv_heads, c.head_dim, base=c.rope_base)
             g.step_attention(b["att"], b["qr"], self.kc[l], self.vc[l], (1, s, c.max_seq, c.heads, c.kv_heads, c.head_dim, c.head_dim),
                              scale, q_dtype=be.F32, kv_dtype=be.F16, window=be.CAUSAL,
                              query_positions=b["positions"], kv_lengths=b["kv_len"])

@@ -135,6 +135,18 @@ int aionhip_step_matmul_batch(aionhip_ctx *ctx, size_t count, const aionhip_weig
                               aionhip_handle a, size_t lda, const aionhip_handle *c, const size_t *ldc,
                               float alpha, float beta);
 
+/* Decode fusion of one attention block's input side for ONE new token of ONE sequence: RMSNorm(x) -> the
+ * q, k and v matmuls (StepMatMul x3 on the same activation) -> RoPE on q and k (StepRope, chunked halves,
+ * cpu/kernels/rope.zig:20-98) -> f32->f16 cast and append of k and v at the device-resident write index
+ * (StepSequenceAppend, cpu/exec/sequence_append.zig:12-104), as one launch. q_out receives the rotated
+ * query [h_q, d] f32; the caches are [t_cap, h_kv, d] f16 (batch 1). Same arithmetic as the separate steps
+ * (aionhip_step_rmsnorm_matmul + aionhip_step_rope_append). AIONHIP_UNSUPPORTED when the shape does not
+ * qualify (k above 4096, misaligned operands): the caller then issues the separate steps. */
+int aionhip_step_rmsnorm_qkv_rope_append(aionhip_ctx *ctx, const aionhip_weight *wq, const aionhip_weight *wk, const aionhip_weight *wv,
+                                         aionhip_handle x, aionhip_handle gamma, aionhip_handle beta_norm, float eps,
+                                         aionhip_handle q_out, aionhip_handle k_cache, aionhip_handle v_cache,
+                                         aionhip_handle positions, aionhip_handle write_index, size_t t_cap, size_t h_q, size_t h_kv,
+                                         size_t d, float base_frequency, float scale_factor, float rope_proportion);
 /* StepRMSNorm feeding MatMul steps, and the fused gate feeding a MatMul step, as one call each:
  * the normalised (or gated) activation is not written out; for one row it is built inside the GEMV
  * kernel. Same arithmetic as aionhip_step_rmsnorm / aionhip_step_gate_gelu followed by the matmul

@@ -145,3 +145,50 @@ def test_rope_append_equals_the_separate_steps(gpu, orc):
     assert np.array_equal(gpu.download(kc2, np.float16, want_k.shape), got_k)
     for t in (qb, kb, vb, pb, wb, qo, kc, vc, qo2, kr, kc2):
         t.free()
+
+
+@pytest.mark.parametrize("dtype", ["q4", "q8"])
+@pytest.mark.parametrize("D,Hq,Hkv,K", [(256, 8, 1, 2048), (64, 4, 2, 512)])
+def test_qkv_rope_append_fusion_equals_the_separate_steps(gpu, orc, dtype, D, Hq, Hkv, K):
+    """RMSNorm -> q/k/v matmuls -> RoPE -> f16 append in one launch against the same steps issued one by one
+    (and through them against the oracle, which the separate steps are tested against)."""
+    from aion_amd import backend as be
+    rng = np.random.default_rng(D + K)
+    dt = be.Q4_0 if dtype == "q4" else be.Q8_0
+    ws = []
+    for n in (Hq * D, Hkv * D, Hkv * D):
+        w = (rng.standard_normal((K, n)) * 0.05).astype(np.float32)
+        ws.append(gpu.upload_weight(dt, be.KMAJOR_KN, n, K, be.quantize_blocks(dt, w, 0)))
+    T, widx, pos = 9, 5, 37
+    x = gpu.upload(rng.standard_normal((1, K)).astype(np.float32))
+    gamma = gpu.upload((1 + 0.1 * rng.standard_normal(K)).astype(np.float32))
+    pb, wb = gpu.upload(np.array([[pos]], np.int32)), gpu.upload(np.array([widx], np.int32))
+    # separate steps
+    q, k, v = gpu.alloc(Hq * D * 4), gpu.alloc(Hkv * D * 4), gpu.alloc(Hkv * D * 4)
+    qr = gpu.alloc(Hq * D * 4)
+    kc, vc = gpu.zeros(T * Hkv * D * 2), gpu.zeros(T * Hkv * D * 2)
+    gpu.step_rmsnorm_matmul(ws, x, gamma, 1, [q, k, v], 1e-6)
+    gpu.step_rope_append(qr, q, k, v, kc, vc, pb, wb, 1, 1, T, Hq, Hkv, D, proportion=0.75)
+    # one launch
+    qr2 = gpu.alloc(Hq * D * 4)
+    kc2, vc2 = gpu.zeros(T * Hkv * D * 2), gpu.zeros(T * Hkv * D * 2)
+    gpu.step_rmsnorm_qkv_rope_append(ws[0], ws[1], ws[2], x, gamma, 1e-6, qr2, kc2, vc2, pb, wb, T, Hq, Hkv, D, proportion=0.75)
+    assert gpu.last_kernel() == "gemv_%s_rmsnorm_rope" % dtype
+    a, b2 = gpu.download(qr, np.float32, (Hq, D)), gpu.download(qr2, np.float32, (Hq, D))
+    # same integer dots and scales; only the f32 summation order over lanes differs between 1 and 8 rows per wavefront
+    assert np.abs(a - b2).max() <= 1e-5 * np.sqrt((a ** 2).mean())
+    ka, kb2 = gpu.download(kc, np.float16, (T, Hkv, D)), gpu.download(kc2, np.float16, (T, Hkv, D))
+    va, vb2 = gpu.download(vc, np.float16, (T, Hkv, D)), gpu.download(vc2, np.float16, (T, Hkv, D))
+    assert np.abs(ka.astype(np.float32) - kb2.astype(np.float32)).max() <= 2e-3 * max(1.0, np.abs(ka.astype(np.float32)).max())
+    assert np.abs(va.astype(np.float32) - vb2.astype(np.float32)).max() <= 2e-3 * max(1.0, np.abs(va.astype(np.float32)).max())
+    assert not kb2[:widx].any() and not kb2[widx + 1:].any() and kb2[widx].any()
+    assert not vb2[:widx].any() and not vb2[widx + 1:].any() and vb2[widx].any()
+    # a write index outside the cache writes nothing
+    wb_bad = gpu.upload(np.array([T], np.int32))
+    kc3, vc3 = gpu.zeros(T * Hkv * D * 2), gpu.zeros(T * Hkv * D * 2)
+    gpu.step_rmsnorm_qkv_rope_append(ws[0], ws[1], ws[2], x, gamma, 1e-6, qr2, kc3, vc3, pb, wb_bad, T, Hq, Hkv, D)
+    assert not gpu.download(kc3, np.float16, (T, Hkv, D)).any() and not gpu.download(vc3, np.float16, (T, Hkv, D)).any()
+    for t in (x, gamma, pb, wb, wb_bad, q, k, v, qr, kc, vc, qr2, kc2, vc2, kc3, vc3):
+        t.free()
+    for w in ws:
+        w.free()
