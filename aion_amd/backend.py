@@ -198,6 +198,12 @@ class HipBackend:
             q_out.handle, k_cache.handle, v_cache.handle, positions.handle, write_index.handle, t_cap, h_q, h_kv, d,
             base, scale_factor, proportion))
 
+    def step_rmsnorm_geglu_matmul(self, w_gate, w_up, w_down, x, gamma, eps, c_buf, alpha=1.0, beta=0.0, beta_norm=None):
+        """One activation row: RMSNorm -> gate/up matmuls -> gelu gate -> down matmul, two launches."""
+        self._check(self._lib.aionhip_step_rmsnorm_geglu_matmul(
+            self._ctx, w_gate.ptr, w_up.ptr, w_down.ptr, x.handle, gamma.handle, beta_norm.handle if beta_norm is not None else 0, eps,
+            c_buf.handle, alpha, beta))
+
     def step_add_i32(self, out, a, b, n):
         self._check(self._lib.aionhip_step_add_i32(self._ctx, out.handle, a.handle, b.handle, n))
 

@@ -165,12 +165,19 @@ struct FusedIn {
 // attention block; a wavefront owns the rows e..e+3 and e+D/2..e+D/2+3 of one head, i.e. both halves
 // of four RoPE pairs, rotates them (q, k) and writes q as f32 and k, v as f16 rows of the KV cache at
 // the device-resident write index: the q/k/v GEMV, RoPE, the f16 cast and the cache append in one launch.
-enum { EPI_NONE = 0, EPI_ROPE_APPEND = 1 };
+// EPI_GATE_QUANT: the two weights are the gate and up projections of a GeGLU block; a workgroup owns 32
+// consecutive outputs j of both (a wavefront: rows j..j+3 of each, twice), forms h_j = gelu_tanh(g_j) * u_j
+// and writes the block's int8 activation preparation (codes, scale, code sum) for the down projection:
+// neither g, u nor h goes to memory and no separate gate / preparation launch is needed.
+enum { EPI_NONE = 0, EPI_ROPE_APPEND = 1, EPI_GATE_QUANT = 2 };
 struct FusedEpi {
     const int *positions, *write_index;
     const float *freq;
     __half *k_cache, *v_cache;
     int t_cap, h_kv, d, rope_pairs;
+    int *act_q;          // EPI_GATE_QUANT: prepared activation planes of the down projection
+    float *act_scale;
+    int *act_sum;
 };
 constexpr size_t FUSED_MAX_K = 8192;
 // above this K the per-workgroup prologue costs more than a separate preparation launch
@@ -178,6 +185,7 @@ constexpr size_t FUSED_PAYS_K = 4096;
 int launch_gemv_fused(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count,
                       int prologue, FusedIn in, float alpha, float beta);
 int launch_gemv_fused_rope(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *q_out, FusedIn in, FusedEpi epi);
+int launch_gemv_fused_geglu(aionhip_ctx *ctx, const aionhip_weight *gate, const aionhip_weight *up, FusedIn in, PreparedAct out);
 int launch_rmsnorm(aionhip_ctx *ctx, float *out, const float *x, const float *gamma, const float *beta, const float *residual,
                    size_t rows, size_t cols, float eps);
 int launch_gate_gelu(aionhip_ctx *ctx, float *out, const float *a, const float *b, size_t n);

@@ -20,7 +20,7 @@ namespace {
 // K bytes of codes, K/32 scales, K/32 code sums, 4 reduction slots.
 template <int DT, int R, int PRO, int NCH, int EPI>
 __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedIn in, int K, float alpha, float beta, FusedEpi epi) {
-    static_assert(EPI == EPI_NONE || R == 8, "the RoPE epilogue owns 4 + 4 rows per wavefront");
+    static_assert(EPI == EPI_NONE || R == 8, "the epilogues own 4 + 4 rows per wavefront");
     extern __shared__ __attribute__((aligned(16))) unsigned char s_mem[];
     int *s_aq = (int *)s_mem;
     float *s_scale = (float *)(s_mem + K);
@@ -32,15 +32,15 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedI
     const int wave_stride = gridDim.x * 4;
     // the wavefront index is uniform: read through a scalar, the row-group bookkeeping and the
     // base addresses then stay in scalar registers
-    int gwave = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(tid >> 6);
+    int gwave = blockIdx.x * (EPI == EPI_GATE_QUANT ? 8 : 4) + __builtin_amdgcn_readfirstlane(tid >> 6);
     const int KB = K >> 5;
     constexpr bool Q8 = DT == AIONHIP_Q8_0;
     const int chunks = Q8 ? (K >> 4) : KB;
 
     // the row group of wavefront index `gw`: segment, first row, row offsets
     struct Group {
-        const u32x4 *qs;
-        const __half *sc;
+        const u32x4 *qs, *qs2;      // qs2 / sc2: rows 4..7 of a gate/up group come from the second weight
+        const __half *sc, *sc2;
         float *c;
         int n, row0, seg;
         size_t rowq[R], rows[R];
@@ -51,8 +51,8 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedI
 #pragma unroll
         for (int i = 1; i < 4; ++i)
             if (i < batch.count && gw >= batch.seg[i].first_wave) si = i;
-        gr.qs = batch.seg[si].qs;
-        gr.sc = batch.seg[si].sc;
+        gr.qs = gr.qs2 = batch.seg[si].qs;
+        gr.sc = gr.sc2 = batch.seg[si].sc;
         gr.c = batch.seg[si].c;
         gr.n = batch.seg[si].n;
         gr.seg = si;
@@ -62,9 +62,19 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedI
             const int per_head = epi.d >> 3, task = gw - batch.seg[si].first_wave;
             gr.row0 = (task / per_head) * epi.d + (task % per_head) * 4;
         }
+        if (EPI == EPI_GATE_QUANT) {
+            // gw = (task * 2 + sub) * 4 + wavefront: outputs j0 .. j0+3 of the gate (rows 0..3) and the up weight (rows 4..7)
+            gr.row0 = (gw >> 2) * 16 + (gw & 3) * 4;
+            gr.qs = batch.seg[0].qs;
+            gr.sc = batch.seg[0].sc;
+            gr.qs2 = batch.seg[1].qs;
+            gr.sc2 = batch.seg[1].sc;
+        }
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int row = EPI == EPI_ROPE_APPEND ? gr.row0 + (r & 3) + (r >> 2) * (epi.d >> 1) : min(gr.row0 + r, gr.n - 1);
+            const int row = EPI == EPI_ROPE_APPEND ? gr.row0 + (r & 3) + (r >> 2) * (epi.d >> 1)
+                          : EPI == EPI_GATE_QUANT ? gr.row0 + (r & 3)
+                          : min(gr.row0 + r, gr.n - 1);
             gr.rowq[r] = (size_t)row * chunks;
             gr.rows[r] = (size_t)row * KB;
         }
@@ -97,8 +107,8 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedI
     const int l0 = min(lane, chunks - 1);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        w0[r] = __builtin_nontemporal_load(cur.qs + cur.rowq[r] + l0);
-        hs0[r] = cur.sc[cur.rows[r] + (Q8 ? (l0 >> 1) : l0)];
+        w0[r] = __builtin_nontemporal_load((EPI == EPI_GATE_QUANT && r >= 4 ? cur.qs2 : cur.qs) + cur.rowq[r] + l0);
+        hs0[r] = (EPI == EPI_GATE_QUANT && r >= 4 ? cur.sc2 : cur.sc)[cur.rows[r] + (Q8 ? (l0 >> 1) : l0)];
     }
 
     float ss = 0.f;
@@ -217,8 +227,8 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedI
                 const int ch = min(ch0 + 64 * u, chunks - 1);
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
-                    w[u][r] = __builtin_nontemporal_load(cur.qs + cur.rowq[r] + ch);
-                    hs[u][r] = cur.sc[cur.rows[r] + (Q8 ? (ch >> 1) : ch)];
+                    w[u][r] = __builtin_nontemporal_load((EPI == EPI_GATE_QUANT && r >= 4 ? cur.qs2 : cur.qs) + cur.rowq[r] + ch);
+                    hs[u][r] = (EPI == EPI_GATE_QUANT && r >= 4 ? cur.sc2 : cur.sc)[cur.rows[r] + (Q8 ? (ch >> 1) : ch)];
                 }
             }
 #pragma unroll
@@ -258,6 +268,47 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedI
                     }
                 }
             }
+        } else if (EPI == EPI_GATE_QUANT) {
+            // lanes 0..3: h_j; after the second 16 outputs the workgroup's 32 values are one quant block
+            float *s_h = s_red + 4;
+            if (lane < 4) {
+                const float gv = alpha * (lane == 0 ? acc[0] : lane == 1 ? acc[1] : lane == 2 ? acc[2] : acc[3 % R]);
+                const float uv = alpha * (lane == 0 ? acc[4 % R] : lane == 1 ? acc[5 % R] : lane == 2 ? acc[6 % R] : acc[7 % R]);
+                s_h[(cur.row0 & 31) + lane] = aion_gate_gelu(gv, uv);       // row0 & 31 = sub * 16 + wavefront * 4
+            }
+            if ((gwave >> 2) & 1) {
+                __syncthreads();
+                if (tid < 8) {
+                    // the arithmetic of prepare_act_kernel (aion cpu/kernels/matmul_q_i8.zig:187-203), 8 lanes x 4 values
+                    const float v0 = s_h[tid * 4], v1 = s_h[tid * 4 + 1], v2 = s_h[tid * 4 + 2], v3 = s_h[tid * 4 + 3];
+                    float amax = fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3)));
+                    amax = fmaxf(amax, dpp_f<DPP_QUAD_XOR1>(amax));
+                    amax = fmaxf(amax, dpp_f<DPP_QUAD_XOR2>(amax));
+                    amax = fmaxf(amax, dpp_f<DPP_ROW_HALF_MIRROR>(amax));
+                    int word = 0, sq = 0;
+                    float scale = 0.f;
+                    if (amax != 0.f) {
+                        scale = amax / 127.f;
+                        const float inv = 127.f / amax;
+                        const int q0 = (int)fminf(127.f, fmaxf(-127.f, roundf(v0 * inv)));
+                        const int q1 = (int)fminf(127.f, fmaxf(-127.f, roundf(v1 * inv)));
+                        const int q2 = (int)fminf(127.f, fmaxf(-127.f, roundf(v2 * inv)));
+                        const int q3 = (int)fminf(127.f, fmaxf(-127.f, roundf(v3 * inv)));
+                        word = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
+                        sq = q0 + q1 + q2 + q3;
+                    }
+                    sq += dpp_i<DPP_QUAD_XOR1>(sq);
+                    sq += dpp_i<DPP_QUAD_XOR2>(sq);
+                    sq += dpp_i<DPP_ROW_HALF_MIRROR>(sq);
+                    const int blk = gwave >> 3;                     // task = quant block of the down projection's activation
+                    epi.act_q[blk * 8 + tid] = word;
+                    if (tid == 0) {
+                        epi.act_scale[blk] = scale;
+                        epi.act_sum[blk] = sq;
+                    }
+                }
+                __syncthreads();                                    // s_h is reused by the next task
+            }
         } else if (lane == 0) {
 #pragma unroll
             for (int r = 0; r < R; ++r) {
@@ -266,14 +317,15 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedI
                 cur.c[cur.row0 + r] = beta == 0.f ? val : val + beta * cur.c[cur.row0 + r];
             }
         }
-        gwave += wave_stride;
+        if (EPI == EPI_GATE_QUANT) gwave = ((gwave >> 2) & 1) ? gwave - 4 + 8 * (int)gridDim.x : gwave + 4;
+        else gwave += wave_stride;
         active = gwave < batch.total_waves;
         if (active) {
             cur = locate(gwave);
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                w0[r] = __builtin_nontemporal_load(cur.qs + cur.rowq[r] + l0);
-                hs0[r] = cur.sc[cur.rows[r] + (Q8 ? (l0 >> 1) : l0)];
+                w0[r] = __builtin_nontemporal_load((EPI == EPI_GATE_QUANT && r >= 4 ? cur.qs2 : cur.qs) + cur.rowq[r] + l0);
+                hs0[r] = (EPI == EPI_GATE_QUANT && r >= 4 ? cur.sc2 : cur.sc)[cur.rows[r] + (Q8 ? (l0 >> 1) : l0)];
             }
         }
     }
@@ -342,7 +394,41 @@ void launch_rope(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *q_out
     launch_k(ctx, gemv_fused_kernel<DT, 8, PRO_RMSNORM, NCH, EPI_ROPE_APPEND>, grid, block, lds, batch, in, K, 1.f, 0.f, epi);
 }
 
+template <int DT, int NCH>
+void launch_geglu(aionhip_ctx *ctx, const aionhip_weight *gate, const aionhip_weight *up, FusedIn in, PreparedAct out) {
+    const int K = (int)gate->k, tasks = (int)gate->n / 32;
+    GemvBatch batch{};
+    batch.count = 2;
+    batch.seg[0] = GemvSeg{(const u32x4 *)gate->qs, gate->sc, nullptr, gate->n, (int)gate->n, 0};
+    batch.seg[1] = GemvSeg{(const u32x4 *)up->qs, up->sc, nullptr, up->n, (int)up->n, 0};
+    batch.total_waves = tasks * 8;
+    const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
+    const dim3 grid((unsigned)(tasks < cus * 8 ? tasks : cus * 8)), block(256);
+    const size_t lds = (size_t)K + (size_t)(K >> 5) * 8 + 16 + 32 * sizeof(float);
+    FusedEpi epi{};
+    epi.act_q = (int *)out.q;
+    epi.act_scale = out.scale;
+    epi.act_sum = out.sum;
+    launch_k(ctx, gemv_fused_kernel<DT, 8, PRO_RMSNORM, NCH, EPI_GATE_QUANT>, grid, block, lds, batch, in, K, 1.f, 0.f, epi);
+}
+
 }  // namespace
+
+int launch_gemv_fused_geglu(aionhip_ctx *ctx, const aionhip_weight *gate, const aionhip_weight *up, FusedIn in, PreparedAct out) {
+    const bool q8 = gate->dtype == AIONHIP_Q8_0;
+    const char *name = q8 ? "gemv_q8_rmsnorm_geglu" : "gemv_q4_rmsnorm_geglu";
+    ProfScope scope(ctx, name);
+    const size_t k = gate->k;
+    if (q8) {
+        if (k <= 2048) launch_geglu<AIONHIP_Q8_0, 2>(ctx, gate, up, in, out);
+        else launch_geglu<AIONHIP_Q8_0, 4>(ctx, gate, up, in, out);
+    } else {
+        if (k <= 2048) launch_geglu<AIONHIP_Q4_0, 2>(ctx, gate, up, in, out);
+        else launch_geglu<AIONHIP_Q4_0, 4>(ctx, gate, up, in, out);
+    }
+    LAUNCH_CHECK(ctx, name);
+    return AIONHIP_OK;
+}
 
 int launch_gemv_fused_rope(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *q_out, FusedIn in, FusedEpi epi) {
     const bool q8 = ws[0]->dtype == AIONHIP_Q8_0;

@@ -163,6 +163,28 @@ int aionhip_step_rmsnorm_qkv_rope_append(aionhip_ctx *ctx, const aionhip_weight 
     return launch_gemv_fused_rope(ctx, ws, (float *)(uintptr_t)q_out, in, epi);
 }
 
+int aionhip_step_rmsnorm_geglu_matmul(aionhip_ctx *ctx, const aionhip_weight *w_gate, const aionhip_weight *w_up, const aionhip_weight *w_down,
+                                      aionhip_handle x, aionhip_handle gamma, aionhip_handle beta_norm, float eps,
+                                      aionhip_handle c, float alpha, float beta) {
+    if (!ctx || !w_gate || !w_up || !w_down) return AIONHIP_INVALID_ARGUMENT;
+    if (!x || !gamma || !c) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "geglu_matmul: null operand");
+    if (!(eps > 0.f) || !(eps < INFINITY)) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "geglu_matmul: eps must be positive and finite");
+    if (w_gate->k != w_up->k || w_gate->n != w_up->n || w_gate->dtype != w_up->dtype || w_down->k != w_gate->n)
+        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "geglu_matmul: gate and up must match, down must take their outputs");
+    if (c & 3) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "geglu_matmul: C not 4-byte aligned");
+    if (w_gate->k > FUSED_PAYS_K || w_gate->n % 32 != 0 || ((x | gamma | beta_norm) & 15))
+        return set_err(ctx, AIONHIP_UNSUPPORTED, "geglu_matmul: needs k <= %zu, a hidden size that is a multiple of 32 and 16-byte aligned x/gamma/beta", FUSED_PAYS_K);
+    int rc = ensure_scratch(ctx, prepared_act_bytes(1, w_down->k));
+    if (rc) return rc;
+    PreparedAct act = prepared_act_carve(ctx->scratch, 1, w_down->k);
+    FusedIn in{(const float *)(uintptr_t)x, nullptr, (const float *)(uintptr_t)gamma, (const float *)(uintptr_t)beta_norm, eps};
+    rc = launch_gemv_fused_geglu(ctx, w_gate, w_up, in, act);
+    if (rc) return rc;
+    float *cp = (float *)(uintptr_t)c;
+    const size_t ldc = w_down->n;
+    return launch_gemv_batch(ctx, &w_down, &cp, &ldc, 1, 1, act, alpha, beta);
+}
+
 int aionhip_step_gate_matmul(aionhip_ctx *ctx, const aionhip_weight *w, size_t rows, aionhip_handle gate, aionhip_handle up,
                              aionhip_handle c, size_t ldc, float alpha, float beta) {
     if (!ctx || !w) return AIONHIP_INVALID_ARGUMENT;

@@ -163,9 +163,14 @@ class Decoder:
                              query_positions=b["positions"], kv_lengths=b["kv_len"])
             # MatMul o with beta = 1: x = x + att @ Wo (the residual add rides on the matmul's beta)
             g.step_matmul(self.w[p + "wo"], b["att"], s, b["x"], beta=1.0)
-            g.step_rmsnorm_matmul([self.w[p + "wgate"], self.w[p + "wup"]], b["x"], self.gamma, s, [b["gate"], b["up"]], c.eps)
-            # gate(gelu) -> MatMul down, beta = 1
-            g.step_gate_matmul(self.w[p + "wdown"], b["gate"], b["up"], s, b["x"], beta=1.0)
+            if s == 1 and c.hidden <= 4096 and c.ffn % 32 == 0:
+                # one row: RMSNorm -> MatMul gate, up -> gate(gelu) -> MatMul down (beta = 1), two launches
+                g.step_rmsnorm_geglu_matmul(self.w[p + "wgate"], self.w[p + "wup"], self.w[p + "wdown"], b["x"], self.gamma, c.eps,
+                                            b["x"], beta=1.0)
+            else:
+                g.step_rmsnorm_matmul([self.w[p + "wgate"], self.w[p + "wup"]], b["x"], self.gamma, s, [b["gate"], b["up"]], c.eps)
+                # gate(gelu) -> MatMul down, beta = 1
+                g.step_gate_matmul(self.w[p + "wdown"], b["gate"], b["up"], s, b["x"], beta=1.0)
         last = b["x"].view((s - 1) * c.hidden * 4)
         g.step_rmsnorm_matmul([self.w["lm_head"]], last, self.gamma, 1, [self.logits], c.eps)
         g.step_argmax(self.token, self.logits, 1, c.vocab)

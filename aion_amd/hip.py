@@ -58,6 +58,8 @@ _SIGS = {
     "aionhip_step_rmsnorm_qkv_rope_append": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_float,
                                                        C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_size_t, C.c_size_t, C.c_size_t,
                                                        C.c_size_t, C.c_float, C.c_float, C.c_float]),
+    "aionhip_step_rmsnorm_geglu_matmul": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_float,
+                                                    C.c_uint64, C.c_float, C.c_float]),
     "aionhip_step_gate_matmul": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint64, C.c_uint64, C.c_uint64, C.c_size_t, C.c_float, C.c_float]),
     "aionhip_step_rope_append": (C.c_int, [C.c_void_p] + [C.c_uint64] * 8 + [C.c_size_t] * 6 + [C.c_float] * 3),
     "aionhip_step_add_i32": (C.c_int, [C.c_void_p] + [C.c_uint64] * 3 + [C.c_size_t]),

@@ -147,6 +147,14 @@ int aionhip_step_rmsnorm_qkv_rope_append(aionhip_ctx *ctx, const aionhip_weight 
                                          aionhip_handle q_out, aionhip_handle k_cache, aionhip_handle v_cache,
                                          aionhip_handle positions, aionhip_handle write_index, size_t t_cap, size_t h_q, size_t h_kv,
                                          size_t d, float base_frequency, float scale_factor, float rope_proportion);
+/* Decode fusion of a GeGLU feed-forward block for ONE activation row: RMSNorm(x) -> gate and up matmuls ->
+ * gate(gelu_tanh) * up (cpu/exec/elementwise.zig:25-37) -> int8 activation preparation -> down matmul,
+ * C[1, n_down] = alpha * (...) + beta * C, in two launches; the gate / up / gated rows never reach memory.
+ * Same arithmetic as aionhip_step_rmsnorm_matmul + aionhip_step_gate_matmul. AIONHIP_UNSUPPORTED when the
+ * shape does not qualify (k above 4096, hidden size not a multiple of 32, misaligned operands). */
+int aionhip_step_rmsnorm_geglu_matmul(aionhip_ctx *ctx, const aionhip_weight *w_gate, const aionhip_weight *w_up, const aionhip_weight *w_down,
+                                      aionhip_handle x, aionhip_handle gamma, aionhip_handle beta_norm, float eps,
+                                      aionhip_handle c, float alpha, float beta);
 /* StepRMSNorm feeding MatMul steps, and the fused gate feeding a MatMul step, as one call each:
  * the normalised (or gated) activation is not written out; for one row it is built inside the GEMV
  * kernel. Same arithmetic as aionhip_step_rmsnorm / aionhip_step_gate_gelu followed by the matmul

@@ -192,3 +192,30 @@ def test_qkv_rope_append_fusion_equals_the_separate_steps(gpu, orc, dtype, D, Hq
         t.free()
     for w in ws:
         w.free()
+
+
+@pytest.mark.parametrize("dtype", ["q4", "q8"])
+@pytest.mark.parametrize("K,F", [(2048, 8192), (256, 96), (4096, 1024)])
+def test_geglu_fusion_equals_the_separate_steps(gpu, orc, dtype, K, F):
+    """RMSNorm -> gate/up matmuls -> gelu gate -> int8 preparation -> down matmul in two launches against the
+    separate steps: the prepared codes are the same integers, so the result is the same up to f32 summation order."""
+    from aion_amd import backend as be
+    rng = np.random.default_rng(K + F)
+    dt = be.Q4_0 if dtype == "q4" else be.Q8_0
+    mk = lambda n, k: gpu.upload_weight(dt, be.KMAJOR_KN, n, k, be.quantize_blocks(dt, (rng.standard_normal((k, n)) * 0.05).astype(np.float32), 0))
+    wg, wu, wd = mk(F, K), mk(F, K), mk(K, F)
+    xv = rng.standard_normal((1, K)).astype(np.float32)
+    gamma = gpu.upload((1 + 0.1 * rng.standard_normal(K)).astype(np.float32))
+    x1, x2 = gpu.upload(xv), gpu.upload(xv)
+    g, u = gpu.alloc(F * 4), gpu.alloc(F * 4)
+    gpu.step_rmsnorm_matmul([wg, wu], x1, gamma, 1, [g, u], 1e-6)
+    gpu.step_gate_matmul(wd, g, u, 1, x1, beta=1.0)
+    gpu.step_rmsnorm_geglu_matmul(wg, wu, wd, x2, gamma, 1e-6, x2, beta=1.0)
+    assert gpu.last_kernel() == "gemv_%s" % dtype
+    a, b2 = gpu.download(x1, np.float32, (K,)), gpu.download(x2, np.float32, (K,))
+    # an f32 rounding difference in g or u can flip one int8 code of h: allow that much and no more
+    assert np.abs(a - b2).max() <= 2e-3 * np.sqrt((a ** 2).mean())
+    for t in (gamma, x1, x2, g, u):
+        t.free()
+    for w in (wg, wu, wd):
+        w.free()
