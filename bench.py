@@ -15,7 +15,7 @@ cpu_baseline = the oracle's restatement of the aion CPU kernel for this op (pack
 M=1, aion cpu/exec/matmul.zig) timed on this host's cores on a bounded sample.
 
 `--sweep` adds the q8 legs and batch 4 / 8 (per-shape kernel GB/s) in a "sweep" object.
-`--extras gemm,attention,decoder` adds the other BASELINE configs (prefill GEMM TFLOP/s, attention
+`--extras gemm,attention,decoder[,decoder_eager]` adds the other BASELINE configs (prefill GEMM TFLOP/s, attention
 TFLOP/s and GB/s, end-to-end decode tokens/s of the synthetic 26-layer decoder) in an "extras"
 object of the same JSON line.
 """
@@ -173,6 +173,8 @@ def main():
             out["extras"]["attention"] = run_attention(gpu, be)
         if "decoder" in extras:
             out["extras"]["decoder"] = run_decoder(gpu, be, with_cpu=not args.no_cpu)
+        if "decoder_eager" in extras:
+            out["extras"]["decoder_eager"] = run_decoder_eager(gpu, be)
 
     out["config"]["setup_s"] = round(setup_s, 1)
     print(json.dumps(out))
@@ -268,8 +270,16 @@ def run_attention(gpu, be):
         for _ in range(iters):
             gpu.step_attention(bufs[3], bufs[0], bufs[1], bufs[2], shape, 1 / 16.0, q_dtype=be.BF16, kv_dtype=be.BF16,
                                query_positions=pos, kv_lengths=kl)
-        prof = [ms for (nm, ms) in gpu.profile_stop() if nm in name]
-        return sum(prof) / iters
+        prof = gpu.profile_stop()
+        # per call: the sum of its kernels (split + merge); median over calls (the first call of a kernel
+        # shape may still carry one-time set-up)
+        per_call = []
+        for i in range(iters):
+            per_call.append(0.0)
+        kernels = [ms for (nm, ms) in prof if nm in name]
+        per = len(kernels) // iters
+        per_call = sorted(sum(kernels[i * per:(i + 1) * per]) for i in range(iters))
+        return per_call[iters // 2]
 
     for L in (1024, 4096):
         q = gpu.upload(_bf16_bits(rng.standard_normal((1, L, Hq, D))))
@@ -297,6 +307,22 @@ def run_attention(gpu, be):
             for t in (q, k, v, o, pos, kl):
                 t.free()
     return res
+
+
+def run_decoder_eager(gpu, be, steps=8):
+    """The config-5 decode step issued launch by launch (no program replay): the form a kernel trace can
+    attribute per kernel (rocprofv3 does not survive stream capture in the traced process)."""
+    from aion_amd.decoder import Decoder, DecoderConfig, SyntheticWeights
+    cfg = DecoderConfig()
+    dec = Decoder(gpu, cfg, SyntheticWeights(cfg, 0))
+    prompt = np.random.default_rng(5).integers(0, cfg.vocab, 128).astype(np.int32)
+    tok = dec.prefill(prompt)
+    gpu.sync()
+    t = time.perf_counter()
+    for _ in range(steps):
+        tok = dec.decode_step_eager(tok)
+    gpu.sync()
+    return {"steps": steps, "eager_ms_per_token": round((time.perf_counter() - t) / steps * 1e3, 4)}
 
 
 def run_decoder(gpu, be, with_cpu=True):
