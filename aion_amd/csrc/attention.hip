@@ -443,15 +443,15 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
 //   V^T[dv][key], row stride 72 B: stores and operand reads are bank-conflict-free); the k index of
 //   the second product is permuted (slot s of lane half h <-> key (s/4)*8 + 4h + s%4 of a 16-key step)
 //   so that the probabilities feed the MFMA straight from the S accumulators without a shuffle.
-constexpr int PF_ROWS = 128, PF_VROW = 72;
+constexpr int PF_ROWS = 128, PF_TK = 64, PF_VROW = 136;
 constexpr float PF_LAZY = 8.f;
 using f32x16 = __attribute__((ext_vector_type(16))) float;
 using u32x2 = __attribute__((ext_vector_type(2))) unsigned int;
 
 template <int D>
 struct PrefillCfg {
-    static constexpr int KROW = D * 2 + 16;                         // K tile row: 16 consecutive rows -> 16 distinct 16-byte bank groups
-    static constexpr int K_BYTES = TILE_KEYS * KROW;
+    static constexpr int KROW = D * 2;                              // unpadded (filled by LDS-writing loads), chunk slots swizzled
+    static constexpr int K_BYTES = PF_TK * KROW;
     static constexpr int V_BYTES = D * PF_VROW;
     static constexpr int STAGE = K_BYTES + V_BYTES;
     static constexpr int LDS_BYTES = 2 * STAGE + 64;
@@ -466,14 +466,16 @@ __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
 
 template <int KV, int D, bool CAP>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
     using Cfg = PrefillCfg<D>;
     constexpr int KK = D / 16;          // k-steps of the first product
     constexpr int NJ = D / 32;          // 32-wide dv tiles of the second product
     constexpr int CPK = D / 8;          // 16-byte chunks per key row
-    constexpr int NKL = TILE_KEYS * CPK / 256;   // K chunks per thread per tile
-    constexpr int V_ITEMS = 16 * CPK;            // V (key pair, chunk) items per tile
-    constexpr int NVL = V_ITEMS >= 256 ? V_ITEMS / 256 : 1;
+    constexpr int NKI = PF_TK * Cfg::KROW / 1024 / 4;   // K loads (1 KiB each) per wavefront per tile
+    constexpr int KEYS_PER_KI = 1024 / Cfg::KROW;       // keys covered by one K load
+    constexpr int V_ITEMS = (PF_TK / 2) * CPK;          // V (key pair, chunk) items per tile
+    constexpr int NVL = V_ITEMS / 256;
+    static_assert(NKI >= 1 && NVL >= 1, "head size below 64 is not handled here");
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l31 = lane & 31, lh = lane >> 5;
@@ -530,7 +532,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
         }
         return;
     }
-    const int t_begin = g_lo / TILE_KEYS, t_end = (g_hi + TILE_KEYS - 1) / TILE_KEYS;
+    const int t_begin = g_lo / PF_TK, t_end = (g_hi + PF_TK - 1) / PF_TK;
 
     const unsigned short *kp = (const unsigned short *)a.k;
     const unsigned short *vp = (const unsigned short *)a.v;
@@ -538,37 +540,41 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
     const size_t kv_base = ((size_t)b * a.T * a.Hkv + hk) * D;
     const int key_clamp_hi = g_hi - 1;
 
-    // ---- cooperative tile loads: registers now, LDS after the current tile's MFMAs
-    u32x4 kreg[NKL], vreg[NVL][2];
-    auto load_tile = [&](int t) {
-        const int key0 = t * TILE_KEYS;
+    // ---- cooperative tile loads. K: global -> LDS directly, 1 KiB per instruction; the 16-byte chunk c of key k
+    // sits at slot c ^ swz(k), swz = k & 15 (k >> 1 & 7 for 128-byte rows), so that the 16 consecutive keys of
+    // an operand read hit 16 distinct bank groups. V: registers now, transposed stores after this tile's MFMAs.
+    // Keys outside the union are read from a clamped in-range key (masked scores / exact-zero probabilities).
+    const int k_key_in = (lane * 16) / Cfg::KROW, k_slot = ((lane * 16) % Cfg::KROW) / 16;
+    auto load_k = [&](int t, unsigned char *st) {
+#if defined(__HIP_DEVICE_COMPILE__)   // the builtin exists in the device pass only
+        const int key0 = t * PF_TK;
 #pragma unroll
-        for (int i = 0; i < NKL; ++i) {
-            const int id = tid + 256 * i, key = id / CPK, c = id % CPK;
+        for (int i = 0; i < NKI; ++i) {
+            const int key = (wave * NKI + i) * KEYS_PER_KI + k_key_in;
+            const int swz = CPK >= 16 ? (key & 15) : ((key >> 1) & 7);
             const int kabs = min(max(key0 + key, g_lo), key_clamp_hi);
-            kreg[i] = *(const u32x4 *)(kp + kv_base + (size_t)kabs * kv_row + c * 8);
+            __builtin_amdgcn_global_load_lds(kp + kv_base + (size_t)kabs * kv_row + (k_slot ^ swz) * 8,
+                                             (lds_void *)(st + (wave * NKI + i) * 1024), 16, 0, 0);
         }
+#endif
+    };
+    u32x4 vreg[NVL][2];
+    auto load_v = [&](int t) {
+        const int key0 = t * PF_TK;
 #pragma unroll
         for (int i = 0; i < NVL; ++i) {
-            const int id = min(tid + 256 * i, V_ITEMS - 1), pair = id & 15, c = id >> 4;
+            const int id = tid + 256 * i, pair = (id & 15) + 16 * (id / (16 * CPK)), c = (id >> 4) % CPK;
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                // keys outside the union are read from a clamped in-range key: their probabilities are exact zeros
                 const int kabs = min(max(key0 + pair * 2 + h, g_lo), key_clamp_hi);
                 vreg[i][h] = *(const u32x4 *)(vp + kv_base + (size_t)kabs * kv_row + c * 8);
             }
         }
     };
-    auto store_tile = [&](unsigned char *st) {
-#pragma unroll
-        for (int i = 0; i < NKL; ++i) {
-            const int id = tid + 256 * i, key = id / CPK, c = id % CPK;
-            *(u32x4 *)(st + key * Cfg::KROW + c * 16) = kreg[i];
-        }
+    auto store_v = [&](unsigned char *st) {
 #pragma unroll
         for (int i = 0; i < NVL; ++i) {
-            const int id = tid + 256 * i, pair = id & 15, c = id >> 4;
-            if (V_ITEMS < 256 && id >= V_ITEMS) continue;
+            const int id = tid + 256 * i, pair = (id & 15) + 16 * (id / (16 * CPK)), c = (id >> 4) % CPK;
             unsigned char *vt = st + Cfg::K_BYTES + (c * 8) * PF_VROW + pair * 4;
             const u32x4 x = vreg[i][0], y = vreg[i][1];
             const unsigned xs[4] = {x.x, x.y, x.z, x.w}, ys[4] = {y.x, y.y, y.z, y.w};
@@ -588,51 +594,61 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
     float m_run = -INFINITY, l_run = 0.f;
     const float cap_inv = CAP ? 1.f / a.soft_cap : 0.f;
 
-    load_tile(t_begin);
-    store_tile(lds);
-    __syncthreads();
+    load_k(t_begin, lds);
+    load_v(t_begin);
+    store_v(lds);
+    __syncthreads();                                               // also waits for the K loads (fence)
 
-    const int k_off = l31 * Cfg::KROW + lh * 16;                    // + kk * 32
-    const int v_off = Cfg::K_BYTES + l31 * PF_VROW + lh * 8;        // + j * 32 rows + step * 32 bytes (+16 for the second 4 keys)
+    // operand addresses: K row (kb*32 + l31) at slot (2*kk + lh) ^ swz(row); V^T row (j*32 + l31), keys of step s2
+    const int k_swz = CPK >= 16 ? (l31 & 15) : ((l31 >> 1) & 7);
+    const int k_row = l31 * Cfg::KROW;
+    const int v_off = Cfg::K_BYTES + l31 * PF_VROW + lh * 8;        // + j * 32 rows + s2 * 32 bytes (+16 for the second 4 keys)
     for (int t = t_begin; t < t_end; ++t) {
         const unsigned char *st = lds + ((t - t_begin) & 1) * Cfg::STAGE;
         unsigned char *nx = lds + ((t - t_begin + 1) & 1) * Cfg::STAGE;
         const bool more = t + 1 < t_end;
-        if (more) load_tile(t + 1);
-        const int key0 = t * TILE_KEYS;
-        const bool mine = key0 < w_hi && key0 + TILE_KEYS > w_lo;       // wavefront-uniform
+        if (more) {
+            load_k(t + 1, nx);
+            load_v(t + 1);
+        }
+        const int key0 = t * PF_TK;
+        const bool mine = key0 < w_hi && key0 + PF_TK > w_lo;       // wavefront-uniform
         if (mine) {
-            // -- S^T = K . Q^T, two accumulation chains
-            f32x16 s0, s1;
+            // -- S^T = K . Q^T for the two 32-key halves (two independent accumulation chains)
+            f32x16 s[2];
 #pragma unroll
-            for (int i = 0; i < 16; ++i) { s0[i] = 0.f; s1[i] = 0.f; }
+            for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-            for (int kk = 0; kk < KK; kk += 2) {
-                const u32x4 k0 = *(const u32x4 *)(st + k_off + kk * 32);
-                const u32x4 k1 = *(const u32x4 *)(st + k_off + (kk + 1) * 32);
-                s0 = mfma32<KV>(k0, qf[kk], s0);
-                s1 = mfma32<KV>(k1, qf[kk + 1], s1);
+                for (int i = 0; i < 16; ++i) s[kb][i] = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) {
+                // rows kb*32 + l31: (row & 15) and (row >> 1 & 7) do not depend on kb
+                const int slot = ((2 * kk + lh) ^ k_swz) * 16;
+                const u32x4 k0 = *(const u32x4 *)(st + k_row + slot);
+                const u32x4 k1 = *(const u32x4 *)(st + 32 * Cfg::KROW + k_row + slot);
+                s[0] = mfma32<KV>(k0, qf[kk], s[0]);
+                s[1] = mfma32<KV>(k1, qf[kk], s[1]);
             }
-            // -- lane holds keys key0 + (i/4)*8 + lh*4 + i%4 of row l31
-            float x[16];
-            const bool full = key0 >= w_lo_max && key0 + TILE_KEYS <= w_hi_min;   // every key visible to every row
+            // -- lane holds keys key0 + kb*32 + (i/4)*8 + lh*4 + i%4 of row l31
+            float x[32];
+            const bool full = key0 >= w_lo_max && key0 + PF_TK <= w_hi_min;   // every key visible to every row
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                float v = (s0[i] + s1[i]) * a.scale;
+            for (int i = 0; i < 32; ++i) {
+                float v = s[i >> 4][i & 15] * a.scale;
                 if (CAP) v = a.soft_cap * tanhf(v * cap_inv);
                 x[i] = v;
             }
-            if (!full) {                                                          // wavefront-uniform
-                const int kb = key0 + lh * 4;
+            if (!full) {                                                      // wavefront-uniform
+                const int kbase = key0 + lh * 4;
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int key = kb + (i >> 2) * 8 + (i & 3);
+                for (int i = 0; i < 32; ++i) {
+                    const int key = kbase + (i >> 4) * 32 + ((i >> 2) & 3) * 8 + (i & 3);
                     x[i] = (key >= lo && key < hi) ? x[i] : -INFINITY;
                 }
             }
             float mx = x[0];
 #pragma unroll
-            for (int i = 1; i < 16; ++i) mx = fmaxf(mx, x[i]);
+            for (int i = 1; i < 32; ++i) mx = fmaxf(mx, x[i]);
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
             // the reference maximum only moves when the tile's maximum exceeds it by more than PF_LAZY:
             // probabilities stay below e^PF_LAZY (exact in the f32 sums, fine in the 16-bit operand) and the
@@ -643,21 +659,21 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
                 alpha = m_run > -INFINITY ? __builtin_amdgcn_exp2f((m_run - m_new) * LOG2E) : 1.f;
                 const float mneg = -m_new * LOG2E;
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
+                for (int i = 0; i < 32; ++i) {
                     x[i] = __builtin_amdgcn_exp2f(fmaf(x[i], LOG2E, mneg));      // exp2(-inf) = 0 for masked keys
                     rowsum += x[i];
                 }
             } else {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) x[i] = 0.f;
+                for (int i = 0; i < 32; ++i) x[i] = 0.f;
             }
             rowsum += __shfl_xor(rowsum, 32, 64);
             l_run = l_run * alpha + rowsum;
             m_run = m_new;
             // P^T operand of 16-key step s2: slots 0..7 <- accumulator elements 8*s2 .. 8*s2+7
-            u32x4 pf[2];
+            u32x4 pf[4];
 #pragma unroll
-            for (int s2 = 0; s2 < 2; ++s2)
+            for (int s2 = 0; s2 < 4; ++s2)
                 pf[s2] = u32x4{pack2<KV>(x[8 * s2], x[8 * s2 + 1]), pack2<KV>(x[8 * s2 + 2], x[8 * s2 + 3]),
                                pack2<KV>(x[8 * s2 + 4], x[8 * s2 + 5]), pack2<KV>(x[8 * s2 + 6], x[8 * s2 + 7])};
             // -- O^T += V^T . P^T
@@ -670,7 +686,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
             for (int j = 0; j < NJ; ++j) {
                 f32x16 c = acc[j];
 #pragma unroll
-                for (int s2 = 0; s2 < 2; ++s2) {
+                for (int s2 = 0; s2 < 4; ++s2) {
                     const unsigned char *vrow = st + v_off + j * 32 * PF_VROW + s2 * 32;
                     const u32x2 va = *(const u32x2 *)(vrow), vb = *(const u32x2 *)(vrow + 16);
                     c = mfma32<KV>(u32x4{va.x, va.y, vb.x, vb.y}, pf[s2], c);
@@ -678,8 +694,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
                 acc[j] = c;
             }
         }
-        if (more) store_tile(nx);
-        __syncthreads();
+        if (more) store_v(nx);
+        __syncthreads();                                           // also waits for this wavefront's K loads (fence)
     }
 
     if (row_ok) {
