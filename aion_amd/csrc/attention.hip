@@ -60,13 +60,16 @@ __device__ __forceinline__ float from_half_bits(unsigned short b) {
     return bf16_bits_to_f32(b);
 }
 // two f32 -> one 32-bit word of two halves (RNE), low half first
+using f32x2 = __attribute__((ext_vector_type(2))) float;
+using bf16x2 = __attribute__((ext_vector_type(2))) __bf16;
 template <int KV>
 __device__ __forceinline__ unsigned pack2(float a, float b) {
     if (KV == AIONHIP_F16) {
         const __half2 h = __floats2half2_rn(a, b);
         return *reinterpret_cast<const unsigned *>(&h);
     }
-    return (unsigned)f32_to_bf16_bits(a) | ((unsigned)f32_to_bf16_bits(b) << 16);
+    // one v_cvt_pk_bf16_f32 (round to nearest even) instead of integer rounding per element
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2{a, b}, bf16x2));
 }
 template <int KV>
 __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
@@ -622,7 +625,6 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
                 for (int i = 0; i < 16; ++i) s[kb][i] = 0.f;
 #pragma unroll
             for (int kk = 0; kk < KK; ++kk) {
-                // rows kb*32 + l31: (row & 15) and (row >> 1 & 7) do not depend on kb
                 const int slot = ((2 * kk + lh) ^ k_swz) * 16;
                 const u32x4 k0 = *(const u32x4 *)(st + k_row + slot);
                 const u32x4 k1 = *(const u32x4 *)(st + 32 * Cfg::KROW + k_row + slot);
@@ -682,17 +684,15 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
 #pragma unroll
                 for (int j = 0; j < NJ; ++j) acc[j] *= alpha;
             }
+            // key step outermost: consecutive MFMAs go to different accumulators
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                f32x16 c = acc[j];
+            for (int s2 = 0; s2 < 4; ++s2)
 #pragma unroll
-                for (int s2 = 0; s2 < 4; ++s2) {
+                for (int j = 0; j < NJ; ++j) {
                     const unsigned char *vrow = st + v_off + j * 32 * PF_VROW + s2 * 32;
                     const u32x2 va = *(const u32x2 *)(vrow), vb = *(const u32x2 *)(vrow + 16);
-                    c = mfma32<KV>(u32x4{va.x, va.y, vb.x, vb.y}, pf[s2], c);
+                    acc[j] = mfma32<KV>(u32x4{va.x, va.y, vb.x, vb.y}, pf[s2], acc[j]);
                 }
-                acc[j] = c;
-            }
         }
         if (more) store_v(nx);
         __syncthreads();                                           // also waits for this wavefront's K loads (fence)
