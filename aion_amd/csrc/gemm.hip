@@ -151,8 +151,8 @@ __global__ void act_bf16_kernel(const float *__restrict__ a, size_t lda, unsigne
 }
 
 // ---- wide-tile kernel: workgroup tile (WM*64) x 256, K step 32, v_mfma_f32_32x32x16_bf16.
-// 2 x 2 wavefronts, each (WM*32) x 128 outputs = WM x 4 tiles of 32x32 (accumulators: WM*64
-// registers). Operands go global -> LDS directly (global_load_lds_dwordx4: each wavefront load
+// 2 x 2 wavefronts, each (WM*32) x (WN*32) outputs = WM x WN tiles of 32x32 (accumulators: WM*WN*16
+// registers; WN = 4, or 3 for the narrower tiles of a last partial round). Operands go global -> LDS directly (global_load_lds_dwordx4: each wavefront load
 // fills 1 KiB = 16 rows of 64 B, no staging registers, no LDS store instructions). Rows are not
 // padded; the 16-byte chunk c of row r sits at slot c ^ ((r >> 2) & 3), chosen on the global side
 // of the load, so that the 16 consecutive rows of a fragment read hit 16 distinct bank groups.
@@ -166,28 +166,29 @@ constexpr int G2_BK = 32, G2_ROW = 64, G2_BN = 256;
 using f32x16 = __attribute__((ext_vector_type(16))) float;
 
 
-template <int WM, int NST, int WGS_PER_CU>
-__global__ __launch_bounds__(256, WGS_PER_CU) void gemm_bf16_wide_kernel(const unsigned short *__restrict__ A, const unsigned short *__restrict__ W,
+template <int WM, int NST, int WN>
+__global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const unsigned short *__restrict__ A, const unsigned short *__restrict__ W,
                                                              float *__restrict__ c, int M, int N, int K, size_t ldc, float alpha,
                                                              float beta, int tiles_m, int tiles) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds2[];
     constexpr int BM2 = WM * 64;
-    constexpr int A_BYTES = BM2 * G2_ROW, B_BYTES = G2_BN * G2_ROW, STAGE = A_BYTES + B_BYTES;
-    constexpr int NA = WM, NB = 4;                           // wavefront loads (16 rows each) per stage
+    constexpr int BN2 = WN * 64;                             // 256 columns, or 192 for the last partial round of tiles
+    constexpr int A_BYTES = BM2 * G2_ROW, B_BYTES = BN2 * G2_ROW, STAGE = A_BYTES + B_BYTES;
+    constexpr int NA = WM, NB = WN;                          // wavefront loads (16 rows each) per stage
     constexpr int NL = NA + NB;
     const int per_xcd = (int)gridDim.x >> 3;
     const int t = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
     if (t >= tiles) return;
-    const int m0 = (t % tiles_m) * BM2, n0 = (t / tiles_m) * G2_BN;
+    const int m0 = (t % tiles_m) * BM2, n0 = (t / tiles_m) * BN2;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l31 = lane & 31, lh = lane >> 5;
-    const int wrow = (wave >> 1) * (WM * 32), wcol = (wave & 1) * 128;
+    const int wrow = (wave >> 1) * (WM * 32), wcol = (wave & 1) * (WN * 32);
 
-    f32x16 acc[WM][4];
+    f32x16 acc[WM][WN];
 #pragma unroll
     for (int mi = 0; mi < WM; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < 4; ++ni)
+        for (int ni = 0; ni < WN; ++ni)
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[mi][ni][i] = 0.f;
 
@@ -222,12 +223,12 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void gemm_bf16_wide_kernel(const u
     const int fa = wrow * G2_ROW, fb = A_BYTES + wcol * G2_ROW;
 
     struct Frag {
-        u32x4 a[WM], b[4];
+        u32x4 a[WM], b[WN];
     };
     auto read_frag = [&](Frag &f, int kt, int ks) {
         const unsigned char *st = lds2 + (kt % NST) * STAGE;
 #pragma unroll
-        for (int ni = 0; ni < 4; ++ni) f.b[ni] = *(const u32x4 *)(st + fb + ni * 32 * G2_ROW + foff[ks]);
+        for (int ni = 0; ni < WN; ++ni) f.b[ni] = *(const u32x4 *)(st + fb + ni * 32 * G2_ROW + foff[ks]);
 #pragma unroll
         for (int mi = 0; mi < WM; ++mi) f.a[mi] = *(const u32x4 *)(st + fa + mi * 32 * G2_ROW + foff[ks]);
     };
@@ -235,10 +236,10 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void gemm_bf16_wide_kernel(const u
 #pragma unroll
         for (int mi = 0; mi < WM; ++mi)
 #pragma unroll
-            for (int ni = 0; ni < 4; ++ni)
+            for (int ni = 0; ni < WN; ++ni)
                 acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, f.a[mi]), __builtin_bit_cast(bf16x8, f.b[ni]), acc[mi][ni], 0, 0, 0);
     };
-    constexpr int NMMA = WM * 4, NFR = WM + 4;
+    constexpr int NMMA = WM * WN, NFR = WM + WN;
 
 #pragma unroll
     for (int i = 0; i < NST - 1; ++i) issue_loads(i);
@@ -298,7 +299,7 @@ __global__ __launch_bounds__(256, WGS_PER_CU) void gemm_bf16_wide_kernel(const u
 #pragma unroll
     for (int mi = 0; mi < WM; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < 4; ++ni) {
+        for (int ni = 0; ni < WN; ++ni) {
             const int col = n0 + wcol + ni * 32 + l31;
             if (col >= N) continue;
 #pragma unroll
@@ -361,37 +362,41 @@ int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *cw, size_t m, const
     }
     ProfScope scope(ctx, "gemm_bf16");
     {
-        // 256-row tiles when they still give every CU a workgroup, else 128-row tiles
         const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
         const int tn = (int)((N + G2_BN - 1) / G2_BN);
         // tallest tile that still gives every CU a workgroup; 64-row tiles when even 128-row ones leave half idle
         const int tm4 = (int)((m + 255) / 256), tm2 = (int)((m + 127) / 128), tm1 = (int)((m + 63) / 64);
         const int wm = (long)tm4 * tn >= cus ? 4 : ((long)tm2 * tn * 2 > cus ? 2 : 1);
-        const int tm = wm == 4 ? tm4 : (wm == 2 ? tm2 : tm1), tiles = tm * tn;
-        const dim3 grid((unsigned)((tiles + 7) / 8 * 8));
-        static bool attr[3] = {false, false, false};
+        const int tm = wm == 4 ? tm4 : (wm == 2 ? tm2 : tm1);
+        // Whole rounds of 256-column tiles first; if the columns left over would make a partial round, they are
+        // covered with 192-column tiles when those fit one round (3/4 of the time of a round of full tiles).
+        int tn_wide = tn, tn_narrow = 0;
         if (wm == 4) {
-            constexpr int LDS = 4 * (256 + G2_BN) * G2_ROW;
-            if (!attr[0]) {
-                HIP_TRY(ctx, hipFuncSetAttribute((const void *)gemm_bf16_wide_kernel<4, 4, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
-                attr[0] = true;
+            const int per_round = cus / tm;                     // column tiles per round
+            const int rest = per_round > 0 ? tn % per_round : 0;
+            if (per_round > 0 && rest > 0 && tn > per_round) {
+                const size_t cols_left = N - (size_t)(tn - rest) * G2_BN;
+                const int narrow = (int)((cols_left + 191) / 192);
+                if ((long)narrow * tm <= cus) { tn_wide = tn - rest; tn_narrow = narrow; }
             }
-            launch_k(ctx, gemm_bf16_wide_kernel<4, 4, 1>, grid, dim3(256), LDS, abf, w->bf16, c, (int)m, (int)N, (int)K, ldc, alpha, beta, tm, tiles);
-        } else if (wm == 2) {
-            constexpr int LDS = 4 * (128 + G2_BN) * G2_ROW;
-            if (!attr[1]) {
-                HIP_TRY(ctx, hipFuncSetAttribute((const void *)gemm_bf16_wide_kernel<2, 4, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
-                attr[1] = true;
-            }
-            launch_k(ctx, gemm_bf16_wide_kernel<2, 4, 1>, grid, dim3(256), LDS, abf, w->bf16, c, (int)m, (int)N, (int)K, ldc, alpha, beta, tm, tiles);
-        } else {
-            constexpr int LDS = 4 * (64 + G2_BN) * G2_ROW;
-            if (!attr[2]) {
-                HIP_TRY(ctx, hipFuncSetAttribute((const void *)gemm_bf16_wide_kernel<1, 4, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
-                attr[2] = true;
-            }
-            launch_k(ctx, gemm_bf16_wide_kernel<1, 4, 1>, grid, dim3(256), LDS, abf, w->bf16, c, (int)m, (int)N, (int)K, ldc, alpha, beta, tm, tiles);
         }
+        static bool attr[4] = {false, false, false, false};
+        auto launch = [&](auto kernel, int idx, int lds, const unsigned short *wp, float *cp, size_t ncols, int tiles) -> int {
+            if (!attr[idx]) {
+                HIP_TRY(ctx, hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+                attr[idx] = true;
+            }
+            launch_k(ctx, kernel, dim3((unsigned)((tiles + 7) / 8 * 8)), dim3(256), lds, abf, wp, cp, (int)m, (int)ncols, (int)K, ldc, alpha, beta, tm, tiles);
+            return AIONHIP_OK;
+        };
+        const size_t wide_cols = tn_narrow ? (size_t)tn_wide * G2_BN : N;
+        if (wm == 4) rc = launch(gemm_bf16_wide_kernel<4, 4, 4>, 0, 4 * (256 + 256) * G2_ROW, w->bf16, c, wide_cols, tm * tn_wide);
+        else if (wm == 2) rc = launch(gemm_bf16_wide_kernel<2, 4, 4>, 1, 4 * (128 + 256) * G2_ROW, w->bf16, c, wide_cols, tm * tn_wide);
+        else rc = launch(gemm_bf16_wide_kernel<1, 4, 4>, 2, 4 * (64 + 256) * G2_ROW, w->bf16, c, wide_cols, tm * tn_wide);
+        if (rc) return rc;
+        if (tn_narrow)
+            rc = launch(gemm_bf16_wide_kernel<4, 4, 3>, 3, 4 * (256 + 192) * G2_ROW, w->bf16 + wide_cols * K, c + wide_cols, N - wide_cols, tm * tn_narrow);
+        if (rc) return rc;
     }
     LAUNCH_CHECK(ctx, "gemm_bf16");
     return AIONHIP_OK;
