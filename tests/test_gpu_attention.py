@@ -205,3 +205,46 @@ def test_precise_mode_brings_f32_queries_to_f32_accuracy(gpu, orc):
     e_fast, e_prec = float(np.abs(fast - ref).max()), float(np.abs(precise - ref).max())
     say("  fast", e_fast, "precise", e_prec)
     assert e_fast < 2e-3 and e_prec < 1e-5
+
+
+def test_prefill_config4_sizes(gpu, orc):
+    # BASELINE config 4a at L = 1024: 8 q heads / 1 kv head, head size 256, bf16, scale 1/16, causal; every row
+    # against the f64 reference (1e-2: bf16 MFMA operands). At L = 4096 the oracle is too slow, so the kernel is
+    # held to properties that do not depend on the size: V = const gives that const back (the probabilities of a
+    # row sum to one), and row 0 sees key 0 only.
+    say("prefill config 4 L1024")
+    (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(41, 1, 1024, 1024, 8, 1, 256, "bf16")
+    got = run_attention(gpu, q, k, v, 1 / 16.0, qd, kd)
+    assert gpu.last_kernel() == "attn_prefill"
+    ref = orc.attention_f64(qf, kf, vf, 1 / 16.0)
+    err = float(np.abs(got - ref).max())
+    say("  max err", err)
+    assert err < 1e-2
+    say("prefill config 4 L4096 properties")
+    L = 4096
+    (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(43, 1, L, L, 8, 1, 256, "bf16")
+    ones, _ = to_bf16(np.full((1, L, 1, 256), 0.75, np.float32))
+    got = run_attention(gpu, q, k, ones, 1 / 16.0, qd, kd)
+    assert float(np.abs(got - 0.75).max()) < 1e-2
+    got = run_attention(gpu, q, k, v, 1 / 16.0, qd, kd)
+    # one visible key: its value (the single probability is exp2 of a rounding residue, 1 to within an ulp)
+    assert np.allclose(got[0, 0], np.broadcast_to(vf[0, 0, 0], (8, 256)), rtol=1e-6, atol=0)
+    # the last rows against the reference on the last 16 positions only (full key range)
+    ref_tail = orc.attention_f64(qf[:, L - 16:], kf, vf, 1 / 16.0, positions=np.arange(L - 16, L, dtype=np.int32).reshape(1, 16))
+    assert float(np.abs(got[:, L - 16:] - ref_tail).max()) < 1e-2
+
+
+def test_prefill_chunk_with_positions_over_a_longer_cache(gpu, orc):
+    # a prompt chunk: 96 new rows at positions 160..255 over a cache of capacity 300 holding 256 keys
+    B, Lq, T, Hq, Hkv, D = 2, 96, 300, 8, 2, 128
+    (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(47, B, Lq, T, Hq, Hkv, D, "f16")
+    k[:, 256:] = np.float16(np.nan)                      # beyond the cache length: must not leak
+    v[:, 256:] = np.float16(np.nan)
+    pos = np.tile(np.arange(160, 256, dtype=np.int32), (B, 1))
+    lens = np.array([256, 200], np.int32)                # the second sequence sees keys < 200 only
+    got = run_attention(gpu, q, k, v, 1 / math.sqrt(D), qd, kd, positions=pos, kv_lengths=lens)
+    assert gpu.last_kernel() == "attn_prefill"
+    kz, vz = np.nan_to_num(kf), np.nan_to_num(vf)
+    ref = orc.attention_f64(qf, kz, vz, 1 / math.sqrt(D), positions=pos, kv_lengths=lens)
+    assert np.isfinite(got).all()
+    assert float(np.abs(got - ref).max()) < 2e-3
