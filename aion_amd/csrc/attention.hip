@@ -10,10 +10,12 @@
 //   head); each lane's accumulators, running max and sum belong to ONE query row, so the softmax
 //   bookkeeping is per-lane scalar work. Two launch shapes:
 //     split mode (few query rows: decode) - a workgroup is one 16-row tile x one key segment, its
-//       four wavefronts interleave 32-key tiles and merge through LDS; segments merge in
+//       eight wavefronts interleave 32-key tiles and merge through LDS; segments merge in
 //       attn_merge_kernel (the flash-decoding split of cpu/exec/attention.zig:879-962).
-//     prefill mode - a workgroup is four 16-row tiles, each wavefront walks its own key range
-//       (whole tiles outside every row's interval are skipped: the causal triangle).
+//     per-wavefront mode - a workgroup is four 16-row tiles, each wavefront walks its own key range; used
+//       for many query rows only when the hi+lo precise mode is on (see attn_prefill_kernel otherwise).
+// attn_prefill_kernel - many query rows: 128 rows per workgroup, K/V tiles shared through LDS, 32x32x16 MFMA
+//   (described at the kernel).
 // attn_generic_kernel - any head size / f32 K,V: one wavefront per query row, scores staged in
 //   global scratch. Slow; it exists so that every shape the op allows has a GPU path.
 //

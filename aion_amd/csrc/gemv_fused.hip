@@ -9,10 +9,10 @@
 // gemv_kernel: one wavefront per R rows, 16-byte chunks per lane, v_dot4_i32_i8, DPP fold. The
 // grid is capped at a few workgroups per CU and wavefronts stride over the row groups, so the
 // prologue is paid a bounded number of times however many rows the weight has.
-// K <= 8192 (10 KB of LDS); larger K keeps the separate preparation launch.
+// K <= 8192 fits (10 KB of LDS); the callers use it up to K = 4096, beyond which the prologue repeated per
+// workgroup costs more than one separate preparation launch.
+// Two optional epilogues finish a decode block in the same launch (EPI_ROPE_APPEND, EPI_GATE_QUANT below).
 #include "common.h"
-
-#include <cstdlib>
 
 namespace {
 
@@ -351,10 +351,7 @@ void launch_r(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *c
     batch.total_waves = waves;
     // at most 8 workgroups per CU: beyond that the wavefronts stride over the row groups
     const int wgs = (waves + 3) / 4;
-#ifndef FUSED_CAP
-#define FUSED_CAP 8
-#endif
-    const dim3 grid((unsigned)(wgs < cus * FUSED_CAP ? wgs : cus * FUSED_CAP)), block(256);
+    const dim3 grid((unsigned)(wgs < cus * 8 ? wgs : cus * 8)), block(256);
     const size_t lds = (size_t)K + (size_t)(K >> 5) * 8 + 16;
     if (R == 4) launch_k(ctx, gemv_fused_kernel<DT, 4, PRO, NCH, EPI_NONE>, grid, block, lds, batch, in, K, alpha, beta, FusedEpi{});
     else if (R == 2) launch_k(ctx, gemv_fused_kernel<DT, 2, PRO, NCH, EPI_NONE>, grid, block, lds, batch, in, K, alpha, beta, FusedEpi{});

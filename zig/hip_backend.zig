@@ -158,6 +158,12 @@ pub const HipBackend = struct {
             },
             // ElemwiseBinary(add | gate gelu), Gather(axis 0), Cast(f32->f16), SequenceAppend map to
             // aionhip_step_add / _gate_gelu / _gather_rows / _cast_f32_f16 / _append_f16 the same way;
+            // Optional launch-saving pattern matches over consecutive steps of a decode program (same results as
+            // the separate steps; fall back to them on AIONHIP_UNSUPPORTED):
+            //   RMSNorm, MatMul x3 (q,k,v), RoPE1D x2, Cast f16 x2, SequenceAppend x2 -> aionhip_step_rmsnorm_qkv_rope_append
+            //   RMSNorm, MatMul x2 (gate, up), gate(gelu), MatMul (down)             -> aionhip_step_rmsnorm_geglu_matmul
+            //   RMSNorm, MatMul(s)                                                   -> aionhip_step_rmsnorm_matmul
+            //   gate(gelu), MatMul                                                   -> aionhip_step_gate_matmul
             // Transfer steps go through deviceMemory() exactly as in backend/gpu/backend.zig:416-457.
             else => return BackendError.Unsupported,
         }
