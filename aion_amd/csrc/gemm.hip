@@ -14,6 +14,7 @@
 
 namespace {
 
+using u32x2 = __attribute__((ext_vector_type(2))) unsigned int;
 using i32x4 = __attribute__((ext_vector_type(4))) int;
 using bf16x8 = __attribute__((ext_vector_type(8))) __bf16;
 
@@ -90,6 +91,177 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(const uint8_t *__restrict_
 #pragma unroll
             for (int ni = 0; ni < TN; ++ni) {
                 const int col = n0 + ni * 16 + r;
+                if (col >= N) continue;
+                float *dst = c + (size_t)row * ldc + col;
+                const float v = alpha * acc[mi][ni][i];
+                *dst = beta == 0.f ? v : v + beta * *dst;
+            }
+        }
+}
+
+// ---- LDS-staged exact kernel (more than 16 activation rows): same arithmetic as gemm_i8_kernel - one
+// v_mfma_i32_16x16x32_i8 per 16x16 tile per quant block, then acc += f32(idot) * (a_scale * w_scale) - but
+// the operands of a K step (4 quant blocks) are staged once per workgroup in LDS with coalesced 16-byte
+// loads (a cache line per row), instead of 8-byte operand loads per lane per tile from global memory, which
+// cost several times their payload in L1 bandwidth. q4 nibbles become signed int8 while they are staged
+// (((x | 0x80) - 8) ^ 0x80 per byte), so no per-tile bias correction is left. Workgroup tile (32*WM) x 128,
+// 2 x 2 wavefronts of (16*WM) x 64 outputs; double-buffered, one barrier per K step. The rescale (3 VALU
+// operations per output per block against 32 integer MACs) bounds it at roughly 1/7 of the int8 MFMA peak.
+constexpr int GI_KC = 4;                              // quant blocks per K step
+constexpr int GI_ROW = GI_KC * 32 + 8;                // staged code row: 128 B + 8 B (spreads the 8-byte operand reads over the banks)
+template <int DT, int WM>
+__global__ __launch_bounds__(256, 2) void gemm_i8_lds_kernel(const uint8_t *__restrict__ qs, const __half *__restrict__ sc,
+                                                          const int8_t *__restrict__ aq, const float *__restrict__ a_scale,
+                                                          float *__restrict__ c, int M, int N, int K, size_t ldc,
+                                                          float alpha, float beta) {
+    constexpr bool Q8 = DT == AIONHIP_Q8_0;
+    constexpr int BM3 = 32 * WM, BN3 = 128;
+    constexpr int A_BYTES = BM3 * GI_ROW, B_BYTES = BN3 * GI_ROW;
+    constexpr int AS_BYTES = BM3 * GI_KC * 4, WS_BYTES = BN3 * GI_KC * 4;
+    constexpr int STAGE = A_BYTES + B_BYTES + AS_BYTES + WS_BYTES;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds3[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, g = lane >> 4;
+    const int m0 = blockIdx.y * BM3, n0 = blockIdx.x * BN3;
+    const int wm0 = (wave >> 1) * (16 * WM), wn0 = (wave & 1) * 64;
+    const int KB = K >> 5, KT = (KB + GI_KC - 1) / GI_KC;
+
+    f32x4 acc[WM][4];
+#pragma unroll
+    for (int mi = 0; mi < WM; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni) acc[mi][ni] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // staging assignment. Codes: 16-byte chunks, 8 per row (one 128-byte line per row per K step).
+    constexpr int NAC = BM3 * 8 / 256;                   // activation chunks per thread (WM)
+    constexpr int NBC = Q8 ? 4 : 2;                      // weight chunks per thread: q8 128 rows x 8, q4 128 rows x 4 (16 B = one block)
+    u32x4 ra[NAC], rb[NBC];
+    float ras[(BM3 * GI_KC + 255) / 256], rws[2];
+    auto load_stage = [&](int kt) {
+        const int kb0 = kt * GI_KC;
+#pragma unroll
+        for (int i = 0; i < NAC; ++i) {
+            const int id = tid + 256 * i, row = id >> 3, part = id & 7;
+            const int kbyte = min(kb0 * 32 + part * 16, K - 16);
+            ra[i] = *(const u32x4 *)(aq + (size_t)min(m0 + row, M - 1) * K + kbyte);
+        }
+#pragma unroll
+        for (int i = 0; i < NBC; ++i) {
+            const int id = tid + 256 * i;
+            if (Q8) {
+                const int row = id >> 3, part = id & 7;
+                const int kbyte = min(kb0 * 32 + part * 16, K - 16);
+                rb[i] = *(const u32x4 *)(qs + (size_t)min(n0 + row, N - 1) * K + kbyte);
+            } else {
+                const int row = id >> 2, blk = min(kb0 + (id & 3), KB - 1);
+                rb[i] = *(const u32x4 *)(qs + (size_t)min(n0 + row, N - 1) * (K >> 1) + (size_t)blk * 16);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < (BM3 * GI_KC + 255) / 256; ++i) {
+            const int id = tid + 256 * i, row = id / GI_KC, j = id % GI_KC;
+            ras[i] = (id < BM3 * GI_KC && kb0 + j < KB) ? a_scale[(size_t)min(m0 + row, M - 1) * KB + kb0 + j] : 0.f;   // past the end: no contribution
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int id = tid + 256 * i, row = id / GI_KC, j = id % GI_KC;
+            rws[i] = kb0 + j < KB ? __half2float(sc[(size_t)min(n0 + row, N - 1) * KB + kb0 + j]) : 0.f;
+        }
+    };
+    auto store_stage = [&](unsigned char *st) {
+#pragma unroll
+        for (int i = 0; i < NAC; ++i) {
+            const int id = tid + 256 * i, row = id >> 3, part = id & 7;
+            *(u32x2 *)(st + row * GI_ROW + part * 16) = u32x2{ra[i].x, ra[i].y};
+            *(u32x2 *)(st + row * GI_ROW + part * 16 + 8) = u32x2{ra[i].z, ra[i].w};
+        }
+#pragma unroll
+        for (int i = 0; i < NBC; ++i) {
+            const int id = tid + 256 * i;
+            if (Q8) {
+                const int row = id >> 3, part = id & 7;
+                *(u32x2 *)(st + A_BYTES + row * GI_ROW + part * 16) = u32x2{rb[i].x, rb[i].y};
+                *(u32x2 *)(st + A_BYTES + row * GI_ROW + part * 16 + 8) = u32x2{rb[i].z, rb[i].w};
+            } else {
+                // word w of the device layout holds elements 8w..8w+7: low nibbles 8w..8w+3, high nibbles 8w+4..8w+7
+                const int row = id >> 2, j = id & 3;
+                unsigned char *dst = st + A_BYTES + row * GI_ROW + j * 32;
+                const unsigned ws4[4] = {rb[i].x, rb[i].y, rb[i].z, rb[i].w};
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const unsigned lo = ws4[w] & 0x0F0F0F0Fu, hi = (ws4[w] >> 4) & 0x0F0F0F0Fu;
+                    *(u32x2 *)(dst + w * 8) = u32x2{((lo | 0x80808080u) - 0x08080808u) ^ 0x80808080u,
+                                                   ((hi | 0x80808080u) - 0x08080808u) ^ 0x80808080u};
+                }
+            }
+        }
+        float *as_l = (float *)(st + A_BYTES + B_BYTES), *ws_l = (float *)(st + A_BYTES + B_BYTES + AS_BYTES);
+#pragma unroll
+        for (int i = 0; i < (BM3 * GI_KC + 255) / 256; ++i)
+            if (tid + 256 * i < BM3 * GI_KC) as_l[tid + 256 * i] = ras[i];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) ws_l[tid + 256 * i] = rws[i];
+    };
+
+    load_stage(0);
+    store_stage(lds3);
+    __syncthreads();
+    for (int kt = 0; kt < KT; ++kt) {
+        const unsigned char *st = lds3 + (kt & 1) * STAGE;
+        const bool more = kt + 1 < KT;
+        if (more) load_stage(kt + 1);
+        const f32x4 *as_l = (const f32x4 *)(st + A_BYTES + B_BYTES), *ws_l = (const f32x4 *)(st + A_BYTES + B_BYTES + AS_BYTES);
+        f32x4 wsc[4];
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni) wsc[ni] = ws_l[wn0 + ni * 16 + r];
+        // (row tile, block) steps, software-pipelined: the four dots of a step are issued, then the previous
+        // step's dots are rescaled while they run. The empty asm statements fix that order for the compiler,
+        // which otherwise issues every dot of the K step first and runs out of registers.
+        i32x4 dprev[4];
+        f32x4 asc[4], asc_prev[4];
+#pragma unroll
+        for (int t = 0; t <= WM * GI_KC; ++t) {
+            const int mi = t / GI_KC, j = t % GI_KC;
+            i32x4 dcur[4];
+            if (t < WM * GI_KC) {
+                if (j == 0) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) asc[i] = as_l[wm0 + mi * 16 + g * 4 + i];
+                }
+                const long a = *(const long *)(st + (wm0 + mi * 16 + r) * GI_ROW + j * 32 + g * 8);
+#pragma unroll
+                for (int ni = 0; ni < 4; ++ni) {
+                    const long b = *(const long *)(st + A_BYTES + (wn0 + ni * 16 + r) * GI_ROW + j * 32 + g * 8);
+                    dcur[ni] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b, i32x4{0, 0, 0, 0}, 0, 0, 0);
+                }
+            }
+            if (t > 0) {
+                const int pm = (t - 1) / GI_KC, pj = (t - 1) % GI_KC;
+#pragma unroll
+                for (int ni = 0; ni < 4; ++ni) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[pm][ni][i] += (float)dprev[ni][i] * (asc_prev[i][pj] * wsc[ni][pj]);
+                    asm volatile("" : "+v"(acc[pm][ni]));
+                }
+            }
+#pragma unroll
+            for (int ni = 0; ni < 4; ++ni) dprev[ni] = dcur[ni];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) asc_prev[i] = asc[i];
+        }
+        if (more) store_stage(lds3 + ((kt + 1) & 1) * STAGE);
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int mi = 0; mi < WM; ++mi)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int row = m0 + wm0 + mi * 16 + g * 4 + i;
+            if (row >= M) continue;
+#pragma unroll
+            for (int ni = 0; ni < 4; ++ni) {
+                const int col = n0 + wn0 + ni * 16 + r;
                 if (col >= N) continue;
                 float *dst = c + (size_t)row * ldc + col;
                 const float v = alpha * acc[mi][ni][i];
@@ -313,6 +485,20 @@ __global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const unsigned shor
         }
 }
 
+template <int DT, int WM>
+int launch_i8_lds(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
+    constexpr int BM3 = 32 * WM;
+    constexpr int LDS = 2 * ((BM3 + 128) * GI_ROW + (BM3 + 128) * GI_KC * 4);
+    static bool attr = false;
+    if (!attr) {
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)gemm_i8_lds_kernel<DT, WM>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+        attr = true;
+    }
+    const dim3 grid((unsigned)((w->n + 127) / 128), (unsigned)((m + BM3 - 1) / BM3));
+    launch_k(ctx, gemm_i8_lds_kernel<DT, WM>, grid, dim3(256), LDS, w->qs, w->sc, act.q, act.scale, c, (int)m, (int)w->n, (int)w->k, ldc, alpha, beta);
+    return AIONHIP_OK;
+}
+
 template <int DT>
 void launch_i8(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
     const int M = (int)m, N = (int)w->n, K = (int)w->k;
@@ -331,7 +517,21 @@ void launch_i8(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct 
 int launch_gemm_i8(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
     const char *name = w->dtype == AIONHIP_Q8_0 ? "gemm_i8_q8" : "gemm_i8_q4";
     ProfScope scope(ctx, name);
-    if (w->dtype == AIONHIP_Q8_0) launch_i8<AIONHIP_Q8_0>(ctx, w, m, act, c, ldc, alpha, beta);
+    if (m > 16 && w->k >= 32) {
+        // 128-row tiles when they still give every CU a workgroup, else 64-, else 32-row tiles
+        const long cus = ctx->cu_count > 0 ? ctx->cu_count : 256, tn = (long)((w->n + 127) / 128);
+        const int wm = (long)((m + 127) / 128) * tn >= cus ? 4 : ((long)((m + 63) / 64) * tn >= cus ? 2 : 1);
+        int rc;
+        if (w->dtype == AIONHIP_Q8_0)
+            rc = wm == 4 ? launch_i8_lds<AIONHIP_Q8_0, 4>(ctx, w, m, act, c, ldc, alpha, beta)
+               : wm == 2 ? launch_i8_lds<AIONHIP_Q8_0, 2>(ctx, w, m, act, c, ldc, alpha, beta)
+                         : launch_i8_lds<AIONHIP_Q8_0, 1>(ctx, w, m, act, c, ldc, alpha, beta);
+        else
+            rc = wm == 4 ? launch_i8_lds<AIONHIP_Q4_0, 4>(ctx, w, m, act, c, ldc, alpha, beta)
+               : wm == 2 ? launch_i8_lds<AIONHIP_Q4_0, 2>(ctx, w, m, act, c, ldc, alpha, beta)
+                         : launch_i8_lds<AIONHIP_Q4_0, 1>(ctx, w, m, act, c, ldc, alpha, beta);
+        if (rc) return rc;
+    } else if (w->dtype == AIONHIP_Q8_0) launch_i8<AIONHIP_Q8_0>(ctx, w, m, act, c, ldc, alpha, beta);
     else launch_i8<AIONHIP_Q4_0>(ctx, w, m, act, c, ldc, alpha, beta);
     LAUNCH_CHECK(ctx, name);
     return AIONHIP_OK;

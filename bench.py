@@ -239,7 +239,7 @@ def run_gemm(gpu, be):
                         gpu.step_matmul(w, x, m, y)
                     prof = [ms for (nm, ms) in gpu.profile_stop() if nm == kname]
                     wall = (time.perf_counter() - t0) / 10
-                    ms = sum(prof) / len(prof)
+                    ms = sum(prof) / 10             # a call may be more than one launch of this kernel
                     tf = 2.0 * m * n * k / (ms * 1e-3) / 1e12
                     res["%s M%d N%d %s" % (tag, m, n, "bf16" if mode == be.GEMM_BF16_MFMA else "exact_i8")] = {
                         "kernel_ms": round(ms, 4), "step_wall_ms": round(wall * 1e3, 4), "TFLOPs": round(tf, 1),
