@@ -273,6 +273,10 @@ class HipBackend:
     def step_cast_f32_f16(self, out, x, n):
         self._check(self._lib.aionhip_step_cast_f32_f16(self._ctx, out.handle, x.handle, n))
 
+    def probe_stream_read(self, src, offset, nbytes, sink):
+        """Plain streaming read of nbytes of src (measurement aid; profiled as "stream_read")."""
+        self._check(self._lib.aionhip_probe_stream_read(self._ctx, src.handle, offset, nbytes, sink.handle))
+
     def step_argmax(self, out, x, rows, n):
         self._check(self._lib.aionhip_step_argmax(self._ctx, out.handle, x.handle, rows, n))
 

@@ -334,6 +334,43 @@ int aionhip_step_cast_f32_f16(aionhip_ctx *ctx, aionhip_handle out_f16, aionhip_
     return AIONHIP_OK;
 }
 
+// Measurement aid: nothing but 16-byte non-temporal loads over `bytes` of `src`, 4 in flight per lane,
+// the loaded words folded into a value that is stored only if it hits one unlikely constant. What this
+// kernel reaches on a byte count is the device's practical read rate for that count (launch and ramp
+// included); the GEMV kernels are reported beside it.
+__global__ __launch_bounds__(256) void stream_read_kernel(const u32x4 *__restrict__ p, size_t n16, unsigned *sink) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * 256;
+    unsigned acc = 0;
+    for (; i + 3 * stride < n16; i += 4 * stride) {
+        u32x4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(p + i + u * stride);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) acc += v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    for (; i < n16; i += stride) {
+        const u32x4 v = __builtin_nontemporal_load(p + i);
+        acc += v.x ^ v.y ^ v.z ^ v.w;
+    }
+    if (acc == 0x9E3779B9u) *sink = acc;
+}
+
+int aionhip_probe_stream_read(aionhip_ctx *ctx, aionhip_handle src, size_t offset, size_t bytes, aionhip_handle sink) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (!src || !sink) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "stream_read: null operand");
+    if ((offset | bytes) & 15) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "stream_read: offset and size must be multiples of 16");
+    if (!bytes) return AIONHIP_OK;
+    const size_t n16 = bytes / 16;
+    const size_t cus = ctx->cu_count > 0 ? (size_t)ctx->cu_count : 256;
+    const size_t want = (n16 + 1023) / 1024;
+    const unsigned grid = (unsigned)(want < cus * 8 ? want : cus * 8);
+    ProfScope scope(ctx, "stream_read");
+    launch_k(ctx, stream_read_kernel, dim3(grid), dim3(256), 0, (const u32x4 *)(dp<const unsigned char>(src) + offset), n16, dp<unsigned>(sink));
+    LAUNCH_CHECK(ctx, "stream_read");
+    return AIONHIP_OK;
+}
+
 int aionhip_step_argmax(aionhip_ctx *ctx, aionhip_handle out_i32, aionhip_handle x, size_t rows, size_t n) {
     if (!ctx) return AIONHIP_INVALID_ARGUMENT;
     if (!out_i32 || !x) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "argmax: null operand");

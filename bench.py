@@ -123,6 +123,25 @@ def main():
     gpu.sync()
     cal_src.free(); cal_dst.free()
 
+    # the device's practical read rate on the same byte counts: a plain streaming-read kernel over a region
+    # of a 1 GiB buffer that moves with every launch (nothing is re-read before 1 GiB of other data went by)
+    read_us = {}
+    rd_buf, rd_sink = gpu.alloc(1 << 30), gpu.alloc(16)
+    rd_at = 0
+    for (n, k) in SHAPES:
+        nb = algorithmic_bytes(18, n, k, batch) // 16 * 16
+        gpu.probe_stream_read(rd_buf, 0, 1 << 30, rd_sink)         # first touch of the buffer / evict the previous shape
+        gpu.sync()
+        gpu.profile_start()
+        for _ in range(20):
+            if rd_at + nb > (1 << 30):
+                rd_at = 0
+            gpu.probe_stream_read(rd_buf, rd_at, nb, rd_sink)
+            rd_at += nb
+        tms = sorted(ms for (nm, ms) in gpu.profile_stop() if nm == "stream_read")
+        read_us["%dx%d" % (n, k)] = tms[len(tms) // 2] * 1e3
+    rd_buf.free(); rd_sink.free()
+
     step_bytes = sum(algorithmic_bytes(18, n, k, batch) for (n, k) in SHAPES)
     ms_per_step = total_ms / args.steps
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
@@ -152,7 +171,12 @@ def main():
                      "traffic": round(sum(MEASURED_TRAFFIC[sh] for sh in SHAPES) / len(SHAPES)),
                      "kernel": "gemv_q4 (gemv_fused_kernel for K <= 4096, gemv_kernel after prepare_act above)",
                      "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, profiles/gemv_q4_decode_bench_kernel_stats_and_traffic.md", "avg_launch_us": round(avg_launch_ms * 1e3, 3),
-                     "algorithmic_bytes_per_launch": bytes_per_launch, "per_shape": per_shape},
+                     "algorithmic_bytes_per_launch": bytes_per_launch, "per_shape": per_shape,
+                     "plain_read_same_bytes": {
+                         "kernel_us": {sh: round(us, 2) for sh, us in read_us.items()},
+                         "GBps": round(step_bytes / (sum(read_us.values()) * 1e-6) / 1e9, 1),
+                         "gemv_rate_over_plain_read_rate": round(sum(read_us.values()) / (avg_launch_ms * 1e3 * len(SHAPES)), 3),
+                         "note": "stream_read_kernel: 16-byte non-temporal loads only, cold data, same byte count per launch"}},
     }
 
     if args.sweep:
@@ -350,7 +374,11 @@ def run_decoder(gpu, be, with_cpu=True):
     prefill_ms = (time.perf_counter() - t) * 1e3
     gpu.set_gemm_mode(be.GEMM_EXACT_I8)
     dec.reset()
+    dec.prefill(prompt); dec.reset()
+    gpu.sync()
+    t = time.perf_counter()
     tok_exact = dec.prefill(prompt)              # the decode continues from the exact-arithmetic prefill
+    prefill_exact_ms = (time.perf_counter() - t) * 1e3
     first = tok_exact
     dec.begin_decode(first)
     gpu.sync()
@@ -374,6 +402,7 @@ def run_decoder(gpu, be, with_cpu=True):
         "setup_s": round(setup_s, 1),
         "prefill_128_ms_bf16_mfma": round(prefill_ms, 3),
         "prefill_tokens_per_s": round(128 / (prefill_ms * 1e-3), 1),
+        "prefill_128_ms_exact_i8": round(prefill_exact_ms, 3),
         "prefill_next_token_bf16_vs_exact": [int(tok), int(tok_exact)],
         "decode_tokens_per_s": round(128 / decode_s, 1),
         "decode_ms_per_token": round(decode_s / 128 * 1e3, 4),

@@ -225,6 +225,10 @@ int aionhip_step_gather_rows(aionhip_ctx *ctx, int table_dtype, aionhip_handle o
 int aionhip_step_append_f16(aionhip_ctx *ctx, aionhip_handle cache, aionhip_handle src_f32, aionhip_handle write_index,
                             size_t b, size_t s, size_t t_cap, size_t row_elems);
 int aionhip_step_cast_f32_f16(aionhip_ctx *ctx, aionhip_handle out_f16, aionhip_handle x_f32, size_t n);
+/* Measurement aid with no counterpart in aion: reads `bytes` of `src` from byte `offset` with a plain
+ * streaming kernel and discards them (`sink`: any 4-byte device buffer, normally left untouched). Timed by
+ * the profiler as "stream_read"; bench.py reports the GEMV kernels beside it. offset, bytes: multiples of 16. */
+int aionhip_probe_stream_read(aionhip_ctx *ctx, aionhip_handle src, size_t offset, size_t bytes, aionhip_handle sink);
 /* StepArgMax over the last axis, first maximum wins (cpu/exec/argmax.zig:56-81); out i32 [rows] */
 int aionhip_step_argmax(aionhip_ctx *ctx, aionhip_handle out_i32, aionhip_handle x, size_t rows, size_t n);
 
