@@ -107,24 +107,32 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(const uint8_t *__restrict_
 // (((x | 0x80) - 8) ^ 0x80 per byte), so no per-tile bias correction is left. Workgroup tile (32*WM) x 128,
 // 2 x 2 wavefronts of (16*WM) x 64 outputs; double-buffered, one barrier per K step. The rescale (3 VALU
 // operations per output per block against 32 integer MACs) bounds it at roughly 1/7 of the int8 MFMA peak.
-constexpr int GI_KC = 4;                              // quant blocks per K step
-constexpr int GI_ROW = GI_KC * 32 + 8;                // staged code row: 128 B + 8 B (spreads the 8-byte operand reads over the banks)
-template <int DT, int WM>
-__global__ __launch_bounds__(256, 2) void gemm_i8_lds_kernel(const uint8_t *__restrict__ qs, const __half *__restrict__ sc,
+// KC = quant blocks per K step: 4 when the grid fills the device (two workgroups per CU hide each other's
+// staging), 8 when it does not (few activation rows: fewer, larger steps - a step then costs one memory
+// latency however little it loads).
+template <int KC> struct GiCfg { static constexpr int ROW = KC * 32 + 16; };   // staged code row; +16 B: conflict-free 8-byte operand reads
+// SPLITK (few activation rows, where the tiles above would leave most CUs idle): the workgroup tile shrinks
+// to (16*WM) x 64 and its four wavefronts share it, each taking every fourth quant block of a K step; their
+// partial sums are added in wavefront order through LDS at the end, so the result does not depend on timing.
+template <int DT, int WM, int KC, bool SPLITK>
+__global__ __launch_bounds__(256, KC == 4 || SPLITK ? 2 : 1) void gemm_i8_lds_kernel(const uint8_t *__restrict__ qs, const __half *__restrict__ sc,
                                                           const int8_t *__restrict__ aq, const float *__restrict__ a_scale,
                                                           float *__restrict__ c, int M, int N, int K, size_t ldc,
                                                           float alpha, float beta) {
     constexpr bool Q8 = DT == AIONHIP_Q8_0;
-    constexpr int BM3 = 32 * WM, BN3 = 128;
-    constexpr int A_BYTES = BM3 * GI_ROW, B_BYTES = BN3 * GI_ROW;
-    constexpr int AS_BYTES = BM3 * GI_KC * 4, WS_BYTES = BN3 * GI_KC * 4;
+    static_assert(!SPLITK || KC == 8, "split K: two blocks per wavefront per step");
+    constexpr int BM3 = (SPLITK ? 16 : 32) * WM, BN3 = SPLITK ? 64 : 128, ROW = GiCfg<KC>::ROW;
+    constexpr int KCW = SPLITK ? KC / 4 : KC;            // blocks of a K step this wavefront works on
+    constexpr int A_BYTES = BM3 * ROW, B_BYTES = BN3 * ROW;
+    constexpr int AS_BYTES = BM3 * KC * 4, WS_BYTES = BN3 * KC * 4;
     constexpr int STAGE = A_BYTES + B_BYTES + AS_BYTES + WS_BYTES;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds3[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, g = lane >> 4;
     const int m0 = blockIdx.y * BM3, n0 = blockIdx.x * BN3;
-    const int wm0 = (wave >> 1) * (16 * WM), wn0 = (wave & 1) * 64;
-    const int KB = K >> 5, KT = (KB + GI_KC - 1) / GI_KC;
+    const int wm0 = SPLITK ? 0 : (wave >> 1) * (16 * WM), wn0 = SPLITK ? 0 : (wave & 1) * 64;
+    const int jw = SPLITK ? wave : 0, jstep = SPLITK ? 4 : 1;     // this wavefront's blocks: jw + jstep * jj
+    const int KB = K >> 5, KT = (KB + KC - 1) / KC;
 
     f32x4 acc[WM][4];
 #pragma unroll
@@ -132,16 +140,19 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_lds_kernel(const uint8_t *__re
 #pragma unroll
         for (int ni = 0; ni < 4; ++ni) acc[mi][ni] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // staging assignment. Codes: 16-byte chunks, 8 per row (one 128-byte line per row per K step).
-    constexpr int NAC = BM3 * 8 / 256;                   // activation chunks per thread (WM)
-    constexpr int NBC = Q8 ? 4 : 2;                      // weight chunks per thread: q8 128 rows x 8, q4 128 rows x 4 (16 B = one block)
+    // staging assignment: 16-byte chunks, 2*KC per code row of a K step (q4 weights: KC, one block each)
+    constexpr int CPR = 2 * KC;                          // chunks per int8 row
+    constexpr int NAC = BM3 * CPR / 256;                 // activation chunks per thread
+    constexpr int NBC = (Q8 ? BN3 * CPR : BN3 * KC) / 256;
+    constexpr int NAS = (BM3 * KC + 255) / 256, NWS = BN3 * KC / 256;
     u32x4 ra[NAC], rb[NBC];
-    float ras[(BM3 * GI_KC + 255) / 256], rws[2];
+    float ras[NAS];
+    __half rws[NWS];                                     // converted when stored: a conversion here would wait for the load
     auto load_stage = [&](int kt) {
-        const int kb0 = kt * GI_KC;
+        const int kb0 = kt * KC;
 #pragma unroll
         for (int i = 0; i < NAC; ++i) {
-            const int id = tid + 256 * i, row = id >> 3, part = id & 7;
+            const int id = tid + 256 * i, row = id / CPR, part = id % CPR;
             const int kbyte = min(kb0 * 32 + part * 16, K - 16);
             ra[i] = *(const u32x4 *)(aq + (size_t)min(m0 + row, M - 1) * K + kbyte);
         }
@@ -149,110 +160,158 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_lds_kernel(const uint8_t *__re
         for (int i = 0; i < NBC; ++i) {
             const int id = tid + 256 * i;
             if (Q8) {
-                const int row = id >> 3, part = id & 7;
+                const int row = id / CPR, part = id % CPR;
                 const int kbyte = min(kb0 * 32 + part * 16, K - 16);
                 rb[i] = *(const u32x4 *)(qs + (size_t)min(n0 + row, N - 1) * K + kbyte);
             } else {
-                const int row = id >> 2, blk = min(kb0 + (id & 3), KB - 1);
+                const int row = id / KC, blk = min(kb0 + id % KC, KB - 1);
                 rb[i] = *(const u32x4 *)(qs + (size_t)min(n0 + row, N - 1) * (K >> 1) + (size_t)blk * 16);
             }
         }
 #pragma unroll
-        for (int i = 0; i < (BM3 * GI_KC + 255) / 256; ++i) {
-            const int id = tid + 256 * i, row = id / GI_KC, j = id % GI_KC;
-            ras[i] = (id < BM3 * GI_KC && kb0 + j < KB) ? a_scale[(size_t)min(m0 + row, M - 1) * KB + kb0 + j] : 0.f;   // past the end: no contribution
+        for (int i = 0; i < NAS; ++i) {
+            // unconditional loads at clamped addresses (a predicated load is waited for on the spot)
+            const int id = min(tid + 256 * i, BM3 * KC - 1), row = id / KC, j = id % KC;
+            ras[i] = a_scale[(size_t)min(m0 + row, M - 1) * KB + min(kb0 + j, KB - 1)];
         }
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int id = tid + 256 * i, row = id / GI_KC, j = id % GI_KC;
-            rws[i] = kb0 + j < KB ? __half2float(sc[(size_t)min(n0 + row, N - 1) * KB + kb0 + j]) : 0.f;
+        for (int i = 0; i < NWS; ++i) {
+            const int id = tid + 256 * i, row = id / KC, j = id % KC;
+            rws[i] = sc[(size_t)min(n0 + row, N - 1) * KB + min(kb0 + j, KB - 1)];
         }
     };
-    auto store_stage = [&](unsigned char *st) {
+    auto store_stage = [&](unsigned char *st, int kt) {
+        const int kb0 = kt * KC;
 #pragma unroll
         for (int i = 0; i < NAC; ++i) {
-            const int id = tid + 256 * i, row = id >> 3, part = id & 7;
-            *(u32x2 *)(st + row * GI_ROW + part * 16) = u32x2{ra[i].x, ra[i].y};
-            *(u32x2 *)(st + row * GI_ROW + part * 16 + 8) = u32x2{ra[i].z, ra[i].w};
+            const int id = tid + 256 * i, row = id / CPR, part = id % CPR;
+            *(u32x4 *)(st + row * ROW + part * 16) = ra[i];
         }
 #pragma unroll
         for (int i = 0; i < NBC; ++i) {
             const int id = tid + 256 * i;
             if (Q8) {
-                const int row = id >> 3, part = id & 7;
-                *(u32x2 *)(st + A_BYTES + row * GI_ROW + part * 16) = u32x2{rb[i].x, rb[i].y};
-                *(u32x2 *)(st + A_BYTES + row * GI_ROW + part * 16 + 8) = u32x2{rb[i].z, rb[i].w};
+                const int row = id / CPR, part = id % CPR;
+                *(u32x4 *)(st + A_BYTES + row * ROW + part * 16) = rb[i];
             } else {
                 // word w of the device layout holds elements 8w..8w+7: low nibbles 8w..8w+3, high nibbles 8w+4..8w+7
-                const int row = id >> 2, j = id & 3;
-                unsigned char *dst = st + A_BYTES + row * GI_ROW + j * 32;
+                const int row = id / KC, j = id % KC;
+                unsigned char *dst = st + A_BYTES + row * ROW + j * 32;
                 const unsigned ws4[4] = {rb[i].x, rb[i].y, rb[i].z, rb[i].w};
+                unsigned dec[8];
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
                     const unsigned lo = ws4[w] & 0x0F0F0F0Fu, hi = (ws4[w] >> 4) & 0x0F0F0F0Fu;
-                    *(u32x2 *)(dst + w * 8) = u32x2{((lo | 0x80808080u) - 0x08080808u) ^ 0x80808080u,
-                                                   ((hi | 0x80808080u) - 0x08080808u) ^ 0x80808080u};
+                    dec[2 * w] = ((lo | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
+                    dec[2 * w + 1] = ((hi | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
                 }
+                *(u32x4 *)dst = u32x4{dec[0], dec[1], dec[2], dec[3]};
+                *(u32x4 *)(dst + 16) = u32x4{dec[4], dec[5], dec[6], dec[7]};
             }
         }
         float *as_l = (float *)(st + A_BYTES + B_BYTES), *ws_l = (float *)(st + A_BYTES + B_BYTES + AS_BYTES);
 #pragma unroll
-        for (int i = 0; i < (BM3 * GI_KC + 255) / 256; ++i)
-            if (tid + 256 * i < BM3 * GI_KC) as_l[tid + 256 * i] = ras[i];
+        for (int i = 0; i < NAS; ++i)                            // blocks past the end of K: scale 0, no contribution
+            if (tid + 256 * i < BM3 * KC) as_l[tid + 256 * i] = kb0 + (tid + 256 * i) % KC < KB ? ras[i] : 0.f;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) ws_l[tid + 256 * i] = rws[i];
+        for (int i = 0; i < NWS; ++i) ws_l[tid + 256 * i] = kb0 + (tid + 256 * i) % KC < KB ? __half2float(rws[i]) : 0.f;
     };
 
     load_stage(0);
-    store_stage(lds3);
+    store_stage(lds3, 0);
     __syncthreads();
     for (int kt = 0; kt < KT; ++kt) {
         const unsigned char *st = lds3 + (kt & 1) * STAGE;
         const bool more = kt + 1 < KT;
         if (more) load_stage(kt + 1);
-        const f32x4 *as_l = (const f32x4 *)(st + A_BYTES + B_BYTES), *ws_l = (const f32x4 *)(st + A_BYTES + B_BYTES + AS_BYTES);
-        f32x4 wsc[4];
+        const float *as_l = (const float *)(st + A_BYTES + B_BYTES), *ws_l = (const float *)(st + A_BYTES + B_BYTES + AS_BYTES);
+        float wsc[4][KCW];
 #pragma unroll
-        for (int ni = 0; ni < 4; ++ni) wsc[ni] = ws_l[wn0 + ni * 16 + r];
-        // (row tile, block) steps, software-pipelined: the four dots of a step are issued, then the previous
-        // step's dots are rescaled while they run. The empty asm statements fix that order for the compiler,
-        // which otherwise issues every dot of the K step first and runs out of registers.
-        i32x4 dprev[4];
-        f32x4 asc[4], asc_prev[4];
+        for (int ni = 0; ni < 4; ++ni) {
+            if (SPLITK) {
 #pragma unroll
-        for (int t = 0; t <= WM * GI_KC; ++t) {
-            const int mi = t / GI_KC, j = t % GI_KC;
-            i32x4 dcur[4];
-            if (t < WM * GI_KC) {
-                if (j == 0) {
+                for (int jj = 0; jj < KCW; ++jj) wsc[ni][jj] = ws_l[(wn0 + ni * 16 + r) * KC + jw + 4 * jj];
+            } else {
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) asc[i] = as_l[wm0 + mi * 16 + g * 4 + i];
-                }
-                const long a = *(const long *)(st + (wm0 + mi * 16 + r) * GI_ROW + j * 32 + g * 8);
-#pragma unroll
-                for (int ni = 0; ni < 4; ++ni) {
-                    const long b = *(const long *)(st + A_BYTES + (wn0 + ni * 16 + r) * GI_ROW + j * 32 + g * 8);
-                    dcur[ni] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b, i32x4{0, 0, 0, 0}, 0, 0, 0);
+                for (int q = 0; q < KC / 4; ++q) {
+                    const f32x4 v = *(const f32x4 *)(ws_l + (wn0 + ni * 16 + r) * KC + q * 4);
+                    wsc[ni][q * 4 % KCW] = v.x; wsc[ni][(q * 4 + 1) % KCW] = v.y; wsc[ni][(q * 4 + 2) % KCW] = v.z; wsc[ni][(q * 4 + 3) % KCW] = v.w;
                 }
             }
-            if (t > 0) {
-                const int pm = (t - 1) / GI_KC, pj = (t - 1) % GI_KC;
+        }
+        // (row tile, block) steps, software-pipelined: a step's dots are issued one at a time between the
+        // rescales of the previous step's dots, so the matrix pipe runs under the vector work even with a
+        // single wavefront on the SIMD. The empty asm statements fix that order for the compiler, which
+        // otherwise issues every dot of the K step first and runs out of registers.
+        i32x4 dprev[4];
+        float asc[4][KCW];
 #pragma unroll
-                for (int ni = 0; ni < 4; ++ni) {
+        for (int t = 0; t <= WM * KCW; ++t) {
+            const int mi = t / KCW, jj = t % KCW;
+            const int pm = (t - 1) / KCW, pj = (t - 1) % KCW;
+            i32x4 dcur[4];
+            long a = 0;
+            if (t < WM * KCW) a = *(const long *)(st + (wm0 + mi * 16 + r) * ROW + (jw + jstep * jj) * 32 + g * 8);
+            if (t > 0 && pj == 0) {             // the previous row tile's activation scales
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) acc[pm][ni][i] += (float)dprev[ni][i] * (asc_prev[i][pj] * wsc[ni][pj]);
+                for (int i = 0; i < 4; ++i) {
+                    if (SPLITK) {
+#pragma unroll
+                        for (int q = 0; q < KCW; ++q) asc[i][q] = as_l[(wm0 + pm * 16 + g * 4 + i) * KC + jw + 4 * q];
+                    } else {
+#pragma unroll
+                        for (int q = 0; q < KC / 4; ++q) {
+                            const f32x4 v = *(const f32x4 *)(as_l + (wm0 + pm * 16 + g * 4 + i) * KC + q * 4);
+                            asc[i][q * 4 % KCW] = v.x; asc[i][(q * 4 + 1) % KCW] = v.y; asc[i][(q * 4 + 2) % KCW] = v.z; asc[i][(q * 4 + 3) % KCW] = v.w;
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int ni = 0; ni < 4; ++ni) {
+                if (t < WM * KCW) {
+                    const long b = *(const long *)(st + A_BYTES + (wn0 + ni * 16 + r) * ROW + (jw + jstep * jj) * 32 + g * 8);
+                    dcur[ni] = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b, i32x4{0, 0, 0, 0}, 0, 0, 0);
+                }
+                if (t > 0) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[pm][ni][i] += (float)dprev[ni][i] * (asc[i][pj] * wsc[ni][pj]);
                     asm volatile("" : "+v"(acc[pm][ni]));
                 }
             }
 #pragma unroll
             for (int ni = 0; ni < 4; ++ni) dprev[ni] = dcur[ni];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) asc_prev[i] = asc[i];
         }
-        if (more) store_stage(lds3 + ((kt + 1) & 1) * STAGE);
+        if (more) store_stage(lds3 + ((kt + 1) & 1) * STAGE, kt + 1);
         __syncthreads();
     }
 
+    if (SPLITK) {
+        // partial sums of the four wavefronts -> LDS (the stages are free: the loop ended on a barrier), then
+        // wavefront w adds column tile w in the fixed order 0,1,2,3 and writes it
+        f32x4 *red = (f32x4 *)lds3;                      // [wave][mi][ni][lane]
+#pragma unroll
+        for (int mi = 0; mi < WM; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 4; ++ni) red[((wave * WM + mi) * 4 + ni) * 64 + lane] = acc[mi][ni];
+        __syncthreads();
+#pragma unroll
+        for (int mi = 0; mi < WM; ++mi) {
+            f32x4 sum = red[((0 * WM + mi) * 4 + wave) * 64 + lane];
+#pragma unroll
+            for (int w = 1; w < 4; ++w) sum += red[((w * WM + mi) * 4 + wave) * 64 + lane];
+            const int col = n0 + wave * 16 + r;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int row = m0 + mi * 16 + g * 4 + i;
+                if (row >= M || col >= N) continue;
+                float *dst = c + (size_t)row * ldc + col;
+                const float v = alpha * sum[i];
+                *dst = beta == 0.f ? v : v + beta * *dst;
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int mi = 0; mi < WM; ++mi)
 #pragma unroll
@@ -485,18 +544,36 @@ __global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const unsigned shor
         }
 }
 
-template <int DT, int WM>
+template <int DT, int WM, int KC, bool SPLITK>
 int launch_i8_lds(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
-    constexpr int BM3 = 32 * WM;
-    constexpr int LDS = 2 * ((BM3 + 128) * GI_ROW + (BM3 + 128) * GI_KC * 4);
+    constexpr int BM3 = (SPLITK ? 16 : 32) * WM, BN3 = SPLITK ? 64 : 128;
+    constexpr int LDS = 2 * ((BM3 + BN3) * GiCfg<KC>::ROW + (BM3 + BN3) * KC * 4);
+    static_assert(LDS <= 160 * 1024, "two stages must fit the CU's LDS");
+    static_assert(!SPLITK || 4 * WM * 4 * 64 * 16 <= LDS, "the split-K reduction reuses the stages");
     static bool attr = false;
     if (!attr) {
-        HIP_TRY(ctx, hipFuncSetAttribute((const void *)gemm_i8_lds_kernel<DT, WM>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+        HIP_TRY(ctx, hipFuncSetAttribute((const void *)gemm_i8_lds_kernel<DT, WM, KC, SPLITK>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
         attr = true;
     }
-    const dim3 grid((unsigned)((w->n + 127) / 128), (unsigned)((m + BM3 - 1) / BM3));
-    launch_k(ctx, gemm_i8_lds_kernel<DT, WM>, grid, dim3(256), LDS, w->qs, w->sc, act.q, act.scale, c, (int)m, (int)w->n, (int)w->k, ldc, alpha, beta);
+    const dim3 grid((unsigned)((w->n + BN3 - 1) / BN3), (unsigned)((m + BM3 - 1) / BM3));
+    launch_k(ctx, gemm_i8_lds_kernel<DT, WM, KC, SPLITK>, grid, dim3(256), LDS, w->qs, w->sc, act.q, act.scale, c, (int)m, (int)w->n, (int)w->k, ldc, alpha, beta);
     return AIONHIP_OK;
+}
+
+template <int DT>
+int launch_i8_lds_pick(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
+    const long cus = ctx->cu_count > 0 ? ctx->cu_count : 256, tn = (long)((w->n + 127) / 128);
+    // 128-row tiles when they still give every CU a workgroup, else 64-, else 32-row tiles
+    const int wm = (long)((m + 127) / 128) * tn >= cus ? 4 : ((long)((m + 63) / 64) * tn >= cus ? 2 : 1);
+    if (wm == 4) return launch_i8_lds<DT, 4, 4, false>(ctx, w, m, act, c, ldc, alpha, beta);
+    if (wm == 2) return launch_i8_lds<DT, 2, 4, false>(ctx, w, m, act, c, ldc, alpha, beta);
+    if ((long)((m + 31) / 32) * tn >= 2 * cus || w->k < 512) return launch_i8_lds<DT, 1, 4, false>(ctx, w, m, act, c, ldc, alpha, beta);
+    // too few 32 x 128 tiles for two workgroups per CU: (16*WM) x 64 tiles with K split over the wavefronts,
+    // the tallest that still give two workgroups per CU
+    const long tn64 = (long)((w->n + 63) / 64);
+    if ((long)((m + 63) / 64) * tn64 >= 2 * cus) return launch_i8_lds<DT, 4, 8, true>(ctx, w, m, act, c, ldc, alpha, beta);
+    if ((long)((m + 31) / 32) * tn64 >= 2 * cus) return launch_i8_lds<DT, 2, 8, true>(ctx, w, m, act, c, ldc, alpha, beta);
+    return launch_i8_lds<DT, 1, 8, true>(ctx, w, m, act, c, ldc, alpha, beta);
 }
 
 template <int DT>
@@ -518,18 +595,8 @@ int launch_gemm_i8(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, Prepared
     const char *name = w->dtype == AIONHIP_Q8_0 ? "gemm_i8_q8" : "gemm_i8_q4";
     ProfScope scope(ctx, name);
     if (m > 16 && w->k >= 32) {
-        // 128-row tiles when they still give every CU a workgroup, else 64-, else 32-row tiles
-        const long cus = ctx->cu_count > 0 ? ctx->cu_count : 256, tn = (long)((w->n + 127) / 128);
-        const int wm = (long)((m + 127) / 128) * tn >= cus ? 4 : ((long)((m + 63) / 64) * tn >= cus ? 2 : 1);
-        int rc;
-        if (w->dtype == AIONHIP_Q8_0)
-            rc = wm == 4 ? launch_i8_lds<AIONHIP_Q8_0, 4>(ctx, w, m, act, c, ldc, alpha, beta)
-               : wm == 2 ? launch_i8_lds<AIONHIP_Q8_0, 2>(ctx, w, m, act, c, ldc, alpha, beta)
-                         : launch_i8_lds<AIONHIP_Q8_0, 1>(ctx, w, m, act, c, ldc, alpha, beta);
-        else
-            rc = wm == 4 ? launch_i8_lds<AIONHIP_Q4_0, 4>(ctx, w, m, act, c, ldc, alpha, beta)
-               : wm == 2 ? launch_i8_lds<AIONHIP_Q4_0, 2>(ctx, w, m, act, c, ldc, alpha, beta)
-                         : launch_i8_lds<AIONHIP_Q4_0, 1>(ctx, w, m, act, c, ldc, alpha, beta);
+        const int rc = w->dtype == AIONHIP_Q8_0 ? launch_i8_lds_pick<AIONHIP_Q8_0>(ctx, w, m, act, c, ldc, alpha, beta)
+                                                : launch_i8_lds_pick<AIONHIP_Q4_0>(ctx, w, m, act, c, ldc, alpha, beta);
         if (rc) return rc;
     } else if (w->dtype == AIONHIP_Q8_0) launch_i8<AIONHIP_Q8_0>(ctx, w, m, act, c, ldc, alpha, beta);
     else launch_i8<AIONHIP_Q4_0>(ctx, w, m, act, c, ldc, alpha, beta);
