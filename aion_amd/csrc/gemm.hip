@@ -560,20 +560,36 @@ int launch_i8_lds(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedA
     return AIONHIP_OK;
 }
 
+// Tile choice by a small cost model fitted to measurements on one MI355X (q4, K = 2048..8192, 24..2048
+// rows): a lone workgroup of each shape costs `us_per_block` per quant block of K; workgroups beyond one
+// per CU overlap by the factor `overlap` (two resident per CU hide each other's staging).
+struct GiShape { int wm; bool split; float us_per_block, overlap; };
+constexpr GiShape GI_SHAPES[6] = {
+    {4, false, 0.81f, 1.40f}, {2, false, 0.44f, 1.25f}, {1, false, 0.284f, 1.55f},
+    {4, true, 0.253f, 1.45f}, {2, true, 0.164f, 1.50f}, {1, true, 0.121f, 1.85f},
+};
 template <int DT>
 int launch_i8_lds_pick(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
-    const long cus = ctx->cu_count > 0 ? ctx->cu_count : 256, tn = (long)((w->n + 127) / 128);
-    // 128-row tiles when they still give every CU a workgroup, else 64-, else 32-row tiles
-    const int wm = (long)((m + 127) / 128) * tn >= cus ? 4 : ((long)((m + 63) / 64) * tn >= cus ? 2 : 1);
-    if (wm == 4) return launch_i8_lds<DT, 4, 4, false>(ctx, w, m, act, c, ldc, alpha, beta);
-    if (wm == 2) return launch_i8_lds<DT, 2, 4, false>(ctx, w, m, act, c, ldc, alpha, beta);
-    if ((long)((m + 31) / 32) * tn >= 2 * cus || w->k < 512) return launch_i8_lds<DT, 1, 4, false>(ctx, w, m, act, c, ldc, alpha, beta);
-    // too few 32 x 128 tiles for two workgroups per CU: (16*WM) x 64 tiles with K split over the wavefronts,
-    // the tallest that still give two workgroups per CU
-    const long tn64 = (long)((w->n + 63) / 64);
-    if ((long)((m + 63) / 64) * tn64 >= 2 * cus) return launch_i8_lds<DT, 4, 8, true>(ctx, w, m, act, c, ldc, alpha, beta);
-    if ((long)((m + 31) / 32) * tn64 >= 2 * cus) return launch_i8_lds<DT, 2, 8, true>(ctx, w, m, act, c, ldc, alpha, beta);
-    return launch_i8_lds<DT, 1, 8, true>(ctx, w, m, act, c, ldc, alpha, beta);
+    const float cus = (float)(ctx->cu_count > 0 ? ctx->cu_count : 256);
+    int best = 0;
+    float best_t = 0.f;
+    for (int i = 0; i < 6; ++i) {
+        const GiShape &g = GI_SHAPES[i];
+        if (g.split && w->k < 256) continue;             // a split-K step is 8 blocks
+        const size_t bm = (size_t)(g.split ? 16 : 32) * g.wm, bn = g.split ? 64 : 128;
+        const float wgs = (float)(((m + bm - 1) / bm) * ((w->n + bn - 1) / bn));
+        const float rounds = wgs / (cus * g.overlap);
+        const float t = g.us_per_block * (rounds > 1.f ? rounds : 1.f);
+        if (i == 0 || t < best_t) { best = i; best_t = t; }
+    }
+    switch (best) {
+    case 0: return launch_i8_lds<DT, 4, 4, false>(ctx, w, m, act, c, ldc, alpha, beta);
+    case 1: return launch_i8_lds<DT, 2, 4, false>(ctx, w, m, act, c, ldc, alpha, beta);
+    case 2: return launch_i8_lds<DT, 1, 4, false>(ctx, w, m, act, c, ldc, alpha, beta);
+    case 3: return launch_i8_lds<DT, 4, 8, true>(ctx, w, m, act, c, ldc, alpha, beta);
+    case 4: return launch_i8_lds<DT, 2, 8, true>(ctx, w, m, act, c, ldc, alpha, beta);
+    default: return launch_i8_lds<DT, 1, 8, true>(ctx, w, m, act, c, ldc, alpha, beta);
+    }
 }
 
 template <int DT>
