@@ -500,6 +500,18 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
     if (a.q_dtype == KV) {
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const u32x4 *)((const unsigned short *)a.q + qbase + kk * 16 + lh * 8);
+    } else if (a.q_dtype == AIONHIP_F32 && (((uintptr_t)a.q) & 15) == 0) {
+        // f32 queries (aion's decode graphs: f32 q over an f16 cache): 16-byte loads, all requested before the first is converted
+        f32x4 x0[KK], x1[KK];
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            const f32x4 *qp = (const f32x4 *)((const float *)a.q + qbase + kk * 16 + lh * 8);
+            x0[kk] = qp[0];
+            x1[kk] = qp[1];
+        }
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk)
+            qf[kk] = u32x4{pack2<KV>(x0[kk].x, x0[kk].y), pack2<KV>(x0[kk].z, x0[kk].w), pack2<KV>(x1[kk].x, x1[kk].y), pack2<KV>(x1[kk].z, x1[kk].w)};
     } else {
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) {
@@ -840,7 +852,11 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
     using Cfg = FlashCfg<D, 4>;
     using SplitCfg = FlashCfg<D, SPLIT_NW>;
     const int units = a.B * a.Hkv;
-    const bool split = a.rows_total <= 64;
+    // Few query rows, or so few 128-row prefill workgroups that they would occupy under a quarter of the CUs
+    // (measured: one batch, one kv head, up to ~1024 positions x 8 heads): 16-row tiles spread the K/V reads
+    // over many CUs, which outweighs re-reading K/V per row tile from L2.
+    const int cus0 = ctx->cu_count > 0 ? ctx->cu_count : 256;
+    const bool split = a.rows_total <= 64 || (!HILO && (long)units * ((a.rows_total + PF_ROWS - 1) / PF_ROWS) * 4 <= cus0);
     if (split) {
         // key segments: one 32-key tile per wavefront while that leaves the device under-filled,
         // more tiles per wavefront beyond one workgroup per CU (its LDS tiles fill a CU)

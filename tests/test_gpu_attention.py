@@ -57,14 +57,17 @@ def make_qkv(seed, B, L, T, Hq, Hkv, D, kind):
     return (qb, kb, vb, be.BF16, be.BF16), (qf, kf, vf)
 
 
+# A prompt whose 128-row workgroups would leave three quarters of the CUs idle runs on the 16-row split kernel;
+# L = 150 (2 x 2 units x 5 workgroups) is such a prompt, L = 560 (2 x 2 x 18) is not.
 @pytest.mark.parametrize("kind,tol", [("f16", 2e-3), ("bf16", 1e-2)])
 @pytest.mark.parametrize("D", [64, 128, 256])
-def test_prefill_causal_gqa(gpu, orc, kind, tol, D):
-    B, L, Hq, Hkv = 2, 150, 8, 2
-    say("prefill", kind, D)
+@pytest.mark.parametrize("L,kernel", [(150, "attn_flash_split"), (560, "attn_prefill")])
+def test_prefill_causal_gqa(gpu, orc, kind, tol, D, L, kernel):
+    B, Hq, Hkv = 2, 8, 2
+    say("prefill", kind, D, L)
     (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(D, B, L, L, Hq, Hkv, D, kind)
     got = run_attention(gpu, q, k, v, 1 / math.sqrt(D), qd, kd)
-    assert gpu.last_kernel() == "attn_prefill"
+    assert gpu.last_kernel() == kernel
     ref = orc.attention_f64(qf, kf, vf, 1 / math.sqrt(D))
     err = float(np.abs(got - ref).max())
     say("  max err", err)
@@ -208,23 +211,26 @@ def test_precise_mode_brings_f32_queries_to_f32_accuracy(gpu, orc):
 
 
 def test_prefill_config4_sizes(gpu, orc):
-    # BASELINE config 4a at L = 1024: 8 q heads / 1 kv head, head size 256, bf16, scale 1/16, causal; every row
-    # against the f64 reference (1e-2: bf16 MFMA operands). At L = 4096 the oracle is too slow, so the kernel is
-    # held to properties that do not depend on the size: V = const gives that const back (the probabilities of a
-    # row sum to one), and row 0 sees key 0 only.
-    say("prefill config 4 L1024")
-    (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(41, 1, 1024, 1024, 8, 1, 256, "bf16")
-    got = run_attention(gpu, q, k, v, 1 / 16.0, qd, kd)
-    assert gpu.last_kernel() == "attn_prefill"
-    ref = orc.attention_f64(qf, kf, vf, 1 / 16.0)
-    err = float(np.abs(got - ref).max())
-    say("  max err", err)
-    assert err < 1e-2
+    # BASELINE config 4a at L = 1024 and 2048: 8 q heads / 1 kv head, head size 256, bf16, scale 1/16, causal;
+    # every row against the f64 reference (1e-2: bf16 MFMA operands). L = 1024 is 64 prefill workgroups (a
+    # quarter of the CUs: split kernel), L = 2048 runs on the prefill kernel. At L = 4096 the oracle is too slow,
+    # so the kernel is held to properties that do not depend on the size: V = const gives that const back (the
+    # probabilities of a row sum to one), and row 0 sees key 0 only.
+    for L, kernel in ((1024, "attn_flash_split"), (2048, "attn_prefill")):
+        say("prefill config 4 L%d" % L)
+        (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(41, 1, L, L, 8, 1, 256, "bf16")
+        got = run_attention(gpu, q, k, v, 1 / 16.0, qd, kd)
+        assert gpu.last_kernel() == kernel
+        ref = orc.attention_f64(qf, kf, vf, 1 / 16.0)
+        err = float(np.abs(got - ref).max())
+        say("  max err", err)
+        assert err < 1e-2
     say("prefill config 4 L4096 properties")
     L = 4096
     (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(43, 1, L, L, 8, 1, 256, "bf16")
     ones, _ = to_bf16(np.full((1, L, 1, 256), 0.75, np.float32))
     got = run_attention(gpu, q, k, ones, 1 / 16.0, qd, kd)
+    assert gpu.last_kernel() == "attn_prefill"
     assert float(np.abs(got - 0.75).max()) < 1e-2
     got = run_attention(gpu, q, k, v, 1 / 16.0, qd, kd)
     # one visible key: its value (the single probability is exp2 of a rounding residue, 1 to within an ulp)
@@ -234,16 +240,21 @@ def test_prefill_config4_sizes(gpu, orc):
     assert float(np.abs(got[:, L - 16:] - ref_tail).max()) < 1e-2
 
 
-def test_prefill_chunk_with_positions_over_a_longer_cache(gpu, orc):
-    # a prompt chunk: 96 new rows at positions 160..255 over a cache of capacity 300 holding 256 keys
-    B, Lq, T, Hq, Hkv, D = 2, 96, 300, 8, 2, 128
+@pytest.mark.parametrize("B,Lq,T,lens,kernel", [
+    (2, 96, 300, [256, 200], "attn_flash_split"),                 # 96 new rows at positions 160..255, capacity 300
+    (4, 320, 520, [480, 400, 480, 170], "attn_prefill"),          # 320 new rows at positions 160..479, capacity 520
+])
+def test_prefill_chunk_with_positions_over_a_longer_cache(gpu, orc, B, Lq, T, lens, kernel):
+    # a prompt chunk: new rows at positions 160.. over a longer cache; the sequences see different key counts
+    Hq, Hkv, D = 8, 2, 128
+    filled = 160 + Lq
     (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(47, B, Lq, T, Hq, Hkv, D, "f16")
-    k[:, 256:] = np.float16(np.nan)                      # beyond the cache length: must not leak
-    v[:, 256:] = np.float16(np.nan)
-    pos = np.tile(np.arange(160, 256, dtype=np.int32), (B, 1))
-    lens = np.array([256, 200], np.int32)                # the second sequence sees keys < 200 only
+    k[:, filled:] = np.float16(np.nan)                   # beyond the cache length: must not leak
+    v[:, filled:] = np.float16(np.nan)
+    pos = np.tile(np.arange(160, filled, dtype=np.int32), (B, 1))
+    lens = np.array(lens, np.int32)
     got = run_attention(gpu, q, k, v, 1 / math.sqrt(D), qd, kd, positions=pos, kv_lengths=lens)
-    assert gpu.last_kernel() == "attn_prefill"
+    assert gpu.last_kernel() == kernel
     kz, vz = np.nan_to_num(kf), np.nan_to_num(vf)
     ref = orc.attention_f64(qf, kz, vz, 1 / math.sqrt(D), positions=pos, kv_lengths=lens)
     assert np.isfinite(got).all()
