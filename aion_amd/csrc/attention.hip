@@ -24,6 +24,7 @@
 #include "common.h"
 
 #include <climits>
+#include <type_traits>
 
 namespace {
 
@@ -116,7 +117,9 @@ struct FlashCfg {
     static constexpr int WAVE_LDS = TILE_KEYS * ROW_BYTES;       // one V tile per wavefront
     static constexpr int WG_LDS = NW * WAVE_LDS;
     static constexpr int MERGE_LDS = (NW * (16 * (D + 4) + 32) + 16 * NW + 32) * 4;   // split mode: NW x (acc[16][D+4], m[16], l[16]) f32 + merge factors
-    static constexpr int LDS_BYTES = WG_LDS > MERGE_LDS ? WG_LDS : MERGE_LDS;
+    static constexpr int Q_ROW = D * 2 + 64;                     // split mode: the 16 query rows in the K/V element type
+    static constexpr int Q_OFF = WG_LDS > MERGE_LDS ? WG_LDS : MERGE_LDS;
+    static constexpr int LDS_BYTES = Q_OFF + 16 * Q_ROW;
 };
 constexpr int SPLIT_NW = 8;
 
@@ -145,14 +148,39 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
     const bool row_ok = rt < a.row_tiles && r < a.rows_total;
     const int li = row_ok ? r / a.groups : 0, gi = row_ok ? r % a.groups : 0;
     const int hq = hk * a.groups + gi;
-    const int kv_end_raw = a.kv_lengths ? a.kv_lengths[b] : a.T;
-    const int pos_raw = (row_ok && a.positions) ? a.positions[(size_t)b * a.L + li] : li;
+    // The cache length is read with a vector load (a per-lane zero in the address keeps the compiler from
+    // turning it into a scalar load, which it would wait for on the spot): it is then in flight together with
+    // the position and the query loads instead of ahead of them.
+    // Both loads are unconditional (an absent operand reads a word of q instead and is replaced afterwards): a
+    // load under a branch is waited for at the end of its block.
+    const int lane_zero = (int)__builtin_amdgcn_mbcnt_lo(0u, 0u);
+    const int *len_p = a.kv_lengths ? a.kv_lengths + b : (const int *)a.q;
+    const int *pos_p = a.positions ? a.positions + ((size_t)b * a.L + li) : (const int *)a.q;
+    const int len_ld = len_p[lane_zero], pos_ld = *pos_p;
+    const int kv_end_raw = a.kv_lengths ? len_ld : a.T;
+    const int pos_raw = (row_ok && a.positions) ? pos_ld : li;
 
     const size_t qbase = (((size_t)b * a.L + li) * a.Hq + hq) * D;
     const bool q_f32_vec = a.q_dtype == AIONHIP_F32 && (((uintptr_t)a.q) & 15) == 0;
     const bool q_same = a.q_dtype == KV && (((uintptr_t)a.q) & 15) == 0;
     u32x4 qf[KK], qf_lo[HILO ? KK : 1];
     f32x4 qx0[KK], qx1[KK];
+    // split mode, f32 queries: every wavefront needs the same 16 rows, so the workgroup fetches them once
+    // (two 16-byte loads per thread instead of 2*KK per lane of every wavefront through the one L1), converts
+    // and shares them through LDS; the fragments are read back after the first tile's K/V loads are issued.
+    const bool q_shared = SPLIT && !HILO && q_f32_vec && D * 16 / 8 <= NW * 64;
+    f32x4 qs0 = f32x4{0.f, 0.f, 0.f, 0.f}, qs1 = qs0;
+    constexpr int QT = D / 8;                                    // threads per staged row (8 elements each)
+    const int qs_row = threadIdx.x / QT, qs_col = (threadIdx.x % QT) * 8;
+    if (q_shared) {
+        const int r2 = rt * 16 + qs_row;
+        if (qs_row < 16 && rt < a.row_tiles && r2 < a.rows_total) {
+            const int l2 = r2 / a.groups, g2 = r2 % a.groups;
+            const f32x4 *qp = (const f32x4 *)((const float *)a.q + (((size_t)b * a.L + l2) * a.Hq + hk * a.groups + g2) * D + qs_col);
+            qs0 = qp[0];
+            qs1 = qp[1];
+        }
+    } else
     if (q_same) {                    // already in the MFMA element type: one 16-byte load per k-step
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk)
@@ -178,6 +206,7 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
     // ---- Q^T operand: 8 consecutive d of row n per k-step, converted to the K/V element type
 #pragma unroll
     for (int kk = 0; kk < KK; ++kk) {
+        if (q_shared) break;
         if (q_same) {
             if (!row_ok) qf[kk] = u32x4{0u, 0u, 0u, 0u};
             if (HILO) qf_lo[kk] = u32x4{0u, 0u, 0u, 0u};
@@ -246,35 +275,71 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
     // anything, so the value must only be finite).
     constexpr int NVI = TILE_KEYS * D * 2 / 1024;
     constexpr int KEYS_PER_VI = 1024 / (D * 2);
+    // Addresses: while one batch entry's cache is under 2 GiB (a uniform test) a row is reached by a 32-bit byte
+    // offset from a uniform base - one 24-bit multiply-add per load instead of 64-bit arithmetic, which counts
+    // when a lone workgroup issues a whole short cache's loads.
+    const unsigned row_bytes = (unsigned)(kv_row * 2);
+    const bool near = (size_t)a.T * kv_row * 2 < ((size_t)1 << 31) && a.T < (1 << 24) && row_bytes < (1u << 24);
+    const unsigned char *kb8 = (const unsigned char *)(kp + kv_base), *vb8 = (const unsigned char *)(vp + kv_base);
     u32x4 kf[2][KK];
-    auto load_k = [&](int t) {
+    auto load_k_as = [&](int t, auto near_c) __attribute__((always_inline)) {
+        constexpr bool near = decltype(near_c)::value;
         const int key0 = t * TILE_KEYS;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int kabs = min(key0 + h * 16 + n, a.T - 1);
-            const unsigned short *krow = kp + kv_base + (size_t)kabs * kv_row + g * 8;
+            if (near) {
+                const unsigned char *krow = kb8 + (__umul24((unsigned)kabs, row_bytes) + (unsigned)g * 16u);
 #pragma unroll
-            for (int kk = 0; kk < KK; ++kk) kf[h][kk] = *(const u32x4 *)(krow + kk * 32);
+                for (int kk = 0; kk < KK; ++kk) kf[h][kk] = *(const u32x4 *)(krow + kk * 64);
+            } else {
+                const unsigned short *krow = kp + kv_base + (size_t)kabs * kv_row + g * 8;
+#pragma unroll
+                for (int kk = 0; kk < KK; ++kk) kf[h][kk] = *(const u32x4 *)(krow + kk * 32);
+            }
         }
     };
     const int v_key_in = (lane * 16) / (D * 2);                      // key of this lane within one V load
     const int v_slot = ((lane * 16) % (D * 2)) / 16;                 // its 16-byte slot within the key row
     const int v_hi_key = max(uni_hi - 1, 0);
-    auto load_v = [&](int t) {
+    auto load_k = [&](int t) __attribute__((always_inline)) {
+        if (near) load_k_as(t, std::true_type{});
+        else load_k_as(t, std::false_type{});
+    };
+    auto load_v_as = [&](int t, auto near_c) __attribute__((always_inline)) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the builtin exists in the device pass only
+        constexpr bool near = decltype(near_c)::value;
         const int key0 = t * TILE_KEYS;
 #pragma unroll
         for (int i = 0; i < NVI; ++i) {
             const int key = i * KEYS_PER_VI + v_key_in;
-            const int chunk = v_slot ^ (2 * ((key >> 2) & 3));
+            // (key >> 2) & 3 does not depend on the lane while an instruction covers at most four keys
+            const int grp = KEYS_PER_VI <= 4 ? ((i * KEYS_PER_VI) >> 2) & 3 : (key >> 2) & 3;
+            const int chunk = v_slot ^ (2 * grp);
             const int kabs = min(max(key0 + key, uni_lo), v_hi_key);
-            __builtin_amdgcn_global_load_lds(vp + kv_base + (size_t)kabs * kv_row + chunk * 8, (lds_void *)(vs + i * 1024), 16, 0, 0);
+            if (near)
+                __builtin_amdgcn_global_load_lds(vb8 + (__umul24((unsigned)kabs, row_bytes) + (unsigned)chunk * 16u), (lds_void *)(vs + i * 1024), 16, 0, 0);
+            else
+                __builtin_amdgcn_global_load_lds(vp + kv_base + (size_t)kabs * kv_row + chunk * 8, (lds_void *)(vs + i * 1024), 16, 0, 0);
         }
 #endif
+    };
+    auto load_v = [&](int t) __attribute__((always_inline)) {
+        if (near) load_v_as(t, std::true_type{});
+        else load_v_as(t, std::false_type{});
     };
     if (t_begin < t_end) {
         load_k(t_begin);
         load_v(t_begin);
+    }
+    if (q_shared) {
+        unsigned char *qsm = lds + Cfg::Q_OFF;
+        if (qs_row < 16)
+            *(u32x4 *)(qsm + qs_row * Cfg::Q_ROW + qs_col * 2) =
+                u32x4{pack2<KV>(qs0.x, qs0.y), pack2<KV>(qs0.z, qs0.w), pack2<KV>(qs1.x, qs1.y), pack2<KV>(qs1.z, qs1.w)};
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const u32x4 *)(qsm + n * Cfg::Q_ROW + kk * 64 + g * 16);
     }
     for (int t = t_begin; t < t_end; t += t_step) {
         const int key0 = t * TILE_KEYS;
@@ -389,34 +454,28 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
         if (g == 0) { w[16 * RS + n] = m_run; w[16 * RS + 16 + n] = l_run; }
     }
     __syncthreads();
-    // per (row, wavefront) weights exp2(m_w - m_all), once; kept behind the NW slots
-    float *fac = mg + NW * WSTRIDE;           // [16][NW] factors, then [16] m_all, [16] l_all
-    if (threadIdx.x < 16) {
-        const int row = threadIdx.x;
-        float m_all = -INFINITY;
-#pragma unroll
-        for (int w = 0; w < NW; ++w) m_all = fmaxf(m_all, mg[w * WSTRIDE + 16 * RS + row]);
-        float l_all = 0.f;
-#pragma unroll
-        for (int w = 0; w < NW; ++w) {
-            const float mw = mg[w * WSTRIDE + 16 * RS + row];
-            const float f = mw > -INFINITY ? exp2f((mw - m_all) * LOG2E) : 0.f;
-            fac[row * NW + w] = f;
-            l_all += mg[w * WSTRIDE + 16 * RS + 16 + row] * f;
-        }
-        fac[16 * NW + row] = m_all;
-        fac[16 * NW + 16 + row] = l_all;
-    }
-    __syncthreads();
+    // every thread derives the weights exp2(m_w - m_all) of its own row from the NW maxima (NW LDS reads that
+    // the sixteen lanes of a row share, NW exp2): cheaper than a serial pass by sixteen threads and a third barrier
     // partial slot layout in global memory (read by attn_merge_kernel): [16][D] o, [16] m, [16] l
     constexpr int PSTRIDE = 16 * D + 32;
     const size_t pslot = ((size_t)(unit * a.row_tiles + rt) * a.nseg + seg) * PSTRIDE;
     for (int e = threadIdx.x; e < 16 * D / 4; e += NW * 64) {
         const int row = e / (D / 4), col = (e % (D / 4)) * 4;
-        f32x4 o = f32x4{0.f, 0.f, 0.f, 0.f};
+        float mw[NW];
+        float m_all = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < NW; ++w) o += *(const f32x4 *)(mg + w * WSTRIDE + row * RS + col) * fac[row * NW + w];
-        const float l_all = fac[16 * NW + 16 + row];
+        for (int w = 0; w < NW; ++w) {
+            mw[w] = mg[w * WSTRIDE + 16 * RS + row];
+            m_all = fmaxf(m_all, mw[w]);
+        }
+        f32x4 o = f32x4{0.f, 0.f, 0.f, 0.f};
+        float l_all = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            const float f = mw[w] > -INFINITY ? exp2f((mw[w] - m_all) * LOG2E) : 0.f;
+            l_all += mg[w * WSTRIDE + 16 * RS + 16 + row] * f;
+            o += *(const f32x4 *)(mg + w * WSTRIDE + row * RS + col) * f;
+        }
         if (a.nseg == 1) {
             const int rr = rt * 16 + row;
             if (rr < a.rows_total) {
@@ -427,7 +486,7 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
         } else {
             *(f32x4 *)(a.partial + pslot + row * D + col) = o;
             if (col == 0) {
-                a.partial[pslot + 16 * D + row] = fac[16 * NW + row];
+                a.partial[pslot + 16 * D + row] = m_all;
                 a.partial[pslot + 16 * D + 16 + row] = l_all;
             }
         }
