@@ -219,3 +219,23 @@ def test_geglu_fusion_equals_the_separate_steps(gpu, orc, dtype, K, F):
         t.free()
     for w in (wg, wu, wd):
         w.free()
+
+
+def test_stream_read_probe_runs_and_checks_its_arguments(gpu):
+    # the measurement aid: reads only (the source and the sink stay as they were), 16-byte granularity enforced
+    data = np.arange(1 << 18, dtype=np.uint32)
+    src = gpu.upload(data)
+    sink = gpu.upload(np.array([7, 7, 7, 7], np.uint32))
+    gpu.profile_start()
+    gpu.probe_stream_read(src, 0, data.nbytes, sink)
+    gpu.probe_stream_read(src, 4096, 65536, sink)
+    gpu.probe_stream_read(src, 0, 0, sink)                       # nothing to read: no launch
+    prof = gpu.profile_stop()
+    assert [nm for nm, _ in prof] == ["stream_read", "stream_read"]
+    assert all(ms > 0 for _, ms in prof)
+    assert (gpu.download(src, np.uint32, data.shape) == data).all()
+    assert (gpu.download(sink, np.uint32, (4,)) == 7).all()
+    for off, nb in ((8, 64), (0, 24)):
+        with pytest.raises(be.AionHipError):
+            gpu.probe_stream_read(src, off, nb, sink)
+    src.free(); sink.free()
