@@ -184,6 +184,29 @@ def test_exact_path_rows_above_eight(gpu, orc, dtype, layout):
     w.free()
 
 
+# Shapes that exercise every workgroup shape of the LDS-staged exact kernel and its edges: K that is not a multiple
+# of the 4- or 8-block K step (the blocks past the end must contribute nothing), N that is not a multiple of the
+# 64/128-column tile, row counts around the 16/32/64/128-row tiles, alpha/beta on a pre-filled C.
+@pytest.mark.parametrize("dtype,layout", CASES)
+@pytest.mark.parametrize("m,n,k", [(17, 33, 32), (40, 130, 96), (130, 70, 288), (65, 1100, 1056), (300, 520, 800),
+                                   (128, 2048, 2048), (24, 8192, 2048), (1100, 2100, 544)])
+def test_exact_gemm_shapes_and_edges(gpu, orc, dtype, layout, m, n, k):
+    say("exact gemm edges", dtype, layout, m, n, k)
+    blocks, w = make_weight(gpu, orc, dtype, layout, n, k, seed=m + n + k, std=0.05)
+    rng = np.random.default_rng(m * 7 + k)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    c0 = rng.standard_normal((m, n)).astype(np.float32)
+    gpu.set_gemm_mode(be.GEMM_EXACT_I8)
+    got = gpu.matmul(w, a)
+    assert gpu.last_kernel() == ("gemm_i8_q8" if dtype == be.Q8_0 else "gemm_i8_q4")
+    want = oracle_matmul(orc, dtype, layout, a, blocks, n)
+    assert norm_err(got, want) < TOL and rms_err(got, want) < RMS_TOL
+    got2 = gpu.matmul(w, a, alpha=0.5, beta=-2.0, c=c0)
+    want2 = 0.5 * want - 2.0 * c0
+    assert rms_err(got2, want2) < RMS_TOL
+    w.free()
+
+
 def test_linearity_in_alpha_and_row_independence(gpu, orc):
     # size-independent properties: rows of A never interact (the one-row and the several-row kernels give a row
     # the same int8 codes and block dots; only the order of the f32 additions over lanes may differ); alpha
