@@ -207,6 +207,26 @@ def test_exact_gemm_shapes_and_edges(gpu, orc, dtype, layout, m, n, k):
     w.free()
 
 
+# 2..8 activation rows (gemv_rows_kernel): row counts that fill a 2-, 4- or 8-row instance only partly, N that is
+# not a multiple of the rows a wavefront works on, K of one LDS pass and K long enough to run as several K-range
+# launches (14336 at 8 rows), alpha/beta on a pre-filled C.
+@pytest.mark.parametrize("dtype,layout", CASES)
+@pytest.mark.parametrize("m,n,k", [(2, 70, 96), (3, 1001, 1056), (5, 333, 2048), (8, 1030, 14336), (7, 4100, 7200), (4, 9000, 512)])
+def test_decode_gemv_two_to_eight_rows(gpu, orc, dtype, layout, m, n, k):
+    say("gemv rows", dtype, layout, m, n, k)
+    blocks, w = make_weight(gpu, orc, dtype, layout, n, k, seed=m * 31 + n + k, std=0.05)
+    rng = np.random.default_rng(m + k)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    c0 = rng.standard_normal((m, n)).astype(np.float32)
+    got = gpu.matmul(w, a)
+    assert gpu.last_kernel() == ("gemv_q8" if dtype == be.Q8_0 else "gemv_q4")
+    want = oracle_matmul(orc, dtype, layout, a, blocks, n)
+    assert norm_err(got, want) < TOL and rms_err(got, want) < RMS_TOL
+    got2 = gpu.matmul(w, a, alpha=-1.5, beta=0.25, c=c0)
+    assert rms_err(got2, -1.5 * want + 0.25 * c0) < RMS_TOL
+    w.free()
+
+
 def test_linearity_in_alpha_and_row_independence(gpu, orc):
     # size-independent properties: rows of A never interact (the one-row and the several-row kernels give a row
     # the same int8 codes and block dots; only the order of the f32 additions over lanes may differ); alpha
