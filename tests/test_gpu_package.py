@@ -1,0 +1,96 @@
+"""A decoder `.aion` package (made by oracle/aion_writer.py) run through aion_amd/package.py on the GPU, against the
+CPU oracle decoder fed the same weights, teacher-forced, with the tolerance of tests/test_gpu_decoder.py (the GPU
+must be no further from the oracle than the oracle's own sensitivity to the exp it uses in attention); and against
+the fused step sequence of aion_amd/decoder.py, which must pick the same tokens from the same weights."""
+import sys
+
+import numpy as np
+import pytest
+
+from aion_amd import aion_file, backend as be
+from aion_amd.decoder import Decoder, DecoderConfig, SyntheticWeights, weight_shapes
+from aion_amd.package import PackageRunner, Unsupported
+from oracle import aion_writer
+
+pytestmark = pytest.mark.gpu
+
+SMALL = dict(layers=3, hidden=512, heads=8, kv_heads=1, head_dim=64, ffn=1024, vocab=2048, max_seq=48)
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def package_bytes(cfg, weights):
+    d = dict(layers=cfg.layers, hidden=cfg.hidden, heads=cfg.heads, kv_heads=cfg.kv_heads, head_dim=cfg.head_dim, ffn=cfg.ffn,
+             vocab=cfg.vocab, eps=cfg.eps, rope_base=cfg.rope_base, wdtype="q8_0" if cfg.wdtype == be.Q8_0 else "q4_0")
+    return aion_writer.build_decoder_package(d, weights.blocks, weights.embed())
+
+
+@pytest.mark.parametrize("wdtype", [be.Q4_0, be.Q8_0])
+def test_package_runs_like_the_oracle_decoder(gpu, orc, wdtype):
+    cfg = DecoderConfig(wdtype=wdtype, **SMALL)
+    weights = SyntheticWeights(cfg, 5)
+    pkg = aion_file.parse(package_bytes(cfg, weights))
+    mk = lambda exact: orc.Decoder(cfg.layers, cfg.hidden, cfg.heads, cfg.kv_heads, cfg.head_dim, cfg.ffn, cfg.vocab, cfg.max_seq,
+                                   eps=cfg.eps, rope_base=cfg.rope_base, wdtype=cfg.wdtype, threads=8, attn_exact=exact)
+    ref, alt = mk(False), mk(True)
+    ones = np.ones(cfg.hidden, np.float32)
+    for o in (ref, alt):
+        for name in weight_shapes(cfg):
+            o.set_weight(name, weights.blocks(name))
+        o.set_weight("embed", weights.embed())
+        for l in range(cfg.layers):
+            o.set_weight("l%d.norm1" % l, ones)
+            o.set_weight("l%d.norm2" % l, ones)
+        o.set_weight("norm_f", ones)
+    run = PackageRunner(gpu, pkg, capacity=cfg.max_seq)
+    fused = Decoder(gpu, cfg, weights)
+    try:
+        prompt = np.random.default_rng(9).integers(0, cfg.vocab, 16).astype(np.int32)
+        errs, selfs = [], []
+
+        def step(tokens, pos):
+            out = run.run(tokens, want=("next_token", "logits"))
+            logits, tok = out["logits"][0, -1], int(out["next_token"][0, -1])
+            (otok, ologits), (_, alogits) = ref.forward(tokens, pos), alt.forward(tokens, pos)
+            rms = float(np.sqrt((ologits.astype(np.float64) ** 2).mean()))
+            err, self_err = float(np.abs(logits - ologits).max()) / rms, float(np.abs(alogits - ologits).max()) / rms
+            top2 = np.sort(ologits)[-2:]
+            say("  pos %d: package max|err|/rms %.2e, cpu self-sensitivity %.2e, tokens %d / %d" % (pos, err, self_err, tok, otok))
+            if float(top2[1] - top2[0]) / rms > 2 * err:
+                assert tok == otok
+            errs.append(err); selfs.append(self_err)
+            return tok, logits
+
+        tok, logits = step(prompt, 0)
+        ftok = fused.prefill(prompt)
+        flogits = fused.logits_host()
+        # the fused step sequence sees the same weights: same arithmetic up to summation order
+        assert float(np.abs(flogits - logits).max()) <= 3 * max(selfs) * float(np.sqrt((logits.astype(np.float64) ** 2).mean())) + 1e-3
+        pos = prompt.size
+        for _ in range(6):
+            tok, _ = step(np.array([tok], np.int32), pos)
+            pos += 1
+        assert run.pos == pos
+        assert np.mean(errs) < 2 * np.mean(selfs) + 1e-3 and max(errs) < 3 * max(selfs) + 1e-3
+    finally:
+        run.close(); fused.close()
+
+
+def test_package_runner_refuses_what_the_backend_has_no_step_for(gpu):
+    b = aion_writer.PackageBuilder()
+    seq = b.symbol("seq")
+    x = b.input("tokens", "i32", (1, seq), role="tokens", axis=1)
+    table = b.initializer("f32", (8, 32), b.tensor_plain("f32", np.zeros((8, 32), np.float32)), "embed")
+    e = b.gather(table, x, (1, seq, 32))
+    y = b.unary("tanh", e, (1, seq, 32))
+    b.output("y", y)
+    pkg = aion_file.parse(b.to_bytes())
+    run = PackageRunner(gpu, pkg, capacity=8)
+    try:
+        with pytest.raises(Unsupported):
+            run.run(np.array([1, 2], np.int32), want=("y",))
+    finally:
+        run.close()
