@@ -3,8 +3,11 @@ backend's steps (the subset of aion's lowering `graph/program/compiler.zig:1052-
 needs). One device buffer per produced value; views alias their source; KV caches are the io-aliased inputs and
 stay on the device between runs (roles from the package's `input_roles`, `storage/aion_file/types.zig:164-198`).
 
-Mapping (node -> step), with the three places where consecutive nodes become one step because the step exists
-in that form only:
+A plan is built once per number of new tokens: buffers are allocated then, and a run only writes the inputs,
+issues the plan's steps and reads the outputs back. For one new token the plan can be recorded as a program
+(HIP graph) whose token, position, write index and visible end stay on the device (`begin_decode` / `decode_step`).
+
+Mapping (node -> step). Consecutive nodes become one step where the step exists in that form only:
   Gather axis 0                       -> aionhip_step_gather_rows
   RMSNorm (x, gamma, beta)            -> aionhip_step_rmsnorm
   MatMul (a, W)                       -> aionhip_step_matmul; W is a q4_0 [K,N] quant_axis 0 initializer, or
@@ -19,6 +22,17 @@ in that form only:
   ElemwiseBinary add                  -> aionhip_step_add
   ArgMax axis -1                      -> aionhip_step_argmax
 Anything else raises Unsupported: aion's placement pass keeps such ops on the CPU backend.
+
+On top of that, the step-level fusions of aion's schedule (graph/opt/fuse_steps.zig, graph/program/matmul_rows.zig)
+and this backend's optional fused steps, each found by walking the consumers of a node and applied only when every
+intermediate value has no other reader:
+  RMSNorm -> MatMul(s) on its output                          -> aionhip_step_rmsnorm_matmul
+  gelu(gate) * up -> MatMul                                   -> aionhip_step_gate_matmul
+  MatMul -> add(residual, .) whose residual is dead afterwards -> beta = 1 into the residual's buffer
+  one new token: RMSNorm -> MatMul q,k,v -> reshape -> RoPE1D(q,k) -> Cast -> SequenceAppend(k,v)
+                                                              -> aionhip_step_rmsnorm_qkv_rope_append
+  one new token: RMSNorm -> MatMul gate,up -> gelu*up -> MatMul down -> add(residual, .)
+                                                              -> aionhip_step_rmsnorm_geglu_matmul
 """
 import numpy as np
 
@@ -46,20 +60,31 @@ def _count(shape):
     return n
 
 
+_VIEWS = ("ViewReshape", "ViewSqueeze", "ViewUnsqueeze")
+_OUT = 1 << 30          # "consumer index" of a graph output
+
+
+class _Plan:
+    def __init__(self):
+        self.steps, self.buffers, self.inputs, self.outputs = [], [], {}, {}
+
+
 class PackageRunner:
-    def __init__(self, gpu, pkg, capacity, capacity_symbol="ctx", tokens_symbol="seq"):
-        self.gpu, self.pkg, self.capacity = gpu, pkg, int(capacity)
+    def __init__(self, gpu, pkg, capacity, capacity_symbol="ctx", tokens_symbol="seq", fuse=True):
+        self.gpu, self.pkg, self.capacity, self.fuse = gpu, pkg, int(capacity), fuse
         self.sym_ctx, self.sym_seq = capacity_symbol, tokens_symbol
         self.pos = 0
-        self.consts = {}            # value id -> _Val of an uploaded initializer
+        self.consts = {}            # (value id, transposed) -> _Val of an uploaded initializer
         self.caches = {}            # input index -> device buffer
-        self.consumers = {}
-        for n in pkg.nodes:
-            for i in n.inputs:
-                self.consumers[i] = self.consumers.get(i, 0) + 1
+        self.plans = {}             # new tokens per run -> _Plan
+        self.program = None
+        self.one = None
+        self.uses = {}
+        for i, n in enumerate(pkg.nodes):
+            for v in n.inputs:
+                self.uses.setdefault(v, []).append(i)
         for _name, vid in pkg.outputs:
-            self.consumers[vid] = self.consumers.get(vid, 0) + 1
-        self.producer = {n.output: n for n in pkg.nodes}
+            self.uses.setdefault(vid, []).append(_OUT)
         self.roles = {}
         for idx, (_name, vid) in enumerate(pkg.inputs):
             role = pkg.role_of_input(idx)
@@ -105,46 +130,37 @@ class PackageRunner:
         self.consts[key] = val
         return val
 
-    # ---- one run
-    def run(self, tokens, want=("next_token",)):
-        """Feeds `tokens` (int32 [S]) at positions pos..pos+S-1, runs the graph, advances pos. Returns the
-        requested outputs (by signature name) as numpy arrays."""
-        g, pkg = self.gpu, self.pkg
-        tokens = np.ascontiguousarray(tokens, np.int32).reshape(-1)
-        s = tokens.size
-        if self.pos + s > self.capacity:
-            raise ValueError("the run exceeds the cache capacity")
+    # ---- planning
+    def _plan(self, s):
+        if s in self.plans:
+            return self.plans[s]
+        g, pkg, nodes, uses = self.gpu, self.pkg, self.pkg.nodes, self.uses
         sym = {self.sym_seq: s, self.sym_ctx: self.capacity}
-        vals, temps = {}, []
+        plan = _Plan()
+        vals, skip = {}, set()
+        producer = {n.output: i for i, n in enumerate(nodes)}
 
         def new(shape, dtype):
             buf = g.alloc(max(_count(shape) * _ELEM[dtype], 4))
-            temps.append(buf)
+            plan.buffers.append(buf)
             return buf
+
+        def emit(fn, *args, **kw):
+            plan.steps.append((fn, args, kw))
 
         for vid, (idx, role) in self.roles.items():
             shape = pkg.shape_of(vid, sym)
-            if role.kind == "tokens":
-                arr = tokens
-            elif role.kind == "positions":
-                arr = np.arange(self.pos, self.pos + s, dtype=np.int32)
-            elif role.kind == "cache_write_index":
-                arr = np.array([self.pos], np.int32)
-            elif role.kind == "cache_visible_end":
-                arr = np.array([self.pos + s], np.int32)
-            elif role.kind == "sequence_cache":
+            if role.kind == "sequence_cache":
                 vals[vid] = _Val("dev", self.caches[idx], shape, "f16")
                 continue
-            else:
+            if role.kind not in ("tokens", "positions", "cache_write_index", "cache_visible_end"):
                 raise Unsupported("input role %s" % role.kind)
-            if _count(shape) != arr.size:
-                raise PackageError("InvalidArgument", "input %d: shape %s for %d elements" % (idx, shape, arr.size))
-            buf = g.upload(arr)
-            temps.append(buf)
+            buf = new(shape, "i32")
+            plan.inputs[role.kind] = (buf, shape)
             vals[vid] = _Val("dev", buf, shape, "i32")
 
         def get(vid):
-            """The device value of `vid`, materialising a pending cast."""
+            """The device value of `vid`; a pending cast is materialised."""
             if vid not in vals:
                 if pkg.values[vid].source != "initializer":
                     raise PackageError("InvalidFormat", "value %d is read before it is produced" % vid)
@@ -153,138 +169,388 @@ class PackageRunner:
             if v.kind == "cast":
                 src = get(v.extra)
                 out = new(v.shape, "f16")
-                g.step_cast_f32_f16(out, src.buf, _count(v.shape))
+                emit(g.step_cast_f32_f16, out, src.buf, _count(v.shape))
                 v = vals[vid] = _Val("dev", out, v.shape, "f16")
             elif v.kind == "gelu":
                 raise Unsupported("a gelu that does not feed a multiply (aion's gate step)")
             return v
 
-        try:
-            for n in pkg.nodes:
-                shape = pkg.shape_of(n.output, sym)
-                dtype = pkg.values[n.output].dtype
-                op, a = n.op, n.attrs
-                if op == "Gather":
-                    table, ids = get(n.inputs[0]), get(n.inputs[1])
-                    if a["axis"] != 0 or a["batch_dims"] != 0 or len(table.shape) != 2 or table.dtype != "f32":
-                        raise Unsupported("Gather other than rows of an f32 table")
-                    out = new(shape, "f32")
-                    g.step_gather_rows(be.F32, out, table.buf, ids.buf, _count(ids.shape), table.shape[1], table.shape[0])
-                    vals[n.output] = _Val("dev", out, shape, "f32")
-                elif op == "RMSNorm":
-                    x, gamma, beta = get(n.inputs[0]), get(n.inputs[1]), get(n.inputs[2])
-                    cols = 1
-                    for t in a["normalized_shape"]:
-                        cols *= pkg.dim_term(t, sym)
-                    if cols != x.shape[-1]:
-                        raise Unsupported("RMSNorm over more than the last axis")
-                    out = new(shape, "f32")
-                    g.step_rmsnorm(out, x.buf, gamma.buf, _count(x.shape) // cols, cols, a["eps"], beta=beta.buf)
-                    vals[n.output] = _Val("dev", out, shape, "f32")
-                elif op == "ViewTranspose2D":
-                    src = n.inputs[0]
-                    if pkg.values[src].source != "initializer":
-                        raise Unsupported("ViewTranspose2D of a computed value")
-                    vals[n.output] = self._const(src, transposed=True)
-                elif op == "MatMul":
-                    x = get(n.inputs[0])
-                    w = vals[n.inputs[1]] if n.inputs[1] in vals else self._const(n.inputs[1])
-                    if w.kind != "weight":
-                        raise Unsupported("MatMul whose right operand is not a quantized weight")
-                    if a["beta"] != 0.0:
-                        raise Unsupported("MatMul with beta != 0 in a package")
-                    out = new(shape, "f32")
-                    g.step_matmul(w.buf, x.buf, _count(x.shape[:-1]), out, alpha=a["alpha"])
-                    vals[n.output] = _Val("dev", out, shape, "f32")
-                elif op in ("ViewReshape", "ViewSqueeze", "ViewUnsqueeze"):
-                    x = get(n.inputs[0])
-                    if _count(shape) != _count(x.shape):
-                        raise PackageError("InvalidFormat", "view changes the element count")
-                    vals[n.output] = _Val("dev", x.buf, shape, x.dtype)
-                elif op == "RoPE1D":
-                    x, pos = get(n.inputs[0]), get(n.inputs[1])
-                    if len(x.shape) != 4:
-                        raise Unsupported("RoPE1D on rank %d" % len(x.shape))
-                    out = new(shape, "f32")
-                    g.step_rope(out, x.buf, pos.buf, x.shape[0], x.shape[1], x.shape[2], x.shape[3], base=a["base_frequency"],
-                                scale_factor=a["scale_factor"], proportion=a["rope_proportion"])
-                    vals[n.output] = _Val("dev", out, shape, "f32")
-                elif op == "Cast":
-                    if a["to_dtype"] != "f16" or pkg.values[n.inputs[0]].dtype != "f32":
-                        raise Unsupported("Cast other than f32 -> f16")
-                    vals[n.output] = _Val("cast", None, shape, "f16", extra=n.inputs[0])
-                elif op == "SequenceAppend":
-                    cache, widx = get(n.inputs[0]), get(n.inputs[2])
-                    newv = vals.get(n.inputs[1])
-                    if newv is None or newv.kind != "cast":
-                        raise Unsupported("SequenceAppend whose new rows are not a Cast f32 -> f16")
-                    src = get(newv.extra)
-                    bsz, t_cap = cache.shape[0], cache.shape[1]
-                    g.step_append_f16(cache.buf, src.buf, widx.buf, bsz, newv.shape[1], t_cap, _count(cache.shape[2:]))
-                    vals[n.output] = _Val("dev", cache.buf, shape, "f16")
-                elif op == "Attention":
-                    q, k, v = get(n.inputs[0]), get(n.inputs[1]), get(n.inputs[2])
-                    rest = list(n.inputs[3:])
-                    pos = get(rest.pop(0)) if a["has_query_positions"] else None
-                    lens = get(rest.pop(0)) if a["has_kv_lengths"] else None
-                    w = a["window"]
-                    out = new(shape, "f32")
-                    dts = {"f32": be.F32, "f16": be.F16}
-                    g.step_attention(out, q.buf, k.buf, v.buf,
-                                     (q.shape[0], q.shape[1], k.shape[1], q.shape[2], k.shape[2], q.shape[3], v.shape[3]), a["scale"],
-                                     q_dtype=dts[q.dtype], kv_dtype=dts[k.dtype], window=(w["left"], w["right"], w["chunk"]),
-                                     soft_cap=a["soft_cap"], query_positions=pos.buf if pos else None,
-                                     kv_lengths=lens.buf if lens else None)
-                    vals[n.output] = _Val("dev", out, shape, "f32")
-                elif op == "Unary":
-                    if a["op"] != "gelu":
-                        raise Unsupported("Unary %s" % a["op"])
-                    vals[n.output] = _Val("gelu", None, shape, "f32", extra=n.inputs[0])
-                elif op == "ElemwiseBinary":
-                    if a["op"] == "add":
-                        x, y = get(n.inputs[0]), get(n.inputs[1])
-                        if x.shape != y.shape:
-                            raise Unsupported("broadcasting add")
-                        out = new(shape, "f32")
-                        g.step_add(out, x.buf, y.buf, _count(shape))
-                    elif a["op"] == "mul":
-                        lhs = vals.get(n.inputs[0])
-                        if lhs is None or lhs.kind != "gelu":
-                            raise Unsupported("a multiply that is not gelu(gate) * up")
-                        gate, up = get(lhs.extra), get(n.inputs[1])
-                        out = new(shape, "f32")
-                        g.step_gate_gelu(out, gate.buf, up.buf, _count(shape))
-                    else:
-                        raise Unsupported("ElemwiseBinary %s" % a["op"])
-                    vals[n.output] = _Val("dev", out, shape, "f32")
-                elif op == "ArgMax":
-                    x = get(n.inputs[0])
-                    if a["axis"] not in (-1, len(x.shape) - 1):
-                        raise Unsupported("ArgMax over an inner axis")
-                    out = new(shape, "i32")
-                    g.step_argmax(out, x.buf, _count(x.shape[:-1]), x.shape[-1])
-                    vals[n.output] = _Val("dev", out, shape, "i32")
-                else:
-                    raise Unsupported("operation %s has no step on this backend" % op)
+        def weight_of(vid):
+            if vid in vals:
+                w = vals[vid]
+            elif vid in producer and nodes[producer[vid]].op == "ViewTranspose2D":
+                src = nodes[producer[vid]].inputs[0]
+                if pkg.values[src].source != "initializer":
+                    return None
+                w = vals[vid] = self._const(src, transposed=True)
+                skip.add(producer[vid])
+            elif pkg.values[vid].source == "initializer":
+                w = self._const(vid)
+            else:
+                return None
+            return w if w.kind == "weight" else None
 
-            result = {}
-            for name, vid in pkg.outputs:
-                if name in want:
-                    v = get(vid)
-                    result[name] = g.download(v.buf, {"f32": np.float32, "i32": np.int32, "f16": np.float16}[v.dtype], v.shape)
+        def sole_user(vid, op=None):
+            """The one node that reads `vid` (None if it has several readers or is a graph output)."""
+            u = uses.get(vid, [])
+            if len(u) != 1 or u[0] == _OUT:
+                return None
+            return u[0] if op is None or nodes[u[0]].op in (op if isinstance(op, tuple) else (op,)) else None
+
+        def residual_of(add_idx, produced_vid):
+            """For add(res, produced) / add(produced, res): the value id of res if the sum may overwrite res."""
+            n = nodes[add_idx]
+            if n.op != "ElemwiseBinary" or n.attrs["op"] != "add" or produced_vid not in n.inputs or n.inputs[0] == n.inputs[1]:
+                return None
+            res = n.inputs[1] if n.inputs[0] == produced_vid else n.inputs[0]
+            rv = vals.get(res)
+            if rv is None or rv.kind != "dev" or not rv.owned or rv.dtype != "f32":
+                return None
+            if any(u > add_idx or (u != add_idx and nodes[u].op in _VIEWS + ("SequenceAppend",)) for u in uses.get(res, [])):
+                return None
+            if pkg.shape_of(res, sym) != pkg.shape_of(n.output, sym):
+                return None
+            return res
+
+        def matmul_nodes_on(h_vid):
+            """All readers of h are MatMuls with h on the left and a quantized weight on the right: their indices."""
+            u = uses.get(h_vid, [])
+            if not u or _OUT in u:
+                return None
+            out = []
+            for i in u:
+                n = nodes[i]
+                if n.op != "MatMul" or n.inputs[0] != h_vid or n.attrs["beta"] != 0.0 or n.attrs["alpha"] != 1.0 or weight_of(n.inputs[1]) is None:
+                    return None
+                out.append(i)
+            return out if len(set(weight_of(nodes[i].inputs[1]).dtype for i in out)) == 1 else None
+
+        def try_qkv(i, mms):
+            """One new token: RMSNorm -> q,k,v -> reshape -> RoPE1D(q,k) -> Cast -> SequenceAppend(k,v)."""
+            if s != 1 or len(mms) != 3:
+                return False
+            n0 = nodes[i]
+            x = get(n0.inputs[0])
+            if x.shape[0] != 1 or x.shape[-1] > 4096:
+                return False
+            chains = {}
+            for m in mms:
+                r = sole_user(nodes[m].output, "ViewReshape")
+                if r is None or len(pkg.shape_of(nodes[r].output, sym)) != 4:
+                    return False
+                nxt = sole_user(nodes[r].output)
+                if nxt is None:
+                    return False
+                if nodes[nxt].op == "RoPE1D":
+                    rope = nxt
+                    after = sole_user(nodes[rope].output)
+                    if after is None:
+                        return False
+                    if nodes[after].op == "Attention" and nodes[after].inputs[0] == nodes[rope].output:
+                        chains["q"] = (m, r, rope)
+                    elif nodes[after].op == "Cast":
+                        app = sole_user(nodes[after].output, "SequenceAppend")
+                        if app is None or nodes[app].inputs[1] != nodes[after].output:
+                            return False
+                        chains["k"] = (m, r, rope, after, app)
+                    else:
+                        return False
+                elif nodes[nxt].op == "Cast":
+                    app = sole_user(nodes[nxt].output, "SequenceAppend")
+                    if app is None or nodes[app].inputs[1] != nodes[nxt].output:
+                        return False
+                    chains["v"] = (m, r, nxt, app)
+                else:
+                    return False
+            if set(chains) != {"q", "k", "v"}:
+                return False
+            rq, rk = nodes[chains["q"][2]], nodes[chains["k"][2]]
+            ak, av = nodes[chains["k"][4]], nodes[chains["v"][3]]
+            if rq.attrs != rk.attrs or rq.inputs[1] != rk.inputs[1] or ak.inputs[2] != av.inputs[2]:
+                return False
+            if any(nodes[c].attrs["to_dtype"] != "f16" for c in (chains["k"][3], chains["v"][2])):
+                return False
+            qs, ks = pkg.shape_of(rq.output, sym), pkg.shape_of(rk.output, sym)
+            if qs[:2] != (1, 1) or ks[:2] != (1, 1) or qs[3] != ks[3] or qs[3] % 8:
+                return False
+            kc, vc = get(ak.inputs[0]), get(av.inputs[0])
+            if kc.shape != vc.shape or kc.shape[2:] != ks[2:] or kc.dtype != "f16":
+                return False
+            gamma, beta = get(n0.inputs[1]), get(n0.inputs[2])
+            q_out = new(qs, "f32")
+            emit(g.step_rmsnorm_qkv_rope_append, weight_of(nodes[chains["q"][0]].inputs[1]).buf, weight_of(nodes[chains["k"][0]].inputs[1]).buf,
+                 weight_of(nodes[chains["v"][0]].inputs[1]).buf, x.buf, gamma.buf, n0.attrs["eps"], q_out, kc.buf, vc.buf,
+                 get(rq.inputs[1]).buf, get(ak.inputs[2]).buf, kc.shape[1], qs[2], ks[2], qs[3], base=rq.attrs["base_frequency"],
+                 scale_factor=rq.attrs["scale_factor"], proportion=rq.attrs["rope_proportion"], beta_norm=beta.buf)
+            vals[rq.output] = _Val("dev", q_out, qs, "f32", owned=True)
+            vals[ak.output] = _Val("dev", kc.buf, kc.shape, "f16")
+            vals[av.output] = _Val("dev", vc.buf, vc.shape, "f16")
+            for c in chains.values():
+                skip.update(c)
+            return True
+
+        def try_geglu(i, mms):
+            """One new token: RMSNorm -> gate, up -> gelu(gate) * up -> down -> add(residual, .)."""
+            if s != 1 or len(mms) != 2:
+                return False
+            n0 = nodes[i]
+            x = get(n0.inputs[0])
+            if _count(x.shape[:-1]) != 1 or x.shape[-1] > 4096:
+                return False
+            ge = [m for m in mms if sole_user(nodes[m].output, "Unary") is not None]
+            if len(ge) != 1:
+                return False
+            mg = ge[0]
+            mu = mms[0] if mms[1] == mg else mms[1]
+            un = sole_user(nodes[mg].output, "Unary")
+            if nodes[un].attrs["op"] != "gelu":
+                return False
+            mul = sole_user(nodes[un].output, "ElemwiseBinary")
+            if mul is None or nodes[mul].attrs["op"] != "mul" or nodes[mul].inputs != (nodes[un].output, nodes[mu].output):
+                return False
+            if sole_user(nodes[mu].output) != mul:
+                return False
+            md = sole_user(nodes[mul].output, "MatMul")
+            if md is None or nodes[md].inputs[0] != nodes[mul].output or nodes[md].attrs["beta"] != 0.0 or nodes[md].attrs["alpha"] != 1.0:
+                return False
+            wd = weight_of(nodes[md].inputs[1])
+            add = sole_user(nodes[md].output, "ElemwiseBinary")
+            if wd is None or add is None:
+                return False
+            res = residual_of(add, nodes[md].output)
+            wg, wu = weight_of(nodes[mg].inputs[1]), weight_of(nodes[mu].inputs[1])
+            if res is None or wg.shape != wu.shape or wg.shape[1] % 32 or wd.dtype != wg.dtype:
+                return False
+            gamma, beta = get(n0.inputs[1]), get(n0.inputs[2])
+            rv = vals[res]
+            emit(g.step_rmsnorm_geglu_matmul, wg.buf, wu.buf, wd.buf, x.buf, gamma.buf, n0.attrs["eps"], rv.buf, beta=1.0, beta_norm=beta.buf)
+            vals[nodes[add].output] = _Val("dev", rv.buf, rv.shape, "f32", owned=True)
+            skip.update((mg, mu, un, mul, md, add))
+            return True
+
+        def matmul_into(out_vid, launch):
+            """Emits `launch(c_buf, beta)` for a matmul-like step producing `out_vid`, folding a following residual add."""
+            shape = pkg.shape_of(out_vid, sym)
+            add = sole_user(out_vid, "ElemwiseBinary") if self.fuse else None
+            res = residual_of(add, out_vid) if add is not None else None
+            if res is not None:
+                rv = vals[res]
+                launch(rv.buf, 1.0)
+                vals[nodes[add].output] = _Val("dev", rv.buf, rv.shape, "f32", owned=True)
+                skip.add(add)
+            else:
+                out = new(shape, "f32")
+                launch(out, 0.0)
+                vals[out_vid] = _Val("dev", out, shape, "f32", owned=True)
+
+        for i, n in enumerate(nodes):
+            if i in skip:
+                continue
+            shape = pkg.shape_of(n.output, sym)
+            op, a = n.op, n.attrs
+            if op == "Gather":
+                table, ids = get(n.inputs[0]), get(n.inputs[1])
+                if a["axis"] != 0 or a["batch_dims"] != 0 or len(table.shape) != 2 or table.dtype != "f32":
+                    raise Unsupported("Gather other than rows of an f32 table")
+                out = new(shape, "f32")
+                emit(g.step_gather_rows, be.F32, out, table.buf, ids.buf, _count(ids.shape), table.shape[1], table.shape[0])
+                vals[n.output] = _Val("dev", out, shape, "f32", owned=True)
+            elif op == "RMSNorm":
+                x, gamma, beta = get(n.inputs[0]), get(n.inputs[1]), get(n.inputs[2])
+                cols = 1
+                for t in a["normalized_shape"]:
+                    cols *= pkg.dim_term(t, sym)
+                if cols != x.shape[-1]:
+                    raise Unsupported("RMSNorm over more than the last axis")
+                rows = _count(x.shape) // cols
+                mms = matmul_nodes_on(n.output) if self.fuse else None
+                if mms and (try_qkv(i, mms) or try_geglu(i, mms)):
+                    continue
+                if mms and len(mms) <= 4:
+                    ws = [weight_of(nodes[m].inputs[1]).buf for m in mms]
+                    outs = [new(pkg.shape_of(nodes[m].output, sym), "f32") for m in mms]
+                    emit(g.step_rmsnorm_matmul, ws, x.buf, gamma.buf, rows, outs, a["eps"], beta_norm=beta.buf)
+                    for m, o in zip(mms, outs):
+                        vals[nodes[m].output] = _Val("dev", o, pkg.shape_of(nodes[m].output, sym), "f32", owned=True)
+                    skip.update(mms)
+                    continue
+                out = new(shape, "f32")
+                emit(g.step_rmsnorm, out, x.buf, gamma.buf, rows, cols, a["eps"], beta=beta.buf)
+                vals[n.output] = _Val("dev", out, shape, "f32", owned=True)
+            elif op == "ViewTranspose2D":
+                if weight_of(n.output) is None:
+                    raise Unsupported("ViewTranspose2D of anything but a quantized weight")
+            elif op == "MatMul":
+                x, w = get(n.inputs[0]), weight_of(n.inputs[1])
+                if w is None:
+                    raise Unsupported("MatMul whose right operand is not a quantized weight")
+                if a["beta"] != 0.0:
+                    raise Unsupported("MatMul with beta != 0 in a package")
+                m_rows, alpha = _count(x.shape[:-1]), a["alpha"]
+                matmul_into(n.output, lambda c, beta, w=w, x=x, m_rows=m_rows, alpha=alpha:
+                            emit(g.step_matmul, w.buf, x.buf, m_rows, c, alpha=alpha, beta=beta))
+            elif op in _VIEWS:
+                x = get(n.inputs[0])
+                if _count(shape) != _count(x.shape):
+                    raise PackageError("InvalidFormat", "view changes the element count")
+                vals[n.output] = _Val("dev", x.buf, shape, x.dtype)
+            elif op == "RoPE1D":
+                x, pos = get(n.inputs[0]), get(n.inputs[1])
+                if len(x.shape) != 4:
+                    raise Unsupported("RoPE1D on rank %d" % len(x.shape))
+                out = new(shape, "f32")
+                emit(g.step_rope, out, x.buf, pos.buf, x.shape[0], x.shape[1], x.shape[2], x.shape[3], base=a["base_frequency"],
+                     scale_factor=a["scale_factor"], proportion=a["rope_proportion"])
+                vals[n.output] = _Val("dev", out, shape, "f32", owned=True)
+            elif op == "Cast":
+                if a["to_dtype"] != "f16" or pkg.values[n.inputs[0]].dtype != "f32":
+                    raise Unsupported("Cast other than f32 -> f16")
+                vals[n.output] = _Val("cast", None, shape, "f16", extra=n.inputs[0])
+            elif op == "SequenceAppend":
+                cache, widx = get(n.inputs[0]), get(n.inputs[2])
+                newv = vals.get(n.inputs[1])
+                if newv is None or newv.kind != "cast":
+                    raise Unsupported("SequenceAppend whose new rows are not a Cast f32 -> f16")
+                src = get(newv.extra)
+                emit(g.step_append_f16, cache.buf, src.buf, widx.buf, cache.shape[0], newv.shape[1], cache.shape[1], _count(cache.shape[2:]))
+                vals[n.output] = _Val("dev", cache.buf, shape, "f16")
+            elif op == "Attention":
+                q, k, v = get(n.inputs[0]), get(n.inputs[1]), get(n.inputs[2])
+                rest = list(n.inputs[3:])
+                pos = get(rest.pop(0)) if a["has_query_positions"] else None
+                lens = get(rest.pop(0)) if a["has_kv_lengths"] else None
+                w = a["window"]
+                out = new(shape, "f32")
+                dts = {"f32": be.F32, "f16": be.F16}
+                emit(g.step_attention, out, q.buf, k.buf, v.buf,
+                     (q.shape[0], q.shape[1], k.shape[1], q.shape[2], k.shape[2], q.shape[3], v.shape[3]), a["scale"],
+                     q_dtype=dts[q.dtype], kv_dtype=dts[k.dtype], window=(w["left"], w["right"], w["chunk"]), soft_cap=a["soft_cap"],
+                     query_positions=pos.buf if pos else None, kv_lengths=lens.buf if lens else None)
+                vals[n.output] = _Val("dev", out, shape, "f32", owned=True)
+            elif op == "Unary":
+                if a["op"] != "gelu":
+                    raise Unsupported("Unary %s" % a["op"])
+                vals[n.output] = _Val("gelu", None, shape, "f32", extra=n.inputs[0])
+            elif op == "ElemwiseBinary":
+                if a["op"] == "add":
+                    x, y = get(n.inputs[0]), get(n.inputs[1])
+                    if x.shape != y.shape:
+                        raise Unsupported("broadcasting add")
+                    out = new(shape, "f32")
+                    emit(g.step_add, out, x.buf, y.buf, _count(shape))
+                    vals[n.output] = _Val("dev", out, shape, "f32", owned=True)
+                elif a["op"] == "mul":
+                    lhs = vals.get(n.inputs[0])
+                    if lhs is None or lhs.kind != "gelu":
+                        raise Unsupported("a multiply that is not gelu(gate) * up")
+                    gate, up = get(lhs.extra), get(n.inputs[1])
+                    md = sole_user(n.output, "MatMul") if self.fuse else None
+                    wd = weight_of(nodes[md].inputs[1]) if md is not None and nodes[md].inputs[0] == n.output else None
+                    if wd is not None and nodes[md].attrs["beta"] == 0.0:
+                        rows, alpha = _count(gate.shape[:-1]), nodes[md].attrs["alpha"]
+                        matmul_into(nodes[md].output, lambda c, beta, wd=wd, gate=gate, up=up, rows=rows, alpha=alpha:
+                                    emit(g.step_gate_matmul, wd.buf, gate.buf, up.buf, rows, c, alpha=alpha, beta=beta))
+                        skip.add(md)
+                    else:
+                        out = new(shape, "f32")
+                        emit(g.step_gate_gelu, out, gate.buf, up.buf, _count(shape))
+                        vals[n.output] = _Val("dev", out, shape, "f32", owned=True)
+                else:
+                    raise Unsupported("ElemwiseBinary %s" % a["op"])
+            elif op == "ArgMax":
+                x = get(n.inputs[0])
+                if a["axis"] not in (-1, len(x.shape) - 1):
+                    raise Unsupported("ArgMax over an inner axis")
+                out = new(shape, "i32")
+                emit(g.step_argmax, out, x.buf, _count(x.shape[:-1]), x.shape[-1])
+                vals[n.output] = _Val("dev", out, shape, "i32", owned=True)
+            else:
+                raise Unsupported("operation %s has no step on this backend" % op)
+        for name, vid in pkg.outputs:
+            v = get(vid)
+            plan.outputs[name] = (v.buf, v.shape, v.dtype)
+        self.plans[s] = plan
+        return plan
+
+    # ---- running
+    def _write_inputs(self, plan, tokens, pos):
+        s = len(tokens)
+        feeds = {"tokens": tokens, "positions": np.arange(pos, pos + s, dtype=np.int32),
+                 "cache_write_index": np.array([pos], np.int32), "cache_visible_end": np.array([pos + s], np.int32)}
+        for kind, (buf, shape) in plan.inputs.items():
+            if _count(shape) != feeds[kind].size:
+                raise PackageError("InvalidArgument", "input %s: shape %s for %d elements" % (kind, shape, feeds[kind].size))
+            self.gpu.write(buf, feeds[kind])
+
+    def _issue(self, plan):
+        for fn, args, kw in plan.steps:
+            fn(*args, **kw)
+
+    def _read(self, plan, want):
+        np_t = {"f32": np.float32, "i32": np.int32, "f16": np.float16}
+        return {name: self.gpu.download(buf, np_t[dt], shape) for name, (buf, shape, dt) in plan.outputs.items() if name in want}
+
+    def run(self, tokens, want=("next_token",)):
+        """Feeds `tokens` (int32 [S]) at positions pos..pos+S-1, runs the graph, advances pos. Returns the
+        requested outputs (by signature name) as numpy arrays."""
+        tokens = np.ascontiguousarray(tokens, np.int32).reshape(-1)
+        if self.pos + tokens.size > self.capacity:
+            raise ValueError("the run exceeds the cache capacity")
+        plan = self._plan(tokens.size)
+        self._write_inputs(plan, tokens, self.pos)
+        self._issue(plan)
+        out = self._read(plan, want)
+        self.pos += tokens.size
+        return out
+
+    def step_count(self, s=1):
+        return len(self._plan(s).steps)
+
+    def begin_decode(self, first_token, token_output="next_token"):
+        """Records the one-token plan as a program whose loop state stays on the device: the token the graph
+        produced becomes the next run's token, position / write index / visible end advance by one."""
+        g = self.gpu
+        plan = self._plan(1)
+        self._write_inputs(plan, np.array([first_token], np.int32), self.pos)
+        if self.program is None:
+            self._issue(plan)                    # eager once: scratch buffers reach their final size
             g.sync()
-        finally:
-            for t in temps:
-                t.free()
-        self.pos += s
-        return result
+            self._write_inputs(plan, np.array([first_token], np.int32), self.pos)
+            if self.one is None:
+                self.one = g.upload(np.ones(1, np.int32))
+            tok_buf = plan.outputs[token_output][0]
+            g.program_begin()
+            self._issue(plan)
+            g._check(g._lib.aionhip_d2d(g._ctx, plan.inputs["tokens"][0].handle, 0, tok_buf.handle, 0, 4))
+            for kind in ("positions", "cache_write_index", "cache_visible_end"):
+                g.step_add_i32(plan.inputs[kind][0], plan.inputs[kind][0], self.one, 1)
+            self.program = g.program_end()
+        self._token_output = token_output
+
+    def decode_step(self, read_token=True):
+        if self.pos + 1 > self.capacity:
+            raise ValueError("cache capacity exhausted")
+        self.gpu.program_execute(self.program)
+        self.pos += 1
+        if read_token:
+            buf, shape, _ = self.plans[1].outputs[self._token_output]
+            return int(self.gpu.download(buf, np.int32, shape).reshape(-1)[-1])
+        return None
 
     def reset(self):
         self.pos = 0
 
     def close(self):
+        if self.program is not None:
+            self.gpu.program_destroy(self.program)
+            self.program = None
+        for plan in self.plans.values():
+            for b in plan.buffers:
+                b.free()
         for c in self.consts.values():
             c.buf.free()
         for b in self.caches.values():
             b.free()
-        self.consts, self.caches = {}, {}
+        if self.one is not None:
+            self.one.free()
+        self.plans, self.consts, self.caches, self.one = {}, {}, {}, None

@@ -15,7 +15,7 @@ cpu_baseline = the oracle's restatement of the aion CPU kernel for this op (pack
 M=1, aion cpu/exec/matmul.zig) timed on this host's cores on a bounded sample.
 
 `--sweep` adds the q8 legs and batch 4 / 8 (per-shape kernel GB/s) in a "sweep" object.
-`--extras gemm,attention,decoder[,decoder_eager]` adds the other BASELINE configs (prefill GEMM TFLOP/s, attention
+`--extras gemm,attention,decoder[,decoder_eager,package]` adds the other BASELINE configs (prefill GEMM TFLOP/s, attention
 TFLOP/s and GB/s, end-to-end decode tokens/s of the synthetic 26-layer decoder) in an "extras"
 object of the same JSON line.
 """
@@ -199,6 +199,8 @@ def main():
             out["extras"]["decoder"] = run_decoder(gpu, be, with_cpu=not args.no_cpu)
         if "decoder_eager" in extras:
             out["extras"]["decoder_eager"] = run_decoder_eager(gpu, be)
+        if "package" in extras:
+            out["extras"]["package"] = run_package(gpu, be)
 
     out["config"]["setup_s"] = round(setup_s, 1)
     print(json.dumps(out))
@@ -351,6 +353,49 @@ def run_decoder_eager(gpu, be, steps=8):
         tok = dec.decode_step_eager(tok)
     gpu.sync()
     return {"steps": steps, "eager_ms_per_token": round((time.perf_counter() - t) / steps * 1e3, 4)}
+
+
+def run_package(gpu, be):
+    """BASELINE config 5 as a `.aion` package: written by oracle/aion_writer.py (the reference's writer cannot run
+    here), read by aion_amd/aion_file.py, scheduled and run by aion_amd/package.py. Same weights as run_decoder."""
+    from aion_amd import aion_file
+    from aion_amd.decoder import DecoderConfig, SyntheticWeights
+    from aion_amd.package import PackageRunner
+    from oracle import aion_writer                       # test infrastructure: only used to make the input file
+    cfg = DecoderConfig()
+    t0 = time.time()
+    weights = SyntheticWeights(cfg, 0)
+    d = dict(layers=cfg.layers, hidden=cfg.hidden, heads=cfg.heads, kv_heads=cfg.kv_heads, head_dim=cfg.head_dim, ffn=cfg.ffn,
+             vocab=cfg.vocab, eps=cfg.eps, rope_base=cfg.rope_base, wdtype="q4_0")
+    data = aion_writer.build_decoder_package(d, weights.blocks, weights.embed())
+    t_write = time.time() - t0
+    t0 = time.time()
+    pkg = aion_file.parse(data)
+    t_parse = time.time() - t0
+    run = PackageRunner(gpu, pkg, capacity=cfg.max_seq)
+    prompt = np.random.default_rng(5).integers(0, cfg.vocab, 128).astype(np.int32)
+    t0 = time.time()
+    run.run(prompt); run.reset()                         # uploads the weights, builds the 128-token plan
+    t_first = time.time() - t0
+    gpu.sync()
+    t = time.perf_counter()
+    tok = int(run.run(prompt)["next_token"][0, -1])
+    prefill_ms = (time.perf_counter() - t) * 1e3
+    run.begin_decode(tok)
+    gpu.sync()
+    t = time.perf_counter()
+    for _ in range(127):
+        tok = run.decode_step()
+    gpu.sync()
+    decode_s = time.perf_counter() - t
+    res = {"file_bytes": len(data), "nodes": len(pkg.nodes), "initializers": len(pkg.tensors),
+           "write_s": round(t_write, 1), "parse_s": round(t_parse, 3), "upload_and_plan_s": round(t_first, 1),
+           "steps_prefill_128": run.step_count(128), "steps_decode": run.step_count(1),
+           "program_nodes": int(gpu.program_node_count(run.program)),
+           "prefill_128_ms": round(prefill_ms, 3), "decode_tokens_per_s": round(127 / decode_s, 1),
+           "decode_ms_per_token": round(decode_s / 127 * 1e3, 4)}
+    run.close()
+    return res
 
 
 def run_decoder(gpu, be, with_cpu=True):

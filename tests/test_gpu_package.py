@@ -94,3 +94,54 @@ def test_package_runner_refuses_what_the_backend_has_no_step_for(gpu):
             run.run(np.array([1, 2], np.int32), want=("y",))
     finally:
         run.close()
+
+
+@pytest.mark.parametrize("wdtype", [be.Q4_0, be.Q8_0])
+def test_fused_schedule_counts_steps_and_matches_the_node_by_node_one(gpu, wdtype):
+    cfg = DecoderConfig(wdtype=wdtype, **SMALL)
+    weights = SyntheticWeights(cfg, 7)
+    pkg = aion_file.parse(package_bytes(cfg, weights))
+    fused, plain = PackageRunner(gpu, pkg, capacity=cfg.max_seq), PackageRunner(gpu, pkg, capacity=cfg.max_seq, fuse=False)
+    try:
+        L = cfg.layers
+        # node by node: per layer 2 norms, 7 matmuls, 2 ropes, 2 appends (each with its cast), attention, gate, 2 adds
+        assert plain.step_count(1) == 1 + 17 * L + 3 and plain.step_count(5) == 1 + 17 * L + 3
+        # one new token: qkv+rope+append, attention, o (+residual), norm+gate/up+gelu+down (+residual) per layer
+        assert fused.step_count(1) == 1 + 4 * L + 2
+        # several tokens: norm+qkv, 2 ropes, 2 appends, attention, o (+residual), norm+gate/up, gate+down (+residual)
+        assert fused.step_count(5) == 1 + 9 * L + 2
+        prompt = np.random.default_rng(3).integers(0, cfg.vocab, 5).astype(np.int32)
+        a, b = fused.run(prompt, want=("next_token", "logits")), plain.run(prompt, want=("next_token", "logits"))
+        rms = float(np.sqrt((b["logits"].astype(np.float64) ** 2).mean()))
+        # same int8 codes and block dots; an f32 rounding difference can flip a code now and then (see test_gpu_decoder.py)
+        assert float(np.abs(a["logits"] - b["logits"]).max()) < 0.1 * rms
+        ta, tb = int(a["next_token"][0, -1]), int(b["next_token"][0, -1])
+        for _ in range(4):
+            a, b = fused.run([ta], want=("next_token", "logits")), plain.run([ta], want=("next_token", "logits"))
+            assert float(np.abs(a["logits"] - b["logits"]).max()) < 0.1 * rms
+            ta = int(a["next_token"][0, -1])
+    finally:
+        fused.close(); plain.close()
+
+
+def test_recorded_decode_program_equals_the_eager_runs(gpu):
+    cfg = DecoderConfig(wdtype=be.Q4_0, **SMALL)
+    weights = SyntheticWeights(cfg, 11)
+    pkg = aion_file.parse(package_bytes(cfg, weights))
+    a, b = PackageRunner(gpu, pkg, capacity=cfg.max_seq), PackageRunner(gpu, pkg, capacity=cfg.max_seq)
+    try:
+        prompt = np.random.default_rng(4).integers(0, cfg.vocab, 9).astype(np.int32)
+        ta = int(a.run(prompt)["next_token"][0, -1])
+        tb = int(b.run(prompt)["next_token"][0, -1])
+        assert ta == tb
+        a.begin_decode(ta)
+        assert gpu.program_node_count(a.program) > 10
+        for step in range(8):
+            fed = ta
+            ta = a.decode_step()                                           # replayed graph, loop state on the device
+            tb = int(b.run([fed])["next_token"][0, -1])                    # the same plan issued eagerly
+            gpu.sync()
+            assert ta == tb, step
+        assert a.pos == b.pos == prompt.size + 8
+    finally:
+        a.close(); b.close()
