@@ -242,12 +242,13 @@ class HipBackend:
             c_buf.free()
 
     def step_attention(self, out, q, k, v, shape, scale, q_dtype=F32, kv_dtype=F16, window=CAUSAL, soft_cap=0.0,
-                       query_positions=None, kv_lengths=None):
+                       query_positions=None, kv_lengths=None, rolling=False):
         B, L, T, Hq, Hkv, Dk, Dv = shape
         p = hip.Attention(out.handle, q.handle, k.handle, v.handle,
                           query_positions.handle if query_positions is not None else 0,
                           kv_lengths.handle if kv_lengths is not None else 0,
-                          B, L, T, Hq, Hkv, Dk, Dv, q_dtype, kv_dtype, scale, soft_cap, window[0], window[1], window[2])
+                          B, L, T, Hq, Hkv, Dk, Dv, q_dtype, kv_dtype, scale, soft_cap, window[0], window[1], window[2],
+                          1 if rolling else 0)
         self._check(self._lib.aionhip_step_attention(self._ctx, C.byref(p)))
 
     def step_rmsnorm(self, out, x, gamma, rows, cols, eps, beta=None, residual=None):
@@ -267,8 +268,9 @@ class HipBackend:
     def step_gather_rows(self, table_dtype, out, table, ids, n_ids, d, vocab):
         self._check(self._lib.aionhip_step_gather_rows(self._ctx, table_dtype, out.handle, table.handle, ids.handle, n_ids, d, vocab))
 
-    def step_append_f16(self, cache, src, write_index, b, s, t_cap, row_elems):
-        self._check(self._lib.aionhip_step_append_f16(self._ctx, cache.handle, src.handle, write_index.handle, b, s, t_cap, row_elems))
+    def step_append_f16(self, cache, src, write_index, b, s, t_cap, row_elems, rolling=False):
+        self._check(self._lib.aionhip_step_append_f16(self._ctx, cache.handle, src.handle, write_index.handle, b, s, t_cap, row_elems,
+                                                      1 if rolling else 0))
 
     def step_cast_f32_f16(self, out, x, n):
         self._check(self._lib.aionhip_step_cast_f32_f16(self._ctx, out.handle, x.handle, n))

@@ -40,6 +40,7 @@ struct AttnArgs {
     const int *positions, *kv_lengths;
     float *partial;
     int B, L, T, Hq, Hkv, groups, rows_total, row_tiles, nseg;
+    int ring;      // rolling caches: T (logical key t lives in row t % T); 0: row t is key t
     int q_dtype, kv_dtype;
     float scale, soft_cap;
     unsigned win_left, win_right, win_chunk;
@@ -98,6 +99,27 @@ __device__ __forceinline__ void window_keys(unsigned left, unsigned right, unsig
     hi = (int)h;
 }
 
+// Rolling caches (aion storage/cache.zig:202-207, cpu/exec/attention.zig:1072-1075, 1150-1152): the cache length may
+// exceed the capacity, keys older than length - capacity are gone, and key t is read from row t % capacity.
+__device__ __forceinline__ int phys_key(int ring, int t) { return ring ? (int)((unsigned)t % (unsigned)ring) : t; }
+// The same for the keys of one tile, whose first key key0 is uniform: one modulo per tile (base), then an add and
+// a conditional subtract per key. Valid while a tile is no longer than the ring (the launcher sees to that).
+struct TileMap {
+    int key0, base, wrap;
+    __device__ __forceinline__ TileMap(int ring, int k0) : key0(k0), base(ring ? (int)((unsigned)k0 % (unsigned)ring) : k0), wrap(ring ? ring : INT_MAX) {}
+    __device__ __forceinline__ int row(int key) const {
+        const int r = base + (key - key0);
+        return r >= wrap ? r - wrap : r;
+    }
+};
+__device__ __forceinline__ int clip_kv_end(int ring, int t_cap, int kv_end_raw) {
+    return ring ? max(0, kv_end_raw) : max(0, min(kv_end_raw, t_cap));
+}
+__device__ __forceinline__ void clip_to_ring(int ring, int kv_end, int &lo, int &hi) {
+    if (ring) lo = max(lo, kv_end - ring);
+    if (hi < lo) hi = lo;
+}
+
 __device__ __forceinline__ int wave_min_i(int v) {
 #pragma unroll
     for (int o = 32; o >= 1; o >>= 1) v = min(v, __shfl_xor(v, o, 64));
@@ -126,8 +148,11 @@ constexpr int SPLIT_NW = 8;
 // HILO: q and the probabilities are fed to the MFMAs as a high and a low half-precision part
 // (x = hi + lo, ~2x the mantissa), which keeps an f32 query path at f32-level accuracy; used when
 // q arrives as f32 (aion's cached decode: f32 q over an f16 cache). K and V are exact either way.
-template <int KV, int D, bool SPLIT, bool HILO>
+// RING: the caches are rolling rings (a.ring = T). A template flag, not a run-time test: the identity instances
+// must not carry the ring's extra live values (both kernels sit at their register limit).
+template <int KV, int D, bool SPLIT, bool HILO, bool RING = false>
 __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel(AttnArgs a) {
+    const int ring = RING ? a.ring : 0;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     constexpr int NW = SPLIT ? SPLIT_NW : 4;
     using Cfg = FlashCfg<D, NW>;
@@ -194,11 +219,11 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
         }
     }
 
-    int kv_end = max(0, min(kv_end_raw, a.T));
+    int kv_end = clip_kv_end(ring, a.T, kv_end_raw);
     int lo = 0, hi = 0;
     if (row_ok) {
         window_keys(a.win_left, a.win_right, a.win_chunk, max(pos_raw, 0), kv_end, lo, hi);
-        if (hi < lo) hi = lo;
+        clip_to_ring(ring, kv_end, lo, hi);
     }
     const int uni_lo = wave_min_i(hi > lo ? lo : INT_MAX);
     const int uni_hi = wave_max_i(hi > lo ? hi : 0);
@@ -281,13 +306,15 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
     const unsigned row_bytes = (unsigned)(kv_row * 2);
     const bool near = (size_t)a.T * kv_row * 2 < ((size_t)1 << 31) && a.T < (1 << 24) && row_bytes < (1u << 24);
     const unsigned char *kb8 = (const unsigned char *)(kp + kv_base), *vb8 = (const unsigned char *)(vp + kv_base);
+    const int k_last = RING ? max(uni_hi - 1, 0) : a.T - 1;        // the last key a K load may name
     u32x4 kf[2][KK];
     auto load_k_as = [&](int t, auto near_c) __attribute__((always_inline)) {
         constexpr bool near = decltype(near_c)::value;
         const int key0 = t * TILE_KEYS;
+        const TileMap tm(ring, key0);
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const int kabs = min(key0 + h * 16 + n, a.T - 1);
+            const int kabs = tm.row(min(key0 + h * 16 + n, k_last));
             if (near) {
                 const unsigned char *krow = kb8 + (__umul24((unsigned)kabs, row_bytes) + (unsigned)g * 16u);
 #pragma unroll
@@ -310,13 +337,14 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
 #if defined(__HIP_DEVICE_COMPILE__)   // the builtin exists in the device pass only
         constexpr bool near = decltype(near_c)::value;
         const int key0 = t * TILE_KEYS;
+        const TileMap tm(ring, key0);
 #pragma unroll
         for (int i = 0; i < NVI; ++i) {
             const int key = i * KEYS_PER_VI + v_key_in;
             // (key >> 2) & 3 does not depend on the lane while an instruction covers at most four keys
             const int grp = KEYS_PER_VI <= 4 ? ((i * KEYS_PER_VI) >> 2) & 3 : (key >> 2) & 3;
             const int chunk = v_slot ^ (2 * grp);
-            const int kabs = min(max(key0 + key, uni_lo), v_hi_key);
+            const int kabs = tm.row(min(max(key0 + key, uni_lo), v_hi_key));
             if (near)
                 __builtin_amdgcn_global_load_lds(vb8 + (__umul24((unsigned)kabs, row_bytes) + (unsigned)chunk * 16u), (lds_void *)(vs + i * 1024), 16, 0, 0);
             else
@@ -528,8 +556,9 @@ __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
-template <int KV, int D, bool CAP>
+template <int KV, int D, bool CAP, bool RING = false>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
+    const int ring = RING ? a.ring : 0;
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
     using Cfg = PrefillCfg<D>;
     constexpr int KK = D / 16;          // k-steps of the first product
@@ -585,11 +614,11 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
         for (int kk = 0; kk < KK; ++kk) qf[kk] = u32x4{0u, 0u, 0u, 0u};
     }
 
-    const int kv_end = max(0, min(kv_end_raw, a.T));
+    const int kv_end = clip_kv_end(ring, a.T, kv_end_raw);
     int lo = 0, hi = 0;
     if (row_ok) {
         window_keys(a.win_left, a.win_right, a.win_chunk, max(pos_raw, 0), kv_end, lo, hi);
-        if (hi < lo) hi = lo;
+        clip_to_ring(ring, kv_end, lo, hi);
     }
     const bool live = hi > lo;
     // wavefront: union (which tiles it computes) and intersection (which tiles need no mask)
@@ -624,11 +653,12 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
     auto load_k = [&](int t, unsigned char *st) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the builtin exists in the device pass only
         const int key0 = t * PF_TK;
+        const TileMap tm(ring, key0);
 #pragma unroll
         for (int i = 0; i < NKI; ++i) {
             const int key = (wave * NKI + i) * KEYS_PER_KI + k_key_in;
             const int swz = CPK >= 16 ? (key & 15) : ((key >> 1) & 7);
-            const int kabs = min(max(key0 + key, g_lo), key_clamp_hi);
+            const int kabs = tm.row(min(max(key0 + key, g_lo), key_clamp_hi));
             __builtin_amdgcn_global_load_lds(kp + kv_base + (size_t)kabs * kv_row + (k_slot ^ swz) * 8,
                                              (lds_void *)(st + (wave * NKI + i) * 1024), 16, 0, 0);
         }
@@ -637,12 +667,13 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
     u32x4 vreg[NVL][2];
     auto load_v = [&](int t) {
         const int key0 = t * PF_TK;
+        const TileMap tm(ring, key0);
 #pragma unroll
         for (int i = 0; i < NVL; ++i) {
             const int id = tid + 256 * i, pair = (id & 15) + 16 * (id / (16 * CPK)), c = (id >> 4) % CPK;
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                const int kabs = min(max(key0 + pair * 2 + h, g_lo), key_clamp_hi);
+                const int kabs = tm.row(min(max(key0 + pair * 2 + h, g_lo), key_clamp_hi));
                 vreg[i][h] = *(const u32x4 *)(vp + kv_base + (size_t)kabs * kv_row + c * 8);
             }
         }
@@ -866,11 +897,11 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(AttnArgs a, int d_k, 
     const int li = (int)((row / a.Hq) % a.L);
     const int b = (int)(row / ((size_t)a.Hq * a.L));
     const int hk = hq / a.groups;
-    int kv_end = a.kv_lengths ? a.kv_lengths[b] : a.T;
-    kv_end = max(0, min(kv_end, a.T));
+    const int kv_end = clip_kv_end(a.ring, a.T, a.kv_lengths ? a.kv_lengths[b] : a.T);
     const int pos = a.positions ? a.positions[(size_t)b * a.L + li] : li;
     int lo, hi;
     window_keys(a.win_left, a.win_right, a.win_chunk, max(pos, 0), kv_end, lo, hi);
+    clip_to_ring(a.ring, kv_end, lo, hi);
     float *o = a.out + row * d_v;
     if (hi <= lo) {
         for (int j = lane; j < d_v; j += 64) o[j] = 0.f;
@@ -879,19 +910,22 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(AttnArgs a, int d_k, 
     float *sc = scores + row * a.T;
     const size_t qb = row * d_k;
     float mx = -INFINITY;
+    // scores are kept at the key's physical row: a ring's visible keys span at most T steps
     for (int t = lo + lane; t < hi; t += 64) {
-        const size_t kb = (((size_t)b * a.T + t) * a.Hkv + hk) * d_k;
+        const int tp = phys_key(a.ring, t);
+        const size_t kb = (((size_t)b * a.T + tp) * a.Hkv + hk) * d_k;
         float d = 0.f;
         for (int j = 0; j < d_k; ++j) d += (load_scalar(a.q, a.q_dtype, qb + j) * a.scale) * load_scalar(a.k, a.kv_dtype, kb + j);
         if (a.soft_cap > 0.f) d = a.soft_cap * tanhf(d / a.soft_cap);
-        sc[t] = d;
+        sc[tp] = d;
         mx = fmaxf(mx, d);
     }
     mx = wave_max(mx);
     float sum = 0.f;
     for (int t = lo + lane; t < hi; t += 64) {
-        const float p = exp2f((sc[t] - mx) * LOG2E);
-        sc[t] = p;
+        const int tp = phys_key(a.ring, t);
+        const float p = exp2f((sc[tp] - mx) * LOG2E);
+        sc[tp] = p;
         sum += p;
     }
     sum = wave_sum(sum);
@@ -901,12 +935,15 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(AttnArgs a, int d_k, 
     const float inv = 1.f / sum;
     for (int j = lane; j < d_v; j += 64) {
         float acc = 0.f;
-        for (int t = lo; t < hi; ++t) acc += sc[t] * load_scalar(a.v, a.kv_dtype, (((size_t)b * a.T + t) * a.Hkv + hk) * d_v + j);
+        for (int t = lo; t < hi; ++t) {
+            const int tp = phys_key(a.ring, t);
+            acc += sc[tp] * load_scalar(a.v, a.kv_dtype, (((size_t)b * a.T + tp) * a.Hkv + hk) * d_v + j);
+        }
         o[j] = acc * inv;
     }
 }
 
-template <int KV, int D, bool HILO>
+template <int KV, int D, bool HILO, bool RING = false>
 int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
     using Cfg = FlashCfg<D, 4>;
     using SplitCfg = FlashCfg<D, SPLIT_NW>;
@@ -933,12 +970,12 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
         }
         static bool attr_split = false;   // per kernel instantiation
         if (!attr_split) {
-            HIP_TRY(ctx, hipFuncSetAttribute((const void *)attn_flash_kernel<KV, D, true, HILO>, hipFuncAttributeMaxDynamicSharedMemorySize, SplitCfg::LDS_BYTES));
+            HIP_TRY(ctx, hipFuncSetAttribute((const void *)attn_flash_kernel<KV, D, true, HILO, RING>, hipFuncAttributeMaxDynamicSharedMemorySize, SplitCfg::LDS_BYTES));
             attr_split = true;
         }
         {
             ProfScope scope(ctx, "attn_flash_split");
-            launch_k(ctx, attn_flash_kernel<KV, D, true, HILO>, dim3((unsigned)(a.row_tiles * nseg), (unsigned)units), dim3(SPLIT_NW * 64), SplitCfg::LDS_BYTES, a);
+            launch_k(ctx, attn_flash_kernel<KV, D, true, HILO, RING>, dim3((unsigned)(a.row_tiles * nseg), (unsigned)units), dim3(SPLIT_NW * 64), SplitCfg::LDS_BYTES, a);
         }
         if (nseg > 1) {
             ProfScope scope(ctx, "attn_merge");
@@ -950,15 +987,15 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
         a.nseg = 1;
         static bool attr_pf[2] = {false, false};
         const bool cap = a.soft_cap > 0.f;
-        const void *fn = cap ? (const void *)attn_prefill_kernel<KV, D, true> : (const void *)attn_prefill_kernel<KV, D, false>;
+        const void *fn = cap ? (const void *)attn_prefill_kernel<KV, D, true, RING> : (const void *)attn_prefill_kernel<KV, D, false, RING>;
         if (!attr_pf[cap]) {
             HIP_TRY(ctx, hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, PCfg::LDS_BYTES));
             attr_pf[cap] = true;
         }
         ProfScope scope(ctx, "attn_prefill");
         const dim3 grid((unsigned)((a.rows_total + PF_ROWS - 1) / PF_ROWS), (unsigned)units);
-        if (cap) launch_k(ctx, attn_prefill_kernel<KV, D, true>, grid, dim3(256), PCfg::LDS_BYTES, a);
-        else launch_k(ctx, attn_prefill_kernel<KV, D, false>, grid, dim3(256), PCfg::LDS_BYTES, a);
+        if (cap) launch_k(ctx, attn_prefill_kernel<KV, D, true, RING>, grid, dim3(256), PCfg::LDS_BYTES, a);
+        else launch_k(ctx, attn_prefill_kernel<KV, D, false, RING>, grid, dim3(256), PCfg::LDS_BYTES, a);
         LAUNCH_CHECK(ctx, "attn_prefill");
     } else {
         a.nseg = 1;
@@ -977,6 +1014,11 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
 template <int KV>
 int launch_flash_d(aionhip_ctx *ctx, AttnArgs &a, int d) {
     const bool hilo = a.q_dtype == AIONHIP_F32 && ctx->attn_precise;
+    if (a.ring) {       // rolling caches: the plain instances only (precise mode and soft cap take the generic kernel)
+        if (d == 64) return launch_flash<KV, 64, false, true>(ctx, a);
+        if (d == 128) return launch_flash<KV, 128, false, true>(ctx, a);
+        return launch_flash<KV, 256, false, true>(ctx, a);
+    }
     if (d == 64) return hilo ? launch_flash<KV, 64, true>(ctx, a) : launch_flash<KV, 64, false>(ctx, a);
     if (d == 128) return hilo ? launch_flash<KV, 128, true>(ctx, a) : launch_flash<KV, 128, false>(ctx, a);
     return hilo ? launch_flash<KV, 256, true>(ctx, a) : launch_flash<KV, 256, false>(ctx, a);
@@ -1013,6 +1055,7 @@ extern "C" int aionhip_step_attention(aionhip_ctx *ctx, const aionhip_attention 
     a.q_dtype = p->q_dtype; a.kv_dtype = p->kv_dtype;
     a.scale = p->scale; a.soft_cap = p->attn_logits_soft_cap;
     a.win_left = p->window_left; a.win_right = p->window_right; a.win_chunk = p->window_chunk;
+    a.ring = p->rolling ? a.T : 0;
 
     if (a.T == 0) {
         // no keys at all: every interval is empty -> zeros (cpu/exec/attention.zig:787-815)
@@ -1021,7 +1064,9 @@ extern "C" int aionhip_step_attention(aionhip_ctx *ctx, const aionhip_attention 
 
     const bool flash = p->d_k == p->d_v && (p->d_k == 64 || p->d_k == 128 || p->d_k == 256) &&
                        (p->kv_dtype == AIONHIP_F16 || p->kv_dtype == AIONHIP_BF16) &&
-                       ((p->k | p->v | p->out) & 15) == 0;
+                       ((p->k | p->v | p->out) & 15) == 0 &&
+                       // a ring shorter than a key tile, or a ring in precise / soft-cap mode: generic kernel
+                       (!a.ring || (a.T >= PF_TK && !(a.q_dtype == AIONHIP_F32 && ctx->attn_precise) && a.soft_cap <= 0.f));
     if (flash) {
         if (p->kv_dtype == AIONHIP_F16) return launch_flash_d<AIONHIP_F16>(ctx, a, (int)p->d_k);
         return launch_flash_d<AIONHIP_BF16>(ctx, a, (int)p->d_k);

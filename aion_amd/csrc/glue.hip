@@ -77,7 +77,7 @@ __global__ void rope_append_kernel(float *__restrict__ q_out, const float *__res
     const size_t src = is_q ? (tok * Hq + h) * D : (tok * Hkv + h) * D;
     const float *xp = is_q ? q : k;
     const int pos = positions[tok];
-    const int widx = write_index[0];
+    const int widx = write_index[tok / s_len];                 // one write index per batch entry (sequence_append.zig:58-60)
     const float fr = i < rope_pairs ? freq[i] : 0.f;
     const float xl = xp[src + i], xh = xp[src + half + i];
     float vl = 0.f, vh = 0.f;
@@ -140,13 +140,16 @@ __global__ void cast_f16_kernel(__half *__restrict__ out, const float *__restric
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) out[i] = __float2half_rn(x[i]);
 }
+// rolling: the cache is a ring, logical step t lives in row t % t_cap (storage/cache.zig:202-207)
 __global__ void append_f16_kernel(__half *__restrict__ cache, const float *__restrict__ src, const int *__restrict__ write_index,
-                                  size_t s_len, size_t t_cap, size_t row_elems, size_t total) {
+                                  size_t s_len, size_t t_cap, size_t row_elems, size_t total, int rolling) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= total) return;
     const size_t e = i % row_elems, s = (i / row_elems) % s_len, b = i / (row_elems * s_len);
-    const long t = (long)write_index[0] + (long)s;
-    if (t < 0 || (size_t)t >= t_cap) return;      // never write outside the cache
+    long t = (long)write_index[b] + (long)s;      // one write index per batch entry (sequence_append.zig:58-60)
+    if (t < 0) return;
+    if (rolling) t %= (long)t_cap;
+    if ((size_t)t >= t_cap) return;               // never write outside the cache
     cache[(b * t_cap + (size_t)t) * row_elems + e] = __float2half_rn(src[i]);
 }
 
@@ -313,14 +316,14 @@ int aionhip_step_gather_rows(aionhip_ctx *ctx, int table_dtype, aionhip_handle o
 }
 
 int aionhip_step_append_f16(aionhip_ctx *ctx, aionhip_handle cache, aionhip_handle src_f32, aionhip_handle write_index, size_t b,
-                            size_t s, size_t t_cap, size_t row_elems) {
+                            size_t s, size_t t_cap, size_t row_elems, int rolling) {
     if (!ctx) return AIONHIP_INVALID_ARGUMENT;
     if (!cache || !src_f32 || !write_index) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "append: null operand");
     if (s > t_cap) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "append: %zu new tokens exceed the cache capacity %zu", s, t_cap);
     const size_t total = b * s * row_elems;
     if (!total) return AIONHIP_OK;
     append_f16_kernel<<<dim3(grid_for(total, 256)), dim3(256), 0, ctx->stream>>>(dp<__half>(cache), dp<const float>(src_f32), dp<const int>(write_index),
-                                                                                 s, t_cap, row_elems, total);
+                                                                                 s, t_cap, row_elems, total, rolling);
     LAUNCH_CHECK(ctx, "append_f16");
     return AIONHIP_OK;
 }

@@ -24,7 +24,7 @@ class Attention(C.Structure):
     _fields_ = [(n, C.c_uint64) for n in ("out", "q", "k", "v", "query_positions", "kv_lengths")] + \
                [(n, C.c_size_t) for n in ("batch", "l_q", "t_kv", "h_q", "h_kv", "d_k", "d_v")] + \
                [("q_dtype", C.c_int), ("kv_dtype", C.c_int), ("scale", C.c_float), ("attn_logits_soft_cap", C.c_float),
-                ("window_left", C.c_uint32), ("window_right", C.c_uint32), ("window_chunk", C.c_uint32)]
+                ("window_left", C.c_uint32), ("window_right", C.c_uint32), ("window_chunk", C.c_uint32), ("rolling", C.c_uint32)]
 
 
 _SIGS = {
@@ -76,7 +76,7 @@ _SIGS = {
     "aionhip_step_add": (C.c_int, [C.c_void_p] + [C.c_uint64] * 3 + [C.c_size_t]),
     "aionhip_step_gate_gelu": (C.c_int, [C.c_void_p] + [C.c_uint64] * 3 + [C.c_size_t]),
     "aionhip_step_gather_rows": (C.c_int, [C.c_void_p, C.c_int] + [C.c_uint64] * 3 + [C.c_size_t] * 3),
-    "aionhip_step_append_f16": (C.c_int, [C.c_void_p] + [C.c_uint64] * 3 + [C.c_size_t] * 4),
+    "aionhip_step_append_f16": (C.c_int, [C.c_void_p] + [C.c_uint64] * 3 + [C.c_size_t] * 4 + [C.c_int]),
     "aionhip_step_cast_f32_f16": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64, C.c_size_t]),
     "aionhip_probe_stream_read": (C.c_int, [C.c_void_p, C.c_uint64, C.c_size_t, C.c_size_t, C.c_uint64]),
     "aionhip_step_argmax": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64, C.c_size_t, C.c_size_t]),

@@ -86,6 +86,8 @@ class PackageRunner:
         for _name, vid in pkg.outputs:
             self.uses.setdefault(vid, []).append(_OUT)
         self.roles = {}
+        self.all_rolling = all(r.retained_history_tokens for r in pkg.input_roles if r.kind == "sequence_cache") and \
+            any(r.kind == "sequence_cache" for r in pkg.input_roles)
         for idx, (_name, vid) in enumerate(pkg.inputs):
             role = pkg.role_of_input(idx)
             if role is None:
@@ -151,7 +153,8 @@ class PackageRunner:
         for vid, (idx, role) in self.roles.items():
             shape = pkg.shape_of(vid, sym)
             if role.kind == "sequence_cache":
-                vals[vid] = _Val("dev", self.caches[idx], shape, "f16")
+                # retained_history_tokens > 0: a rolling ring (storage/aion_file/types.zig:195-197, storage/cache.zig:35-38)
+                vals[vid] = _Val("dev", self.caches[idx], shape, "f16", extra="rolling" if role.retained_history_tokens else None)
                 continue
             if role.kind not in ("tokens", "positions", "cache_write_index", "cache_visible_end"):
                 raise Unsupported("input role %s" % role.kind)
@@ -274,8 +277,8 @@ class PackageRunner:
             if qs[:2] != (1, 1) or ks[:2] != (1, 1) or qs[3] != ks[3] or qs[3] % 8:
                 return False
             kc, vc = get(ak.inputs[0]), get(av.inputs[0])
-            if kc.shape != vc.shape or kc.shape[2:] != ks[2:] or kc.dtype != "f16":
-                return False
+            if kc.shape != vc.shape or kc.shape[2:] != ks[2:] or kc.dtype != "f16" or kc.extra or vc.extra:
+                return False                     # (the fused step writes at the write index itself: not for rings)
             gamma, beta = get(n0.inputs[1]), get(n0.inputs[2])
             q_out = new(qs, "f32")
             emit(g.step_rmsnorm_qkv_rope_append, weight_of(nodes[chains["q"][0]].inputs[1]).buf, weight_of(nodes[chains["k"][0]].inputs[1]).buf,
@@ -412,8 +415,9 @@ class PackageRunner:
                 if newv is None or newv.kind != "cast":
                     raise Unsupported("SequenceAppend whose new rows are not a Cast f32 -> f16")
                 src = get(newv.extra)
-                emit(g.step_append_f16, cache.buf, src.buf, widx.buf, cache.shape[0], newv.shape[1], cache.shape[1], _count(cache.shape[2:]))
-                vals[n.output] = _Val("dev", cache.buf, shape, "f16")
+                emit(g.step_append_f16, cache.buf, src.buf, widx.buf, cache.shape[0], newv.shape[1], cache.shape[1], _count(cache.shape[2:]),
+                     rolling=cache.extra == "rolling")
+                vals[n.output] = _Val("dev", cache.buf, shape, "f16", extra=cache.extra)
             elif op == "Attention":
                 q, k, v = get(n.inputs[0]), get(n.inputs[1]), get(n.inputs[2])
                 rest = list(n.inputs[3:])
@@ -425,7 +429,8 @@ class PackageRunner:
                 emit(g.step_attention, out, q.buf, k.buf, v.buf,
                      (q.shape[0], q.shape[1], k.shape[1], q.shape[2], k.shape[2], q.shape[3], v.shape[3]), a["scale"],
                      q_dtype=dts[q.dtype], kv_dtype=dts[k.dtype], window=(w["left"], w["right"], w["chunk"]), soft_cap=a["soft_cap"],
-                     query_positions=pos.buf if pos else None, kv_lengths=lens.buf if lens else None)
+                     query_positions=pos.buf if pos else None, kv_lengths=lens.buf if lens else None,
+                     rolling=k.extra == "rolling")
                 vals[n.output] = _Val("dev", out, shape, "f32", owned=True)
             elif op == "Unary":
                 if a["op"] != "gelu":
@@ -494,7 +499,7 @@ class PackageRunner:
         """Feeds `tokens` (int32 [S]) at positions pos..pos+S-1, runs the graph, advances pos. Returns the
         requested outputs (by signature name) as numpy arrays."""
         tokens = np.ascontiguousarray(tokens, np.int32).reshape(-1)
-        if self.pos + tokens.size > self.capacity:
+        if self.pos + tokens.size > self.capacity and not self.all_rolling:
             raise ValueError("the run exceeds the cache capacity")
         plan = self._plan(tokens.size)
         self._write_inputs(plan, tokens, self.pos)
@@ -528,7 +533,7 @@ class PackageRunner:
         self._token_output = token_output
 
     def decode_step(self, read_token=True):
-        if self.pos + 1 > self.capacity:
+        if self.pos + 1 > self.capacity and not self.all_rolling:
             raise ValueError("cache capacity exhausted")
         self.gpu.program_execute(self.program)
         self.pos += 1

@@ -189,6 +189,10 @@ typedef struct aionhip_attention {
     int kv_dtype;  /* F32 | F16 | BF16 */
     float scale, attn_logits_soft_cap;
     uint32_t window_left, window_right, window_chunk;
+    /* 1: k and v are rolling caches (storage/cache.zig:35-38, 202-207): logical key t lives in row t % T,
+     * kv_lengths may exceed T, and keys older than kv_length - T are gone (cpu/exec/attention.zig:1072-1075,
+     * 1150-1152, 1537-1546). 0: row t is key t and kv_lengths is clipped to T. */
+    uint32_t rolling;
 } aionhip_attention;
 int aionhip_step_attention(aionhip_ctx *ctx, const aionhip_attention *p);
 /* f32 queries over an f16/bf16 cache: off (default) = q rounded to the cache element type, one MFMA
@@ -206,7 +210,7 @@ int aionhip_step_rope(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle x, ai
                       size_t b, size_t t, size_t h, size_t d, float base_frequency, float scale_factor, float rope_proportion);
 /* RoPE1D(q) + RoPE1D(k) + Cast f16 + SequenceAppend(k cache) + Cast f16 + SequenceAppend(v cache)
  * of one step as a single launch (same arithmetic as the separate steps): q,q_out [B,S,Hq,D] f32,
- * k,v [B,S,Hkv,D] f32, caches [B,T,Hkv,D] f16, positions [B,S] i32, write_index [1] i32 on device */
+ * k,v [B,S,Hkv,D] f32, caches [B,T,Hkv,D] f16, positions [B,S] i32, write_index [B] i32 on device */
 int aionhip_step_rope_append(aionhip_ctx *ctx, aionhip_handle q_out, aionhip_handle q, aionhip_handle k, aionhip_handle v,
                              aionhip_handle k_cache, aionhip_handle v_cache, aionhip_handle positions, aionhip_handle write_index,
                              size_t b, size_t s, size_t t_cap, size_t h_q, size_t h_kv, size_t d,
@@ -221,9 +225,10 @@ int aionhip_step_gather_rows(aionhip_ctx *ctx, int table_dtype, aionhip_handle o
                              aionhip_handle ids, size_t n_ids, size_t d, size_t vocab);
 /* StepCast f32 -> f16 (cpu/exec/cast.zig) fused with StepSequenceAppend
  * (cpu/exec/sequence_append.zig:12-104): rows src [B,S,H,D] f32 are written as f16 into
- * cache [B,T,H,D] at token index write_index[0] (i32 on device) .. +S */
+ * cache [B,T,H,D] at token index write_index[b] (i32 [B] on device) .. +S; rolling = 1: the cache is a ring
+ * and logical step t goes to row t % T (storage/cache.zig:202-207) */
 int aionhip_step_append_f16(aionhip_ctx *ctx, aionhip_handle cache, aionhip_handle src_f32, aionhip_handle write_index,
-                            size_t b, size_t s, size_t t_cap, size_t row_elems);
+                            size_t b, size_t s, size_t t_cap, size_t row_elems, int rolling);
 int aionhip_step_cast_f32_f16(aionhip_ctx *ctx, aionhip_handle out_f16, aionhip_handle x_f32, size_t n);
 /* Measurement aid with no counterpart in aion: reads `bytes` of `src` from byte `offset` with a plain
  * streaming kernel and discards them (`sink`: any 4-byte device buffer, normally left untouched). Timed by

@@ -206,7 +206,7 @@ class PackageBuilder:
         return bytes(out)
 
 
-def build_decoder_package(cfg, blocks_of, embed, gammas=None):
+def build_decoder_package(cfg, blocks_of, embed, gammas=None, window=None, retained=0):
     """The config-5 decoder authored as a graph (the pattern of src/bench/models.zig:433-536 trimmed to a plain
     pre-norm block; the weight and cache operands as aion declares them): inputs tokens [1,seq] i32, positions
     [1,seq] i32, write_index [1] i32, visible_end [1] i32, and per layer a k and a v cache [1,ctx,Hkv,D] f16 that
@@ -214,7 +214,9 @@ def build_decoder_package(cfg, blocks_of, embed, gammas=None):
     ArgMax gives it: i32 [1,seq]; output 1 the logits [1,seq,vocab].
 
     cfg: layers, hidden, heads, kv_heads, head_dim, ffn, vocab, eps, rope_base, wdtype ("q4_0" | "q8_0");
-    blocks_of(name) -> packed blocks ([K,N] quant_axis 0 for q4_0, [N,K] quant_axis 1 for q8_0); embed f32 [vocab,hidden]."""
+    blocks_of(name) -> packed blocks ([K,N] quant_axis 0 for q4_0, [N,K] quant_axis 1 for q8_0); embed f32 [vocab,hidden].
+    window: (left, right, chunk) of every Attention (default causal); retained > 0 declares the caches rolling rings
+    that keep that many earlier positions (a sliding-window layer, src/bench/models.zig:440-447)."""
     b = PackageBuilder()
     seq, ctx = b.symbol("seq"), b.symbol("ctx")
     H, Hkv, D, E, F, V = cfg["heads"], cfg["kv_heads"], cfg["head_dim"], cfg["hidden"], cfg["ffn"], cfg["vocab"]
@@ -228,7 +230,7 @@ def build_decoder_package(cfg, blocks_of, embed, gammas=None):
     for l in range(cfg["layers"]):
         for kv in "kv":
             caches.append(b.input("l%d.%s_cache" % (l, kv), "f16", (1, ctx, Hkv, D), role="sequence_cache", axis=1,
-                                  capacity_symbol=0 + 1))           # dim symbol 1 = "ctx"
+                                  capacity_symbol=0 + 1, retained=retained))   # dim symbol 1 = "ctx"
 
     def weight(name, k, n):
         blocks = blocks_of(name)
@@ -263,7 +265,8 @@ def build_decoder_package(cfg, blocks_of, embed, gammas=None):
         vc = b.sequence_append(caches[2 * l + 1], b.cast(v, "f16", (1, seq, Hkv, D)), write_index, "f16", (1, ctx, Hkv, D))
         b.output("l%d.k_cache" % l, kc, alias_of_input=4 + 2 * l)
         b.output("l%d.v_cache" % l, vc, alias_of_input=4 + 2 * l + 1)
-        o = b.attention(q, kc, vc, positions, visible_end, (1, seq, H, D), 1.0 / float(np.sqrt(D)))
+        o = b.attention(q, kc, vc, positions, visible_end, (1, seq, H, D), 1.0 / float(np.sqrt(D)),
+                        window=window if window else (0xFFFFFFFF, 0, 0))
         o = b.matmul(b.reshape(o, "f32", (1, seq, H * D)), weight(p + "wo", H * D, E), (1, seq, E))
         x = b.binary("add", x, o, (1, seq, E))
         h = rms(x, p + "norm2", (1, seq, E))

@@ -206,6 +206,61 @@ def attention_f64(q, k, v, scale, window=CAUSAL, soft_cap=0.0, positions=None, k
     return out
 
 
+def window_keys(window, pos, end):
+    """AttentionWindow.keys (graph/graph.zig:160-167): the key interval [lo, hi) of a query at `pos` over keys [0, end)."""
+    left, right, chunk = window
+    anchor = (pos // chunk) * chunk if chunk > 0 else pos
+    span = chunk if chunk > 0 else 1
+    lo = anchor - min(anchor, left)
+    hi = end if right == UNBOUNDED else min(end, anchor + span + right)
+    return lo, max(hi, lo)
+
+
+def attention_rolling_f64(q, k_ring, v_ring, scale, window, positions, kv_lengths, soft_cap=0.0):
+    """Attention over rolling caches, the reference's generic path in f64 (cpu/exec/attention.zig:1055-1160, 1537-1546):
+    the cache length may exceed the capacity T; keys older than length - T are gone (:1072-1075); logical key t is
+    read from row t % T (:1150-1152). Plain loops: small cases only.
+    Pinned in tests/test_oracle_rolling.py by: ring == the unrolled linear cache through orc_attention_f64 whenever
+    the window stays inside the retained keys, and ring == the linear cache with its overwritten prefix cut off
+    (positions shifted) when it does not."""
+    q = np.asarray(q, np.float64)
+    k = np.asarray(k_ring, np.float64); v = np.asarray(v_ring, np.float64)
+    B, L, Hq, _ = q.shape
+    T, Hkv = k.shape[1], k.shape[2]
+    out = np.zeros((B, L, Hq, v.shape[3]), np.float64)
+    for b in range(B):
+        end = int(kv_lengths[b])
+        start = max(0, end - T)
+        for l in range(L):
+            lo, hi = window_keys(window, int(positions[b, l]), end)
+            lo = max(lo, start)
+            if hi <= lo:
+                continue
+            rows = np.arange(lo, hi) % T
+            for h in range(Hq):
+                hk = h // (Hq // Hkv)
+                sc = (k[b, rows, hk] @ q[b, l, h]) * scale
+                if soft_cap > 0:
+                    sc = soft_cap * np.tanh(sc / soft_cap)
+                p = np.exp(sc - sc.max())
+                out[b, l, h] = (p / p.sum()) @ v[b, rows, hk]
+    return out.astype(np.float32)
+
+
+def sequence_append(cache, new, end_index, rolling=False):
+    """StepSequenceAppend (cpu/exec/sequence_append.zig:58-104): rows new[b, s] go to cache[b, map(end_index[b] + s)];
+    map is the identity (out of range = InvalidArgument) or t % T for a rolling cache (storage/cache.zig:187-207)."""
+    out = np.array(cache, copy=True)
+    T = out.shape[1]
+    for b in range(out.shape[0]):
+        for s_ in range(new.shape[1]):
+            t = int(end_index[b]) + s_
+            if t < 0 or (not rolling and t >= T):
+                raise ValueError("sequence_append: InvalidArgument")
+            out[b, t % T if rolling else t] = new[b, s_]
+    return out
+
+
 def rmsnorm(x, gamma, eps, beta=None, residual=None):
     x = _f32(x); rows, cols = x.shape
     g = _f32(gamma); b = None if beta is None else _f32(beta); r = None if residual is None else _f32(residual)

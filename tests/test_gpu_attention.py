@@ -29,7 +29,7 @@ def to_bf16(x):
     return bits, (bits.astype(np.uint32) << 16).view(np.float32)
 
 
-def run_attention(gpu, q, k, v, scale, q_dtype, kv_dtype, window=be.CAUSAL, soft_cap=0.0, positions=None, kv_lengths=None):
+def run_attention(gpu, q, k, v, scale, q_dtype, kv_dtype, window=be.CAUSAL, soft_cap=0.0, positions=None, kv_lengths=None, rolling=False):
     B, L, Hq, Dk = q.shape
     _, T, Hkv, _ = k.shape
     Dv = v.shape[3]
@@ -38,7 +38,7 @@ def run_attention(gpu, q, k, v, scale, q_dtype, kv_dtype, window=be.CAUSAL, soft
     pos = gpu.upload(np.ascontiguousarray(positions, np.int32)) if positions is not None else None
     kl = gpu.upload(np.ascontiguousarray(kv_lengths, np.int32)) if kv_lengths is not None else None
     gpu.step_attention(out, bufs[0], bufs[1], bufs[2], (B, L, T, Hq, Hkv, Dk, Dv), scale, q_dtype=q_dtype, kv_dtype=kv_dtype,
-                       window=window, soft_cap=soft_cap, query_positions=pos, kv_lengths=kl)
+                       window=window, soft_cap=soft_cap, query_positions=pos, kv_lengths=kl, rolling=rolling)
     res = gpu.download(out, np.float32, (B, L, Hq, Dv))
     for b in bufs + [out] + [x for x in (pos, kl) if x is not None]:
         b.free()
@@ -259,3 +259,48 @@ def test_prefill_chunk_with_positions_over_a_longer_cache(gpu, orc, B, Lq, T, le
     ref = orc.attention_f64(qf, kz, vz, 1 / math.sqrt(D), positions=pos, kv_lengths=lens)
     assert np.isfinite(got).all()
     assert float(np.abs(got - ref).max()) < 2e-3
+
+
+def ring_of(linear, T):
+    """The last T steps of a linear history [B, end, H, D], each at row t % T."""
+    end = linear.shape[1]
+    ring = np.zeros((linear.shape[0], T) + linear.shape[2:], linear.dtype)
+    for t in range(max(0, end - T), end):
+        ring[:, t % T] = linear[:, t]
+    return ring
+
+
+# Rolling caches (aion storage/cache.zig:202-207, cpu/exec/attention.zig:1072-1075, 1150-1152): the cache length
+# exceeds the capacity, keys older than length - capacity are gone, key t is read from row t % capacity. Every
+# kernel against the oracle's rolling attention (pinned to the linear one in tests/test_oracle_rolling.py).
+@pytest.mark.parametrize("case", [
+    # B, L, Hq, Hkv, D, T(capacity), ends, window, kind, kernel
+    (2, 1, 8, 1, 256, 96, [250, 97], be.CAUSAL, "f16", "attn_flash_split"),            # decode, ring wrapped / barely wrapped
+    (3, 1, 8, 2, 128, 2048, [5000, 2048, 700], (1000, 0, 0), "bf16", "attn_flash_split"),  # several segments, sliding window
+    (2, 20, 4, 2, 64, 64, [300, 150], (30, 0, 0), "f16", "attn_flash_split"),          # a short chunk of new rows
+    (4, 320, 8, 2, 128, 512, [1400, 900, 700, 330], (400, 0, 0), "f16", "attn_prefill"),   # long chunk: prefill kernel
+    (2, 3, 4, 2, 80, 40, [130, 41], be.CAUSAL, "f16", "attn_generic"),                 # odd head size
+    (2, 1, 8, 1, 64, 48, [200, 100], be.CAUSAL, "f16", "attn_generic"),                # ring shorter than a key tile
+])
+def test_rolling_caches(gpu, orc, case):
+    B, L, Hq, Hkv, D, T, ends, window, kind, kernel = case
+    say("rolling", case)
+    rng = np.random.default_rng(sum(ends))
+    ends = np.array(ends, np.int32)
+    hist = int(ends.max())
+    (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(hist + L, B, L, hist, Hq, Hkv, D, kind)
+    # every batch entry's ring holds ITS last T steps; queries sit at the end of each entry's history
+    k_ring, v_ring = np.zeros((B, T, Hkv, D), k.dtype), np.zeros((B, T, Hkv, D), v.dtype)
+    kr_f, vr_f = np.zeros((B, T, Hkv, D), np.float32), np.zeros((B, T, Hkv, D), np.float32)
+    pos = np.zeros((B, L), np.int32)
+    for b in range(B):
+        e = int(ends[b])
+        k_ring[b], v_ring[b] = ring_of(k[b:b + 1, :e], T)[0], ring_of(v[b:b + 1, :e], T)[0]
+        kr_f[b], vr_f[b] = ring_of(kf[b:b + 1, :e], T)[0], ring_of(vf[b:b + 1, :e], T)[0]
+        pos[b] = np.arange(e - L, e)
+    got = run_attention(gpu, q, k_ring, v_ring, 1 / math.sqrt(D), qd, kd, window=window, positions=pos, kv_lengths=ends, rolling=True)
+    assert gpu.last_kernel() == kernel
+    want = orc.attention_rolling_f64(qf, kr_f, vr_f, 1 / math.sqrt(D), window, pos, ends)
+    err = float(np.abs(got - want).max())
+    say("  max err", err)
+    assert np.isfinite(got).all() and err < (1e-2 if kind == "bf16" else 2e-3)

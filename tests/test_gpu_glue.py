@@ -98,21 +98,38 @@ def test_kv_append_f16_at_device_write_index(gpu, orc):
     B, S, T, H, D = 2, 3, 10, 1, 64
     cache = np.zeros((B, T, H, D), np.float16)
     cb = gpu.upload(cache)
-    for step, widx in enumerate([0, 3, 6]):
+    for step, widx in enumerate([(0, 4), (3, 0), (6, 7)]):           # one write index per batch entry
         src = rng.standard_normal((B, S, H, D)).astype(np.float32)
-        sb, wb = gpu.upload(src), gpu.upload(np.array([widx], np.int32))
+        sb, wb = gpu.upload(src), gpu.upload(np.array(widx, np.int32))
         gpu.step_append_f16(cb, sb, wb, B, S, T, H * D)
-        cache[:, widx:widx + S] = orc.cast_f32_f16(src)
+        cache = orc.sequence_append(cache, orc.cast_f32_f16(src), widx)
         assert np.array_equal(gpu.download(cb, np.float16, cache.shape), cache)
         sb.free(); wb.free()
     # a write index that would run past the capacity writes only what fits
     src = np.ones((B, S, H, D), np.float32)
-    sb, wb = gpu.upload(src), gpu.upload(np.array([8], np.int32))
+    sb, wb = gpu.upload(src), gpu.upload(np.array([8, 8], np.int32))
     gpu.step_append_f16(cb, sb, wb, B, S, T, H * D)
     cache[:, 8:10] = 1.0
     assert np.array_equal(gpu.download(cb, np.float16, cache.shape), cache)
     for t in (cb, sb, wb):
         t.free()
+
+
+def test_kv_append_into_a_rolling_cache(gpu, orc):
+    rng = np.random.default_rng(8)
+    B, T, H, D = 2, 12, 2, 32
+    cache = np.zeros((B, T, H, D), np.float16)
+    cb = gpu.upload(cache)
+    t0 = np.array([0, 30], np.int32)
+    for n in (5, 9, 1, 12, 7):
+        src = rng.standard_normal((B, n, H, D)).astype(np.float32)
+        sb, wb = gpu.upload(src), gpu.upload(t0)
+        gpu.step_append_f16(cb, sb, wb, B, n, T, H * D, rolling=True)
+        cache = orc.sequence_append(cache, orc.cast_f32_f16(src), t0, rolling=True)
+        assert np.array_equal(gpu.download(cb, np.float16, cache.shape), cache)
+        t0 = t0 + n
+        sb.free(); wb.free()
+    cb.free()
 
 
 def test_rope_append_equals_the_separate_steps(gpu, orc):
@@ -122,7 +139,7 @@ def test_rope_append_equals_the_separate_steps(gpu, orc):
     k = rng.standard_normal((B, S, Hkv, D)).astype(np.float32)
     v = rng.standard_normal((B, S, Hkv, D)).astype(np.float32)
     pos = np.array([[4, 5, 6], [4, 5, 6]], np.int32)
-    qb, kb, vb, pb, wb = gpu.upload(q), gpu.upload(k), gpu.upload(v), gpu.upload(pos), gpu.upload(np.array([4], np.int32))
+    qb, kb, vb, pb, wb = gpu.upload(q), gpu.upload(k), gpu.upload(v), gpu.upload(pos), gpu.upload(np.array([4, 4], np.int32))
     qo = gpu.alloc(q.nbytes)
     kc, vc = gpu.zeros(B * T * Hkv * D * 2), gpu.zeros(B * T * Hkv * D * 2)
     gpu.step_rope_append(qo, qb, kb, vb, kc, vc, pb, wb, B, S, T, Hq, Hkv, D)

@@ -145,3 +145,33 @@ def test_recorded_decode_program_equals_the_eager_runs(gpu):
         assert a.pos == b.pos == prompt.size + 8
     finally:
         a.close(); b.close()
+
+
+def test_sliding_window_package_on_rolling_caches_equals_full_caches(gpu):
+    """A sliding-window decoder whose caches are rolling rings of 64 rows must produce what the same model produces
+    with caches that hold the whole history: the window (24 back) never reaches past what the ring retains. Bit for
+    bit: the same kernels visit the same keys in the same order, only the rows they are read from differ. (A ring
+    shorter than the 64-key tile of the MFMA kernels runs on the generic kernel, which does not round q to f16.)"""
+    cfg = DecoderConfig(wdtype=be.Q4_0, **SMALL)
+    weights = SyntheticWeights(cfg, 13)
+    d = dict(layers=cfg.layers, hidden=cfg.hidden, heads=cfg.heads, kv_heads=cfg.kv_heads, head_dim=cfg.head_dim, ffn=cfg.ffn,
+             vocab=cfg.vocab, eps=cfg.eps, rope_base=cfg.rope_base, wdtype="q4_0")
+    window = (24, 0, 0)
+    ring_pkg = aion_file.parse(aion_writer.build_decoder_package(d, weights.blocks, weights.embed(), window=window, retained=24))
+    full_pkg = aion_file.parse(aion_writer.build_decoder_package(d, weights.blocks, weights.embed(), window=window))
+    assert ring_pkg.role_of_input(4).retained_history_tokens == 24 and full_pkg.role_of_input(4).retained_history_tokens == 0
+    # node by node on both sides, so that both issue the same steps (with fusions on, the ring side keeps its
+    # appends as separate steps while the full side takes the fused one-token q/k/v step: equal up to f32 rounding)
+    ring, full = PackageRunner(gpu, ring_pkg, capacity=64, fuse=False), PackageRunner(gpu, full_pkg, capacity=128, fuse=False)
+    try:
+        prompt = np.random.default_rng(2).integers(0, cfg.vocab, 7).astype(np.int32)
+        a, b = ring.run(prompt, want=("next_token", "logits")), full.run(prompt, want=("next_token", "logits"))
+        assert np.array_equal(a["logits"], b["logits"])
+        tok = int(b["next_token"][0, -1])
+        for step in range(100):                                  # runs well past the ring's 64 rows
+            a, b = ring.run([tok], want=("next_token", "logits")), full.run([tok], want=("next_token", "logits"))
+            assert np.array_equal(a["logits"], b["logits"]), step
+            tok = int(b["next_token"][0, -1])
+        assert ring.pos == 107
+    finally:
+        ring.close(); full.close()

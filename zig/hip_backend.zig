@@ -137,6 +137,8 @@ pub const HipBackend = struct {
                 p.q_dtype = @intFromEnum(qm.dtype); p.kv_dtype = @intFromEnum(km.dtype);
                 p.scale = s.scale; p.attn_logits_soft_cap = s.attn_logits_soft_cap;
                 p.window_left = s.window.left; p.window_right = s.window.right; p.window_chunk = s.window.chunk;
+                // a rolling sequence cache reads key t from row t % capacity (cpu/exec/attention.zig:1537-1546)
+                p.rolling = if (store.sequenceCachePolicyInfo(s.k).kind == .rolling) 1 else 0;
                 try check(c.aionhip_step_attention(self.ctx, &p));
             },
             .RMSNorm => |s| {
