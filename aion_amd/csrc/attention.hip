@@ -719,8 +719,11 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
             load_v(t + 1);
         }
         const int key0 = t * PF_TK;
-        const bool mine = key0 < w_hi && key0 + PF_TK > w_lo;       // wavefront-uniform
-        if (mine) {
+        // Every wavefront computes every tile of the workgroup's union, also one that none of its own rows sees
+        // (all of its scores are then masked and it adds exact zeros): the wavefronts meet at the barrier below
+        // anyway, and a branch around the MFMAs makes the compiler carry the accumulators in vector registers
+        // and copy all of them to and from the accumulation registers on every tile.
+        {
             // -- S^T = K . Q^T for the two 32-key halves (two independent accumulation chains)
             f32x16 s[2];
 #pragma unroll
@@ -784,9 +787,21 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
                                pack2<KV>(x[8 * s2 + 4], x[8 * s2 + 5]), pack2<KV>(x[8 * s2 + 6], x[8 * s2 + 7])};
             // -- O^T += V^T . P^T
             if (__any(alpha != 1.f)) {              // wavefront-uniform and rare: must stay a branch, not a select
-                asm volatile("" ::: "memory");
+                // The accumulators live in accumulation registers for the MFMAs. Written as plain C++ the multiply
+                // makes the compiler keep them in vector registers around this branch and copy all of them back and
+                // forth on the common path (several hundred moves per key tile). So: read, scale and write back each
+                // one here, with the register class pinned. The s_nops cover the waits between an MFMA result and
+                // its read, and between the write-back and the next MFMA, which the compiler cannot see in here.
+                asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory");
 #pragma unroll
-                for (int j = 0; j < NJ; ++j) acc[j] *= alpha;
+                for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        float tmp;
+                        asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 1\n\tv_accvgpr_write_b32 %0, %1"
+                                     : "+a"(acc[j][i]), "=&v"(tmp) : "v"(alpha));
+                    }
+                asm volatile("s_nop 7" ::: "memory");
             }
             // key step outermost: consecutive MFMAs go to different accumulators
 #pragma unroll
