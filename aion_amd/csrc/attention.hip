@@ -537,6 +537,9 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
 //   so that the probabilities feed the MFMA straight from the S accumulators without a shuffle.
 constexpr int PF_ROWS = 128, PF_TK = 64, PF_VROW = 136;
 constexpr float PF_LAZY = 8.f;
+#ifndef PF_AHEAD
+#define PF_AHEAD 3
+#endif
 using f32x16 = __attribute__((ext_vector_type(16))) float;
 using u32x2 = __attribute__((ext_vector_type(2))) unsigned int;
 
@@ -738,6 +741,17 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
                 s[0] = mfma32<KV>(k0, qf[kk], s[0]);
                 s[1] = mfma32<KV>(k1, qf[kk], s[1]);
             }
+#ifndef PF_NO_PIPE
+            // issue order: the LDS reads run PF_AHEAD k-steps ahead of the MFMAs that consume them (left alone the
+            // compiler issues each read right before its MFMA, which then waits out the whole LDS latency)
+            __builtin_amdgcn_sched_group_barrier(0x100, 2 * PF_AHEAD, 0);
+#pragma unroll
+            for (int kk = 0; kk < KK - PF_AHEAD; ++kk) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, 2 * PF_AHEAD, 0);
+#endif
             // -- lane holds keys key0 + kb*32 + (i/4)*8 + lh*4 + i%4 of row l31
             float x[32];
             const bool full = key0 >= w_lo_max && key0 + PF_TK <= w_hi_min;   // every key visible to every row
@@ -812,6 +826,15 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
                     const u32x2 va = *(const u32x2 *)(vrow), vb = *(const u32x2 *)(vrow + 16);
                     acc[j] = mfma32<KV>(u32x4{va.x, va.y, vb.x, vb.y}, pf[s2], acc[j]);
                 }
+#ifndef PF_NO_PIPE
+            __builtin_amdgcn_sched_group_barrier(0x100, 2 * PF_AHEAD, 1);
+#pragma unroll
+            for (int i = 0; i < 4 * NJ - 2 * PF_AHEAD; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 1);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, 2 * PF_AHEAD, 1);
+#endif
         }
         if (more) store_v(nx);
         __syncthreads();                                           // also waits for this wavefront's K loads (fence)
