@@ -578,7 +578,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
     const int unit = blockIdx.y, b = unit / a.Hkv, hk = unit % a.Hkv;
 
     // ---- this lane's query row (lanes l and l+32 share it)
-    const int r = blockIdx.x * PF_ROWS + wave * 32 + l31;
+    // row tiles in descending order: under a causal mask the last rows see the most keys, and workgroups are
+    // dispatched in index order - the long ones start first and the short ones fill the gaps at the end
+    const int r = ((int)gridDim.x - 1 - (int)blockIdx.x) * PF_ROWS + wave * 32 + l31;
     const bool row_ok = r < a.rows_total;
     const int li = row_ok ? r / a.groups : 0, gi = row_ok ? r % a.groups : 0;
     const int hq = hk * a.groups + gi;
