@@ -272,6 +272,22 @@ class HipBackend:
         self._check(self._lib.aionhip_step_append_f16(self._ctx, cache.handle, src.handle, write_index.handle, b, s, t_cap, row_elems,
                                                       1 if rolling else 0))
 
+    def cache_grow(self, dst, src, outer, old_run_bytes, new_run_bytes):
+        """dst [outer, new_run_bytes] <- the runs of src [outer, old_run_bytes], zero elsewhere (storage/manager/grow.zig:37-78)."""
+        self._check(self._lib.aionhip_cache_grow(self._ctx, dst.handle, src.handle, outer, old_run_bytes, new_run_bytes))
+
+    def cache_grow_rolling(self, dst, src, logical_ends, b, old_capacity, new_capacity, row_bytes, retained_history):
+        """Ring growth: the retained logical steps move to row t % new_capacity (storage/manager/grow.zig:107-150)."""
+        self._check(self._lib.aionhip_cache_grow_rolling(self._ctx, dst.handle, src.handle, logical_ends.handle, b, old_capacity,
+                                                         new_capacity, row_bytes, retained_history))
+
+    def cache_grow_target(self, current, num, den):
+        """Next capacity of the geometric schedule (storage/manager.zig:69-76); raises on invalid arguments."""
+        t = int(self._lib.aionhip_cache_grow_target(current, num, den))
+        if t == 0:
+            raise ValueError("cache_grow_target: InvalidArgument")
+        return t
+
     def step_cast_f32_f16(self, out, x, n):
         self._check(self._lib.aionhip_step_cast_f32_f16(self._ctx, out.handle, x.handle, n))
 

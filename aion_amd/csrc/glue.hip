@@ -153,6 +153,40 @@ __global__ void append_f16_kernel(__half *__restrict__ cache, const float *__res
     cache[(b * t_cap + (size_t)t) * row_elems + e] = __float2half_rn(src[i]);
 }
 
+// Growth of a sequence cache along its time axis (storage/manager/grow.zig:37-78): the wider backing is zero
+// except for the `outer` preserved runs, each copied to the start of its wider slot. One pass over the new
+// backing in 4-byte words (the reference's device path also moves whole words).
+__global__ void cache_grow_kernel(unsigned *__restrict__ dst, const unsigned *__restrict__ src, size_t old_words, size_t new_words, size_t total) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const size_t o = i / new_words, r = i % new_words;
+    dst[i] = r < old_words ? src[o * old_words + r] : 0u;
+}
+// The same for a ring (grow.zig:107-150): row t % capacity changes with the capacity, so the retained logical
+// steps of batch entry b - the last min(end, retained_history, old_capacity) before end = logical_ends[b] - are
+// re-placed; every other row of the new ring is zero. A new row p holds the step t = end-1 - ((end-1-p) mod
+// new_capacity) if that step is retained (at most one retained step maps to a row, as kept <= old < new capacity).
+__global__ void cache_grow_rolling_kernel(unsigned *__restrict__ dst, const unsigned *__restrict__ src, const int *__restrict__ logical_ends,
+                                          size_t old_cap, size_t new_cap, size_t row_words, size_t retained, size_t total) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const size_t w = i % row_words, p = (i / row_words) % new_cap, b = i / (row_words * new_cap);
+    const long end = logical_ends[b];
+    unsigned v = 0u;
+    if (end > 0) {
+        const size_t e = (size_t)end;
+        size_t kept = e < retained ? e : retained;
+        if (old_cap < kept) kept = old_cap;
+        const size_t last = e - 1;
+        const size_t back = (last % new_cap + new_cap - p) % new_cap;      // steps from `last` back to the one living in row p
+        if (back < kept) {
+            const size_t t = last - back;
+            v = src[(b * old_cap + t % old_cap) * row_words + w];
+        }
+    }
+    dst[i] = v;
+}
+
 // cpu/exec/argmax.zig:56-81: strict > keeps the first maximum. Two stages: ARGMAX_PARTS workgroups
 // per row each reduce a contiguous slice to (value, index), then one workgroup picks among them
 // (ties -> the smaller index, which is the first maximum).
@@ -325,6 +359,48 @@ int aionhip_step_append_f16(aionhip_ctx *ctx, aionhip_handle cache, aionhip_hand
     append_f16_kernel<<<dim3(grid_for(total, 256)), dim3(256), 0, ctx->stream>>>(dp<__half>(cache), dp<const float>(src_f32), dp<const int>(write_index),
                                                                                  s, t_cap, row_elems, total, rolling);
     LAUNCH_CHECK(ctx, "append_f16");
+    return AIONHIP_OK;
+}
+
+size_t aionhip_cache_grow_target(size_t current, size_t num, size_t den) {
+    if (!current || !num || !den) return 0;
+    if (current > SIZE_MAX / num) return 0;
+    const size_t prod = current * num;
+    if (prod > SIZE_MAX - (den - 1)) return 0;
+    const size_t next = (prod + den - 1) / den;
+    if (next <= current) return current == SIZE_MAX ? 0 : current + 1;
+    return next;
+}
+
+int aionhip_cache_grow(aionhip_ctx *ctx, aionhip_handle dst, aionhip_handle src, size_t outer, size_t old_run_bytes, size_t new_run_bytes) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (!dst || !src) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "cache_grow: null operand");
+    if (dst == src) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "cache_grow: the grown cache needs a backing of its own");
+    if ((old_run_bytes | new_run_bytes) & 3) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "cache_grow: runs of %zu and %zu bytes are not whole 4-byte words", old_run_bytes, new_run_bytes);
+    if (new_run_bytes < old_run_bytes) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "cache_grow: %zu -> %zu bytes per run is not a growth", old_run_bytes, new_run_bytes);
+    if (new_run_bytes && outer > SIZE_MAX / new_run_bytes) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "cache_grow: size overflow");
+    const size_t total = outer * (new_run_bytes / 4);
+    if (!total) return AIONHIP_OK;
+    cache_grow_kernel<<<dim3(grid_for(total, 256)), dim3(256), 0, ctx->stream>>>(dp<unsigned>(dst), dp<const unsigned>(src), old_run_bytes / 4, new_run_bytes / 4, total);
+    LAUNCH_CHECK(ctx, "cache_grow");
+    return AIONHIP_OK;
+}
+
+int aionhip_cache_grow_rolling(aionhip_ctx *ctx, aionhip_handle dst, aionhip_handle src, aionhip_handle logical_ends, size_t b,
+                               size_t old_capacity, size_t new_capacity, size_t row_bytes, size_t retained_history) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (!dst || !src || !logical_ends) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "cache_grow_rolling: null operand");
+    if (dst == src) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "cache_grow_rolling: the grown cache needs a backing of its own");
+    if (!old_capacity || new_capacity <= old_capacity)
+        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "cache_grow_rolling: capacity %zu -> %zu is not a growth", old_capacity, new_capacity);
+    if (row_bytes & 3) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "cache_grow_rolling: rows of %zu bytes are not whole 4-byte words", row_bytes);
+    if (row_bytes && (new_capacity > SIZE_MAX / row_bytes || (b && new_capacity * row_bytes > SIZE_MAX / b)))
+        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "cache_grow_rolling: size overflow");
+    const size_t total = b * new_capacity * (row_bytes / 4);
+    if (!total) return AIONHIP_OK;
+    cache_grow_rolling_kernel<<<dim3(grid_for(total, 256)), dim3(256), 0, ctx->stream>>>(dp<unsigned>(dst), dp<const unsigned>(src), dp<const int>(logical_ends),
+                                                                                         old_capacity, new_capacity, row_bytes / 4, retained_history, total);
+    LAUNCH_CHECK(ctx, "cache_grow_rolling");
     return AIONHIP_OK;
 }
 

@@ -70,8 +70,15 @@ class _Plan:
 
 
 class PackageRunner:
-    def __init__(self, gpu, pkg, capacity, capacity_symbol="ctx", tokens_symbol="seq", fuse=True):
+    def __init__(self, gpu, pkg, capacity, capacity_symbol="ctx", tokens_symbol="seq", fuse=True, growth=None):
+        """growth: None = the capacity is fixed and a run that needs more is an error. A dict with "numerator",
+        "denominator" and optionally "max_capacity" = the sequence caches grow on the device when a run needs more
+        rows, on the schedule of aion's session (api/loaded_model.zig:735-827: geometric steps, then a power of
+        two and at least four times the old capacity, since every capacity is a set of plans of its own; rolling
+        caches use the factor 2/1 and are re-placed row by row)."""
         self.gpu, self.pkg, self.capacity, self.fuse = gpu, pkg, int(capacity), fuse
+        self.growth = growth
+        self.cache_meta = {}        # input index -> (value id, retained history tokens)
         self.sym_ctx, self.sym_seq = capacity_symbol, tokens_symbol
         self.pos = 0
         self.consts = {}            # (value id, transposed) -> _Val of an uploaded initializer
@@ -97,7 +104,10 @@ class PackageRunner:
                 shape = pkg.shape_of(vid, {self.sym_ctx: self.capacity, self.sym_seq: 1})
                 if pkg.values[vid].dtype != "f16":
                     raise Unsupported("sequence cache of dtype %s" % pkg.values[vid].dtype)
+                if growth is not None and not (role.flags & 2) and not role.retained_history_tokens:
+                    raise Unsupported("input %d does not allow growth (InputRoleFlags.allow_growable)" % idx)
                 self.caches[idx] = gpu.zeros(_count(shape) * 2)
+                self.cache_meta[idx] = (vid, int(role.retained_history_tokens))
 
     # ---- initializers
     def _const(self, vid, transposed=False):
@@ -495,12 +505,71 @@ class PackageRunner:
         np_t = {"f32": np.float32, "i32": np.int32, "f16": np.float16}
         return {name: self.gpu.download(buf, np_t[dt], shape) for name, (buf, shape, dt) in plan.outputs.items() if name in want}
 
+    # ---- cache growth
+    def _required(self, s):
+        """Rows the caches must hold for a run of s tokens at self.pos (api/loaded_model/sequence_cache.zig:45-51)."""
+        need = 0
+        for _vid, retained in self.cache_meta.values():
+            need = max(need, (min(self.pos, retained) if retained else self.pos) + s)
+        return need
+
+    def _grow(self, required):
+        g, gr = self.gpu, self.growth
+        num, den = (2, 1) if self.all_rolling else (int(gr["numerator"]), int(gr["denominator"]))
+        ceiling = 0 if self.all_rolling else int(gr.get("max_capacity", 0))
+        target = self.capacity
+        while target < required:
+            target = g.cache_grow_target(target, num, den)
+        p2 = 1
+        while p2 < target:
+            p2 *= 2
+        target = max(p2, self.capacity * 4)
+        if ceiling:
+            if required > ceiling:
+                raise ValueError("the run exceeds the caches' growth ceiling")
+            target = min(target, ceiling)
+        ends = None
+        for idx, (vid, retained) in self.cache_meta.items():
+            old_shape = self.pkg.shape_of(vid, {self.sym_ctx: self.capacity, self.sym_seq: 1})
+            new_shape = self.pkg.shape_of(vid, {self.sym_ctx: target, self.sym_seq: 1})
+            if old_shape[1] != self.capacity or new_shape[1] != target or old_shape[:1] + old_shape[2:] != new_shape[:1] + new_shape[2:]:
+                raise Unsupported("cache input %d: the capacity symbol is not its time axis" % idx)
+            b, row_bytes = old_shape[0], _count(old_shape[2:]) * 2
+            new = g.alloc(_count(new_shape) * 2)          # every byte is written by the growth kernel
+            if retained:
+                if ends is None:
+                    ends = g.upload(np.full(b, self.pos, np.int32))
+                g.cache_grow_rolling(new, self.caches[idx], ends, b, self.capacity, target, row_bytes, retained)
+            else:
+                g.cache_grow(new, self.caches[idx], b, self.capacity * row_bytes, target * row_bytes)
+            g.sync()
+            self.caches[idx].free()
+            self.caches[idx] = new
+        if ends is not None:
+            ends.free()
+        # every plan holds the old caches and the old capacity in its shapes
+        if self.program is not None:
+            g.program_destroy(self.program)
+            self.program = None
+        for plan in self.plans.values():
+            for buf in plan.buffers:
+                buf.free()
+        self.plans = {}
+        self.capacity = target
+
+    def _ensure_capacity(self, s):
+        required = self._required(s)
+        if required <= self.capacity:
+            return
+        if self.growth is None:
+            raise ValueError("the run exceeds the cache capacity")
+        self._grow(required)
+
     def run(self, tokens, want=("next_token",)):
         """Feeds `tokens` (int32 [S]) at positions pos..pos+S-1, runs the graph, advances pos. Returns the
         requested outputs (by signature name) as numpy arrays."""
         tokens = np.ascontiguousarray(tokens, np.int32).reshape(-1)
-        if self.pos + tokens.size > self.capacity and not self.all_rolling:
-            raise ValueError("the run exceeds the cache capacity")
+        self._ensure_capacity(tokens.size)
         plan = self._plan(tokens.size)
         self._write_inputs(plan, tokens, self.pos)
         self._issue(plan)
@@ -533,8 +602,13 @@ class PackageRunner:
         self._token_output = token_output
 
     def decode_step(self, read_token=True):
-        if self.pos + 1 > self.capacity and not self.all_rolling:
-            raise ValueError("cache capacity exhausted")
+        if self._required(1) > self.capacity:
+            if self.growth is None:
+                raise ValueError("cache capacity exhausted")
+            # the loop state lives in the old plan's buffers: take the pending token out, grow, record again
+            token = int(self.gpu.download(self.plans[1].inputs["tokens"][0], np.int32, (1,))[0])
+            self._grow(self._required(1))
+            self.begin_decode(token, self._token_output)
         self.gpu.program_execute(self.program)
         self.pos += 1
         if read_token:

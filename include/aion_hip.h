@@ -230,6 +230,24 @@ int aionhip_step_gather_rows(aionhip_ctx *ctx, int table_dtype, aionhip_handle o
 int aionhip_step_append_f16(aionhip_ctx *ctx, aionhip_handle cache, aionhip_handle src_f32, aionhip_handle write_index,
                             size_t b, size_t s, size_t t_cap, size_t row_elems, int rolling);
 int aionhip_step_cast_f32_f16(aionhip_ctx *ctx, aionhip_handle out_f16, aionhip_handle x_f32, size_t n);
+/* Growth of a sequence cache along its time axis with the data kept on the device
+ * (storage/manager/grow.zig:37-78 growAxisOnDevice, driven by api/loaded_model.zig:791-827 and
+ * storage/manager/store_view.zig:104-124): dst is the new backing [outer, new_run_bytes], src the old one
+ * [outer, old_run_bytes]; every run is copied to the start of its wider slot and the rest of dst is zero. Runs are
+ * whole 4-byte words (grow.zig:51-52) and new_run_bytes >= old_run_bytes. For a cache [B,T,H,D] grown to T':
+ * outer = B, runs = T*H*D and T'*H*D elements. dst and src are distinct buffers; the caller frees src afterwards
+ * (stream order keeps it alive for this copy). */
+int aionhip_cache_grow(aionhip_ctx *ctx, aionhip_handle dst, aionhip_handle src, size_t outer, size_t old_run_bytes,
+                       size_t new_run_bytes);
+/* The same for a rolling cache [B, capacity, row] (grow.zig:107-150 ensureRollingCacheCapacity, which goes through the
+ * host; here one kernel): the row of logical step t is t % capacity, so the retained steps of batch entry b - the last
+ * min(end, retained_history, old_capacity) steps before end = logical_ends[b] (i32 [B] on device) - move to row
+ * t % new_capacity; all other rows of dst are zero. new_capacity > old_capacity > 0. */
+int aionhip_cache_grow_rolling(aionhip_ctx *ctx, aionhip_handle dst, aionhip_handle src, aionhip_handle logical_ends, size_t b,
+                               size_t old_capacity, size_t new_capacity, size_t row_bytes, size_t retained_history);
+/* The next capacity of a geometric growth schedule (storage/manager.zig:69-76 growTarget, storage/cache.zig:129-137):
+ * ceil(current * num / den), or current + 1 where that is no growth. 0 = invalid argument or overflow. Host only. */
+size_t aionhip_cache_grow_target(size_t current, size_t num, size_t den);
 /* Measurement aid with no counterpart in aion: reads `bytes` of `src` from byte `offset` with a plain
  * streaming kernel and discards them (`sink`: any 4-byte device buffer, normally left untouched). Timed by
  * the profiler as "stream_read"; bench.py reports the GEMV kernels beside it. offset, bytes: multiples of 16. */

@@ -206,7 +206,7 @@ class PackageBuilder:
         return bytes(out)
 
 
-def build_decoder_package(cfg, blocks_of, embed, gammas=None, window=None, retained=0):
+def build_decoder_package(cfg, blocks_of, embed, gammas=None, window=None, retained=0, growable=False):
     """The config-5 decoder authored as a graph (the pattern of src/bench/models.zig:433-536 trimmed to a plain
     pre-norm block; the weight and cache operands as aion declares them): inputs tokens [1,seq] i32, positions
     [1,seq] i32, write_index [1] i32, visible_end [1] i32, and per layer a k and a v cache [1,ctx,Hkv,D] f16 that
@@ -216,7 +216,8 @@ def build_decoder_package(cfg, blocks_of, embed, gammas=None, window=None, retai
     cfg: layers, hidden, heads, kv_heads, head_dim, ffn, vocab, eps, rope_base, wdtype ("q4_0" | "q8_0");
     blocks_of(name) -> packed blocks ([K,N] quant_axis 0 for q4_0, [N,K] quant_axis 1 for q8_0); embed f32 [vocab,hidden].
     window: (left, right, chunk) of every Attention (default causal); retained > 0 declares the caches rolling rings
-    that keep that many earlier positions (a sliding-window layer, src/bench/models.zig:440-447)."""
+    that keep that many earlier positions (a sliding-window layer, src/bench/models.zig:440-447); growable sets the
+    caches' allow_growable role flag."""
     b = PackageBuilder()
     seq, ctx = b.symbol("seq"), b.symbol("ctx")
     H, Hkv, D, E, F, V = cfg["heads"], cfg["kv_heads"], cfg["head_dim"], cfg["hidden"], cfg["ffn"], cfg["vocab"]
@@ -230,7 +231,8 @@ def build_decoder_package(cfg, blocks_of, embed, gammas=None, window=None, retai
     for l in range(cfg["layers"]):
         for kv in "kv":
             caches.append(b.input("l%d.%s_cache" % (l, kv), "f16", (1, ctx, Hkv, D), role="sequence_cache", axis=1,
-                                  capacity_symbol=0 + 1, retained=retained))   # dim symbol 1 = "ctx"
+                                  capacity_symbol=0 + 1, retained=retained,      # dim symbol 1 = "ctx"
+                                  flags=3 if growable else 1))                  # zero_init | allow_growable (types.zig:179-183)
 
     def weight(name, k, n):
         blocks = blocks_of(name)

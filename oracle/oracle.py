@@ -261,6 +261,64 @@ def sequence_append(cache, new, end_index, rolling=False):
     return out
 
 
+def grow_target(current, num, den):
+    """StorageManager.growTarget (storage/manager.zig:69-76; the same rule as storage/cache.zig:129-137)."""
+    if current == 0 or num == 0 or den == 0:
+        raise ValueError("grow_target: InvalidArgument")
+    nxt = (current * num + den - 1) // den
+    return current + 1 if nxt <= current else nxt
+
+
+def grow_axis(cache, axis, new_size):
+    """growAxisOnDevice / growAxisPreserveScalar (storage/manager/grow.zig:37-78): the tensor grows along `axis`, existing
+    elements keep their indices, new elements are zero."""
+    cache = np.asarray(cache)
+    if new_size < cache.shape[axis]:
+        raise ValueError("grow_axis: InvalidArgument")
+    shape = list(cache.shape)
+    shape[axis] = new_size
+    out = np.zeros(shape, cache.dtype)
+    out[tuple(slice(0, n) for n in cache.shape)] = cache
+    return out
+
+
+def grow_rolling(cache, new_capacity, retained_history, logical_ends):
+    """ensureRollingCacheCapacity (storage/manager/grow.zig:107-150): cache [B, T, ...] is a ring; the last
+    min(end, retained_history, T) logical steps before each batch entry's end move to row t % new_capacity, the rest
+    of the new ring is zero."""
+    cache = np.asarray(cache)
+    B, T = cache.shape[0], cache.shape[1]
+    if len(logical_ends) != B or T == 0:
+        raise ValueError("grow_rolling: InvalidArgument")
+    if T >= new_capacity:
+        return cache.copy()
+    out = np.zeros((B, new_capacity) + cache.shape[2:], cache.dtype)
+    for b, end in enumerate(logical_ends):
+        end = int(end)
+        kept = min(end, retained_history, T)
+        for t in range(end - kept, end):
+            out[b, t % new_capacity] = cache[b, t % T]
+    return out
+
+
+def session_growth_target(capacity, required, num, den, max_capacity=0):
+    """growSequenceCache (api/loaded_model.zig:791-827): geometric steps until `required` fits, then rounded up to a
+    power of two and to at least four times the old capacity (each capacity is a compiled shape), clipped to the
+    policy's ceiling. Rolling caches use the factor 2/1 and no ceiling."""
+    target = capacity
+    while target < required:
+        target = grow_target(target, num, den)
+    p2 = 1
+    while p2 < target:
+        p2 *= 2
+    target = max(p2, capacity * 4)
+    if max_capacity:
+        if required > max_capacity:
+            raise ValueError("session_growth_target: InvalidArgument")
+        target = min(target, max_capacity)
+    return target
+
+
 def rmsnorm(x, gamma, eps, beta=None, residual=None):
     x = _f32(x); rows, cols = x.shape
     g = _f32(gamma); b = None if beta is None else _f32(beta); r = None if residual is None else _f32(residual)

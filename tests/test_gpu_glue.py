@@ -256,3 +256,53 @@ def test_stream_read_probe_runs_and_checks_its_arguments(gpu):
         with pytest.raises(be.AionHipError):
             gpu.probe_stream_read(src, off, nb, sink)
     src.free(); sink.free()
+
+
+def test_cache_growth_golden_vectors(gpu):
+    # storage/test_storage.zig:883-898: ring [4,5,0,3], end 6, 3 retained, grown to 7
+    src, ends = gpu.upload(np.array([4, 5, 0, 3], np.float32)), gpu.upload(np.array([6], np.int32))
+    dst = gpu.upload(np.full(7, 77, np.float32))
+    gpu.cache_grow_rolling(dst, src, ends, 1, 4, 7, 4, 3)
+    assert gpu.download(dst, np.float32, (7,)).tolist() == [0, 0, 0, 3, 4, 5, 0]
+    # backend/cpu/test_cpu_backend.zig:4718-4790: [0,1,2,3] grown to 8, then [90,91] appended at 5 (here an f16 cache)
+    old = gpu.upload(np.array([0, 1, 2, 3], np.float16))
+    new = gpu.upload(np.full(8, 77, np.float16))
+    gpu.cache_grow(new, old, 1, 8, 16)
+    app, wi = gpu.upload(np.array([90, 91], np.float32)), gpu.upload(np.array([5], np.int32))
+    gpu.step_append_f16(new, app, wi, 1, 2, 8, 1)
+    assert gpu.download(new, np.float16, (8,)).tolist() == [0, 1, 2, 3, 0, 90, 91, 0]
+    # storage/test_storage.zig:862-873 and the schedule's corner cases
+    assert gpu.cache_grow_target(8, 2, 1) == 16 and gpu.cache_grow_target(3, 3, 2) == 5 and gpu.cache_grow_target(5, 1, 1) == 6
+    with pytest.raises(ValueError):
+        gpu.cache_grow_target(0, 2, 1)
+    for t in (src, ends, dst, old, new, app, wi):
+        t.free()
+
+
+@pytest.mark.parametrize("B,T,new_T,H,D", [(1, 4, 16, 1, 2), (3, 7, 9, 2, 64), (2, 128, 512, 1, 256)])
+def test_cache_growth_against_the_oracle(gpu, orc, B, T, new_T, H, D):
+    rng = np.random.default_rng(11)
+    cache = rng.standard_normal((B, T, H, D)).astype(np.float16)
+    src = gpu.upload(cache)
+    dst = gpu.upload(np.full((B, new_T, H, D), 7, np.float16))             # stale contents must not survive
+    gpu.cache_grow(dst, src, B, T * H * D * 2, new_T * H * D * 2)
+    assert np.array_equal(gpu.download(dst, np.float16, (B, new_T, H, D)), orc.grow_axis(cache, 1, new_T))
+    for retained, ends in ((T, [T + 3] * B), (max(1, T // 2), list(range(1, 2 * T, max(1, (2 * T - 1) // B)))[:B]), (10 * T, [0] * B), (3, [5 * T + b for b in range(B)])):
+        eb = gpu.upload(np.array(ends, np.int32))
+        gpu.write(dst, np.full((B, new_T, H, D), 7, np.float16))
+        gpu.cache_grow_rolling(dst, src, eb, B, T, new_T, H * D * 2, retained)
+        assert np.array_equal(gpu.download(dst, np.float16, (B, new_T, H, D)), orc.grow_rolling(cache, new_T, retained, ends)), (retained, ends)
+        eb.free()
+    src.free(); dst.free()
+
+
+def test_cache_growth_rejects_bad_arguments(gpu):
+    from aion_amd.hip import AionHipError
+    a, b, e = gpu.zeros(64), gpu.zeros(64), gpu.zeros(4)
+    for call in (lambda: gpu.cache_grow(a, a, 1, 8, 16), lambda: gpu.cache_grow(a, b, 1, 16, 8), lambda: gpu.cache_grow(a, b, 1, 6, 16),
+                 lambda: gpu.cache_grow_rolling(a, b, e, 1, 4, 4, 4, 3), lambda: gpu.cache_grow_rolling(a, b, e, 1, 0, 4, 4, 3),
+                 lambda: gpu.cache_grow_rolling(a, b, e, 1, 4, 8, 6, 3), lambda: gpu.cache_grow_rolling(a, a, e, 1, 4, 8, 4, 3)):
+        with pytest.raises(AionHipError):
+            call()
+    gpu.cache_grow(a, b, 0, 8, 16)          # nothing to do
+    a.free(); b.free(); e.free()

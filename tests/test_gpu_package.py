@@ -175,3 +175,80 @@ def test_sliding_window_package_on_rolling_caches_equals_full_caches(gpu):
         assert ring.pos == 107
     finally:
         ring.close(); full.close()
+
+
+def test_growing_caches_match_preallocated_ones(gpu):
+    """A session whose caches start at 8 rows and grow on the device (8 -> 32 -> 128) must produce the tokens of one
+    whose caches were allocated at 128 rows from the start (api/test_sequence_cache.zig:228 "a growable cache matches
+    a preallocated one"): growth keeps every row where it was. Logits are compared to f32 rounding, not bit for bit:
+    the attention kernels split their key range by the cache's capacity."""
+    cfg = DecoderConfig(wdtype=be.Q4_0, **SMALL)
+    weights = SyntheticWeights(cfg, 17)
+    d = dict(layers=cfg.layers, hidden=cfg.hidden, heads=cfg.heads, kv_heads=cfg.kv_heads, head_dim=cfg.head_dim, ffn=cfg.ffn,
+             vocab=cfg.vocab, eps=cfg.eps, rope_base=cfg.rope_base, wdtype="q4_0")
+    pkg = aion_file.parse(aion_writer.build_decoder_package(d, weights.blocks, weights.embed(), growable=True))
+    fixed_pkg = aion_file.parse(aion_writer.build_decoder_package(d, weights.blocks, weights.embed()))
+    assert pkg.role_of_input(4).flags == 3 and fixed_pkg.role_of_input(4).flags == 1
+    with pytest.raises(Unsupported):
+        PackageRunner(gpu, fixed_pkg, capacity=8, growth=dict(numerator=2, denominator=1))
+    grow = PackageRunner(gpu, pkg, capacity=8, growth=dict(numerator=2, denominator=1, max_capacity=128))
+    full = PackageRunner(gpu, pkg, capacity=128)
+    try:
+        prompt = np.random.default_rng(3).integers(0, cfg.vocab, 11).astype(np.int32)      # 11 rows: the first growth, 8 -> 32
+        a, b = grow.run(prompt, want=("next_token", "logits")), full.run(prompt, want=("next_token", "logits"))
+        assert grow.capacity == 32
+        assert np.allclose(a["logits"], b["logits"], atol=2e-4, rtol=1e-4)
+        assert np.array_equal(a["next_token"], b["next_token"])
+        tok = int(b["next_token"][0, -1])
+        # eager single tokens up to the edge of 32, then the recorded program across the second growth
+        for step in range(15):
+            a, b = grow.run([tok], want=("next_token", "logits")), full.run([tok], want=("next_token", "logits"))
+            assert np.allclose(a["logits"], b["logits"], atol=2e-4, rtol=1e-4), step
+            assert np.array_equal(a["next_token"], b["next_token"]), step
+            tok = int(b["next_token"][0, -1])
+        grow.begin_decode(tok); full.begin_decode(tok)
+        for step in range(60):
+            ta, tb = grow.decode_step(), full.decode_step()
+            assert ta == tb, step
+        assert grow.capacity == 128 and grow.pos == full.pos == 86
+        # the grown caches hold what the preallocated ones hold
+        for idx in grow.caches:
+            got = gpu.download(grow.caches[idx], np.float16, (128, cfg.kv_heads * cfg.head_dim))
+            want = gpu.download(full.caches[idx], np.float16, (128, cfg.kv_heads * cfg.head_dim))
+            assert np.allclose(got[:86].astype(np.float32), want[:86].astype(np.float32), atol=4e-3) and not got[86:].any()
+        with pytest.raises(ValueError):
+            grow.run(np.zeros(60, np.int32))                                            # 146 rows: past the ceiling
+    finally:
+        grow.close(); full.close()
+
+
+def test_rolling_caches_grow_for_a_long_run(gpu):
+    """A ring of 64 rows (12 retained) asked to take a 60-token run needs 12 + 60 rows: it grows to 256 with its
+    retained rows re-placed (storage/manager/grow.zig:107-150), and the session goes on as one that had 256 rows all
+    along, also after the positions wrap around the ring. (Both rings are at least one 64-key tile long, so both
+    sessions run on the same kernel family from the first run on.)"""
+    cfg = DecoderConfig(wdtype=be.Q4_0, **SMALL)
+    weights = SyntheticWeights(cfg, 19)
+    d = dict(layers=cfg.layers, hidden=cfg.hidden, heads=cfg.heads, kv_heads=cfg.kv_heads, head_dim=cfg.head_dim, ffn=cfg.ffn,
+             vocab=cfg.vocab, eps=cfg.eps, rope_base=cfg.rope_base, wdtype="q4_0")
+    pkg = aion_file.parse(aion_writer.build_decoder_package(d, weights.blocks, weights.embed(), window=(12, 0, 0), retained=12))
+    grow = PackageRunner(gpu, pkg, capacity=64, growth=dict(numerator=2, denominator=1), fuse=False)
+    full = PackageRunner(gpu, pkg, capacity=256, fuse=False)
+    fixed = PackageRunner(gpu, pkg, capacity=64, fuse=False)
+    try:
+        rng = np.random.default_rng(4)
+        first, second = rng.integers(0, cfg.vocab, 14).astype(np.int32), rng.integers(0, cfg.vocab, 60).astype(np.int32)
+        for r in (grow, full, fixed):
+            r.run(first)
+        with pytest.raises(ValueError):
+            fixed.run(second)
+        a, b = grow.run(second, want=("next_token", "logits")), full.run(second, want=("next_token", "logits"))
+        assert grow.capacity == 256
+        assert np.allclose(a["logits"], b["logits"], atol=2e-4, rtol=1e-4)
+        tok = int(b["next_token"][0, -1])
+        for step in range(200):                                    # positions 74 .. 273: around the ring
+            a, b = grow.run([tok], want=("next_token", "logits")), full.run([tok], want=("next_token", "logits"))
+            assert np.allclose(a["logits"], b["logits"], atol=2e-4, rtol=1e-4), step
+            tok = int(b["next_token"][0, -1])
+    finally:
+        grow.close(); full.close(); fixed.close()
