@@ -540,6 +540,9 @@ constexpr float PF_LAZY = 8.f;
 #ifndef PF_AHEAD
 #define PF_AHEAD 3
 #endif
+#ifndef PF_PIPE_D
+#define PF_PIPE_D 256      // head sizes from here on run the software-pipelined tile loop
+#endif
 using f32x16 = __attribute__((ext_vector_type(16))) float;
 using u32x2 = __attribute__((ext_vector_type(2))) unsigned int;
 
@@ -706,6 +709,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
     float m_run = -INFINITY, l_run = 0.f;
     const float cap_inv = CAP ? 1.f / a.soft_cap : 0.f;
 
+    if constexpr (D < PF_PIPE_D) {
     load_k(t_begin, lds);
     load_v(t_begin);
     store_v(lds);
@@ -743,7 +747,6 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
                 s[0] = mfma32<KV>(k0, qf[kk], s[0]);
                 s[1] = mfma32<KV>(k1, qf[kk], s[1]);
             }
-#ifndef PF_NO_PIPE
             // issue order: the LDS reads run PF_AHEAD k-steps ahead of the MFMAs that consume them (left alone the
             // compiler issues each read right before its MFMA, which then waits out the whole LDS latency)
             __builtin_amdgcn_sched_group_barrier(0x100, 2 * PF_AHEAD, 0);
@@ -753,7 +756,6 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
                 __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
             }
             __builtin_amdgcn_sched_group_barrier(0x008, 2 * PF_AHEAD, 0);
-#endif
             // -- lane holds keys key0 + kb*32 + (i/4)*8 + lh*4 + i%4 of row l31
             float x[32];
             const bool full = key0 >= w_lo_max && key0 + PF_TK <= w_hi_min;   // every key visible to every row
@@ -828,7 +830,6 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
                     const u32x2 va = *(const u32x2 *)(vrow), vb = *(const u32x2 *)(vrow + 16);
                     acc[j] = mfma32<KV>(u32x4{va.x, va.y, vb.x, vb.y}, pf[s2], acc[j]);
                 }
-#ifndef PF_NO_PIPE
             __builtin_amdgcn_sched_group_barrier(0x100, 2 * PF_AHEAD, 1);
 #pragma unroll
             for (int i = 0; i < 4 * NJ - 2 * PF_AHEAD; ++i) {
@@ -836,10 +837,223 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
                 __builtin_amdgcn_sched_group_barrier(0x100, 1, 1);
             }
             __builtin_amdgcn_sched_group_barrier(0x008, 2 * PF_AHEAD, 1);
-#endif
         }
         if (more) store_v(nx);
         __syncthreads();                                           // also waits for this wavefront's K loads (fence)
+    }
+
+    } else {
+    // operand addresses: K row (kb*32 + l31) at slot (2*kk + lh) ^ swz(row); V^T row (j*32 + l31), keys of step s2
+    const int k_swz = CPK >= 16 ? (l31 & 15) : ((l31 >> 1) & 7);
+    const int k_row = l31 * Cfg::KROW;
+    const int v_off = Cfg::K_BYTES + l31 * PF_VROW + lh * 8;        // + j * 32 rows + s2 * 32 bytes (+16 for the second 4 keys)
+
+    // Head size 256 and up (below, the serial loop above is faster: fewer MFMAs per tile to hide anything behind).
+    // The loop is software-pipelined over the key tiles: iteration t computes S_t = K_t . Q^T, then the softmax of
+    // S_t (vector ALU) TOGETHER WITH O += V_(t-1)^T . P_(t-1) (matrix pipe) - one wavefront per SIMD has nobody else
+    // to fill the matrix pipe while it computes exponentials, so it has to overlap the two itself. P_(t-1) and the
+    // running statistics of tile t-1 are consistent with the accumulators; the rescale by alpha_t follows the product.
+    // LDS: K_t sits in stage t&1 (requested an iteration ahead), V_t is requested into registers in iteration t-1,
+    // transposed into stage t&1 at the top of iteration t and consumed in iteration t+1: one barrier per tile.
+    f32x16 sc[2];
+    u32x4 pf[4] = {};
+    auto tile_qk = [&](const unsigned char *st) __attribute__((always_inline)) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) sc[kb][i] = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            const int slot = ((2 * kk + lh) ^ k_swz) * 16;
+            const u32x4 k0 = *(const u32x4 *)(st + k_row + slot);
+            const u32x4 k1 = *(const u32x4 *)(st + 32 * Cfg::KROW + k_row + slot);
+            sc[0] = mfma32<KV>(k0, qf[kk], sc[0]);
+            sc[1] = mfma32<KV>(k1, qf[kk], sc[1]);
+        }
+    };
+    // scaled (capped, masked) scores of the tile: lane holds keys key0 + kb*32 + (i/4)*8 + lh*4 + i%4 of row l31.
+    // No branch in this kernel may contain an MFMA on the output accumulators (the compiler would then carry them in
+    // vector registers and copy all of them to and from the accumulation registers on every tile), so the one
+    // wavefront-uniform branch of a tile - mask or no mask - sits here, around vector instructions only.
+    float x[32];
+    auto tile_scores = [&](int key0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            float v = sc[i >> 4][i & 15] * a.scale;
+            if (CAP) v = a.soft_cap * tanhf(v * cap_inv);
+            x[i] = v;
+        }
+        const bool full = key0 >= w_lo_max && key0 + PF_TK <= w_hi_min;   // every key visible to every row
+        if (!full) {
+            // key = key0 + 4*lh + c_i is visible iff lo <= key < hi, i.e. (unsigned)(c_i - lo_rel) < span
+            const int lo_rel = lo - (key0 + lh * 4);
+            const unsigned span = (unsigned)(hi - lo);
+#pragma unroll
+            for (int i = 0; i < 32; ++i) {
+                const int c = (i >> 4) * 32 + ((i >> 2) & 3) * 8 + (i & 3);
+                x[i] = (unsigned)(c - lo_rel) < span ? x[i] : -INFINITY;
+            }
+        }
+    };
+    // softmax of x -> pf (next iteration's P^T operand), interleaved with the product of the previous tile
+    auto tile_softmax_pv = [&](auto with_pv_c, const unsigned char *vst) __attribute__((always_inline)) {
+        constexpr bool WITH_PV = decltype(with_pv_c)::value;
+        // The softmax is cut into 32 units of a few vector instructions, and the product of the previous tile into its
+        // NM MFMAs; unit group k is issued right behind MFMA k and a scheduling barrier keeps the pairs in this order
+        // (left to itself the compiler issues the whole softmax first and the MFMAs behind it). The V^T operand of
+        // MFMA k + PV_AHEAD is requested behind MFMA k.
+        //   units 0..7    partial maxima of four scores each (two chains)
+        //   unit  8       row maximum across the two lane halves, new reference maximum, alpha, exponent offset
+        //   units 9..24   two exponentials each, partial sums (two chains)
+        //   units 25..28  the four P^T operands of the next product
+        //   unit  29      row sum across the lane halves, running sum and maximum
+        constexpr int NM = 4 * NJ, UPM = 32 / NM, PV_AHEAD = NM >= 16 ? 4 : 2;
+        float mxp[2] = {-INFINITY, -INFINITY}, rs[2] = {0.f, 0.f};
+        float m_new = m_run, alpha = 1.f, mneg = 0.f;
+        u32x4 pn[4];
+        auto unit = [&](int u) __attribute__((always_inline)) {
+            if (u < 8) {
+                mxp[u & 1] = fmaxf(fmaxf(mxp[u & 1], fmaxf(x[4 * u], x[4 * u + 1])), fmaxf(x[4 * u + 2], x[4 * u + 3]));
+            } else if (u == 8) {
+                float mx = fmaxf(mxp[0], mxp[1]);
+                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                // the reference maximum only moves when the tile's maximum exceeds it by more than PF_LAZY:
+                // probabilities stay below e^PF_LAZY (exact in the f32 sums, fine in the 16-bit operand) and the
+                // 2*D-register rescale of the accumulators becomes rare after the first tiles
+                m_new = mx > m_run + PF_LAZY ? mx : m_run;
+                // branch-free: with nothing visible so far (m_new = -inf) the exponent's offset is 0 and every
+                // masked score still gives exp2(-inf) = 0
+                alpha = m_run > -INFINITY ? __builtin_amdgcn_exp2f((m_run - m_new) * LOG2E) : 1.f;
+                mneg = m_new > -INFINITY ? -m_new * LOG2E : 0.f;
+            } else if (u < 25) {
+                const int i0 = 2 * (u - 9);
+                x[i0] = __builtin_amdgcn_exp2f(fmaf(x[i0], LOG2E, mneg));
+                x[i0 + 1] = __builtin_amdgcn_exp2f(fmaf(x[i0 + 1], LOG2E, mneg));
+                rs[0] += x[i0];
+                rs[1] += x[i0 + 1];
+            } else if (u < 29) {
+                const int s2 = u - 25;
+                // P^T operand of 16-key step s2: slots 0..7 <- accumulator elements 8*s2 .. 8*s2+7
+                pn[s2] = u32x4{pack2<KV>(x[8 * s2], x[8 * s2 + 1]), pack2<KV>(x[8 * s2 + 2], x[8 * s2 + 3]),
+                               pack2<KV>(x[8 * s2 + 4], x[8 * s2 + 5]), pack2<KV>(x[8 * s2 + 6], x[8 * s2 + 7])};
+            } else if (u == 29) {
+                float rowsum = rs[0] + rs[1];
+                rowsum += __shfl_xor(rowsum, 32, 64);
+                l_run = l_run * alpha + rowsum;
+                m_run = m_new;
+            }
+        };
+        if (WITH_PV) {
+            // -- O^T += V^T . P^T of the previous tile; key step outermost: consecutive MFMAs go to different accumulators
+            auto v_operand = [&](int idx) __attribute__((always_inline)) {
+                const unsigned char *vrow = vst + v_off + (idx % NJ) * 32 * PF_VROW + (idx / NJ) * 32;
+                const u32x2 va = *(const u32x2 *)(vrow), vb = *(const u32x2 *)(vrow + 16);
+                return u32x4{va.x, va.y, vb.x, vb.y};
+            };
+            u32x4 vop[PV_AHEAD];
+#pragma unroll
+            for (int k = 0; k < PV_AHEAD; ++k) vop[k] = v_operand(k);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int k = 0; k < NM; ++k) {
+                acc[k % NJ] = mfma32<KV>(vop[k % PV_AHEAD], pf[k / NJ], acc[k % NJ]);
+                if (k + PV_AHEAD < NM) vop[k % PV_AHEAD] = v_operand(k + PV_AHEAD);
+#pragma unroll
+                for (int u = k * UPM; u < (k + 1) * UPM; ++u) unit(u);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < 30; ++u) unit(u);
+        }
+        if (__any(alpha != 1.f)) {              // wavefront-uniform and rare: must stay a branch, not a select
+            // The accumulators live in accumulation registers for the MFMAs. Written as plain C++ the multiply
+            // makes the compiler keep them in vector registers around this branch and copy all of them back and
+            // forth on the common path (several hundred moves per key tile). So: read, scale and write back each
+            // one here, with the register class pinned. The s_nops cover the waits between an MFMA result and
+            // its read, and between the write-back and the next MFMA, which the compiler cannot see in here.
+            asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory");
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    float tmp;
+                    asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 1\n\tv_accvgpr_write_b32 %0, %1"
+                                 : "+a"(acc[j][i]), "=&v"(tmp) : "v"(alpha));
+                }
+            asm volatile("s_nop 7" ::: "memory");
+        }
+#pragma unroll
+        for (int s2 = 0; s2 < 4; ++s2) pf[s2] = pn[s2];
+    };
+    auto pin_acc = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) asm volatile("" : "+a"(acc[j][i]));
+    };
+    using yes = std::integral_constant<bool, true>;
+    using no = std::integral_constant<bool, false>;
+
+    // one tile's front half: V_t to LDS for the next iteration's product, requests for tile t+1, S_t
+    auto tile_front = [&](int t) __attribute__((always_inline)) {
+        unsigned char *st = lds + ((t - t_begin) & 1) * Cfg::STAGE;
+        unsigned char *other = lds + ((t - t_begin + 1) & 1) * Cfg::STAGE;
+        store_v(st);
+        // unconditional (a branch would split the block): past the end the last tile is requested once more, into
+        // the stage and the registers that nobody reads again
+        const int tn = min(t + 1, t_end - 1);
+        load_k(tn, other);
+        load_v(tn);
+        tile_qk(st);
+        // issue order: the LDS reads run PF_AHEAD k-steps ahead of the MFMAs that consume them (left alone the
+        // compiler issues each read right before its MFMA, which then waits out the whole LDS latency)
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * PF_AHEAD, 0);
+#pragma unroll
+        for (int kk = 0; kk < KK - PF_AHEAD; ++kk) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 2 * PF_AHEAD, 0);
+        tile_scores(t * PF_TK);
+    };
+
+    load_k(t_begin, lds);
+    load_v(t_begin);
+    __syncthreads();                                               // K of the first tile has landed (fence)
+    // first tile, peeled: there is no previous product to overlap with
+    tile_front(t_begin);
+    tile_softmax_pv(no{}, lds);
+    __syncthreads();
+    for (int t = t_begin + 1; t < t_end; ++t) {
+        // the accumulators are declared to sit in accumulation registers here and after the front half: without
+        // these two pins the register allocator parks them in vector registers while S_t is computed and copies all
+        // of them back for the product (2 x D/2 moves per tile)
+        pin_acc();
+        tile_front(t);
+        pin_acc();
+        tile_softmax_pv(yes{}, lds + ((t - t_begin + 1) & 1) * Cfg::STAGE);
+        __syncthreads();                                           // also waits for this wavefront's K loads (fence)
+    }
+    {   // the last tile's product
+        const unsigned char *vst = lds + ((t_end - 1 - t_begin) & 1) * Cfg::STAGE;
+        constexpr int NM = 4 * NJ, PV_AHEAD = 4;
+        auto v_operand = [&](int idx) __attribute__((always_inline)) {
+            const unsigned char *vrow = vst + v_off + (idx % NJ) * 32 * PF_VROW + (idx / NJ) * 32;
+            const u32x2 va = *(const u32x2 *)(vrow), vb = *(const u32x2 *)(vrow + 16);
+            return u32x4{va.x, va.y, vb.x, vb.y};
+        };
+        u32x4 vop[PV_AHEAD];
+#pragma unroll
+        for (int k = 0; k < PV_AHEAD; ++k) vop[k] = v_operand(k);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int k = 0; k < NM; ++k) {
+            acc[k % NJ] = mfma32<KV>(vop[k % PV_AHEAD], pf[k / NJ], acc[k % NJ]);
+            if (k + PV_AHEAD < NM) vop[k % PV_AHEAD] = v_operand(k + PV_AHEAD);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
     }
 
     if (row_ok) {
