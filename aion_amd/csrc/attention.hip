@@ -540,6 +540,12 @@ constexpr float PF_LAZY = 8.f;
 #ifndef PF_AHEAD
 #define PF_AHEAD 3
 #endif
+#ifndef PF_FLASH_BELOW
+#define PF_FLASH_BELOW 8   // prompts whose 128-row workgroups would fill under 1/PF_FLASH_BELOW of the CUs run on the 16-row split kernel
+#endif
+#ifndef PF_SEG_TILES
+#define PF_SEG_TILES 4     // fewest 64-key tiles a key segment of the prefill kernel is worth
+#endif
 #ifndef PF_PIPE_D
 #define PF_PIPE_D 256      // head sizes from here on run the software-pipelined tile loop
 #endif
@@ -638,14 +644,30 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
     __syncthreads();
     const int g_lo = min(min(s_rng[0], s_rng[1]), min(s_rng[2], s_rng[3]));
     const int g_hi = max(max(s_rng[4], s_rng[5]), max(s_rng[6], s_rng[7]));
-    if (g_hi <= g_lo) {                                 // nothing visible to any row: zeros
+    // key segments (a.nseg > 1: few row tiles on many CUs): workgroup z takes the z-th part of the union's tiles and
+    // leaves its unnormalized accumulators, reference maximum and sum in the partial buffer for attn_merge_kernel
+    const int nseg = a.nseg, seg = blockIdx.z;
+    int t_begin = g_lo / PF_TK, t_end = (g_hi + PF_TK - 1) / PF_TK;
+    bool nothing = g_hi <= g_lo;
+    if (nseg > 1 && !nothing) {
+        const int per = (t_end - t_begin + nseg - 1) / nseg;
+        t_begin += seg * per;
+        t_end = min(t_end, t_begin + per);
+        nothing = t_begin >= t_end;
+    }
+    float *part = nullptr;
+    if (nseg > 1) part = a.partial + ((size_t)(unit * a.row_tiles + (r >> 4)) * nseg + seg) * (16 * D + 32);
+    if (nothing) {                                      // nothing visible to any row: zeros / an empty partial
         if (row_ok) {
-            float *o = a.out + qbase;
+            float *o = nseg > 1 ? part + (r & 15) * D : a.out + qbase;
             for (int d = lh * (D / 2); d < (lh + 1) * (D / 2); d += 4) *(f32x4 *)(o + d) = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (nseg > 1 && lh == 0) {
+                part[16 * D + (r & 15)] = -INFINITY;
+                part[16 * D + 16 + (r & 15)] = 0.f;
+            }
         }
         return;
     }
-    const int t_begin = g_lo / PF_TK, t_end = (g_hi + PF_TK - 1) / PF_TK;
 
     const unsigned short *kp = (const unsigned short *)a.k;
     const unsigned short *vp = (const unsigned short *)a.v;
@@ -1057,8 +1079,12 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
     }
 
     if (row_ok) {
-        const float inv = l_run > 0.f ? 1.f / l_run : 0.f;          // empty interval -> zeros
-        float *o = a.out + qbase;
+        const float inv = nseg > 1 ? 1.f : (l_run > 0.f ? 1.f / l_run : 0.f);          // empty interval -> zeros
+        float *o = nseg > 1 ? part + (r & 15) * D : a.out + qbase;
+        if (nseg > 1 && lh == 0) {
+            part[16 * D + (r & 15)] = m_run;
+            part[16 * D + 16 + (r & 15)] = l_run;
+        }
 #pragma unroll
         for (int j = 0; j < NJ; ++j)
 #pragma unroll
@@ -1141,6 +1167,53 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnArgs a) {
     }
 }
 
+// The same merge for many rows and few segments (the prefill kernel's key segments): one thread per (row, four
+// consecutive dv), so that a wavefront reads whole contiguous rows of every segment's accumulators.
+template <int D>
+__global__ __launch_bounds__(256) void attn_merge_rows_kernel(AttnArgs a) {
+    constexpr int WSTRIDE = 16 * D + 32;
+    constexpr int TPR = D / 4, RPB = 256 / TPR;          // threads per row, rows per workgroup
+    constexpr int UN = 4;
+    const int unit = blockIdx.y, b = unit / a.Hkv, hk = unit % a.Hkv;
+    const int rr = blockIdx.x * RPB + (int)threadIdx.x / TPR, dv = ((int)threadIdx.x % TPR) * 4;
+    if (rr >= a.rows_total) return;
+    const int rt = rr >> 4, row = rr & 15;
+    const float *base = a.partial + (size_t)(unit * a.row_tiles + rt) * a.nseg * WSTRIDE;
+    float m_all = -INFINITY, l_all = 0.f;
+    f32x4 o = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < a.nseg; s0 += UN) {
+        float ms[UN], ls[UN];
+        f32x4 os[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const float *p = base + (size_t)min(s0 + u, a.nseg - 1) * WSTRIDE;      // clamped: every load is unconditional
+            ms[u] = p[16 * D + row];
+            ls[u] = p[16 * D + 16 + row];
+            os[u] = *(const f32x4 *)(p + row * D + dv);
+        }
+        float m_new = m_all;
+#pragma unroll
+        for (int u = 0; u < UN; ++u)
+            if (s0 + u < a.nseg) m_new = fmaxf(m_new, ms[u]);
+        if (m_new > -INFINITY) {
+            const float f0 = m_all > -INFINITY ? exp2f((m_all - m_new) * LOG2E) : 0.f;
+            o *= f0;
+            l_all *= f0;
+#pragma unroll
+            for (int u = 0; u < UN; ++u) {
+                const bool live = s0 + u < a.nseg && ms[u] > -INFINITY;
+                const float f = live ? exp2f((ms[u] - m_new) * LOG2E) : 0.f;
+                o += os[u] * f;
+                l_all += ls[u] * f;
+            }
+            m_all = m_new;
+        }
+    }
+    const int l2 = rr / a.groups, g3 = rr % a.groups;
+    const float inv = l_all > 0.f ? 1.f / l_all : 0.f;
+    *(f32x4 *)(a.out + (((size_t)b * a.L + l2) * a.Hq + hk * a.groups + g3) * D + dv) = o * inv;
+}
+
 // One wavefront per query row; any head sizes and element types. scores: [rows][T] f32 scratch.
 __global__ __launch_bounds__(256) void attn_generic_kernel(AttnArgs a, int d_k, int d_v, float *scores) {
     const int lane = threadIdx.x & 63;
@@ -1206,7 +1279,7 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
     // (measured: one batch, one kv head, up to ~1024 positions x 8 heads): 16-row tiles spread the K/V reads
     // over many CUs, which outweighs re-reading K/V per row tile from L2.
     const int cus0 = ctx->cu_count > 0 ? ctx->cu_count : 256;
-    const bool split = a.rows_total <= 64 || (!HILO && (long)units * ((a.rows_total + PF_ROWS - 1) / PF_ROWS) * 4 <= cus0);
+    const bool split = a.rows_total <= 64 || (!HILO && (long)units * ((a.rows_total + PF_ROWS - 1) / PF_ROWS) * PF_FLASH_BELOW <= cus0);
     if (split) {
         // key segments: one 32-key tile per wavefront while that leaves the device under-filled,
         // more tiles per wavefront beyond one workgroup per CU (its LDS tiles fill a CU)
@@ -1238,7 +1311,18 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
         LAUNCH_CHECK(ctx, "attn_flash_split");
     } else if (!HILO) {
         using PCfg = PrefillCfg<D>;
-        a.nseg = 1;
+        // Fewer workgroups than half the CUs: the key range of every row tile is cut into segments (at least
+        // PF_SEG_TILES tiles each) and the partial results are merged, as in the decode path.
+        const int wgs = units * ((a.rows_total + PF_ROWS - 1) / PF_ROWS);
+        const int key_tiles = (a.T + PF_TK - 1) / PF_TK;
+        int nseg = max(1, min(min(cus0 / max(wgs, 1), key_tiles / PF_SEG_TILES), 16));
+        a.nseg = nseg;
+        if (nseg > 1) {
+            const size_t bytes = (size_t)units * a.row_tiles * nseg * (16 * D + 32) * sizeof(float);
+            int rc = ensure_scratch2(ctx, bytes);
+            if (rc) return rc;
+            a.partial = (float *)ctx->scratch2;
+        }
         static bool attr_pf[2] = {false, false};
         const bool cap = a.soft_cap > 0.f;
         const void *fn = cap ? (const void *)attn_prefill_kernel<KV, D, true, RING> : (const void *)attn_prefill_kernel<KV, D, false, RING>;
@@ -1246,10 +1330,17 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
             HIP_TRY(ctx, hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, PCfg::LDS_BYTES));
             attr_pf[cap] = true;
         }
-        ProfScope scope(ctx, "attn_prefill");
-        const dim3 grid((unsigned)((a.rows_total + PF_ROWS - 1) / PF_ROWS), (unsigned)units);
-        if (cap) launch_k(ctx, attn_prefill_kernel<KV, D, true, RING>, grid, dim3(256), PCfg::LDS_BYTES, a);
-        else launch_k(ctx, attn_prefill_kernel<KV, D, false, RING>, grid, dim3(256), PCfg::LDS_BYTES, a);
+        {
+            ProfScope scope(ctx, "attn_prefill");
+            const dim3 grid((unsigned)((a.rows_total + PF_ROWS - 1) / PF_ROWS), (unsigned)units, (unsigned)nseg);
+            if (cap) launch_k(ctx, attn_prefill_kernel<KV, D, true, RING>, grid, dim3(256), PCfg::LDS_BYTES, a);
+            else launch_k(ctx, attn_prefill_kernel<KV, D, false, RING>, grid, dim3(256), PCfg::LDS_BYTES, a);
+        }
+        if (nseg > 1) {
+            ProfScope scope(ctx, "attn_merge");
+            constexpr int RPB = 256 / (D / 4);
+            launch_k(ctx, attn_merge_rows_kernel<D>, dim3((unsigned)((a.rows_total + RPB - 1) / RPB), (unsigned)units), dim3(256), 0, a);
+        }
         LAUNCH_CHECK(ctx, "attn_prefill");
     } else {
         a.nseg = 1;

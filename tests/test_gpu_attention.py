@@ -212,11 +212,12 @@ def test_precise_mode_brings_f32_queries_to_f32_accuracy(gpu, orc):
 
 def test_prefill_config4_sizes(gpu, orc):
     # BASELINE config 4a at L = 1024 and 2048: 8 q heads / 1 kv head, head size 256, bf16, scale 1/16, causal;
-    # every row against the f64 reference (1e-2: bf16 MFMA operands). L = 1024 is 64 prefill workgroups (a
-    # quarter of the CUs: split kernel), L = 2048 runs on the prefill kernel. At L = 4096 the oracle is too slow,
+    # every row against the f64 reference (1e-2: bf16 MFMA operands). L = 512 is 32 prefill workgroups (an
+    # eighth of the CUs: 16-row split kernel); L = 1024 and 2048 run on the prefill kernel with the key range of
+    # every row tile cut into 4 and 2 segments that a merge pass folds. At L = 4096 the oracle is too slow,
     # so the kernel is held to properties that do not depend on the size: V = const gives that const back (the
     # probabilities of a row sum to one), and row 0 sees key 0 only.
-    for L, kernel in ((1024, "attn_flash_split"), (2048, "attn_prefill")):
+    for L, kernel in ((512, "attn_flash_split"), (1024, "attn_prefill"), (2048, "attn_prefill")):
         say("prefill config 4 L%d" % L)
         (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(41, 1, L, L, 8, 1, 256, "bf16")
         got = run_attention(gpu, q, k, v, 1 / 16.0, qd, kd)
@@ -304,3 +305,27 @@ def test_rolling_caches(gpu, orc, case):
     err = float(np.abs(got - want).max())
     say("  max err", err)
     assert np.isfinite(got).all() and err < (1e-2 if kind == "bf16" else 2e-3)
+
+
+@pytest.mark.parametrize("window,rolling", [(be.CAUSAL, False), ((300, 0, 0), False), ((200, 40, 64), False), ((300, 0, 0), True)])
+def test_prefill_key_segments_with_windows_and_ragged_lengths(gpu, orc, window, rolling):
+    """The prefill kernel with its key range cut into segments (few row tiles on many CUs) and the merge pass: ragged
+    cache lengths, positions that start inside the cache, windows that leave whole segments of a row tile empty, and
+    a rolling cache. The profile must show the merge pass, or the case did not run in segments."""
+    B, Lq, T, Hq, Hkv, D = 2, 400, 1536, 8, 2, 128
+    ends = np.array([1500, 1000], np.int32)
+    (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(53, B, Lq, T, Hq, Hkv, D, "f16")
+    pos = np.stack([np.arange(e - Lq, e, dtype=np.int32) for e in ends])
+    if rolling:
+        ends = ends + 2 * T                                   # the ring has wrapped twice
+        pos = pos + 2 * T
+    gpu.profile_start()
+    got = run_attention(gpu, q, k, v, 1 / math.sqrt(D), qd, kd, window=window, positions=pos, kv_lengths=ends, rolling=rolling)
+    names = [n for n, _ in gpu.profile_stop()]
+    assert names == ["attn_prefill", "attn_merge"], names
+    if rolling:
+        ref = orc.attention_rolling_f64(qf, kf, vf, 1 / math.sqrt(D), window, pos, ends)
+    else:
+        ref = orc.attention_f64(qf, kf, vf, 1 / math.sqrt(D), window=window, positions=pos, kv_lengths=ends)
+    assert np.isfinite(got).all()
+    assert float(np.abs(got - ref).max()) < 2e-3
