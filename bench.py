@@ -301,9 +301,6 @@ def run_attention(gpu, be):
         prof = gpu.profile_stop()
         # per call: the sum of its kernels (split + merge); median over calls (the first call of a kernel
         # shape may still carry one-time set-up)
-        per_call = []
-        for i in range(iters):
-            per_call.append(0.0)
         kernels = [ms for (nm, ms) in prof if nm in name]
         per = len(kernels) // iters
         per_call = sorted(sum(kernels[i * per:(i + 1) * per]) for i in range(iters))
@@ -314,7 +311,8 @@ def run_attention(gpu, be):
         k = gpu.upload(_bf16_bits(rng.standard_normal((1, L, Hkv, D))))
         v = gpu.upload(_bf16_bits(rng.standard_normal((1, L, Hkv, D))))
         o = gpu.alloc(L * Hq * D * 4)
-        # a prompt whose 128-row workgroups would fill under a quarter of the CUs runs on the split kernel
+        # the 128-row prefill kernel; where its row tiles alone would leave CUs idle (L = 1024, 2048) every row
+        # tile's key range is cut into segments and a merge pass folds them (both kernels are timed)
         ms = timed(("attn_prefill", "attn_flash_split", "attn_merge"), (1, L, L, Hq, Hkv, D, D), (q, k, v, o))
         flops = 4.0 * Hq * D * L * (L + 1) / 2
         tf = flops / (ms * 1e-3) / 1e12
