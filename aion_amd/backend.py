@@ -191,12 +191,12 @@ class HipBackend:
                                                        positions.handle, write_index.handle, b, s, t_cap, h_q, h_kv, d, base, scale_factor, proportion))
 
     def step_rmsnorm_qkv_rope_append(self, wq, wk, wv, x, gamma, eps, q_out, k_cache, v_cache, positions, write_index,
-                                     t_cap, h_q, h_kv, d, base=10000.0, scale_factor=1.0, proportion=1.0, beta_norm=None):
-        """One new token of one sequence: RMSNorm -> q/k/v matmuls -> RoPE -> f16 cache append, one launch."""
+                                     t_cap, h_q, h_kv, d, base=10000.0, scale_factor=1.0, proportion=1.0, beta_norm=None, rolling=False):
+        """One new token of one sequence: RMSNorm -> q/k/v matmuls -> RoPE -> f16 cache append (rolling: into rings), one launch."""
         self._check(self._lib.aionhip_step_rmsnorm_qkv_rope_append(
             self._ctx, wq.ptr, wk.ptr, wv.ptr, x.handle, gamma.handle, beta_norm.handle if beta_norm is not None else 0, eps,
             q_out.handle, k_cache.handle, v_cache.handle, positions.handle, write_index.handle, t_cap, h_q, h_kv, d,
-            base, scale_factor, proportion))
+            base, scale_factor, proportion, 1 if rolling else 0))
 
     def step_rmsnorm_geglu_matmul(self, w_gate, w_up, w_down, x, gamma, eps, c_buf, alpha=1.0, beta=0.0, beta_norm=None):
         """One activation row: RMSNorm -> gate/up matmuls -> gelu gate -> down matmul, two launches."""

@@ -175,6 +175,7 @@ struct FusedEpi {
     const float *freq;
     __half *k_cache, *v_cache;
     int t_cap, h_kv, d, rope_pairs;
+    int rolling;         // the caches are rings: logical step t lives in row t % t_cap
     int *act_q;          // EPI_GATE_QUANT: prepared activation planes of the down projection
     float *act_scale;
     int *act_sum;

@@ -260,7 +260,8 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedI
                     cur.c[head * epi.d + i] = yl;
                     cur.c[head * epi.d + half + i] = yh;
                 } else {
-                    const long t = (long)epi.write_index[0];
+                    long t = (long)epi.write_index[0];
+                    if (epi.rolling && t >= 0) t %= (long)epi.t_cap;                  // storage/cache.zig:202-207
                     if (t >= 0 && t < (long)epi.t_cap) {                               // never write outside the cache
                         __half *dst = (cur.seg == 1 ? epi.k_cache : epi.v_cache) + ((size_t)t * epi.h_kv + head) * epi.d;
                         dst[i] = __float2half_rn(yl);

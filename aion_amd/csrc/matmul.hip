@@ -136,7 +136,7 @@ int aionhip_step_rmsnorm_qkv_rope_append(aionhip_ctx *ctx, const aionhip_weight 
                                          aionhip_handle x, aionhip_handle gamma, aionhip_handle beta_norm, float eps,
                                          aionhip_handle q_out, aionhip_handle k_cache, aionhip_handle v_cache,
                                          aionhip_handle positions, aionhip_handle write_index, size_t t_cap, size_t h_q, size_t h_kv,
-                                         size_t d, float base_frequency, float scale_factor, float rope_proportion) {
+                                         size_t d, float base_frequency, float scale_factor, float rope_proportion, int rolling) {
     if (!ctx || !wq || !wk || !wv) return AIONHIP_INVALID_ARGUMENT;
     if (!x || !gamma || !q_out || !k_cache || !v_cache || !positions || !write_index)
         return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "qkv_rope_append: null operand");
@@ -160,7 +160,7 @@ int aionhip_step_rmsnorm_qkv_rope_append(aionhip_ctx *ctx, const aionhip_weight 
     int rc = rope_table(ctx, (int)rope_pairs, freq_step, scale_factor, &freq);
     if (rc) return rc;
     FusedEpi epi{(const int *)(uintptr_t)positions, (const int *)(uintptr_t)write_index, freq, (__half *)(uintptr_t)k_cache,
-                 (__half *)(uintptr_t)v_cache, (int)t_cap, (int)h_kv, (int)d, (int)rope_pairs};
+                 (__half *)(uintptr_t)v_cache, (int)t_cap, (int)h_kv, (int)d, (int)rope_pairs, rolling ? 1 : 0};
     FusedIn in{(const float *)(uintptr_t)x, nullptr, (const float *)(uintptr_t)gamma, (const float *)(uintptr_t)beta_norm, eps};
     return launch_gemv_fused_rope(ctx, ws, (float *)(uintptr_t)q_out, in, epi);
 }

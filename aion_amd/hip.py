@@ -57,7 +57,7 @@ _SIGS = {
     "aionhip_step_rmsnorm_matmul": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_void_p), C.c_size_t, C.c_uint64, C.c_uint64, C.c_uint64, C.c_float, C.POINTER(C.c_uint64), C.POINTER(C.c_size_t), C.c_float, C.c_float]),
     "aionhip_step_rmsnorm_qkv_rope_append": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_float,
                                                        C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_size_t, C.c_size_t, C.c_size_t,
-                                                       C.c_size_t, C.c_float, C.c_float, C.c_float]),
+                                                       C.c_size_t, C.c_float, C.c_float, C.c_float, C.c_int]),
     "aionhip_step_rmsnorm_geglu_matmul": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_float,
                                                     C.c_uint64, C.c_float, C.c_float]),
     "aionhip_step_gate_matmul": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint64, C.c_uint64, C.c_uint64, C.c_size_t, C.c_float, C.c_float]),

@@ -287,17 +287,18 @@ class PackageRunner:
             if qs[:2] != (1, 1) or ks[:2] != (1, 1) or qs[3] != ks[3] or qs[3] % 8:
                 return False
             kc, vc = get(ak.inputs[0]), get(av.inputs[0])
-            if kc.shape != vc.shape or kc.shape[2:] != ks[2:] or kc.dtype != "f16" or kc.extra or vc.extra:
-                return False                     # (the fused step writes at the write index itself: not for rings)
+            if kc.shape != vc.shape or kc.shape[2:] != ks[2:] or kc.dtype != "f16" or kc.extra != vc.extra or kc.extra not in (None, "rolling"):
+                return False
             gamma, beta = get(n0.inputs[1]), get(n0.inputs[2])
             q_out = new(qs, "f32")
             emit(g.step_rmsnorm_qkv_rope_append, weight_of(nodes[chains["q"][0]].inputs[1]).buf, weight_of(nodes[chains["k"][0]].inputs[1]).buf,
                  weight_of(nodes[chains["v"][0]].inputs[1]).buf, x.buf, gamma.buf, n0.attrs["eps"], q_out, kc.buf, vc.buf,
                  get(rq.inputs[1]).buf, get(ak.inputs[2]).buf, kc.shape[1], qs[2], ks[2], qs[3], base=rq.attrs["base_frequency"],
-                 scale_factor=rq.attrs["scale_factor"], proportion=rq.attrs["rope_proportion"], beta_norm=beta.buf)
+                 scale_factor=rq.attrs["scale_factor"], proportion=rq.attrs["rope_proportion"], beta_norm=beta.buf,
+                 rolling=kc.extra == "rolling")
             vals[rq.output] = _Val("dev", q_out, qs, "f32", owned=True)
-            vals[ak.output] = _Val("dev", kc.buf, kc.shape, "f16")
-            vals[av.output] = _Val("dev", vc.buf, vc.shape, "f16")
+            vals[ak.output] = _Val("dev", kc.buf, kc.shape, "f16", extra=kc.extra)
+            vals[av.output] = _Val("dev", vc.buf, vc.shape, "f16", extra=vc.extra)
             for c in chains.values():
                 skip.update(c)
             return True

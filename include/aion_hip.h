@@ -140,13 +140,14 @@ int aionhip_step_matmul_batch(aionhip_ctx *ctx, size_t count, const aionhip_weig
  * cpu/kernels/rope.zig:20-98) -> f32->f16 cast and append of k and v at the device-resident write index
  * (StepSequenceAppend, cpu/exec/sequence_append.zig:12-104), as one launch. q_out receives the rotated
  * query [h_q, d] f32; the caches are [t_cap, h_kv, d] f16 (batch 1). Same arithmetic as the separate steps
- * (aionhip_step_rmsnorm_matmul + aionhip_step_rope_append). AIONHIP_UNSUPPORTED when the shape does not
- * qualify (k above 4096, misaligned operands): the caller then issues the separate steps. */
+ * (aionhip_step_rmsnorm_matmul + aionhip_step_rope_append); rolling = 1: the caches are rings, as in
+ * aionhip_step_append_f16. AIONHIP_UNSUPPORTED when the shape does not qualify (k above 4096, misaligned
+ * operands): the caller then issues the separate steps. */
 int aionhip_step_rmsnorm_qkv_rope_append(aionhip_ctx *ctx, const aionhip_weight *wq, const aionhip_weight *wk, const aionhip_weight *wv,
                                          aionhip_handle x, aionhip_handle gamma, aionhip_handle beta_norm, float eps,
                                          aionhip_handle q_out, aionhip_handle k_cache, aionhip_handle v_cache,
                                          aionhip_handle positions, aionhip_handle write_index, size_t t_cap, size_t h_q, size_t h_kv,
-                                         size_t d, float base_frequency, float scale_factor, float rope_proportion);
+                                         size_t d, float base_frequency, float scale_factor, float rope_proportion, int rolling);
 /* Decode fusion of a GeGLU feed-forward block for ONE activation row: RMSNorm(x) -> gate and up matmuls ->
  * gate(gelu_tanh) * up (cpu/exec/elementwise.zig:25-37) -> int8 activation preparation -> down matmul,
  * C[1, n_down] = alpha * (...) + beta * C, in two launches; the gate / up / gated rows never reach memory.

@@ -205,6 +205,11 @@ def test_qkv_rope_append_fusion_equals_the_separate_steps(gpu, orc, dtype, D, Hq
     kc3, vc3 = gpu.zeros(T * Hkv * D * 2), gpu.zeros(T * Hkv * D * 2)
     gpu.step_rmsnorm_qkv_rope_append(ws[0], ws[1], ws[2], x, gamma, 1e-6, qr2, kc3, vc3, pb, wb_bad, T, Hq, Hkv, D)
     assert not gpu.download(kc3, np.float16, (T, Hkv, D)).any() and not gpu.download(vc3, np.float16, (T, Hkv, D)).any()
+    # rolling caches: the same out-of-range step lands in row step % T, with the values the in-range write gave
+    wb_ring = gpu.upload(np.array([3 * T + widx], np.int32))
+    gpu.step_rmsnorm_qkv_rope_append(ws[0], ws[1], ws[2], x, gamma, 1e-6, qr2, kc3, vc3, pb, wb_ring, T, Hq, Hkv, D, proportion=0.75, rolling=True)
+    assert np.array_equal(gpu.download(kc3, np.float16, (T, Hkv, D)), kb2) and np.array_equal(gpu.download(vc3, np.float16, (T, Hkv, D)), vb2)
+    wb_ring.free()
     for t in (x, gamma, pb, wb, wb_bad, q, k, v, qr, kc, vc, qr2, kc2, vc2, kc3, vc3):
         t.free()
     for w in ws:

@@ -160,9 +160,9 @@ def test_sliding_window_package_on_rolling_caches_equals_full_caches(gpu):
     ring_pkg = aion_file.parse(aion_writer.build_decoder_package(d, weights.blocks, weights.embed(), window=window, retained=24))
     full_pkg = aion_file.parse(aion_writer.build_decoder_package(d, weights.blocks, weights.embed(), window=window))
     assert ring_pkg.role_of_input(4).retained_history_tokens == 24 and full_pkg.role_of_input(4).retained_history_tokens == 0
-    # node by node on both sides, so that both issue the same steps (with fusions on, the ring side keeps its
-    # appends as separate steps while the full side takes the fused one-token q/k/v step: equal up to f32 rounding)
-    ring, full = PackageRunner(gpu, ring_pkg, capacity=64, fuse=False), PackageRunner(gpu, full_pkg, capacity=128, fuse=False)
+    # both sides issue the same steps, fused ones included (the one-token q/k/v step appends into rings too)
+    ring, full = PackageRunner(gpu, ring_pkg, capacity=64), PackageRunner(gpu, full_pkg, capacity=128)
+    assert ring.step_count(1) == full.step_count(1) == 1 + 4 * cfg.layers + 2
     try:
         prompt = np.random.default_rng(2).integers(0, cfg.vocab, 7).astype(np.int32)
         a, b = ring.run(prompt, want=("next_token", "logits")), full.run(prompt, want=("next_token", "logits"))
