@@ -288,6 +288,17 @@ class HipBackend:
             raise ValueError("cache_grow_target: InvalidArgument")
         return t
 
+    UNARY = {"relu": 0, "gelu": 1, "silu": 2, "sigmoid": 3, "tanh": 4, "sqrt": 5, "log": 6}
+    BINARY = {"add": 0, "sub": 1, "mul": 2, "div": 3}
+
+    def step_unary(self, op, out, x, n):
+        """StepUnary on f32; op by aion's name (backend/types.zig:119-128)."""
+        self._check(self._lib.aionhip_step_unary(self._ctx, self.UNARY[op], out.handle, x.handle, n))
+
+    def step_binary(self, op, out, a, b, n, nb=None):
+        """StepElemwiseBinary add/sub/mul/div on f32: out[i] = a[i] op b[i % nb] (nb = n: same shape; 1: scalar)."""
+        self._check(self._lib.aionhip_step_binary(self._ctx, self.BINARY[op], out.handle, a.handle, b.handle, n, n if nb is None else nb))
+
     def step_cast_f32_f16(self, out, x, n):
         self._check(self._lib.aionhip_step_cast_f32_f16(self._ctx, out.handle, x.handle, n))
 

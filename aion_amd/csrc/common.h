@@ -251,6 +251,10 @@ __device__ __forceinline__ float aion_tanh_approx(float x) {
     sg = fminf(1.f, fmaxf(0.f, sg));
     return fminf(1.f, fmaxf(-1.f, 2.f * sg - 1.f));
 }
+__device__ __forceinline__ float aion_sigmoid_approx(float x) {
+    const float e = aion_exp_approx(-fabsf(x));
+    return fminf(1.f, fmaxf(0.f, (x >= 0.f ? 1.f : e) / (1.f + e)));
+}
 // aion cpu/exec/elementwise.zig:25-37 (gate) + cpu/kernels/gelu.zig:8-14: gelu_tanh(x) * up
 __device__ __forceinline__ float aion_gate_gelu(float x, float up) {
     const float t = 0.7978845608028654f * (x + 0.044715f * (x * x * x));

@@ -112,6 +112,32 @@ __global__ void gate_gelu_kernel(float *__restrict__ out, const float *__restric
     out[i] = aion_gate_gelu(a[i], b[i]);
 }
 
+// StepUnary on f32 (backend/types.zig:119-125, cpu/exec/unary.zig:55-64) with aion's exp-based approximations of
+// sigmoid and tanh (cpu/kernels/fast_math.zig:53-148; gelu is the tanh form, cpu/kernels/gelu.zig:8-14)
+template <int OP>
+__global__ void unary_kernel(float *__restrict__ out, const float *__restrict__ x, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float v = x[i];
+    float r;
+    if (OP == AIONHIP_UNARY_RELU) r = v > 0.f ? v : 0.f;
+    else if (OP == AIONHIP_UNARY_GELU) r = 0.5f * v * (1.f + aion_tanh_approx(0.7978845608028654f * (v + 0.044715f * (v * v * v))));
+    else if (OP == AIONHIP_UNARY_SILU) r = v * aion_sigmoid_approx(v);
+    else if (OP == AIONHIP_UNARY_SIGMOID) r = aion_sigmoid_approx(v);
+    else if (OP == AIONHIP_UNARY_TANH) r = aion_tanh_approx(v);
+    else r = sqrtf(v);
+    out[i] = r;
+}
+// StepElemwiseBinary add / sub / mul / div on f32 where b has a's shape, is one element, or is a contiguous suffix of
+// a's shape (cpu/exec/elementwise.zig:38-60: identical, scalar_b, contiguous_suffix_b): out[i] = a[i] op b[i % nb]
+template <int OP>
+__global__ void binary_kernel(float *__restrict__ out, const float *__restrict__ a, const float *__restrict__ b, size_t n, size_t nb) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float x = a[i], y = b[nb == n ? i : i % nb];
+    out[i] = OP == AIONHIP_BINARY_ADD ? x + y : OP == AIONHIP_BINARY_SUB ? x - y : OP == AIONHIP_BINARY_MUL ? x * y : x / y;
+}
+
 // cpu/exec/gather.zig:60-87: one workgroup per gathered row; ids outside [0, vocab) give zeros
 __global__ __launch_bounds__(256) void gather_rows_kernel(int dtype, float *__restrict__ out, const void *__restrict__ table,
                                                           const int *__restrict__ ids, size_t d, size_t vocab) {
@@ -326,6 +352,46 @@ int aionhip_step_add(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle a, aio
     if (!n) return AIONHIP_OK;
     add_kernel<<<dim3(grid_for(n, 256)), dim3(256), 0, ctx->stream>>>(dp<float>(out), dp<const float>(a), dp<const float>(b), n);
     LAUNCH_CHECK(ctx, "add");
+    return AIONHIP_OK;
+}
+
+int aionhip_step_unary(aionhip_ctx *ctx, int op, aionhip_handle out, aionhip_handle x, size_t n) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (!out || !x) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "unary: null operand");
+    if (op == 6) return set_err(ctx, AIONHIP_UNSUPPORTED, "unary: log has no step on this backend");
+    if (op < 0 || op > 6) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "unary: unknown op %d", op);
+    if (!n) return AIONHIP_OK;
+    const dim3 grid(grid_for(n, 256)), block(256);
+    float *o = dp<float>(out);
+    const float *p = dp<const float>(x);
+    switch (op) {
+    case AIONHIP_UNARY_RELU: unary_kernel<AIONHIP_UNARY_RELU><<<grid, block, 0, ctx->stream>>>(o, p, n); break;
+    case AIONHIP_UNARY_GELU: unary_kernel<AIONHIP_UNARY_GELU><<<grid, block, 0, ctx->stream>>>(o, p, n); break;
+    case AIONHIP_UNARY_SILU: unary_kernel<AIONHIP_UNARY_SILU><<<grid, block, 0, ctx->stream>>>(o, p, n); break;
+    case AIONHIP_UNARY_SIGMOID: unary_kernel<AIONHIP_UNARY_SIGMOID><<<grid, block, 0, ctx->stream>>>(o, p, n); break;
+    case AIONHIP_UNARY_TANH: unary_kernel<AIONHIP_UNARY_TANH><<<grid, block, 0, ctx->stream>>>(o, p, n); break;
+    default: unary_kernel<AIONHIP_UNARY_SQRT><<<grid, block, 0, ctx->stream>>>(o, p, n); break;
+    }
+    LAUNCH_CHECK(ctx, "unary");
+    return AIONHIP_OK;
+}
+
+int aionhip_step_binary(aionhip_ctx *ctx, int op, aionhip_handle out, aionhip_handle a, aionhip_handle b, size_t n, size_t nb) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (!out || !a || !b) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "binary: null operand");
+    if (op < AIONHIP_BINARY_ADD || op > AIONHIP_BINARY_DIV) return set_err(ctx, AIONHIP_UNSUPPORTED, "binary: op %d has no step on this backend (add, sub, mul, div do)", op);
+    if (!n) return AIONHIP_OK;
+    if (nb == 0 || n % nb != 0) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "binary: b's %zu elements do not tile a's %zu", nb, n);
+    const dim3 grid(grid_for(n, 256)), block(256);
+    float *o = dp<float>(out);
+    const float *pa = dp<const float>(a), *pb = dp<const float>(b);
+    switch (op) {
+    case AIONHIP_BINARY_ADD: binary_kernel<AIONHIP_BINARY_ADD><<<grid, block, 0, ctx->stream>>>(o, pa, pb, n, nb); break;
+    case AIONHIP_BINARY_SUB: binary_kernel<AIONHIP_BINARY_SUB><<<grid, block, 0, ctx->stream>>>(o, pa, pb, n, nb); break;
+    case AIONHIP_BINARY_MUL: binary_kernel<AIONHIP_BINARY_MUL><<<grid, block, 0, ctx->stream>>>(o, pa, pb, n, nb); break;
+    default: binary_kernel<AIONHIP_BINARY_DIV><<<grid, block, 0, ctx->stream>>>(o, pa, pb, n, nb); break;
+    }
+    LAUNCH_CHECK(ctx, "binary");
     return AIONHIP_OK;
 }
 

@@ -66,7 +66,7 @@ _OUT = 1 << 30          # "consumer index" of a graph output
 
 class _Plan:
     def __init__(self):
-        self.steps, self.buffers, self.inputs, self.outputs = [], [], {}, {}
+        self.steps, self.buffers, self.inputs, self.outputs, self.values = [], [], {}, {}, {}
 
 
 class PackageRunner:
@@ -78,7 +78,7 @@ class PackageRunner:
         caches use the factor 2/1 and are re-placed row by row)."""
         self.gpu, self.pkg, self.capacity, self.fuse = gpu, pkg, int(capacity), fuse
         self.growth = growth
-        self.cache_meta = {}        # input index -> (value id, retained history tokens)
+        self.cache_meta = {}        # input index -> (value id, retained history tokens, rows if the capacity is a constant else None)
         self.sym_ctx, self.sym_seq = capacity_symbol, tokens_symbol
         self.pos = 0
         self.consts = {}            # (value id, transposed) -> _Val of an uploaded initializer
@@ -107,7 +107,7 @@ class PackageRunner:
                 if growth is not None and not (role.flags & 2) and not role.retained_history_tokens:
                     raise Unsupported("input %d does not allow growth (InputRoleFlags.allow_growable)" % idx)
                 self.caches[idx] = gpu.zeros(_count(shape) * 2)
-                self.cache_meta[idx] = (vid, int(role.retained_history_tokens))
+                self.cache_meta[idx] = (vid, int(role.retained_history_tokens), None if role.capacity_symbol != 0xFFFFFFFF else shape[1])
 
     # ---- initializers
     def _const(self, vid, transposed=False):
@@ -129,6 +129,14 @@ class PackageRunner:
             elif t.scheme == "q8_0" and t.quant_axis == 1 and transposed:
                 n, k = shape
                 w = self.gpu.upload_weight(be.Q8_0, be.ROWS_NK, n, k, np.asarray(t.data))
+            elif t.scheme == "q8_0" and t.quant_axis == 1:
+                # rows of 34-byte blocks as the file holds them: a Gather table (cpu/exec/gather.zig:60-87). The same
+                # initializer under a ViewTranspose2D (a tied logits head) is uploaded a second time in the matmul layout.
+                if shape[1] % 32:
+                    raise Unsupported("a q8_0 gather table whose rows are not whole blocks")
+                val = _Val("qtable", self.gpu.upload(np.asarray(t.data)), shape, "q8_0")
+                self.consts[key] = val
+                return val
             else:
                 raise Unsupported("%s initializer with quant_axis %d%s as a matmul operand" %
                                   (t.scheme, t.quant_axis, " under a transpose" if transposed else ""))
@@ -184,8 +192,11 @@ class PackageRunner:
                 out = new(v.shape, "f16")
                 emit(g.step_cast_f32_f16, out, src.buf, _count(v.shape))
                 v = vals[vid] = _Val("dev", out, v.shape, "f16")
-            elif v.kind == "gelu":
-                raise Unsupported("a gelu that does not feed a multiply (aion's gate step)")
+            elif v.kind == "gelu":              # a gelu that does not feed a multiply: the plain unary step
+                src = get(v.extra)
+                out = new(v.shape, "f32")
+                emit(g.step_unary, "gelu", out, src.buf, _count(v.shape))
+                v = vals[vid] = _Val("dev", out, v.shape, "f32", owned=True)
             return v
 
         def weight_of(vid):
@@ -364,10 +375,11 @@ class PackageRunner:
             op, a = n.op, n.attrs
             if op == "Gather":
                 table, ids = get(n.inputs[0]), get(n.inputs[1])
-                if a["axis"] != 0 or a["batch_dims"] != 0 or len(table.shape) != 2 or table.dtype != "f32":
-                    raise Unsupported("Gather other than rows of an f32 table")
+                if a["axis"] != 0 or a["batch_dims"] != 0 or len(table.shape) != 2 or table.dtype not in ("f32", "q8_0"):
+                    raise Unsupported("Gather other than rows of an f32 or row-quantized q8_0 table")
                 out = new(shape, "f32")
-                emit(g.step_gather_rows, be.F32, out, table.buf, ids.buf, _count(ids.shape), table.shape[1], table.shape[0])
+                emit(g.step_gather_rows, be.F32 if table.dtype == "f32" else be.Q8_0, out, table.buf, ids.buf, _count(ids.shape),
+                     table.shape[1], table.shape[0])
                 vals[n.output] = _Val("dev", out, shape, "f32", owned=True)
             elif op == "RMSNorm":
                 x, gamma, beta = get(n.inputs[0]), get(n.inputs[1]), get(n.inputs[2])
@@ -444,21 +456,36 @@ class PackageRunner:
                      rolling=k.extra == "rolling")
                 vals[n.output] = _Val("dev", out, shape, "f32", owned=True)
             elif op == "Unary":
-                if a["op"] != "gelu":
-                    raise Unsupported("Unary %s" % a["op"])
-                vals[n.output] = _Val("gelu", None, shape, "f32", extra=n.inputs[0])
-            elif op == "ElemwiseBinary":
-                if a["op"] == "add":
-                    x, y = get(n.inputs[0]), get(n.inputs[1])
-                    if x.shape != y.shape:
-                        raise Unsupported("broadcasting add")
+                if a["op"] == "gelu":           # pending: gelu(gate) * up is aion's gate step
+                    vals[n.output] = _Val("gelu", None, shape, "f32", extra=n.inputs[0])
+                elif a["op"] in ("relu", "silu", "sigmoid", "tanh", "sqrt"):
+                    x = get(n.inputs[0])
                     out = new(shape, "f32")
-                    emit(g.step_add, out, x.buf, y.buf, _count(shape))
+                    emit(g.step_unary, a["op"], out, x.buf, _count(shape))
+                    vals[n.output] = _Val("dev", out, shape, "f32", owned=True)
+                else:
+                    raise Unsupported("Unary %s" % a["op"])
+            elif op == "ElemwiseBinary":
+                lhs = vals.get(n.inputs[0])
+                if a["op"] in ("add", "sub", "mul", "div") and not (a["op"] == "mul" and lhs is not None and lhs.kind == "gelu"):
+                    # same shape, a scalar, or a contiguous suffix of the left operand's shape (cpu/exec/elementwise.zig:38-60)
+                    x, y = get(n.inputs[0]), get(n.inputs[1])
+                    if x.dtype != "f32" or y.dtype != "f32":
+                        raise Unsupported("ElemwiseBinary on %s" % x.dtype)
+                    ys = tuple(d for d in y.shape)
+                    while len(ys) > 1 and ys[0] == 1:
+                        ys = ys[1:]
+                    if not (x.shape == y.shape or _count(ys) == 1 or (len(ys) <= len(x.shape) and tuple(x.shape[len(x.shape) - len(ys):]) == ys)):
+                        raise Unsupported("ElemwiseBinary with a general broadcast")
+                    if tuple(shape) != tuple(x.shape):
+                        raise Unsupported("ElemwiseBinary that broadcasts its left operand")
+                    out = new(shape, "f32")
+                    if a["op"] == "add" and x.shape == y.shape:
+                        emit(g.step_add, out, x.buf, y.buf, _count(shape))
+                    else:
+                        emit(g.step_binary, a["op"], out, x.buf, y.buf, _count(shape), _count(ys))
                     vals[n.output] = _Val("dev", out, shape, "f32", owned=True)
                 elif a["op"] == "mul":
-                    lhs = vals.get(n.inputs[0])
-                    if lhs is None or lhs.kind != "gelu":
-                        raise Unsupported("a multiply that is not gelu(gate) * up")
                     gate, up = get(lhs.extra), get(n.inputs[1])
                     md = sole_user(n.output, "MatMul") if self.fuse else None
                     wd = weight_of(nodes[md].inputs[1]) if md is not None and nodes[md].inputs[0] == n.output else None
@@ -485,6 +512,9 @@ class PackageRunner:
         for name, vid in pkg.outputs:
             v = get(vid)
             plan.outputs[name] = (v.buf, v.shape, v.dtype)
+        # every value that ended up in a device buffer of its own, by value id (fused-away values are absent): lets a
+        # caller read an intermediate result after a run
+        plan.values = {vid: (v.buf, v.shape, v.dtype) for vid, v in vals.items() if v.kind == "dev" and v.buf is not None}
         self.plans[s] = plan
         return plan
 
@@ -510,8 +540,12 @@ class PackageRunner:
     def _required(self, s):
         """Rows the caches must hold for a run of s tokens at self.pos (api/loaded_model/sequence_cache.zig:45-51)."""
         need = 0
-        for _vid, retained in self.cache_meta.values():
-            need = max(need, (min(self.pos, retained) if retained else self.pos) + s)
+        for idx, (_vid, retained, fixed_rows) in self.cache_meta.items():
+            rows = (min(self.pos, retained) if retained else self.pos) + s
+            if fixed_rows is None:
+                need = max(need, rows)
+            elif rows > fixed_rows:             # a cache of constant shape (a local layer's ring): nothing to grow
+                raise ValueError("the run needs %d rows of cache input %d, which holds %d" % (rows, idx, fixed_rows))
         return need
 
     def _grow(self, required):
@@ -530,7 +564,9 @@ class PackageRunner:
                 raise ValueError("the run exceeds the caches' growth ceiling")
             target = min(target, ceiling)
         ends = None
-        for idx, (vid, retained) in self.cache_meta.items():
+        for idx, (vid, retained, fixed_rows) in self.cache_meta.items():
+            if fixed_rows is not None:
+                continue
             old_shape = self.pkg.shape_of(vid, {self.sym_ctx: self.capacity, self.sym_seq: 1})
             new_shape = self.pkg.shape_of(vid, {self.sym_ctx: target, self.sym_seq: 1})
             if old_shape[1] != self.capacity or new_shape[1] != target or old_shape[:1] + old_shape[2:] != new_shape[:1] + new_shape[2:]:

@@ -220,6 +220,18 @@ int aionhip_step_rope_append(aionhip_ctx *ctx, aionhip_handle q_out, aionhip_han
  * (backend/types.zig:105-109, cpu/exec/elementwise.zig:25-37, cpu/kernels/gelu.zig:8-14) */
 int aionhip_step_add(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle a, aionhip_handle b, size_t n);
 int aionhip_step_gate_gelu(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle a, aionhip_handle b, size_t n);
+/* StepUnary on f32 (backend/types.zig:119-128 UnaryOp, the ids below are its ids; cpu/exec/unary.zig:55-64):
+ * sigmoid and tanh are aion's exp-based approximations (cpu/kernels/fast_math.zig:53-148), gelu the tanh form
+ * (cpu/kernels/gelu.zig:8-14), silu = x * sigmoid(x). log (id 6): AIONHIP_UNSUPPORTED. out may alias x. */
+enum { AIONHIP_UNARY_RELU = 0, AIONHIP_UNARY_GELU = 1, AIONHIP_UNARY_SILU = 2, AIONHIP_UNARY_SIGMOID = 3,
+       AIONHIP_UNARY_TANH = 4, AIONHIP_UNARY_SQRT = 5 };
+int aionhip_step_unary(aionhip_ctx *ctx, int op, aionhip_handle out, aionhip_handle x, size_t n);
+/* StepElemwiseBinary add / sub / mul / div on f32 (backend/types.zig:92-96 ElemwiseBinaryOp ids;
+ * cpu/exec/elementwise.zig:38-60): b has a's n elements (identical), one element (scalar_b) or the nb elements of
+ * a contiguous suffix of a's shape (contiguous_suffix_b): out[i] = a[i] op b[i % nb]. The comparison ops and general
+ * broadcasts: AIONHIP_UNSUPPORTED. out may alias a. */
+enum { AIONHIP_BINARY_ADD = 0, AIONHIP_BINARY_SUB = 1, AIONHIP_BINARY_MUL = 2, AIONHIP_BINARY_DIV = 3 };
+int aionhip_step_binary(aionhip_ctx *ctx, int op, aionhip_handle out, aionhip_handle a, aionhip_handle b, size_t n, size_t nb);
 /* StepGather axis 0 (cpu/exec/gather.zig:60-87): rows of an f32 or q8_0 (quant_axis 1, packed
  * 34-byte blocks) table [V,D] -> out f32 [n_ids, D]; ids i32 on device */
 int aionhip_step_gather_rows(aionhip_ctx *ctx, int table_dtype, aionhip_handle out, aionhip_handle table,

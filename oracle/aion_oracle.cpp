@@ -610,6 +610,33 @@ void orc_gate_gelu(const float *a, const float *b, size_t n, float *out) {
     }
 }
 
+// cpu/exec/unary.zig:55-64 over cpu/kernels/{relu,gelu,silu,sigmoid,tanh}.zig; op ids of backend/types.zig:119-125
+int orc_unary(int op, const float *x, size_t n, float *out) {
+    for (size_t i = 0; i < n; ++i) {
+        const float v = x[i];
+        switch (op) {
+        case 0: out[i] = v > 0.0f ? v : 0.0f; break;
+        case 1: out[i] = 0.5f * v * (1.0f + tanh_approx(0.7978845608028654f * (v + 0.044715f * (v * v * v)))); break;
+        case 2: out[i] = v * sigmoid_approx(v); break;
+        case 3: out[i] = sigmoid_approx(v); break;
+        case 4: out[i] = tanh_approx(v); break;
+        case 5: out[i] = std::sqrt(v); break;
+        default: return -1;
+        }
+    }
+    return 0;
+}
+
+// cpu/exec/elementwise.zig:38-60: same shape, scalar b, or b a contiguous suffix of a's shape; op ids of backend/types.zig:92-96
+int orc_binary(int op, const float *a, const float *b, size_t n, size_t nb, float *out) {
+    if (nb == 0 || n % nb != 0 || op < 0 || op > 3) return -1;
+    for (size_t i = 0; i < n; ++i) {
+        const float x = a[i], y = b[i % nb];
+        out[i] = op == 0 ? x + y : op == 1 ? x - y : op == 2 ? x * y : x / y;
+    }
+    return 0;
+}
+
 void orc_gather_rows(int dtype, const void *table, size_t d, const int32_t *ids, size_t n_ids, float *out) {
     for (size_t i = 0; i < n_ids; ++i) {
         const size_t row = (size_t)ids[i];

@@ -111,6 +111,14 @@ void orc_rope(const float *x, const int32_t *positions, size_t b, size_t t, size
               float base, float scale_factor, float proportion, float *out);
 /* cpu/exec/elementwise.zig:25-37, kernels/gelu.zig:8-14: out = gelu_tanh_approx(a) * b */
 void orc_gate_gelu(const float *a, const float *b, size_t n, float *out);
+/* cpu/exec/unary.zig:55-64 over cpu/kernels/{relu,gelu,silu,sigmoid,tanh}.zig and fast_math.zig:53-148; op = UnaryOp id
+ * (backend/types.zig:119-125: relu 0, gelu 1, silu 2, sigmoid 3, tanh 4, sqrt 5). Pinned by definition checks, by
+ * gelu(a) * b == orc_gate_gelu(a, b) bit for bit and by the approximations' distance from the true functions
+ * (tests/test_graph_oracle.py). -1: unknown op */
+int orc_unary(int op, const float *x, size_t n, float *out);
+/* cpu/exec/elementwise.zig:38-60: add 0 / sub 1 / mul 2 / div 3 with b identical, scalar or a contiguous suffix of a's
+ * shape (nb elements, nb divides n): out[i] = a[i] op b[i % nb]. Pinned against numpy broadcasting. -1: invalid */
+int orc_binary(int op, const float *a, const float *b, size_t n, size_t nb, float *out);
 /* cpu/exec/gather.zig:60-87: rows of a q8_0 [V,D] axis-1 table (or f32 when dtype==0) */
 void orc_gather_rows(int dtype, const void *table, size_t d, const int32_t *ids, size_t n_ids, float *out);
 /* cpu/exec/argmax.zig:56-81: first maximum wins */

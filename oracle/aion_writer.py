@@ -286,3 +286,94 @@ def build_decoder_package(cfg, blocks_of, embed, gammas=None, window=None, retai
     b.add_metadata("arch", "synthetic-decoder")
     b.add_metadata("layers", str(cfg["layers"]))
     return b.to_bytes()
+
+
+def build_sandwich_decoder_package(cfg, blocks_of, table_blocks, gammas):
+    """A decoder in the shape of aion's own bench model (src/bench/models.zig:433-536, without its per-layer-input
+    branch and kv sharing): a tied, block-quantized embedding table that is gathered from AND contracted against
+    (through a ViewTranspose2D) for the logits; the embedding scaled by sqrt(hidden); per-head RMSNorm on q, k and v;
+    attention with scale 1; RMSNorm on the attention and feed-forward outputs before their residual adds; local layers
+    with a sliding window over rolling caches of `local_window` rows (window left = local_window - 1, that many
+    positions retained: models.zig:66-68, 301-310, 440-445) and every `global_every`-th layer global over [1,ctx,..]
+    caches with its own RoPE base; logits soft-capped as scale * tanh(logits / scale) before the ArgMax.
+
+    cfg: layers, hidden, heads, kv_heads, head_dim, ffn, vocab, eps, rope_base_local, rope_base_global, local_window,
+    global_every, logit_softcap, wdtype. blocks_of(name) as in build_decoder_package; table_blocks: the embedding
+    table [vocab, hidden] as q8_0 blocks along its rows (quant_axis 1); gammas: name -> f32 vector for every norm
+    ("l%d.norm_in", "l%d.q_norm", "l%d.k_norm", "l%d.v_norm", "l%d.norm_attn", "l%d.norm_ffn_in", "l%d.norm_ffn", "norm_f")."""
+    b = PackageBuilder()
+    seq, ctx = b.symbol("seq"), b.symbol("ctx")
+    H, Hkv, D, E, F, V = cfg["heads"], cfg["kv_heads"], cfg["head_dim"], cfg["hidden"], cfg["ffn"], cfg["vocab"]
+    W = cfg["local_window"]
+    q8 = cfg["wdtype"] == "q8_0"
+    is_global = lambda l: l % cfg["global_every"] == cfg["global_every"] - 1
+
+    tokens = b.input("tokens", "i32", (1, seq), role="tokens", axis=1)
+    positions = b.input("positions", "i32", (1, seq), role="positions", axis=1)
+    write_index = b.input("write_index", "i32", (1,), role="cache_write_index")
+    visible_end = b.input("visible_end", "i32", (1,), role="cache_visible_end")
+    caches = []
+    for l in range(cfg["layers"]):
+        for kv in "kv":
+            if is_global(l):
+                caches.append(b.input("l%d.%s_cache" % (l, kv), "f16", (1, ctx, Hkv, D), role="sequence_cache", axis=1, capacity_symbol=1))
+            else:
+                caches.append(b.input("l%d.%s_cache" % (l, kv), "f16", (1, W, Hkv, D), role="sequence_cache", axis=1, retained=W - 1))
+
+    def weight(name, k, n):
+        blocks = blocks_of(name)
+        if q8:
+            w = b.initializer("q8_0", (n, k), b.tensor_quantized("q8_0", blocks, 1), name)
+            return b.transpose2d(w, "q8_0", (k, n))
+        return b.initializer("q4_0", (k, n), b.tensor_quantized("q4_0", blocks, 0), name)
+
+    def vec(name, values):
+        return b.initializer("f32", (len(values),), b.tensor_plain("f32", np.asarray(values, np.float32)), name)
+
+    def scalar(value):
+        return b.initializer("f32", (1,), b.tensor_plain("f32", np.asarray([value], np.float32)))
+
+    betas = {n: vec("beta%d" % n, np.zeros(n, np.float32)) for n in (E, D)}
+
+    def rms(x, name, shape):
+        n = shape[-1]
+        return b.rmsnorm(x, vec(name, gammas[name]), betas[n], cfg["eps"], shape, (n,))
+
+    table = b.initializer("q8_0", (V, E), b.tensor_quantized("q8_0", table_blocks, 1), "embed")
+    x = b.binary("mul", b.gather(table, tokens, (1, seq, E)), scalar(float(np.sqrt(np.float32(E)))), (1, seq, E))
+    for l in range(cfg["layers"]):
+        p = "l%d." % l
+        base = cfg["rope_base_global"] if is_global(l) else cfg["rope_base_local"]
+        t_len = ctx if is_global(l) else W
+        h = rms(x, p + "norm_in", (1, seq, E))
+        q = b.reshape(b.matmul(h, weight(p + "wq", E, H * D), (1, seq, H * D)), "f32", (1, seq, H, D))
+        q = b.rope(rms(q, p + "q_norm", (1, seq, H, D)), positions, (1, seq, H, D), base)
+        k = b.reshape(b.matmul(h, weight(p + "wk", E, Hkv * D), (1, seq, Hkv * D)), "f32", (1, seq, Hkv, D))
+        k = b.rope(rms(k, p + "k_norm", (1, seq, Hkv, D)), positions, (1, seq, Hkv, D), base)
+        v = b.reshape(b.matmul(h, weight(p + "wv", E, Hkv * D), (1, seq, Hkv * D)), "f32", (1, seq, Hkv, D))
+        v = rms(v, p + "v_norm", (1, seq, Hkv, D))
+        kc = b.sequence_append(caches[2 * l], b.cast(k, "f16", (1, seq, Hkv, D)), write_index, "f16", (1, t_len, Hkv, D))
+        vc = b.sequence_append(caches[2 * l + 1], b.cast(v, "f16", (1, seq, Hkv, D)), write_index, "f16", (1, t_len, Hkv, D))
+        b.output("l%d.k_cache" % l, kc, alias_of_input=4 + 2 * l)
+        b.output("l%d.v_cache" % l, vc, alias_of_input=4 + 2 * l + 1)
+        window = (0xFFFFFFFF, 0, 0) if is_global(l) else (W - 1, 0, 0)
+        o = b.attention(q, kc, vc, positions, visible_end, (1, seq, H, D), 1.0, window=window)
+        o = b.matmul(b.reshape(o, "f32", (1, seq, H * D)), weight(p + "wo", H * D, E), (1, seq, E))
+        x = b.binary("add", x, rms(o, p + "norm_attn", (1, seq, E)), (1, seq, E))
+        h = rms(x, p + "norm_ffn_in", (1, seq, E))
+        gate = b.matmul(h, weight(p + "wgate", E, F), (1, seq, F))
+        up = b.matmul(h, weight(p + "wup", E, F), (1, seq, F))
+        act = b.binary("mul", b.unary("gelu", gate, (1, seq, F)), up, (1, seq, F))
+        ff = b.matmul(act, weight(p + "wdown", F, E), (1, seq, E))
+        x = b.binary("add", x, rms(ff, p + "norm_ffn", (1, seq, E)), (1, seq, E))
+    h = rms(x, "norm_f", (1, seq, E))
+    logits = b.matmul(h, b.transpose2d(table, "q8_0", (E, V)), (1, seq, V))
+    cap = cfg["logit_softcap"]
+    capped = b.binary("mul", b.unary("tanh", b.binary("mul", logits, scalar(1.0 / cap), (1, seq, V)), (1, seq, V)), scalar(cap), (1, seq, V))
+    token = b.argmax(capped, (1, seq))
+    b.outputs.insert(0, (b.string("next_token"), token))
+    b.outputs.insert(1, (b.string("logits"), capped))
+    b.io_aliases = [(i, o + 2) for i, o in b.io_aliases]
+    b.add_metadata("arch", "synthetic-sandwich-decoder")
+    b.add_metadata("layers", str(cfg["layers"]))
+    return b.to_bytes()

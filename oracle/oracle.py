@@ -43,6 +43,8 @@ def _load():
     lib.orc_rmsnorm.argtypes = [vp, vp, vp, vp, sz, sz, f, vp]; lib.orc_rmsnorm.restype = None
     lib.orc_rope.argtypes = [vp, vp, sz, sz, sz, sz, f, f, f, vp]; lib.orc_rope.restype = None
     lib.orc_gate_gelu.argtypes = [vp, vp, sz, vp]; lib.orc_gate_gelu.restype = None
+    lib.orc_unary.argtypes = [C.c_int, vp, sz, vp]; lib.orc_unary.restype = C.c_int
+    lib.orc_binary.argtypes = [C.c_int, vp, vp, sz, sz, vp]; lib.orc_binary.restype = C.c_int
     lib.orc_gather_rows.argtypes = [i, vp, sz, vp, sz, vp]; lib.orc_gather_rows.restype = None
     lib.orc_argmax.argtypes = [vp, sz, sz, vp]; lib.orc_argmax.restype = None
     lib.orc_cast_f32_f16.argtypes = [vp, sz, vp]; lib.orc_cast_f32_f16.restype = None
@@ -339,6 +341,27 @@ def gate_gelu(a, b):
     a = _f32(a); b = _f32(b)
     out = np.zeros_like(a)
     _lib.orc_gate_gelu(_p(a), _p(b), a.size, _p(out))
+    return out
+
+
+UNARY_OPS = {"relu": 0, "gelu": 1, "silu": 2, "sigmoid": 3, "tanh": 4, "sqrt": 5}
+BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3}
+
+
+def unary(op, x):
+    x = _f32(x)
+    out = np.zeros_like(x)
+    if _lib.orc_unary(UNARY_OPS[op], _p(x), x.size, _p(out)):
+        raise ValueError("orc_unary: InvalidArgument")
+    return out
+
+
+def binary(op, a, b):
+    """b has a's shape, one element, or a contiguous suffix of a's shape."""
+    a = _f32(a); b = _f32(b)
+    out = np.zeros_like(a)
+    if _lib.orc_binary(BINARY_OPS[op], _p(a), _p(b), a.size, b.size, _p(out)):
+        raise ValueError("orc_binary: InvalidArgument")
     return out
 
 

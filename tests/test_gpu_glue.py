@@ -311,3 +311,36 @@ def test_cache_growth_rejects_bad_arguments(gpu):
             call()
     gpu.cache_grow(a, b, 0, 8, 16)          # nothing to do
     a.free(); b.free(); e.free()
+
+
+def test_unary_and_binary_steps(gpu, orc):
+    rng = np.random.default_rng(31)
+    from aion_amd.hip import AionHipError
+    x = np.concatenate([rng.standard_normal(5000).astype(np.float32) * 4, np.array([0, -0.0, 30, -30, 88, -88, 1e-6], np.float32)])
+    xb, ob = gpu.upload(x), gpu.alloc(x.nbytes)
+    for op in ("relu", "gelu", "silu", "sigmoid", "tanh", "sqrt"):
+        src = np.abs(x) if op == "sqrt" else x
+        gpu.write(xb, src)
+        gpu.step_unary(op, ob, xb, x.size)
+        got, want = gpu.download(ob, np.float32, x.shape), orc.unary(op, src)
+        # the same exp polynomial and the same operations; only mul+add contraction may differ by an ulp or two
+        assert np.abs(got - want).max() <= 4e-7 * max(1.0, float(np.abs(want).max())), op
+    with pytest.raises(AionHipError):
+        gpu.step_unary("log", ob, xb, x.size)
+    a = rng.standard_normal((6, 5, 64)).astype(np.float32)
+    ab, outb = gpu.upload(a), gpu.alloc(a.nbytes)
+    for b in (rng.standard_normal((6, 5, 64)).astype(np.float32) + 3, np.array([0.37], np.float32), rng.standard_normal(64).astype(np.float32) + 3,
+              rng.standard_normal((5, 64)).astype(np.float32) + 3):
+        bb = gpu.upload(b)
+        for op in ("add", "sub", "mul", "div"):
+            gpu.step_binary(op, outb, ab, bb, a.size, b.size)
+            assert np.array_equal(gpu.download(outb, np.float32, a.shape), orc.binary(op, a, b)), (op, b.shape)
+        bb.free()
+    bad = gpu.upload(np.ones(7, np.float32))
+    with pytest.raises(AionHipError):
+        gpu.step_binary("add", outb, ab, bad, a.size, 7)
+    # in place
+    gpu.step_binary("mul", ab, ab, ab, a.size)
+    assert np.array_equal(gpu.download(ab, np.float32, a.shape), a * a)
+    for t in (xb, ob, ab, outb, bad):
+        t.free()

@@ -85,7 +85,7 @@ def test_package_runner_refuses_what_the_backend_has_no_step_for(gpu):
     x = b.input("tokens", "i32", (1, seq), role="tokens", axis=1)
     table = b.initializer("f32", (8, 32), b.tensor_plain("f32", np.zeros((8, 32), np.float32)), "embed")
     e = b.gather(table, x, (1, seq, 32))
-    y = b.unary("tanh", e, (1, seq, 32))
+    y = b.unary("log", b.unary("tanh", e, (1, seq, 32)), (1, seq, 32))        # tanh has a step, log has none
     b.output("y", y)
     pkg = aion_file.parse(b.to_bytes())
     run = PackageRunner(gpu, pkg, capacity=8)
@@ -252,3 +252,91 @@ def test_rolling_caches_grow_for_a_long_run(gpu):
             tok = int(b["next_token"][0, -1])
     finally:
         grow.close(); full.close(); fixed.close()
+
+
+def test_bench_model_shaped_package_against_the_graph_oracle(gpu, orc):
+    """A package in the shape of aion's own bench model (tied row-quantized embedding table gathered from and
+    contracted against, scaled embedding, per-head q/k/v norms, norms on the block outputs, local layers with
+    sliding windows over rolling caches of constant size beside global layers, soft-capped logits: oracle/aion_writer.py
+    build_sandwich_decoder_package) through the package runner, against the node-by-node CPU interpreter
+    (oracle/graph_oracle.py) fed the same package. The tolerance is the decoder tests': the GPU may be no further from
+    the interpreter than the interpreter is from itself when one operand rounding changes (queries rounded to f16, as
+    the MFMA kernels do) - a flipped int8 activation code is worth ~5e-3 of a matmul's output, whatever flipped it;
+    and the tokens the interpreter picks wherever its top two logits are further apart than the error."""
+    from oracle import graph_oracle
+    cfg = dict(layers=3, hidden=256, heads=4, kv_heads=1, head_dim=64, ffn=512, vocab=1024, eps=1e-6, rope_base_local=10000.0,
+               rope_base_global=1000000.0, local_window=64, global_every=3, logit_softcap=30.0, wdtype="q4_0")
+    E, H, Hkv, D, F, V, W = cfg["hidden"], cfg["heads"], cfg["kv_heads"], cfg["head_dim"], cfg["ffn"], cfg["vocab"], cfg["local_window"]
+    rng = np.random.default_rng(23)
+    shapes = {"wq": (E, H * D), "wk": (E, Hkv * D), "wv": (E, Hkv * D), "wo": (H * D, E), "wgate": (E, F), "wup": (E, F), "wdown": (F, E)}
+    blocks = {"l%d.%s" % (l, n): orc.quantize(orc.Q4_0, (rng.standard_normal(s) * 0.06).astype(np.float32), 0)
+              for l in range(cfg["layers"]) for n, s in shapes.items()}
+    table = orc.quantize(orc.Q8_0, (rng.standard_normal((V, E)) * 0.05).astype(np.float32), 1)
+    gammas = {}
+    for l in range(cfg["layers"]):
+        for n, width in (("norm_in", E), ("q_norm", D), ("k_norm", D), ("v_norm", D), ("norm_attn", E), ("norm_ffn_in", E), ("norm_ffn", E)):
+            # attention runs with scale 1 on normalized heads: gammas of 0.35 on q and k put the scores where a trained
+            # model's are (unit gammas give |q.k| up to the head size and a softmax that magnifies every rounding)
+            g0 = 0.35 if n in ("q_norm", "k_norm") else 1.0
+            gammas["l%d.%s" % (l, n)] = (g0 * (1 + 0.1 * rng.standard_normal(width))).astype(np.float32)
+    gammas["norm_f"] = (1 + 0.1 * rng.standard_normal(E)).astype(np.float32)
+    pkg = aion_file.parse(aion_writer.build_sandwich_decoder_package(cfg, lambda name: blocks[name], table, gammas))
+    T = 128
+    run = PackageRunner(gpu, pkg, capacity=T)
+    plain = PackageRunner(gpu, pkg, capacity=T, fuse=False)
+    caches, rings = {}, []
+    for idx, (name, vid) in enumerate(pkg.inputs):
+        role = pkg.role_of_input(idx)
+        if role.kind == "sequence_cache":
+            caches[name] = np.zeros(pkg.shape_of(vid, {"ctx": T, "seq": 1}), np.float16)
+            if role.retained_history_tokens:
+                rings.append(name)
+    assert len(rings) == 4 and len(caches) == 6
+    try:
+        pos, tok, errs, selfs = 0, None, [], []
+        prompt = rng.integers(0, V, 40).astype(np.int32)
+        for step in range(1 + 45):                        # 40 prompt tokens, then single tokens past the rings' 64 rows
+            tokens = prompt if step == 0 else np.array([tok], np.int32)
+            s = tokens.size
+            feeds = dict(caches)
+            by_role = {"tokens": tokens.reshape(1, s), "positions": np.arange(pos, pos + s, dtype=np.int32).reshape(1, s),
+                       "cache_write_index": np.array([pos], np.int32), "cache_visible_end": np.array([pos + s], np.int32)}
+            for idx, (name, _vid) in enumerate(pkg.inputs):
+                if pkg.role_of_input(idx).kind in by_role:
+                    feeds[name] = by_role[pkg.role_of_input(idx).kind]
+            want = graph_oracle.run_graph(pkg, feeds, {"seq": s, "ctx": T}, rolling_inputs=rings)
+            alt = graph_oracle.run_graph(pkg, feeds, {"seq": s, "ctx": T}, rolling_inputs=rings, round_q_f16=True)
+            for name in caches:
+                caches[name] = want[name]
+            got = run.run(tokens, want=("next_token", "logits"))
+            got_plain = plain.run(tokens, want=("next_token", "logits"))
+            if step in (0, 1, 30):
+                # node by node: every step of the unfused plan against the interpreter ON THE DEVICE'S OWN INPUTS
+                # (no amplification between nodes). Prompt, first single token, and a token after the rings wrapped.
+                np_t = {"f32": np.float32, "i32": np.int32, "f16": np.float16}
+                dev = {vid: gpu.download(buf, np_t[dt], shape) for vid, (buf, shape, dt) in plain.plans[s].values.items()}
+                report = graph_oracle.check_nodes(pkg, feeds, {"seq": s, "ctx": T}, dev, rolling_inputs=rings)
+                assert len(report) > 50
+                for i, op, e in report:
+                    assert e < (4e-3 if op == "Attention" else 2e-5), (step, i, op, e)
+            ol, gl = want["logits"][0, -1], got["logits"][0, -1]
+            rms = float(np.sqrt((ol.astype(np.float64) ** 2).mean()))
+            err = float(np.abs(gl - ol).max()) / rms
+            errs.append(err)
+            selfs.append(float(np.abs(alt["logits"][0, -1] - ol).max()) / rms)
+            # the fused schedule against the node-by-node one on the same device: f32 summation order only
+            assert float(np.abs(got_plain["logits"][0, -1] - gl).max()) / rms < 2e-3
+            top2 = np.sort(ol)[-2:]
+            otok = int(want["next_token"][0, -1])
+            if float(top2[1] - top2[0]) / rms > 2 * err:
+                assert int(got["next_token"][0, -1]) == otok, step
+            tok = otok
+            pos += s
+        say("bench-shaped package: max err/rms %.2e, mean %.2e (interpreter against itself: %.2e, %.2e) over %d runs; steps per token %d (node by node %d)"
+            % (max(errs), float(np.mean(errs)), max(selfs), float(np.mean(selfs)), len(errs), run.step_count(1), plain.step_count(1)))
+        assert np.mean(errs) < 2 * np.mean(selfs) + 1e-3 and max(errs) < 3 * max(selfs) + 1e-3
+        assert np.abs(got["logits"]).max() <= 30.0
+        with pytest.raises(ValueError):
+            run.run(np.zeros(30, np.int32))               # 63 retained + 30 new rows do not fit a 64-row ring
+    finally:
+        run.close(); plain.close()
