@@ -402,13 +402,20 @@ def run_decoder(gpu, be, with_cpu=True):
     from aion_amd.decoder import Decoder, DecoderConfig, SyntheticWeights, weight_shapes
     cfg = DecoderConfig()
     t0 = time.time()
-    oracle = None
+    oracle = oracle_alt = None
     if with_cpu:
         from oracle import oracle as orc
         threads = min(16, os.cpu_count() or 1)
-        oracle = orc.Decoder(cfg.layers, cfg.hidden, cfg.heads, cfg.kv_heads, cfg.head_dim, cfg.ffn, cfg.vocab, cfg.max_seq,
-                             eps=cfg.eps, rope_base=cfg.rope_base, wdtype=cfg.wdtype, threads=threads)
-    dec = Decoder(gpu, cfg, SyntheticWeights(cfg, 0), on_weight=oracle.set_weight if oracle else None)
+        mk = lambda exact: orc.Decoder(cfg.layers, cfg.hidden, cfg.heads, cfg.kv_heads, cfg.head_dim, cfg.ffn, cfg.vocab, cfg.max_seq,
+                                       eps=cfg.eps, rope_base=cfg.rope_base, wdtype=cfg.wdtype, threads=threads, attn_exact=exact)
+        # the second one differs by one thing (exact exp in attention instead of aion's polynomial): how far the CPU
+        # path moves under a 4e-5 perturbation is the yardstick for the GPU's distance from it
+        oracle, oracle_alt = mk(False), mk(True)
+
+    def on_weight(name, data):
+        oracle.set_weight(name, data)
+        oracle_alt.set_weight(name, data)
+    dec = Decoder(gpu, cfg, SyntheticWeights(cfg, 0), on_weight=on_weight if oracle else None)
     setup_s = time.time() - t0
     prompt = np.random.default_rng(5).integers(0, cfg.vocab, 128).astype(np.int32)
     weight_bytes = sum(n * k // 32 * 18 for (n, k) in weight_shapes(cfg).values())
@@ -447,9 +454,9 @@ def run_decoder(gpu, be, with_cpu=True):
     res = {
         "config": "26 layers, hidden 2048, 8q/1kv heads x 256, ffn 8192 (GeGLU), vocab 262144, q4_0 weights, f16 KV cache, prompt 128, greedy 128, batch 1",
         "setup_s": round(setup_s, 1),
-        "prefill_128_ms_bf16_mfma": round(prefill_ms, 3),
-        "prefill_tokens_per_s": round(128 / (prefill_ms * 1e-3), 1),
-        "prefill_128_ms_exact_i8": round(prefill_exact_ms, 3),
+        "prefill_128_ms_exact_i8": round(prefill_exact_ms, 3),          # the default mode: aion's arithmetic
+        "prefill_tokens_per_s": round(128 / (prefill_exact_ms * 1e-3), 1),
+        "prefill_128_ms_bf16_mfma": round(prefill_ms, 3),               # pays off from a few hundred rows on
         "prefill_next_token_bf16_vs_exact": [int(tok), int(tok_exact)],
         "decode_tokens_per_s": round(128 / decode_s, 1),
         "decode_ms_per_token": round(decode_s / 128 * 1e3, 4),
@@ -463,6 +470,8 @@ def run_decoder(gpu, be, with_cpu=True):
         t = time.perf_counter()
         otok, ologits = oracle.forward(prompt, 0)
         cpu_prefill_s = time.perf_counter() - t
+        atok, alogits = oracle_alt.forward(prompt, 0)
+        self_err = float(np.abs(alogits - ologits).max()) / float(np.sqrt((ologits.astype(np.float64) ** 2).mean()))
         dec.reset()
         gtok = dec.prefill(prompt)
         glogits = dec.logits_host()
@@ -488,7 +497,12 @@ def run_decoder(gpu, be, with_cpu=True):
                                 "prefill_128_s": round(cpu_prefill_s, 2), "decode_tokens_per_s": round(n_cpu / cpu_decode_s, 3),
                                 "sample": "prompt + %d teacher-forced decode steps" % n_cpu,
                                 "gpu_vs_cpu_logits_max_err_over_rms": [round(e, 4) for e in errs],
-                                "greedy_token_agreement": agree}
+                                "greedy_token_agreement": agree,
+                                "cpu_vs_cpu_exact_exp_logits_max_err_over_rms_prefill": round(self_err, 4),
+                                "cpu_vs_cpu_exact_exp_token_agreement_prefill": int(atok == otok),
+                                "note": "aion re-quantizes activations to int8 before every matmul: any perturbation flips codes and "
+                                        "saturates after a few layers, so the CPU path against itself (exact exp instead of aion's "
+                                        "polynomial in attention) moves as far as the GPU is from it"}
     dec.close()
     return res
 
