@@ -607,6 +607,11 @@ void launch_i8(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct 
 
 }  // namespace
 
+int launch_gemm_i8_few_rows(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
+    return w->dtype == AIONHIP_Q8_0 ? launch_i8_lds_pick<AIONHIP_Q8_0>(ctx, w, m, act, c, ldc, alpha, beta)
+                                    : launch_i8_lds_pick<AIONHIP_Q4_0>(ctx, w, m, act, c, ldc, alpha, beta);
+}
+
 int launch_gemm_i8(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
     const char *name = w->dtype == AIONHIP_Q8_0 ? "gemm_i8_q8" : "gemm_i8_q4";
     ProfScope scope(ctx, name);

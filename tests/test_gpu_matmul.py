@@ -209,9 +209,11 @@ def test_exact_gemm_shapes_and_edges(gpu, orc, dtype, layout, m, n, k):
 
 # 2..8 activation rows (gemv_rows_kernel): row counts that fill a 2-, 4- or 8-row instance only partly, N that is
 # not a multiple of the rows a wavefront works on, K of one LDS pass and K long enough to run as several K-range
-# launches (14336 at 8 rows), alpha/beta on a pre-filled C.
+# launches (14336 at 8 rows), alpha/beta on a pre-filled C. The last three shapes (5..8 rows, at least 16384 columns,
+# K up to 4096) run on the 16-row tile of the LDS-staged MFMA kernel instead: ragged N, K of one and of many steps.
 @pytest.mark.parametrize("dtype,layout", CASES)
-@pytest.mark.parametrize("m,n,k", [(2, 70, 96), (3, 1001, 1056), (5, 333, 2048), (8, 1030, 14336), (7, 4100, 7200), (4, 9000, 512)])
+@pytest.mark.parametrize("m,n,k", [(2, 70, 96), (3, 1001, 1056), (5, 333, 2048), (8, 1030, 14336), (7, 4100, 7200), (4, 9000, 512),
+                                   (5, 16390, 256), (8, 20001, 2048), (6, 16384, 4096)])
 def test_decode_gemv_two_to_eight_rows(gpu, orc, dtype, layout, m, n, k):
     say("gemv rows", dtype, layout, m, n, k)
     blocks, w = make_weight(gpu, orc, dtype, layout, n, k, seed=m * 31 + n + k, std=0.05)
