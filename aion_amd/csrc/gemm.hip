@@ -1,11 +1,10 @@
 // Prefill GEMM back ends (more than 8 activation rows): C[m,n] = alpha * A[m,:] . W[n,:] + beta * C.
 //
-// gemm_i8_kernel (AIONHIP_GEMM_EXACT_I8) - aion's CPU arithmetic (cpu/kernels/matmul_q_i8.zig:
+// gemm_i8_lds_kernel (AIONHIP_GEMM_EXACT_I8) - aion's CPU arithmetic (cpu/kernels/matmul_q_i8.zig:
 //   384-497): activations int8 per (row, 32-block), one v_mfma_i32_16x16x32_i8 per 16x16 output
 //   tile per quant block (K=32 IS one block, so the i32 tile is the exact block dot), then
-//   acc += f32(idot) * (a_scale * w_scale) on the VALU. Operands come straight from global
-//   memory in MFMA layout (8 bytes per lane per tile). The per-block rescale (3 VALU ops per
-//   output element per block) is what bounds it, not the MFMA pipe.
+//   acc += f32(idot) * (a_scale * w_scale) on the VALU. Operands are staged through LDS. The per-block
+//   rescale (3 VALU ops per output element per block) is what bounds it, not the MFMA pipe.
 //
 // gemm_bf16_wide_kernel (AIONHIP_GEMM_BF16_MFMA) - weights dequantized once to bf16 [N,K] (kept
 //   per weight: 288 GB of HBM makes the 2 B/weight copy affordable), activations rounded to bf16,
@@ -19,87 +18,7 @@ using i32x4 = __attribute__((ext_vector_type(4))) int;
 using bf16x8 = __attribute__((ext_vector_type(8))) __bf16;
 
 // ------------------------------------------------------------------------------------ exact int8
-template <int DT, int TM>
-__global__ __launch_bounds__(256) void gemm_i8_kernel(const uint8_t *__restrict__ qs, const __half *__restrict__ sc,
-                                                      const int8_t *__restrict__ aq, const float *__restrict__ a_scale,
-                                                      const int *__restrict__ a_sum, float *__restrict__ c,
-                                                      int M, int N, int K, size_t ldc, float alpha, float beta) {
-    constexpr int TN = 4;
-    constexpr bool Q8 = DT == AIONHIP_Q8_0;
-    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int r = lane & 15, g = lane >> 4;
-    const int n0 = (blockIdx.x * 4 + wave) * (TN * 16);
-    const int m0 = blockIdx.y * (TM * 16);
-    if (n0 >= N) return;
-    const int KB = K >> 5;
-
-    f32x4 acc[TM][TN];
-#pragma unroll
-    for (int mi = 0; mi < TM; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < TN; ++ni) acc[mi][ni] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    size_t arow[TM], srow[TM][4], wrow[TN];
-#pragma unroll
-    for (int mi = 0; mi < TM; ++mi) {
-        arow[mi] = (size_t)min(m0 + mi * 16 + r, M - 1) * K;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) srow[mi][i] = (size_t)min(m0 + mi * 16 + g * 4 + i, M - 1) * KB;
-    }
-#pragma unroll
-    for (int ni = 0; ni < TN; ++ni) wrow[ni] = (size_t)min(n0 + ni * 16 + r, N - 1);
-
-    for (int kb = 0; kb < KB; ++kb) {
-        long a[TM], b[TN];
-        float ws[TN];
-#pragma unroll
-        for (int mi = 0; mi < TM; ++mi) a[mi] = *(const long *)(aq + arow[mi] + kb * 32 + g * 8);
-#pragma unroll
-        for (int ni = 0; ni < TN; ++ni) {
-            if (Q8) {
-                b[ni] = *(const long *)(qs + wrow[ni] * K + kb * 32 + g * 8);
-            } else {
-                const unsigned w = *(const unsigned *)(qs + wrow[ni] * (K >> 1) + kb * 16 + g * 4);
-                b[ni] = (long)(((unsigned long)((w >> 4) & 0x0F0F0F0Fu) << 32) | (unsigned long)(w & 0x0F0F0F0Fu));
-            }
-            ws[ni] = __half2float(sc[wrow[ni] * KB + kb]);
-        }
-#pragma unroll
-        for (int mi = 0; mi < TM; ++mi) {
-            float as[4];
-            int bias[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                as[i] = a_scale[srow[mi][i] + kb];
-                bias[i] = Q8 ? 0 : 8 * a_sum[srow[mi][i] + kb];
-            }
-#pragma unroll
-            for (int ni = 0; ni < TN; ++ni) {
-                const i32x4 d = __builtin_amdgcn_mfma_i32_16x16x32_i8(a[mi], b[ni], i32x4{0, 0, 0, 0}, 0, 0, 0);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[mi][ni][i] += (float)(d[i] - bias[i]) * (as[i] * ws[ni]);
-            }
-        }
-    }
-
-#pragma unroll
-    for (int mi = 0; mi < TM; ++mi)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int row = m0 + mi * 16 + g * 4 + i;
-            if (row >= M) continue;
-#pragma unroll
-            for (int ni = 0; ni < TN; ++ni) {
-                const int col = n0 + ni * 16 + r;
-                if (col >= N) continue;
-                float *dst = c + (size_t)row * ldc + col;
-                const float v = alpha * acc[mi][ni][i];
-                *dst = beta == 0.f ? v : v + beta * *dst;
-            }
-        }
-}
-
-// ---- LDS-staged exact kernel (more than 16 activation rows): same arithmetic as gemm_i8_kernel - one
+// ---- LDS-staged exact kernel: one
 // v_mfma_i32_16x16x32_i8 per 16x16 tile per quant block, then acc += f32(idot) * (a_scale * w_scale) - but
 // the operands of a K step (4 quant blocks) are staged once per workgroup in LDS with coalesced 16-byte
 // loads (a cache line per row), instead of 8-byte operand loads per lane per tile from global memory, which
@@ -592,19 +511,6 @@ int launch_i8_lds_pick(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, Prep
     }
 }
 
-template <int DT>
-void launch_i8(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
-    const int M = (int)m, N = (int)w->n, K = (int)w->k;
-    const unsigned gx = (unsigned)((N + 255) / 256);
-    if (M > 32) {
-        launch_k(ctx, gemm_i8_kernel<DT, 4>, dim3(gx, (unsigned)((M + 63) / 64)), dim3(256), 0, w->qs, w->sc, act.q, act.scale, act.sum, c, M, N, K, ldc, alpha, beta);
-    } else if (M > 16) {
-        launch_k(ctx, gemm_i8_kernel<DT, 2>, dim3(gx, (unsigned)((M + 31) / 32)), dim3(256), 0, w->qs, w->sc, act.q, act.scale, act.sum, c, M, N, K, ldc, alpha, beta);
-    } else {
-        launch_k(ctx, gemm_i8_kernel<DT, 1>, dim3(gx, (unsigned)((M + 15) / 16)), dim3(256), 0, w->qs, w->sc, act.q, act.scale, act.sum, c, M, N, K, ldc, alpha, beta);
-    }
-}
-
 }  // namespace
 
 int launch_gemm_i8_few_rows(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
@@ -615,12 +521,8 @@ int launch_gemm_i8_few_rows(aionhip_ctx *ctx, const aionhip_weight *w, size_t m,
 int launch_gemm_i8(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
     const char *name = w->dtype == AIONHIP_Q8_0 ? "gemm_i8_q8" : "gemm_i8_q4";
     ProfScope scope(ctx, name);
-    if (m > 16 && w->k >= 32) {
-        const int rc = w->dtype == AIONHIP_Q8_0 ? launch_i8_lds_pick<AIONHIP_Q8_0>(ctx, w, m, act, c, ldc, alpha, beta)
-                                                : launch_i8_lds_pick<AIONHIP_Q4_0>(ctx, w, m, act, c, ldc, alpha, beta);
-        if (rc) return rc;
-    } else if (w->dtype == AIONHIP_Q8_0) launch_i8<AIONHIP_Q8_0>(ctx, w, m, act, c, ldc, alpha, beta);
-    else launch_i8<AIONHIP_Q4_0>(ctx, w, m, act, c, ldc, alpha, beta);
+    const int rc = launch_gemm_i8_few_rows(ctx, w, m, act, c, ldc, alpha, beta);
+    if (rc) return rc;
     LAUNCH_CHECK(ctx, name);
     return AIONHIP_OK;
 }

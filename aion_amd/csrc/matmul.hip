@@ -2,8 +2,9 @@
 // graph/program/compiler.zig:189-239,337-357), activation preparation, kernel routing
 // (the counterpart of cpu/exec/matmul.zig:233-296 `matvecRoute` / `gemm2D`):
 //   m == 1, k <= 4096, 16-byte aligned A  -> gemv_fused_kernel (activation prepared in the kernel)
-//   m <= 8                                -> prepare_act_kernel + gemv_kernel
-//   m  > 8                                -> gemm_i8_kernel (exact) or gemm_bf16_wide_kernel
+//   m <= 8                                -> prepare_act_kernel + gemv_kernel / gemv_rows_kernel (5..8 rows against a
+//                                            wide short weight: the 16-row tile of gemm_i8_lds_kernel)
+//   m  > 8                                -> gemm_i8_lds_kernel (exact) or gemm_bf16_wide_kernel
 // and the decode fusions built on the single-row kernel: RMSNorm / gelu-gate prologues, the q/k/v + RoPE +
 // cache-append launch and the GeGLU block (two launches).
 #include "common.h"
