@@ -11,7 +11,7 @@ import ctypes as C
 import numpy as np
 
 from . import hip
-from .hip import (BF16, F16, F32, GEMM_BF16_MFMA, GEMM_EXACT_I8, I32, KMAJOR_KN, Q4_0, Q8_0, ROWS_NK, UNBOUNDED,  # noqa: F401
+from .hip import (BF16, F16, F32, GEMM_BF16_MFMA, GEMM_BF16_MFMA_ALWAYS, GEMM_EXACT_I8, I32, KMAJOR_KN, Q4_0, Q8_0, ROWS_NK, UNBOUNDED,  # noqa: F401
                   AionHipError)
 
 BLOCK_BYTES = {Q4_0: 18, Q8_0: 34}

@@ -170,7 +170,7 @@ void *aionhip_stream(aionhip_ctx *ctx) { return ctx ? (void *)ctx->stream : null
 
 int aionhip_set_gemm_mode(aionhip_ctx *ctx, int mode) {
     if (!ctx) return AIONHIP_INVALID_ARGUMENT;
-    if (mode != AIONHIP_GEMM_EXACT_I8 && mode != AIONHIP_GEMM_BF16_MFMA) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "unknown gemm mode %d", mode);
+    if (mode != AIONHIP_GEMM_EXACT_I8 && mode != AIONHIP_GEMM_BF16_MFMA && mode != AIONHIP_GEMM_BF16_MFMA_ALWAYS) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "unknown gemm mode %d", mode);
     ctx->gemm_mode = mode;
     return AIONHIP_OK;
 }

@@ -487,20 +487,26 @@ constexpr GiShape GI_SHAPES[6] = {
     {4, false, 0.81f, 1.40f}, {2, false, 0.44f, 1.25f}, {1, false, 0.284f, 1.55f},
     {4, true, 0.253f, 1.45f}, {2, true, 0.164f, 1.50f}, {1, true, 0.121f, 1.85f},
 };
-template <int DT>
-int launch_i8_lds_pick(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
+// the cheapest shape for m rows against an n x k weight and its modelled time per quant block of K
+int pick_i8_shape(const aionhip_ctx *ctx, size_t m, size_t n, size_t k, float *us_per_block) {
     const float cus = (float)(ctx->cu_count > 0 ? ctx->cu_count : 256);
     int best = 0;
     float best_t = 0.f;
     for (int i = 0; i < 6; ++i) {
         const GiShape &g = GI_SHAPES[i];
-        if (g.split && w->k < 256) continue;             // a split-K step is 8 blocks
+        if (g.split && k < 256) continue;                // a split-K step is 8 blocks
         const size_t bm = (size_t)(g.split ? 16 : 32) * g.wm, bn = g.split ? 64 : 128;
-        const float wgs = (float)(((m + bm - 1) / bm) * ((w->n + bn - 1) / bn));
+        const float wgs = (float)(((m + bm - 1) / bm) * ((n + bn - 1) / bn));
         const float rounds = wgs / (cus * g.overlap);
         const float t = g.us_per_block * (rounds > 1.f ? rounds : 1.f);
         if (i == 0 || t < best_t) { best = i; best_t = t; }
     }
+    if (us_per_block) *us_per_block = best_t;
+    return best;
+}
+template <int DT>
+int launch_i8_lds_pick(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
+    const int best = pick_i8_shape(ctx, m, w->n, w->k, nullptr);
     switch (best) {
     case 0: return launch_i8_lds<DT, 4, 4, false>(ctx, w, m, act, c, ldc, alpha, beta);
     case 1: return launch_i8_lds<DT, 2, 4, false>(ctx, w, m, act, c, ldc, alpha, beta);
@@ -512,6 +518,22 @@ int launch_i8_lds_pick(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, Prep
 }
 
 }  // namespace
+
+// In bf16 mode: is the bf16 MFMA kernel expected to beat the exact kernel for this shape? Up to a few hundred rows it
+// is not - it streams a 2-byte copy of every weight (3.5x the q4 bytes), its 256-column tiles leave most CUs idle and
+// one workgroup's K loop is a latency chain - and the exact kernel is then both the faster and the exact one.
+// Modelled times in microseconds, constants fitted to a sweep of 9..512 rows over four weight shapes.
+bool gemm_bf16_pays(const aionhip_ctx *ctx, size_t m, size_t n, size_t k) {
+    float per_block = 0.f;
+    pick_i8_shape(ctx, m, n, k, &per_block);
+    const float blocks = (float)(k / 32);
+    const float exact_us = per_block * blocks + 5.f + (float)m * (float)k * 4.f / 2.0e6f;       // + the int8 preparation of A
+    const float copy_us = (float)n * (float)k * 2.f / 4.0e6f;                                  // weight bytes at ~4 TB/s
+    const float flop_us = 2.f * (float)m * (float)n * (float)k / 9.0e8f;                        // ~900 TFLOP/s
+    const float chain_us = blocks * 0.27f;                                                       // one workgroup's K loop
+    const float bf16_us = fmaxf(fmaxf(copy_us, flop_us), chain_us) + 15.f;
+    return bf16_us < exact_us;
+}
 
 int launch_gemm_i8_few_rows(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
     return w->dtype == AIONHIP_Q8_0 ? launch_i8_lds_pick<AIONHIP_Q8_0>(ctx, w, m, act, c, ldc, alpha, beta)

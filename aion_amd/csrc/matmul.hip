@@ -46,12 +46,18 @@ int run_rows(aionhip_ctx *ctx, const Batch &b, size_t m, const float *a, size_t 
     if (m > 0x7FFFFFFFu) return set_err(ctx, AIONHIP_UNSUPPORTED, "matmul: m exceeds 2^31-1");
     if (m == 1 && b.k <= FUSED_PAYS_K && ((uintptr_t)a & 15) == 0)
         return launch_gemv_fused(ctx, b.w, b.c, b.ldc, (int)b.count, PRO_QUANT, FusedIn{a, nullptr, nullptr, nullptr, 0.f}, alpha, beta);
-    if (m > GEMV_MAX_M && ctx->gemm_mode == AIONHIP_GEMM_BF16_MFMA) {
-        for (size_t i = 0; i < b.count; ++i) {
-            int rc = launch_gemm_bf16(ctx, b.w[i], m, a, lda, b.c[i], b.ldc[i], alpha, beta);
-            if (rc) return rc;
+    if (m > GEMV_MAX_M && ctx->gemm_mode != AIONHIP_GEMM_EXACT_I8) {
+        // the bf16 kernel where it is expected to win (or always, if so asked), the exact kernel (below) for the rest
+        bool all_bf16 = true;
+        if (ctx->gemm_mode == AIONHIP_GEMM_BF16_MFMA)
+            for (size_t i = 0; i < b.count; ++i) all_bf16 = all_bf16 && gemm_bf16_pays(ctx, m, b.w[i]->n, b.k);
+        if (all_bf16) {
+            for (size_t i = 0; i < b.count; ++i) {
+                int rc = launch_gemm_bf16(ctx, b.w[i], m, a, lda, b.c[i], b.ldc[i], alpha, beta);
+                if (rc) return rc;
+            }
+            return AIONHIP_OK;
         }
-        return AIONHIP_OK;
     }
     int rc = ensure_scratch(ctx, prepared_act_bytes(m, b.k));
     if (rc) return rc;

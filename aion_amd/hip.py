@@ -10,7 +10,7 @@ OK, INVALID_ARGUMENT, OUT_OF_MEMORY, UNSUPPORTED, EXECUTION_FAILED = range(5)
 STATUS_NAMES = {0: "OK", 1: "InvalidArgument", 2: "OutOfMemory", 3: "Unsupported", 4: "ExecutionFailed"}
 F32, F16, I8, Q4_0, Q8_0, I32, BF16 = 0, 1, 2, 3, 4, 5, 16
 ROWS_NK, KMAJOR_KN = 0, 1
-GEMM_EXACT_I8, GEMM_BF16_MFMA = 0, 1
+GEMM_EXACT_I8, GEMM_BF16_MFMA, GEMM_BF16_MFMA_ALWAYS = 0, 1, 2
 UNBOUNDED = 0xFFFFFFFF
 
 

@@ -256,7 +256,7 @@ def run_gemm(gpu, be):
             for m in (512, 2048):
                 x = gpu.upload(rng.standard_normal((m, k)).astype(np.float32))
                 y = gpu.alloc(m * n * 4)
-                for mode, kname, peak in ((be.GEMM_BF16_MFMA, "gemm_bf16", "bf16"), (be.GEMM_EXACT_I8, "gemm_i8_" + tag, "int8")):
+                for mode, kname, peak in ((be.GEMM_BF16_MFMA_ALWAYS, "gemm_bf16", "bf16"), (be.GEMM_EXACT_I8, "gemm_i8_" + tag, "int8")):
                     gpu.set_gemm_mode(mode)
                     for _ in range(2):
                         gpu.step_matmul(w, x, m, y)
@@ -269,7 +269,7 @@ def run_gemm(gpu, be):
                     wall = (time.perf_counter() - t0) / 10
                     ms = sum(prof) / 10             # a call may be more than one launch of this kernel
                     tf = 2.0 * m * n * k / (ms * 1e-3) / 1e12
-                    res["%s M%d N%d %s" % (tag, m, n, "bf16" if mode == be.GEMM_BF16_MFMA else "exact_i8")] = {
+                    res["%s M%d N%d %s" % (tag, m, n, "bf16" if mode == be.GEMM_BF16_MFMA_ALWAYS else "exact_i8")] = {
                         "kernel_ms": round(ms, 4), "step_wall_ms": round(wall * 1e3, 4), "TFLOPs": round(tf, 1),
                         "frac_mfma_peak": round(tf / MFMA_PEAK[peak], 4), "peak": peak}
                 x.free(); y.free()
@@ -456,7 +456,7 @@ def run_decoder(gpu, be, with_cpu=True):
         "setup_s": round(setup_s, 1),
         "prefill_128_ms_exact_i8": round(prefill_exact_ms, 3),          # the default mode: aion's arithmetic
         "prefill_tokens_per_s": round(128 / (prefill_exact_ms * 1e-3), 1),
-        "prefill_128_ms_bf16_mfma": round(prefill_ms, 3),               # pays off from a few hundred rows on
+        "prefill_128_ms_bf16_mode": round(prefill_ms, 3),               # bf16 mode keeps the exact kernel at 128 rows (the bf16 one pays from a few hundred on)
         "prefill_next_token_bf16_vs_exact": [int(tok), int(tok_exact)],
         "decode_tokens_per_s": round(128 / decode_s, 1),
         "decode_ms_per_token": round(decode_s / 128 * 1e3, 4),

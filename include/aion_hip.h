@@ -170,8 +170,10 @@ int aionhip_step_gate_matmul(aionhip_ctx *ctx, const aionhip_weight *b, size_t r
 
 /* How m > 8 rows are multiplied. EXACT_I8 (default): int8 activations, integer MFMA, per-block
  * f32 scaling - the same numbers as the decode path. BF16_MFMA: weights dequantized to bf16,
- * activations rounded to bf16, f32 accumulation - faster, judged at 1e-2 instead of 2e-3. */
-typedef enum aionhip_gemm_mode { AIONHIP_GEMM_EXACT_I8 = 0, AIONHIP_GEMM_BF16_MFMA = 1 } aionhip_gemm_mode;
+ * activations rounded to bf16, f32 accumulation - judged at 1e-2 instead of 2e-3; used where it is expected to
+ * be the faster kernel (from a few hundred rows on; below that the exact kernel runs, which is then both faster
+ * and exact). BF16_MFMA_ALWAYS: the bf16 kernel for every m > 8, whatever the shape. */
+typedef enum aionhip_gemm_mode { AIONHIP_GEMM_EXACT_I8 = 0, AIONHIP_GEMM_BF16_MFMA = 1, AIONHIP_GEMM_BF16_MFMA_ALWAYS = 2 } aionhip_gemm_mode;
 int aionhip_set_gemm_mode(aionhip_ctx *ctx, int mode);
 /* Name of the kernel the last matmul/attention step launched (the reference's tests assert
  * which kernel ran after a parity check, backend/gpu/test_gpu_backend.zig:1116-1162). */

@@ -97,7 +97,7 @@ def test_config3_exact_full_size_on_row_sample(gpu, orc, dtype, layout, m, n):
 @pytest.mark.parametrize("m,n,k", [(9, 64, 64), (100, 130, 256), (300, 520, 1024)])
 def test_bf16_gemm_ragged_shapes(gpu, orc, dtype, layout, m, n, k):
     say("bf16", dtype, layout, m, n, k)
-    gpu.set_gemm_mode(be.GEMM_BF16_MFMA)
+    gpu.set_gemm_mode(be.GEMM_BF16_MFMA_ALWAYS)         # shapes this small run on the exact kernel in the plain bf16 mode
     try:
         blocks, w = make_weight(gpu, dtype, layout, n, k, seed=m * n)
         a = bf16_round(np.random.default_rng(k).standard_normal((m, k)).astype(np.float32))
@@ -125,7 +125,7 @@ def test_bf16_gemm_ragged_shapes(gpu, orc, dtype, layout, m, n, k):
 def test_config3_bf16_full_size_on_row_sample(gpu, orc, dtype, layout, m, n):
     k = 4096
     say("config3 bf16", dtype, m, n)
-    gpu.set_gemm_mode(be.GEMM_BF16_MFMA)
+    gpu.set_gemm_mode(be.GEMM_BF16_MFMA_ALWAYS)
     try:
         blocks, w = make_weight(gpu, dtype, layout, n, k, seed=n + 1)
         a = bf16_round(np.random.default_rng(m + 1).standard_normal((m, k)).astype(np.float32))
@@ -140,3 +140,24 @@ def test_config3_bf16_full_size_on_row_sample(gpu, orc, dtype, layout, m, n):
         w.free()
     finally:
         gpu.set_gemm_mode(be.GEMM_EXACT_I8)
+
+
+def test_bf16_mode_runs_the_bf16_kernel_only_where_it_pays(gpu, orc):
+    """In bf16 mode a shape the bf16 kernel is not expected to win (few rows: it streams a 2-byte copy of the weight
+    through 256-column tiles) stays on the exact kernel - same numbers as the exact mode - and a large one moves."""
+    blocks, w = make_weight(gpu, be.Q4_0, be.KMAJOR_KN, 4096, 4096, seed=5)
+    rng = np.random.default_rng(6)
+    small, large = rng.standard_normal((48, 4096)).astype(np.float32), rng.standard_normal((2048, 4096)).astype(np.float32)
+    exact_small = gpu.matmul(w, small)
+    gpu.set_gemm_mode(be.GEMM_BF16_MFMA)
+    try:
+        got = gpu.matmul(w, small)
+        assert gpu.last_kernel() == "gemm_i8_q4" and np.array_equal(got, exact_small)
+        gpu.matmul(w, large)
+        assert gpu.last_kernel() == "gemm_bf16"
+        gpu.set_gemm_mode(be.GEMM_BF16_MFMA_ALWAYS)
+        gpu.matmul(w, small)
+        assert gpu.last_kernel() == "gemm_bf16"
+    finally:
+        gpu.set_gemm_mode(be.GEMM_EXACT_I8)
+    w.free()
