@@ -307,8 +307,9 @@ def test_rolling_caches(gpu, orc, case):
     assert np.isfinite(got).all() and err < (1e-2 if kind == "bf16" else 2e-3)
 
 
-@pytest.mark.parametrize("window,rolling", [(be.CAUSAL, False), ((300, 0, 0), False), ((200, 40, 64), False), ((300, 0, 0), True)])
-def test_prefill_key_segments_with_windows_and_ragged_lengths(gpu, orc, window, rolling):
+@pytest.mark.parametrize("window,rolling,soft_cap", [(be.CAUSAL, False, 0.0), ((300, 0, 0), False, 0.0), ((200, 40, 64), False, 0.0),
+                                                     ((300, 0, 0), True, 0.0), (be.CAUSAL, False, 5.0)])
+def test_prefill_key_segments_with_windows_and_ragged_lengths(gpu, orc, window, rolling, soft_cap):
     """The prefill kernel with its key range cut into segments (few row tiles on many CUs) and the merge pass: ragged
     cache lengths, positions that start inside the cache, windows that leave whole segments of a row tile empty, and
     a rolling cache. The profile must show the merge pass, or the case did not run in segments."""
@@ -320,12 +321,12 @@ def test_prefill_key_segments_with_windows_and_ragged_lengths(gpu, orc, window, 
         ends = ends + 2 * T                                   # the ring has wrapped twice
         pos = pos + 2 * T
     gpu.profile_start()
-    got = run_attention(gpu, q, k, v, 1 / math.sqrt(D), qd, kd, window=window, positions=pos, kv_lengths=ends, rolling=rolling)
+    got = run_attention(gpu, q, k, v, 1 / math.sqrt(D), qd, kd, window=window, positions=pos, kv_lengths=ends, rolling=rolling, soft_cap=soft_cap)
     names = [n for n, _ in gpu.profile_stop()]
     assert names == ["attn_prefill", "attn_merge"], names
     if rolling:
         ref = orc.attention_rolling_f64(qf, kf, vf, 1 / math.sqrt(D), window, pos, ends)
     else:
-        ref = orc.attention_f64(qf, kf, vf, 1 / math.sqrt(D), window=window, positions=pos, kv_lengths=ends)
+        ref = orc.attention_f64(qf, kf, vf, 1 / math.sqrt(D), window=window, soft_cap=soft_cap, positions=pos, kv_lengths=ends)
     assert np.isfinite(got).all()
     assert float(np.abs(got - ref).max()) < 2e-3
