@@ -299,6 +299,16 @@ class HipBackend:
         """StepElemwiseBinary add/sub/mul/div on f32: out[i] = a[i] op b[i % nb] (nb = n: same shape; 1: scalar)."""
         self._check(self._lib.aionhip_step_binary(self._ctx, self.BINARY[op], out.handle, a.handle, b.handle, n, n if nb is None else nb))
 
+    def step_headnorm_rope_append(self, q_out, q, k, v, gammas, betas, eps, k_cache, v_cache, positions, write_index, b, s, t_cap,
+                                  h_q, h_kv, d, base=10000.0, scale_factor=1.0, proportion=1.0, rolling=False):
+        """Per-head RMSNorm on q, k, v (gammas / betas: three buffers each, a beta may be None) -> RoPE(q, k) -> f16
+        cache append of k and v, one launch."""
+        hb = [x.handle if x is not None else 0 for x in betas]
+        self._check(self._lib.aionhip_step_headnorm_rope_append(
+            self._ctx, q_out.handle, q.handle, k.handle, v.handle, gammas[0].handle, hb[0], gammas[1].handle, hb[1], gammas[2].handle, hb[2],
+            eps, k_cache.handle, v_cache.handle, positions.handle, write_index.handle, b, s, t_cap, h_q, h_kv, d, base, scale_factor,
+            proportion, 1 if rolling else 0))
+
     def step_cast_f32_f16(self, out, x, n):
         self._check(self._lib.aionhip_step_cast_f32_f16(self._ctx, out.handle, x.handle, n))
 

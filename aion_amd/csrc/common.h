@@ -218,6 +218,14 @@ constexpr int DPP_ROW_HALF_MIRROR = 0x141;
 constexpr int DPP_ROW_MIRROR = 0x140;
 
 // sum over the 64 lanes of a wavefront; every lane returns the total
+// The rotation of one RoPE pair with every product and the sum rounded on its own, as aion's CPU kernel computes it
+// (cpu/kernels/rope.zig:90-91, no fused multiply-add) - and so the same bits from every kernel that rotates.
+__device__ __forceinline__ void rope_rotate(float xl, float xh, float sn, float cs, float &yl, float &yh) {
+#pragma clang fp contract(off)
+    yl = xl * cs - xh * sn;
+    yh = xl * sn + xh * cs;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
     v += dpp_f<DPP_QUAD_XOR1>(v);
     v += dpp_f<DPP_QUAD_XOR2>(v);

@@ -255,7 +255,8 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedI
                 const bool rot = cur.seg < 2 && i < epi.rope_pairs;
                 float sn = 0.f, cs = 1.f;
                 if (rot) sincosf((float)epi.positions[0] * epi.freq[i], &sn, &cs);
-                const float yl = rot ? xl * cs - xh * sn : xl, yh = rot ? xl * sn + xh * cs : xh;
+                float yl = xl, yh = xh;
+                if (rot) rope_rotate(xl, xh, sn, cs, yl, yh);
                 if (cur.seg == 0) {
                     cur.c[head * epi.d + i] = yl;
                     cur.c[head * epi.d + half + i] = yh;

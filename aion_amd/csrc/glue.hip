@@ -51,8 +51,7 @@ __global__ void rope_kernel(float *__restrict__ out, const float *__restrict__ x
     sincosf(ang, &sn, &cs);
     for (int h = 0; h < H; ++h) {
         const float xl = xr[h * D + i], xh = xr[h * D + half + i];
-        orow[h * D + i] = xl * cs - xh * sn;
-        orow[h * D + half + i] = xl * sn + xh * cs;
+        rope_rotate(xl, xh, sn, cs, orow[h * D + i], orow[h * D + half + i]);
     }
 }
 
@@ -84,7 +83,8 @@ __global__ void rope_append_kernel(float *__restrict__ q_out, const float *__res
     if (!is_q) { vl = v[src + i]; vh = v[src + half + i]; }
     float sn = 0.f, cs = 1.f;
     if (rot) sincosf((float)pos * fr, &sn, &cs);
-    const float yl = rot ? xl * cs - xh * sn : xl, yh = rot ? xl * sn + xh * cs : xh;
+    float yl = xl, yh = xh;
+    if (rot) rope_rotate(xl, xh, sn, cs, yl, yh);
     if (is_q) {
         q_out[src + i] = yl;
         q_out[src + half + i] = yh;
@@ -98,6 +98,74 @@ __global__ void rope_append_kernel(float *__restrict__ q_out, const float *__res
     kcache[dst + half + i] = __float2half_rn(yh);
     vcache[dst + i] = __float2half_rn(vl);
     vcache[dst + half + i] = __float2half_rn(vh);
+}
+
+// The input side of an attention block in a model that normalizes its heads (aion's bench model,
+// src/bench/models.zig:455-473): RMSNorm over the head dimension on q, k and v (cpu/kernels/layernorm.zig:69-147), RoPE on
+// q and k, f16 cast and cache append of k and v - eight to ten steps of a few microseconds each as one launch. One
+// wavefront per (token, head): q heads first, then k, then v; lane l holds the pairs (i, i + D/2), i = l, l + 64, ...
+__global__ __launch_bounds__(256) void headnorm_rope_append_kernel(
+    float *__restrict__ q_out, const float *__restrict__ q, const float *__restrict__ k, const float *__restrict__ v,
+    const float *__restrict__ gq, const float *__restrict__ bq, const float *__restrict__ gk, const float *__restrict__ bk,
+    const float *__restrict__ gv, const float *__restrict__ bv, float eps, __half *__restrict__ kcache, __half *__restrict__ vcache,
+    const int *__restrict__ positions, const int *__restrict__ write_index, size_t batch, size_t s_len, size_t t_cap, int Hq, int Hkv,
+    int D, int rope_pairs, const float *__restrict__ freq, int rolling) {
+    const int half = D / 2, slots = Hq + 2 * Hkv, lane = threadIdx.x & 63;
+    const size_t item = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (item >= batch * s_len * (size_t)slots) return;                     // wavefront-uniform
+    const int slot = (int)(item % slots);
+    const size_t tok = item / slots;
+    const int kind = slot < Hq ? 0 : slot < Hq + Hkv ? 1 : 2;             // q, k, v
+    const int h = kind == 0 ? slot : kind == 1 ? slot - Hq : slot - Hq - Hkv;
+    const float *src = (kind == 0 ? q + (tok * Hq + h) * D : (kind == 1 ? k : v) + (tok * Hkv + h) * D);
+    const float *gamma = kind == 0 ? gq : kind == 1 ? gk : gv, *beta = kind == 0 ? bq : kind == 1 ? bk : bv;
+    const int pos = positions[tok];
+    const int widx = write_index[tok / s_len];
+    constexpr int MAXP = 4;                                                // pairs per lane: head sizes up to 512
+    float xl[MAXP], xh[MAXP];
+#pragma unroll
+    for (int u = 0; u < MAXP; ++u) {
+        const int i = lane + 64 * u;
+        xl[u] = i < half ? src[i] : 0.f;
+        xh[u] = i < half ? src[half + i] : 0.f;
+    }
+    // the sum of squares in rmsnorm_kernel's order (thread c of 256 adds x[c]^2, x[c + 256]^2; four wavefront sums; their
+    // pairwise sum), so that the fused step gives the bits of the separate ones: the row is read a second time, from L1
+    float part[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int c = lane + 64 * j;
+        float ssj = 0.f;
+        if (c < D) ssj += src[c] * src[c];
+        if (c + 256 < D) ssj += src[c + 256] * src[c + 256];
+        part[j] = wave_sum(ssj);
+    }
+    const float ss = (part[0] + part[1]) + (part[2] + part[3]);
+    const float inv = 1.f / sqrtf(ss * (1.f / (float)D) + eps);
+    const size_t b = tok / s_len, s = tok % s_len;
+    long t = (long)widx + (long)s;
+    if (rolling && t >= 0) t %= (long)t_cap;
+    const bool in_cache = t >= 0 && (size_t)t < t_cap;                     // never write outside the cache
+    __half *dst = (kind == 1 ? kcache : vcache) + ((b * t_cap + (size_t)(in_cache ? t : 0)) * Hkv + h) * D;
+#pragma unroll
+    for (int u = 0; u < MAXP; ++u) {
+        const int i = lane + 64 * u;
+        if (i >= half) break;
+        float yl = (xl[u] * inv) * gamma[i] + (beta ? beta[i] : 0.f);
+        float yh = (xh[u] * inv) * gamma[half + i] + (beta ? beta[half + i] : 0.f);
+        if (kind != 2 && i < rope_pairs) {
+            float sn, cs;
+            sincosf((float)pos * freq[i], &sn, &cs);
+            rope_rotate(yl, yh, sn, cs, yl, yh);
+        }
+        if (kind == 0) {
+            q_out[(tok * Hq + h) * D + i] = yl;
+            q_out[(tok * Hq + h) * D + half + i] = yh;
+        } else if (in_cache) {
+            dst[i] = __float2half_rn(yl);
+            dst[half + i] = __float2half_rn(yh);
+        }
+    }
 }
 
 __global__ void add_kernel(float *__restrict__ out, const float *__restrict__ a, const float *__restrict__ b, size_t n) {
@@ -343,6 +411,40 @@ int aionhip_step_rope_append(aionhip_ctx *ctx, aionhip_handle q_out, aionhip_han
         dp<float>(q_out), dp<const float>(q), dp<const float>(k), dp<const float>(v), dp<__half>(k_cache), dp<__half>(v_cache),
         dp<const int>(positions), dp<const int>(write_index), b, s, t_cap, (int)h_q, (int)h_kv, (int)d, (int)rope_pairs, freq);
     LAUNCH_CHECK(ctx, "rope_append");
+    return AIONHIP_OK;
+}
+
+int aionhip_step_headnorm_rope_append(aionhip_ctx *ctx, aionhip_handle q_out, aionhip_handle q, aionhip_handle k, aionhip_handle v,
+                                      aionhip_handle gamma_q, aionhip_handle beta_q, aionhip_handle gamma_k, aionhip_handle beta_k,
+                                      aionhip_handle gamma_v, aionhip_handle beta_v, float eps, aionhip_handle k_cache,
+                                      aionhip_handle v_cache, aionhip_handle positions, aionhip_handle write_index, size_t b, size_t s,
+                                      size_t t_cap, size_t h_q, size_t h_kv, size_t d, float base_frequency, float scale_factor,
+                                      float rope_proportion, int rolling) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (!q_out || !q || !k || !v || !gamma_q || !gamma_k || !gamma_v || !k_cache || !v_cache || !positions || !write_index)
+        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "headnorm_rope_append: null operand");
+    if (!(eps > 0.f) || !(eps < INFINITY)) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "headnorm_rope_append: eps must be positive and finite");
+    if (!(base_frequency > 0.f) || !(base_frequency < INFINITY) || !(scale_factor > 0.f) || !(scale_factor < INFINITY) ||
+        !(rope_proportion >= 0.f && rope_proportion <= 1.f))
+        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "headnorm_rope_append: base/scale must be positive and finite, proportion in [0,1]");
+    if (d % 2 != 0 || h_q > 65535 || h_kv > 65535) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "headnorm_rope_append: head size must be even");
+    if (d > 512) return set_err(ctx, AIONHIP_UNSUPPORTED, "headnorm_rope_append: head size %zu above 512 (issue the separate steps)", d);
+    if (s > t_cap) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "headnorm_rope_append: %zu new tokens exceed the cache capacity %zu", s, t_cap);
+    const size_t items = b * s * (h_q + 2 * h_kv);
+    if (!items || !h_q || !h_kv || !d) return AIONHIP_OK;
+    const size_t half = d / 2;
+    size_t rope_pairs = (size_t)floorf(rope_proportion * (float)half);
+    if (rope_pairs > half) rope_pairs = half;
+    const float freq_step = (float)pow((double)base_frequency, (double)(-2.0f / (float)d));
+    const float *freq = nullptr;
+    int rc = rope_table(ctx, (int)rope_pairs, freq_step, scale_factor, &freq);
+    if (rc) return rc;
+    headnorm_rope_append_kernel<<<dim3(grid_for(items, 4)), dim3(256), 0, ctx->stream>>>(
+        dp<float>(q_out), dp<const float>(q), dp<const float>(k), dp<const float>(v), dp<const float>(gamma_q), dp<const float>(beta_q),
+        dp<const float>(gamma_k), dp<const float>(beta_k), dp<const float>(gamma_v), dp<const float>(beta_v), eps, dp<__half>(k_cache),
+        dp<__half>(v_cache), dp<const int>(positions), dp<const int>(write_index), b, s, t_cap, (int)h_q, (int)h_kv, (int)d,
+        (int)rope_pairs, freq, rolling);
+    LAUNCH_CHECK(ctx, "headnorm_rope_append");
     return AIONHIP_OK;
 }
 

@@ -314,6 +314,89 @@ class PackageRunner:
                 skip.update(c)
             return True
 
+        def try_headnorm(i):
+            """Per-head norms between the projections and the cache (src/bench/models.zig:455-473):
+            q,k,v -> reshape -> RMSNorm over the head size -> RoPE1D(q,k) -> Cast -> SequenceAppend(k,v), one launch.
+            Called at the first of the three norms; the three projections are already on the device."""
+            n0 = nodes[i]
+            r0 = producer.get(n0.inputs[0])
+            if r0 is None or nodes[r0].op != "ViewReshape":
+                return False
+            m0 = producer.get(nodes[r0].inputs[0])
+            if m0 is None or nodes[m0].op != "MatMul":
+                return False
+            sibs = uses.get(nodes[m0].inputs[0], [])
+            if len(sibs) != 3 or _OUT in sibs or any(nodes[m].op != "MatMul" or nodes[m].output not in vals for m in sibs):
+                return False
+            chains, src = {}, {}
+            for m in sibs:
+                r = sole_user(nodes[m].output, "ViewReshape")
+                if r is None or len(pkg.shape_of(nodes[r].output, sym)) != 4:
+                    return False
+                nrm = sole_user(nodes[r].output, "RMSNorm")
+                if nrm is None or nodes[nrm].inputs[0] != nodes[r].output or nrm in skip or nrm < i:
+                    return False
+                hs = pkg.shape_of(nodes[nrm].output, sym)
+                if [pkg.dim_term(t, sym) for t in nodes[nrm].attrs["normalized_shape"]] != [hs[3]]:
+                    return False
+                nxt = sole_user(nodes[nrm].output)
+                if nxt is None:
+                    return False
+                if nodes[nxt].op == "RoPE1D" and nodes[nxt].inputs[0] == nodes[nrm].output:
+                    after = sole_user(nodes[nxt].output)
+                    if after is None:
+                        return False
+                    if nodes[after].op == "Attention" and nodes[after].inputs[0] == nodes[nxt].output:
+                        chains["q"], src["q"] = (nrm, nxt), m
+                    elif nodes[after].op == "Cast":
+                        app = sole_user(nodes[after].output, "SequenceAppend")
+                        if app is None or nodes[app].inputs[1] != nodes[after].output:
+                            return False
+                        chains["k"], src["k"] = (nrm, nxt, after, app), m
+                    else:
+                        return False
+                elif nodes[nxt].op == "Cast":
+                    app = sole_user(nodes[nxt].output, "SequenceAppend")
+                    if app is None or nodes[app].inputs[1] != nodes[nxt].output:
+                        return False
+                    chains["v"], src["v"] = (nrm, nxt, app), m
+                else:
+                    return False
+            if set(chains) != {"q", "k", "v"} or chains["q"][0] != i:
+                return False
+            nq, nk, nv = (nodes[chains[c][0]] for c in "qkv")
+            rq, rk = nodes[chains["q"][1]], nodes[chains["k"][1]]
+            ak, av = nodes[chains["k"][3]], nodes[chains["v"][2]]
+            if rq.attrs != rk.attrs or rq.inputs[1] != rk.inputs[1] or ak.inputs[2] != av.inputs[2]:
+                return False
+            if nq.attrs["eps"] != nk.attrs["eps"] or nq.attrs["eps"] != nv.attrs["eps"]:
+                return False
+            if any(nodes[c].attrs["to_dtype"] != "f16" for c in (chains["k"][2], chains["v"][1])):
+                return False
+            qs, ks, vs = (pkg.shape_of(x.output, sym) for x in (nq, nk, nv))
+            if qs[:2] != ks[:2] or ks != vs or qs[3] != ks[3] or qs[3] % 2 or qs[3] > 512:
+                return False
+            kc, vc = get(ak.inputs[0]), get(av.inputs[0])
+            if kc.shape != vc.shape or kc.shape[0] != ks[0] or kc.shape[2:] != ks[2:] or kc.dtype != "f16" or kc.extra != vc.extra \
+                    or kc.extra not in (None, "rolling") or ks[1] > kc.shape[1]:
+                return False
+            srcs = [get(nodes[src[c]].output) for c in "qkv"]          # the reshapes between are views of these
+            if any(x.dtype != "f32" for x in srcs):
+                return False
+            gammas = [get(x.inputs[1]).buf for x in (nq, nk, nv)]
+            betas = [get(x.inputs[2]).buf for x in (nq, nk, nv)]
+            q_out = new(qs, "f32")
+            emit(g.step_headnorm_rope_append, q_out, srcs[0].buf, srcs[1].buf, srcs[2].buf, gammas, betas, nq.attrs["eps"], kc.buf, vc.buf,
+                 get(rq.inputs[1]).buf, get(ak.inputs[2]).buf, qs[0], qs[1], kc.shape[1], qs[2], ks[2], qs[3],
+                 base=rq.attrs["base_frequency"], scale_factor=rq.attrs["scale_factor"], proportion=rq.attrs["rope_proportion"],
+                 rolling=kc.extra == "rolling")
+            vals[rq.output] = _Val("dev", q_out, qs, "f32", owned=True)
+            vals[ak.output] = _Val("dev", kc.buf, kc.shape, "f16", extra=kc.extra)
+            vals[av.output] = _Val("dev", vc.buf, vc.shape, "f16", extra=vc.extra)
+            for c in chains.values():
+                skip.update(c)
+            return True
+
         def try_geglu(i, mms):
             """One new token: RMSNorm -> gate, up -> gelu(gate) * up -> down -> add(residual, .)."""
             if s != 1 or len(mms) != 2:
@@ -389,6 +472,8 @@ class PackageRunner:
                 if cols != x.shape[-1]:
                     raise Unsupported("RMSNorm over more than the last axis")
                 rows = _count(x.shape) // cols
+                if self.fuse and len(x.shape) == 4 and try_headnorm(i):
+                    continue
                 mms = matmul_nodes_on(n.output) if self.fuse else None
                 if mms and (try_qkv(i, mms) or try_geglu(i, mms)):
                     continue

@@ -218,6 +218,16 @@ int aionhip_step_rope_append(aionhip_ctx *ctx, aionhip_handle q_out, aionhip_han
                              aionhip_handle k_cache, aionhip_handle v_cache, aionhip_handle positions, aionhip_handle write_index,
                              size_t b, size_t s, size_t t_cap, size_t h_q, size_t h_kv, size_t d,
                              float base_frequency, float scale_factor, float rope_proportion);
+/* The same with an RMSNorm over the head dimension on q, k and v in front (StepRMSNorm x3, gamma / beta of width d,
+ * a beta may be 0; cpu/exec/layernorm.zig:54-155): the input side of an attention block in models that normalize
+ * their heads (src/bench/models.zig:455-473), one launch instead of eight to ten. rope_proportion 0 = no rotation;
+ * rolling = 1: ring caches. Head sizes up to 512 (AIONHIP_UNSUPPORTED above: issue the separate steps). */
+int aionhip_step_headnorm_rope_append(aionhip_ctx *ctx, aionhip_handle q_out, aionhip_handle q, aionhip_handle k, aionhip_handle v,
+                                      aionhip_handle gamma_q, aionhip_handle beta_q, aionhip_handle gamma_k, aionhip_handle beta_k,
+                                      aionhip_handle gamma_v, aionhip_handle beta_v, float eps, aionhip_handle k_cache,
+                                      aionhip_handle v_cache, aionhip_handle positions, aionhip_handle write_index, size_t b, size_t s,
+                                      size_t t_cap, size_t h_q, size_t h_kv, size_t d, float base_frequency, float scale_factor,
+                                      float rope_proportion, int rolling);
 /* StepElemwiseBinary: add, and the fused gate act(a)*b with act = gelu (tanh form)
  * (backend/types.zig:105-109, cpu/exec/elementwise.zig:25-37, cpu/kernels/gelu.zig:8-14) */
 int aionhip_step_add(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle a, aionhip_handle b, size_t n);

@@ -164,6 +164,67 @@ def test_rope_append_equals_the_separate_steps(gpu, orc):
         t.free()
 
 
+@pytest.mark.parametrize("B,S,T,Hq,Hkv,D,rolling,with_beta,proportion", [
+    (1, 1, 16, 8, 1, 256, False, False, 1.0),      # one new token, the bench model's head shape
+    (2, 3, 12, 4, 2, 64, False, True, 0.5),        # several tokens, two sequences, biased norms, half the pairs rotated
+    (1, 5, 8, 4, 1, 128, True, False, 1.0),        # a ring: rows 6, 7, 0, 1, 2
+    (1, 2, 9, 3, 3, 512, False, True, 1.0),        # the largest head size of the fused step
+    (1, 1, 4, 2, 1, 6, True, False, 1.0),          # fewer pairs than lanes
+])
+def test_headnorm_rope_append_equals_the_separate_steps(gpu, orc, B, S, T, Hq, Hkv, D, rolling, with_beta, proportion):
+    """Per-head RMSNorm(q, k, v) -> RoPE(q, k) -> f16 append(k, v) in one launch, against the oracle's separate steps
+    (f32 rounding of the sum of squares, 1e-5) and against this backend's own, whose bits it reproduces."""
+    rng = np.random.default_rng(B * 100 + D)
+    q = rng.standard_normal((B, S, Hq, D)).astype(np.float32)
+    k = rng.standard_normal((B, S, Hkv, D)).astype(np.float32)
+    v = rng.standard_normal((B, S, Hkv, D)).astype(np.float32)
+    gam = [(1 + 0.2 * rng.standard_normal(D)).astype(np.float32) for _ in range(3)]
+    bet = [(0.1 * rng.standard_normal(D)).astype(np.float32) if with_beta else None for _ in range(3)]
+    start = 6 if rolling and S > 1 else 3
+    pos = np.tile(np.arange(start, start + S, dtype=np.int32), (B, 1))
+    widx = np.full(B, start, np.int32)
+    eps = 1e-6
+    bufs = [gpu.upload(x) for x in (q, k, v, pos, widx)]
+    qb, kb, vb, pb, wb = bufs
+    gb = [gpu.upload(x) for x in gam]
+    bb = [gpu.upload(x) if x is not None else None for x in bet]
+    qo = gpu.alloc(q.nbytes)
+    seed = rng.standard_normal((B, T, Hkv, D)).astype(np.float16)          # earlier rows must survive
+    kc, vc = gpu.upload(seed), gpu.upload(seed)
+    gpu.step_headnorm_rope_append(qo, qb, kb, vb, gb, bb, eps, kc, vc, pb, wb, B, S, T, Hq, Hkv, D, proportion=proportion, rolling=rolling)
+    norm = lambda x, i: orc.rmsnorm(x.reshape(-1, D), gam[i], eps, beta=bet[i]).reshape(x.shape)
+    want_q = orc.rope(norm(q, 0), pos, proportion=proportion)
+    want_k = orc.cast_f32_f16(orc.rope(norm(k, 1), pos, proportion=proportion))
+    want_v = orc.cast_f32_f16(norm(v, 2))
+    rows = [(start + s) % T if rolling else start + s for s in range(S)]
+    exp_k, exp_v = seed.copy(), seed.copy()
+    exp_k[:, rows], exp_v[:, rows] = want_k, want_v
+    got_q = gpu.download(qo, np.float32, q.shape)
+    got_k, got_v = gpu.download(kc, np.float16, seed.shape), gpu.download(vc, np.float16, seed.shape)
+    assert np.allclose(got_q, want_q, atol=1e-5, rtol=1e-5)
+    assert np.allclose(got_k.astype(np.float32), exp_k.astype(np.float32), atol=4e-3)      # one f16 ulp at |x| < 8
+    assert np.allclose(got_v.astype(np.float32), exp_v.astype(np.float32), atol=4e-3)
+    untouched = [t for t in range(T) if t not in rows]
+    assert np.array_equal(got_k[:, untouched], seed[:, untouched]) and np.array_equal(got_v[:, untouched], seed[:, untouched])
+    # the separate steps of this backend on the same operands
+    nq, nk, nv, q2, k2 = (gpu.alloc(x.nbytes) for x in (q, k, v, q, k))
+    kc2, vc2 = gpu.upload(seed), gpu.upload(seed)
+    for out, x, i, heads in ((nq, qb, 0, Hq), (nk, kb, 1, Hkv), (nv, vb, 2, Hkv)):
+        gpu.step_rmsnorm(out, x, gb[i], B * S * heads, D, eps, beta=bb[i])
+    gpu.step_rope(q2, nq, pb, B, S, Hq, D, proportion=proportion)
+    gpu.step_rope(k2, nk, pb, B, S, Hkv, D, proportion=proportion)
+    gpu.step_append_f16(kc2, k2, wb, B, S, T, Hkv * D, rolling=rolling)
+    gpu.step_append_f16(vc2, nv, wb, B, S, T, Hkv * D, rolling=rolling)
+    # identical arithmetic in the identical order: identical bits
+    assert np.array_equal(gpu.download(q2, np.float32, q.shape), got_q)
+    assert np.array_equal(gpu.download(kc2, np.float16, seed.shape), got_k)
+    assert np.array_equal(gpu.download(vc2, np.float16, seed.shape), got_v)
+    with pytest.raises(Exception):
+        gpu.step_headnorm_rope_append(qo, qb, kb, vb, gb, bb, eps, kc, vc, pb, wb, B, S, T, Hq, Hkv, 1024)
+    for t in bufs + gb + [x for x in bb if x is not None] + [qo, kc, vc, nq, nk, nv, q2, k2, kc2, vc2]:
+        t.free()
+
+
 @pytest.mark.parametrize("dtype", ["q4", "q8"])
 @pytest.mark.parametrize("D,Hq,Hkv,K", [(256, 8, 1, 2048), (64, 4, 2, 512)])
 def test_qkv_rope_append_fusion_equals_the_separate_steps(gpu, orc, dtype, D, Hq, Hkv, K):

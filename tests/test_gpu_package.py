@@ -336,6 +336,12 @@ def test_bench_model_shaped_package_against_the_graph_oracle(gpu, orc):
             % (max(errs), float(np.mean(errs)), max(selfs), float(np.mean(selfs)), len(errs), run.step_count(1), plain.step_count(1)))
         assert np.mean(errs) < 2 * np.mean(selfs) + 1e-3 and max(errs) < 3 * max(selfs) + 1e-3
         assert np.abs(got["logits"]).max() <= 30.0
+        # the head norms, the rotations and the appends of a block are one step, for the prompt and for single tokens
+        for s_len in (40, 1):
+            names = [fn.__name__ for fn, _a, _k in run.plans[s_len].steps]
+            assert names.count("step_headnorm_rope_append") == cfg["layers"]
+            assert not any(x in names for x in ("step_rope", "step_append_f16", "step_cast_f32_f16"))
+            assert "step_headnorm_rope_append" not in [fn.__name__ for fn, _a, _k in plain.plans[s_len].steps]
         with pytest.raises(ValueError):
             run.run(np.zeros(30, np.int32))               # 63 retained + 30 new rows do not fit a 64-row ring
     finally:

@@ -163,6 +163,7 @@ pub const HipBackend = struct {
             // Optional launch-saving pattern matches over consecutive steps of a decode program (same results as
             // the separate steps; fall back to them on AIONHIP_UNSUPPORTED):
             //   RMSNorm, MatMul x3 (q,k,v), RoPE1D x2, Cast f16 x2, SequenceAppend x2 -> aionhip_step_rmsnorm_qkv_rope_append
+            //   RMSNorm x3 (per head, q,k,v), RoPE1D x2, Cast f16 x2, SequenceAppend x2 -> aionhip_step_headnorm_rope_append
             //   RMSNorm, MatMul x2 (gate, up), gate(gelu), MatMul (down)             -> aionhip_step_rmsnorm_geglu_matmul
             //   RMSNorm, MatMul(s)                                                   -> aionhip_step_rmsnorm_matmul
             //   gate(gelu), MatMul                                                   -> aionhip_step_gate_matmul
