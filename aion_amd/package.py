@@ -422,18 +422,25 @@ class PackageRunner:
             if md is None or nodes[md].inputs[0] != nodes[mul].output or nodes[md].attrs["beta"] != 0.0 or nodes[md].attrs["alpha"] != 1.0:
                 return False
             wd = weight_of(nodes[md].inputs[1])
-            add = sole_user(nodes[md].output, "ElemwiseBinary")
-            if wd is None or add is None:
+            if wd is None:
                 return False
-            res = residual_of(add, nodes[md].output)
+            add = sole_user(nodes[md].output, "ElemwiseBinary")
+            res = residual_of(add, nodes[md].output) if add is not None else None
             wg, wu = weight_of(nodes[mg].inputs[1]), weight_of(nodes[mu].inputs[1])
-            if res is None or wg.shape != wu.shape or wg.shape[1] % 32 or wd.dtype != wg.dtype:
+            if wg.shape != wu.shape or wg.shape[1] % 32 or wd.dtype != wg.dtype:
                 return False
             gamma, beta = get(n0.inputs[1]), get(n0.inputs[2])
-            rv = vals[res]
-            emit(g.step_rmsnorm_geglu_matmul, wg.buf, wu.buf, wd.buf, x.buf, gamma.buf, n0.attrs["eps"], rv.buf, beta=1.0, beta_norm=beta.buf)
-            vals[nodes[add].output] = _Val("dev", rv.buf, rv.shape, "f32", owned=True)
-            skip.update((mg, mu, un, mul, md, add))
+            if res is not None:
+                rv = vals[res]
+                emit(g.step_rmsnorm_geglu_matmul, wg.buf, wu.buf, wd.buf, x.buf, gamma.buf, n0.attrs["eps"], rv.buf, beta=1.0, beta_norm=beta.buf)
+                vals[nodes[add].output] = _Val("dev", rv.buf, rv.shape, "f32", owned=True)
+                skip.update((mg, mu, un, mul, md, add))
+            else:                                   # the down projection feeds something else (a norm): a buffer of its own
+                oshape = pkg.shape_of(nodes[md].output, sym)
+                out = new(oshape, "f32")
+                emit(g.step_rmsnorm_geglu_matmul, wg.buf, wu.buf, wd.buf, x.buf, gamma.buf, n0.attrs["eps"], out, beta=0.0, beta_norm=beta.buf)
+                vals[nodes[md].output] = _Val("dev", out, oshape, "f32", owned=True)
+                skip.update((mg, mu, un, mul, md))
             return True
 
         def matmul_into(out_vid, launch):
@@ -484,6 +491,15 @@ class PackageRunner:
                     for m, o in zip(mms, outs):
                         vals[nodes[m].output] = _Val("dev", o, pkg.shape_of(nodes[m].output, sym), "f32", owned=True)
                     skip.update(mms)
+                    continue
+                add = sole_user(n.output, "ElemwiseBinary") if self.fuse else None
+                res = residual_of(add, n.output) if add is not None else None
+                if res is not None and vals[res].buf is not x.buf:
+                    # add(residual, norm(x)): the norm step's own residual operand, summed in place (the same two roundings)
+                    rv = vals[res]
+                    emit(g.step_rmsnorm, rv.buf, x.buf, gamma.buf, rows, cols, a["eps"], beta=beta.buf, residual=rv.buf)
+                    vals[nodes[add].output] = _Val("dev", rv.buf, rv.shape, "f32", owned=True)
+                    skip.add(add)
                     continue
                 out = new(shape, "f32")
                 emit(g.step_rmsnorm, out, x.buf, gamma.buf, rows, cols, a["eps"], beta=beta.buf)

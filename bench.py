@@ -15,7 +15,7 @@ cpu_baseline = the oracle's restatement of the aion CPU kernel for this op (pack
 M=1, aion cpu/exec/matmul.zig) timed on this host's cores on a bounded sample.
 
 `--sweep` adds the q8 legs and batch 4 / 8 (per-shape kernel GB/s) in a "sweep" object.
-`--extras gemm,attention,decoder[,decoder_eager,package]` adds the other BASELINE configs (prefill GEMM TFLOP/s, attention
+`--extras gemm,attention,decoder[,decoder_eager,package,package_bench_shape]` adds the other BASELINE configs (prefill GEMM TFLOP/s, attention
 TFLOP/s and GB/s, end-to-end decode tokens/s of the synthetic 26-layer decoder) in an "extras"
 object of the same JSON line.
 """
@@ -201,6 +201,8 @@ def main():
             out["extras"]["decoder_eager"] = run_decoder_eager(gpu, be)
         if "package" in extras:
             out["extras"]["package"] = run_package(gpu, be)
+        if "package_bench_shape" in extras:
+            out["extras"]["package_bench_shape"] = run_package_bench_shape(gpu, be)
 
     out["config"]["setup_s"] = round(setup_s, 1)
     print(json.dumps(out))
@@ -392,6 +394,59 @@ def run_package(gpu, be):
            "program_nodes": int(gpu.program_node_count(run.program)),
            "prefill_128_ms": round(prefill_ms, 3), "decode_tokens_per_s": round(127 / decode_s, 1),
            "decode_ms_per_token": round(decode_s / 127 * 1e3, 4)}
+    run.close()
+    return res
+
+
+def run_package_bench_shape(gpu, be):
+    """A package with the block structure of aion's own bench model (src/bench/models.zig:433-536: tied row-quantized
+    q8_0 table, scaled embedding, per-head q/k/v norms, norms on the block outputs, local layers on 512-row rings beside
+    every fifth layer global, soft-capped logits) at BASELINE config 5's sizes, through the package runner. Random
+    weights; the arithmetic is checked on a small instance of the same writer in the GPU tests."""
+    from aion_amd import aion_file
+    from aion_amd.decoder import DecoderConfig, SyntheticWeights
+    from aion_amd.package import PackageRunner
+    from oracle import aion_writer                       # test infrastructure: only used to make the input file
+    cfg = DecoderConfig()
+    weights = SyntheticWeights(cfg, 0)
+    d = dict(layers=cfg.layers, hidden=cfg.hidden, heads=cfg.heads, kv_heads=cfg.kv_heads, head_dim=cfg.head_dim, ffn=cfg.ffn,
+             vocab=cfg.vocab, eps=cfg.eps, rope_base_local=10000.0, rope_base_global=1000000.0, local_window=512, global_every=5,
+             logit_softcap=30.0, wdtype="q4_0")
+    rng = np.random.default_rng(11)
+    gammas = {}
+    for l in range(cfg.layers):
+        for n, width in (("norm_in", cfg.hidden), ("q_norm", cfg.head_dim), ("k_norm", cfg.head_dim), ("v_norm", cfg.head_dim),
+                         ("norm_attn", cfg.hidden), ("norm_ffn_in", cfg.hidden), ("norm_ffn", cfg.hidden)):
+            gammas["l%d.%s" % (l, n)] = ((0.35 if n in ("q_norm", "k_norm") else 1.0) * (1 + 0.1 * rng.standard_normal(width))).astype(np.float32)
+    gammas["norm_f"] = np.ones(cfg.hidden, np.float32)
+    t0 = time.time()
+    table = be.quantize_blocks(be.Q8_0, weights.embed(), 1)
+    data = aion_writer.build_sandwich_decoder_package(d, weights.blocks, table, gammas)
+    del table
+    t_write = time.time() - t0
+    pkg = aion_file.parse(data)
+    capacity, n_prompt, n_decode = 1024, 128, 511        # the 512-row rings wrap during the decode
+    run = PackageRunner(gpu, pkg, capacity=capacity)
+    prompt = rng.integers(0, cfg.vocab, n_prompt).astype(np.int32)
+    run.run(prompt); run.reset()                         # uploads the weights, builds the prompt's plan
+    gpu.sync()
+    t = time.perf_counter()
+    tok = int(run.run(prompt)["next_token"][0, -1])
+    prefill_ms = (time.perf_counter() - t) * 1e3
+    run.begin_decode(tok)
+    gpu.sync()
+    t = time.perf_counter()
+    for _ in range(n_decode):
+        tok = run.decode_step()
+    gpu.sync()
+    decode_s = time.perf_counter() - t
+    stream = sum(t_.data.nbytes for t_ in pkg.tensors if t_.quantized)
+    res = {"file_bytes": len(data), "nodes": len(pkg.nodes), "write_s": round(t_write, 1),
+           "steps_prefill_128": run.step_count(n_prompt), "steps_decode": run.step_count(1),
+           "program_nodes": int(gpu.program_node_count(run.program)), "prefill_128_ms": round(prefill_ms, 3),
+           "decode_tokens": n_decode, "decode_tokens_per_s": round(n_decode / decode_s, 1),
+           "decode_ms_per_token": round(decode_s / n_decode * 1e3, 4), "weight_bytes_per_token": int(stream),
+           "weight_GBps": round(stream * n_decode / decode_s / 1e9, 1)}
     run.close()
     return res
 

@@ -342,6 +342,11 @@ def test_bench_model_shaped_package_against_the_graph_oracle(gpu, orc):
             assert names.count("step_headnorm_rope_append") == cfg["layers"]
             assert not any(x in names for x in ("step_rope", "step_append_f16", "step_cast_f32_f16"))
             assert "step_headnorm_rope_append" not in [fn.__name__ for fn, _a, _k in plain.plans[s_len].steps]
+        # seven steps per block for a single token (norm + q/k/v, head norms + RoPE + append, attention, o, norm + residual,
+        # norm + GeGLU + down, norm + residual) and seven around the blocks
+        assert run.step_count(1) <= 7 * cfg["layers"] + 7
+        residual_norms = [k for fn, _a, k in run.plans[1].steps if fn.__name__ == "step_rmsnorm" and k.get("residual") is not None]
+        assert len(residual_norms) == 2 * cfg["layers"]
         with pytest.raises(ValueError):
             run.run(np.zeros(30, np.int32))               # 63 retained + 30 new rows do not fit a 64-row ring
     finally:
