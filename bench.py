@@ -15,7 +15,7 @@ cpu_baseline = the oracle's restatement of the aion CPU kernel for this op (pack
 M=1, aion cpu/exec/matmul.zig) timed on this host's cores on a bounded sample.
 
 `--sweep` adds the q8 legs and batch 4 / 8 (per-shape kernel GB/s) in a "sweep" object.
-`--extras gemm,attention,decoder[,decoder_eager,package,package_bench_shape]` adds the other BASELINE configs (prefill GEMM TFLOP/s, attention
+`--extras gemm,attention,decoder[,decoder_eager,package,package_bench_shape,package_bench_shape_eager]` adds the other BASELINE configs (prefill GEMM TFLOP/s, attention
 TFLOP/s and GB/s, end-to-end decode tokens/s of the synthetic 26-layer decoder) in an "extras"
 object of the same JSON line.
 """
@@ -203,6 +203,8 @@ def main():
             out["extras"]["package"] = run_package(gpu, be)
         if "package_bench_shape" in extras:
             out["extras"]["package_bench_shape"] = run_package_bench_shape(gpu, be)
+        if "package_bench_shape_eager" in extras:
+            out["extras"]["package_bench_shape_eager"] = run_package_bench_shape(gpu, be, eager=True)
 
     out["config"]["setup_s"] = round(setup_s, 1)
     print(json.dumps(out))
@@ -398,8 +400,9 @@ def run_package(gpu, be):
     return res
 
 
-def run_package_bench_shape(gpu, be):
-    """A package with the block structure of aion's own bench model (src/bench/models.zig:433-536: tied row-quantized
+def run_package_bench_shape(gpu, be, eager=False):
+    """eager: the single-token steps are issued launch by launch (no program replay), the form a kernel trace can
+    attribute per kernel. A package with the block structure of aion's own bench model (src/bench/models.zig:433-536: tied row-quantized
     q8_0 table, scaled embedding, per-head q/k/v norms, norms on the block outputs, local layers on 512-row rings beside
     every fifth layer global, soft-capped logits) at BASELINE config 5's sizes, through the package runner. Random
     weights; the arithmetic is checked on a small instance of the same writer in the GPU tests."""
@@ -433,6 +436,15 @@ def run_package_bench_shape(gpu, be):
     t = time.perf_counter()
     tok = int(run.run(prompt)["next_token"][0, -1])
     prefill_ms = (time.perf_counter() - t) * 1e3
+    if eager:
+        gpu.sync()
+        t = time.perf_counter()
+        for _ in range(32):
+            tok = int(run.run(np.array([tok], np.int32))["next_token"][0, -1])
+        gpu.sync()
+        res = {"steps_decode": run.step_count(1), "eager_tokens": 32, "eager_ms_per_token": round((time.perf_counter() - t) / 32 * 1e3, 4)}
+        run.close()
+        return res
     run.begin_decode(tok)
     gpu.sync()
     t = time.perf_counter()

@@ -8,9 +8,10 @@ from aion_amd import hip
 pytestmark = pytest.mark.gpu
 
 
-def test_rmsnorm_with_and_without_residual(gpu, orc):
+@pytest.mark.parametrize("rows,cols", [(5, 2048), (1, 2048), (3, 7), (2, 100), (4, 256), (2, 2049), (3, 4096)])
+def test_rmsnorm_with_and_without_residual(gpu, orc, rows, cols):
+    """Rows of up to 2048 columns run on the kernel that holds the row in registers, longer ones on the two-pass one."""
     rng = np.random.default_rng(1)
-    rows, cols = 5, 2048
     x = rng.standard_normal((rows, cols)).astype(np.float32)
     g = rng.standard_normal(cols).astype(np.float32)
     bt = rng.standard_normal(cols).astype(np.float32)
@@ -21,6 +22,10 @@ def test_rmsnorm_with_and_without_residual(gpu, orc):
     assert np.allclose(gpu.download(out, np.float32, x.shape), orc.rmsnorm(x, g, 1e-6), rtol=1e-5, atol=1e-5)
     gpu.step_rmsnorm(out, xb, gb, rows, cols, 1e-6, beta=bb, residual=rb)
     assert np.allclose(gpu.download(out, np.float32, x.shape), orc.rmsnorm(x, g, 1e-6, beta=bt, residual=r), rtol=1e-5, atol=1e-5)  # three-term sum: fused multiply-add vs separate rounding
+    want = orc.rmsnorm(x, g, 1e-6, beta=bt, residual=r)
+    gpu.step_rmsnorm(rb, xb, gb, rows, cols, 1e-6, beta=bb, residual=rb)          # summed into the residual in place
+    assert np.array_equal(gpu.download(rb, np.float32, x.shape), gpu.download(out, np.float32, x.shape))
+    assert np.allclose(gpu.download(rb, np.float32, x.shape), want, rtol=1e-5, atol=1e-5)
     with pytest.raises(be.AionHipError) as e:
         gpu.step_rmsnorm(out, xb, gb, rows, cols, 0.0)
     assert e.value.status == hip.INVALID_ARGUMENT
