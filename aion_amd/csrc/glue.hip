@@ -157,12 +157,20 @@ __global__ __launch_bounds__(256) void headnorm_rope_append_kernel(
     const int pos = positions[tok];
     const int widx = write_index[tok / s_len];
     constexpr int MAXP = 4;                                                // pairs per lane: head sizes up to 512
-    float xl[MAXP], xh[MAXP];
+    // everything the second half needs is requested here, at clamped addresses without branches, so that the launch is one
+    // memory round trip: the row, gamma, beta and the rotation frequencies
+    float xl[MAXP], xh[MAXP], gl[MAXP], gh[MAXP], bl[MAXP], bh[MAXP], fr[MAXP];
+    const float *bsrc = beta ? beta : gamma;
 #pragma unroll
     for (int u = 0; u < MAXP; ++u) {
-        const int i = lane + 64 * u;
-        xl[u] = i < half ? src[i] : 0.f;
-        xh[u] = i < half ? src[half + i] : 0.f;
+        const int i = min(lane + 64 * u, half - 1);
+        xl[u] = src[i];
+        xh[u] = src[half + i];
+        gl[u] = gamma[i];
+        gh[u] = gamma[half + i];
+        bl[u] = bsrc[i];
+        bh[u] = bsrc[half + i];
+        fr[u] = freq[rope_pairs > 0 ? min(i, rope_pairs - 1) : 0];
     }
     // the sum of squares in rmsnorm_kernel's order (thread c of 256 adds x[c]^2, x[c + 256]^2; four wavefront sums; their
     // pairwise sum), so that the fused step gives the bits of the separate ones: the row is read a second time, from L1
@@ -186,11 +194,11 @@ __global__ __launch_bounds__(256) void headnorm_rope_append_kernel(
     for (int u = 0; u < MAXP; ++u) {
         const int i = lane + 64 * u;
         if (i >= half) break;
-        float yl = (xl[u] * inv) * gamma[i] + (beta ? beta[i] : 0.f);
-        float yh = (xh[u] * inv) * gamma[half + i] + (beta ? beta[half + i] : 0.f);
+        float yl = (xl[u] * inv) * gl[u] + (beta ? bl[u] : 0.f);
+        float yh = (xh[u] * inv) * gh[u] + (beta ? bh[u] : 0.f);
         if (kind != 2 && i < rope_pairs) {
             float sn, cs;
-            sincosf((float)pos * freq[i], &sn, &cs);
+            sincosf((float)pos * fr[u], &sn, &cs);
             rope_rotate(yl, yh, sn, cs, yl, yh);
         }
         if (kind == 0) {
