@@ -200,6 +200,8 @@ int launch_gemm_i8(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, Prepared
 // bf16 mode only: whether the bf16 MFMA kernel is expected to be the faster one for m rows against an n x k weight
 bool gemm_bf16_pays(const aionhip_ctx *ctx, size_t m, size_t n, size_t k);
 // the LDS-staged MFMA kernel for a handful of rows (no profile scope of its own: the caller's name stays)
+int launch_gemm_i8_batch(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count, size_t m,
+                         PreparedAct act, float alpha, float beta);
 int launch_gemm_i8_few_rows(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta);
 int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, const float *a, size_t lda, float *c, size_t ldc, float alpha, float beta);
 

@@ -29,15 +29,23 @@ using bf16x8 = __attribute__((ext_vector_type(8))) __bf16;
 // KC = quant blocks per K step: 4 when the grid fills the device (two workgroups per CU hide each other's
 // staging), 8 when it does not (few activation rows: fewer, larger steps - a step then costs one memory
 // latency however little it loads).
+// up to four weights with the same K and block format against one prepared activation: column tiles first_tile[i] .. of weight i
+struct GemmSegs {
+    const uint8_t *qs[4];
+    const __half *sc[4];
+    float *c[4];
+    size_t ldc[4];
+    int n[4], first_tile[4];
+    int count;
+};
 template <int KC> struct GiCfg { static constexpr int ROW = KC * 32 + 16; };   // staged code row; +16 B: conflict-free 8-byte operand reads
 // SPLITK (few activation rows, where the tiles above would leave most CUs idle): the workgroup tile shrinks
 // to (16*WM) x 64 and its four wavefronts share it, each taking every fourth quant block of a K step; their
 // partial sums are added in wavefront order through LDS at the end, so the result does not depend on timing.
 template <int DT, int WM, int KC, bool SPLITK>
-__global__ __launch_bounds__(256, KC == 4 || SPLITK ? 2 : 1) void gemm_i8_lds_kernel(const uint8_t *__restrict__ qs, const __half *__restrict__ sc,
+__global__ __launch_bounds__(256, KC == 4 || SPLITK ? 2 : 1) void gemm_i8_lds_kernel(GemmSegs segs,
                                                           const int8_t *__restrict__ aq, const float *__restrict__ a_scale,
-                                                          float *__restrict__ c, int M, int N, int K, size_t ldc,
-                                                          float alpha, float beta) {
+                                                          int M, int K, float alpha, float beta) {
     constexpr bool Q8 = DT == AIONHIP_Q8_0;
     static_assert(!SPLITK || KC == 8, "split K: two blocks per wavefront per step");
     constexpr int BM3 = (SPLITK ? 16 : 32) * WM, BN3 = SPLITK ? 64 : 128, ROW = GiCfg<KC>::ROW;
@@ -48,7 +56,17 @@ __global__ __launch_bounds__(256, KC == 4 || SPLITK ? 2 : 1) void gemm_i8_lds_ke
     extern __shared__ __attribute__((aligned(16))) unsigned char lds3[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, g = lane >> 4;
-    const int m0 = blockIdx.y * BM3, n0 = blockIdx.x * BN3;
+    // the weight this column tile belongs to (sibling weights over one activation share a launch)
+    int si = 0;
+#pragma unroll
+    for (int i = 1; i < 4; ++i)
+        if (i < segs.count && (int)blockIdx.x >= segs.first_tile[i]) si = i;
+    const uint8_t *__restrict__ qs = segs.qs[si];
+    const __half *__restrict__ sc = segs.sc[si];
+    float *__restrict__ c = segs.c[si];
+    const int N = segs.n[si];
+    const size_t ldc = segs.ldc[si];
+    const int m0 = blockIdx.y * BM3, n0 = ((int)blockIdx.x - segs.first_tile[si]) * BN3;
     const int wm0 = SPLITK ? 0 : (wave >> 1) * (16 * WM), wn0 = SPLITK ? 0 : (wave & 1) * 64;
     const int jw = SPLITK ? wave : 0, jstep = SPLITK ? 4 : 1;     // this wavefront's blocks: jw + jstep * jj
     const int KB = K >> 5, KT = (KB + KC - 1) / KC;
@@ -464,7 +482,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const unsigned shor
 }
 
 template <int DT, int WM, int KC, bool SPLITK>
-int launch_i8_lds(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
+int launch_i8_lds(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count, size_t m, PreparedAct act,
+                  float alpha, float beta) {
     constexpr int BM3 = (SPLITK ? 16 : 32) * WM, BN3 = SPLITK ? 64 : 128;
     constexpr int LDS = 2 * ((BM3 + BN3) * GiCfg<KC>::ROW + (BM3 + BN3) * KC * 4);
     static_assert(LDS <= 160 * 1024, "two stages must fit the CU's LDS");
@@ -474,8 +493,20 @@ int launch_i8_lds(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedA
         HIP_TRY(ctx, hipFuncSetAttribute((const void *)gemm_i8_lds_kernel<DT, WM, KC, SPLITK>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
         attr = true;
     }
-    const dim3 grid((unsigned)((w->n + BN3 - 1) / BN3), (unsigned)((m + BM3 - 1) / BM3));
-    launch_k(ctx, gemm_i8_lds_kernel<DT, WM, KC, SPLITK>, grid, dim3(256), LDS, w->qs, w->sc, act.q, act.scale, c, (int)m, (int)w->n, (int)w->k, ldc, alpha, beta);
+    GemmSegs segs{};
+    segs.count = count;
+    int tiles = 0;
+    for (int i = 0; i < count; ++i) {
+        segs.qs[i] = ws[i]->qs;
+        segs.sc[i] = ws[i]->sc;
+        segs.c[i] = cs[i];
+        segs.ldc[i] = ldcs[i];
+        segs.n[i] = (int)ws[i]->n;
+        segs.first_tile[i] = tiles;
+        tiles += (int)((ws[i]->n + BN3 - 1) / BN3);
+    }
+    const dim3 grid((unsigned)tiles, (unsigned)((m + BM3 - 1) / BM3));
+    launch_k(ctx, gemm_i8_lds_kernel<DT, WM, KC, SPLITK>, grid, dim3(256), LDS, segs, act.q, act.scale, (int)m, (int)ws[0]->k, alpha, beta);
     return AIONHIP_OK;
 }
 
@@ -504,16 +535,20 @@ int pick_i8_shape(const aionhip_ctx *ctx, size_t m, size_t n, size_t k, float *u
     if (us_per_block) *us_per_block = best_t;
     return best;
 }
+// the tile shape is chosen for the columns of all the weights together (their tiles share the launch)
 template <int DT>
-int launch_i8_lds_pick(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
-    const int best = pick_i8_shape(ctx, m, w->n, w->k, nullptr);
+int launch_i8_lds_pick(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count, size_t m,
+                       PreparedAct act, float alpha, float beta) {
+    size_t n_total = 0;
+    for (int i = 0; i < count; ++i) n_total += ws[i]->n;
+    const int best = pick_i8_shape(ctx, m, n_total, ws[0]->k, nullptr);
     switch (best) {
-    case 0: return launch_i8_lds<DT, 4, 4, false>(ctx, w, m, act, c, ldc, alpha, beta);
-    case 1: return launch_i8_lds<DT, 2, 4, false>(ctx, w, m, act, c, ldc, alpha, beta);
-    case 2: return launch_i8_lds<DT, 1, 4, false>(ctx, w, m, act, c, ldc, alpha, beta);
-    case 3: return launch_i8_lds<DT, 4, 8, true>(ctx, w, m, act, c, ldc, alpha, beta);
-    case 4: return launch_i8_lds<DT, 2, 8, true>(ctx, w, m, act, c, ldc, alpha, beta);
-    default: return launch_i8_lds<DT, 1, 8, true>(ctx, w, m, act, c, ldc, alpha, beta);
+    case 0: return launch_i8_lds<DT, 4, 4, false>(ctx, ws, cs, ldcs, count, m, act, alpha, beta);
+    case 1: return launch_i8_lds<DT, 2, 4, false>(ctx, ws, cs, ldcs, count, m, act, alpha, beta);
+    case 2: return launch_i8_lds<DT, 1, 4, false>(ctx, ws, cs, ldcs, count, m, act, alpha, beta);
+    case 3: return launch_i8_lds<DT, 4, 8, true>(ctx, ws, cs, ldcs, count, m, act, alpha, beta);
+    case 4: return launch_i8_lds<DT, 2, 8, true>(ctx, ws, cs, ldcs, count, m, act, alpha, beta);
+    default: return launch_i8_lds<DT, 1, 8, true>(ctx, ws, cs, ldcs, count, m, act, alpha, beta);
     }
 }
 
@@ -536,8 +571,21 @@ bool gemm_bf16_pays(const aionhip_ctx *ctx, size_t m, size_t n, size_t k) {
 }
 
 int launch_gemm_i8_few_rows(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {
-    return w->dtype == AIONHIP_Q8_0 ? launch_i8_lds_pick<AIONHIP_Q8_0>(ctx, w, m, act, c, ldc, alpha, beta)
-                                    : launch_i8_lds_pick<AIONHIP_Q4_0>(ctx, w, m, act, c, ldc, alpha, beta);
+    return w->dtype == AIONHIP_Q8_0 ? launch_i8_lds_pick<AIONHIP_Q8_0>(ctx, &w, &c, &ldc, 1, m, act, alpha, beta)
+                                    : launch_i8_lds_pick<AIONHIP_Q4_0>(ctx, &w, &c, &ldc, 1, m, act, alpha, beta);
+}
+
+// 1..4 weights of one dtype, layout and K against the same prepared rows, one launch
+int launch_gemm_i8_batch(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count, size_t m,
+                         PreparedAct act, float alpha, float beta) {
+    if (count < 1 || count > 4) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "gemm: %d weights in one launch (1..4)", count);
+    const char *name = ws[0]->dtype == AIONHIP_Q8_0 ? "gemm_i8_q8" : "gemm_i8_q4";
+    ProfScope scope(ctx, name);
+    const int rc = ws[0]->dtype == AIONHIP_Q8_0 ? launch_i8_lds_pick<AIONHIP_Q8_0>(ctx, ws, cs, ldcs, count, m, act, alpha, beta)
+                                                 : launch_i8_lds_pick<AIONHIP_Q4_0>(ctx, ws, cs, ldcs, count, m, act, alpha, beta);
+    if (rc) return rc;
+    LAUNCH_CHECK(ctx, name);
+    return AIONHIP_OK;
 }
 
 int launch_gemm_i8(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta) {

@@ -65,8 +65,10 @@ int run_rows(aionhip_ctx *ctx, const Batch &b, size_t m, const float *a, size_t 
     rc = launch_prepare_act(ctx, a, lda, m, b.k, act);
     if (rc) return rc;
     if (m <= GEMV_MAX_M) return launch_gemv_batch(ctx, b.w, b.c, b.ldc, (int)b.count, (int)m, act, alpha, beta);
-    for (size_t i = 0; i < b.count; ++i) {
-        rc = launch_gemm_i8(ctx, b.w[i], m, act, b.c[i], b.ldc[i], alpha, beta);
+    // sibling weights (q/k/v, gate/up) share one launch, four at a time
+    for (size_t i = 0; i < b.count; i += 4) {
+        const size_t cnt = b.count - i < 4 ? b.count - i : 4;
+        rc = launch_gemm_i8_batch(ctx, b.w + i, b.c + i, b.ldc + i, (int)cnt, m, act, alpha, beta);
         if (rc) return rc;
     }
     return AIONHIP_OK;

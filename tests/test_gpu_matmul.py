@@ -192,6 +192,34 @@ def test_single_row_long_k(gpu, orc, dtype, layout, n, k, kernel):
     w.free()
 
 
+# Sibling weights over one activation (q/k/v, gate/up) with more than eight rows: one launch of the exact GEMM whose
+# column tiles are dealt out to the weights in order. Column counts that do not fill a tile, one to four weights,
+# row counts around the tile heights, alpha/beta on pre-filled outputs - each output against the oracle.
+@pytest.mark.parametrize("dtype,layout", CASES)
+@pytest.mark.parametrize("m,ns,k", [(37, (200, 64, 70), 256), (128, (2048, 256, 256), 2048), (9, (130,), 544), (300, (520, 1000, 8, 129), 1056)])
+def test_sibling_weights_share_a_gemm_launch(gpu, orc, dtype, layout, m, ns, k):
+    say("sibling gemm", dtype, layout, m, ns, k)
+    made = [make_weight(gpu, orc, dtype, layout, n, k, seed=n + 7 * i, std=0.1) for i, n in enumerate(ns)]
+    rng = np.random.default_rng(m)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    c0 = [rng.standard_normal((m, n)).astype(np.float32) for n in ns]
+    a_buf = gpu.upload(a)
+    for alpha, beta in ((1.0, 0.0), (0.5, -2.0)):
+        c_bufs = [gpu.upload(c) for c in c0]
+        gpu.profile_start()
+        gpu.step_matmul_batch([w for _b, w in made], a_buf, m, c_bufs, alpha=alpha, beta=beta)
+        launches = [nm for nm, _ms in gpu.profile_stop() if nm.startswith("gemm_i8")]
+        assert len(launches) == 1
+        for (blocks, _w), cb, c, n in zip(made, c_bufs, c0, ns):
+            got = gpu.download(cb, np.float32, (m, n))
+            want = oracle_matmul(orc, dtype, layout, a, blocks, n, alpha=alpha, beta=beta, c=c)
+            assert norm_err(got, want) < TOL and rms_err(got, want) < RMS_TOL, (n, alpha)
+            cb.free()
+    a_buf.free()
+    for _b, w in made:
+        w.free()
+
+
 @pytest.mark.parametrize("dtype,layout", CASES)
 def test_exact_path_rows_above_eight(gpu, orc, dtype, layout):
     say("exact gemm", dtype, layout)
