@@ -18,9 +18,12 @@ namespace {
 
 // NCH = float4 activation chunks per thread (K <= 1024 * NCH). LDS is sized per launch:
 // K bytes of codes, K/32 scales, K/32 code sums, 4 reduction slots.
-template <int DT, int R, int PRO, int NCH, int EPI>
-__global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedIn in, int K, float alpha, float beta, FusedEpi epi) {
+// NT = threads per workgroup (K <= 4 * NT * NCH): 256, or more for the plain preparation - the wavefronts of a workgroup
+// share one preparation, and every workgroup reads the whole activation at the same moment.
+template <int DT, int R, int PRO, int NCH, int EPI, int NT = 256>
+__global__ __launch_bounds__(NT) void gemv_fused_kernel(GemvBatch batch, FusedIn in, int K, float alpha, float beta, FusedEpi epi) {
     static_assert(EPI == EPI_NONE || R == 8, "the epilogues own 4 + 4 rows per wavefront");
+    static_assert(NT == 256 || (PRO == PRO_QUANT && EPI == EPI_NONE), "wide workgroups: plain preparation only");
     extern __shared__ __attribute__((aligned(16))) unsigned char s_mem[];
     int *s_aq = (int *)s_mem;
     float *s_scale = (float *)(s_mem + K);
@@ -29,10 +32,10 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedI
     constexpr int MAX_CH4 = NCH;
 
     const int tid = threadIdx.x, lane = tid & 63;
-    const int wave_stride = gridDim.x * 4;
+    const int wave_stride = gridDim.x * (NT / 64);
     // the wavefront index is uniform: read through a scalar, the row-group bookkeeping and the
     // base addresses then stay in scalar registers
-    int gwave = blockIdx.x * (EPI == EPI_GATE_QUANT ? 8 : 4) + __builtin_amdgcn_readfirstlane(tid >> 6);
+    int gwave = blockIdx.x * (EPI == EPI_GATE_QUANT ? 8 : NT / 64) + __builtin_amdgcn_readfirstlane(tid >> 6);
     const int KB = K >> 5;
     constexpr bool Q8 = DT == AIONHIP_Q8_0;
     const int chunks = Q8 ? (K >> 4) : KB;
@@ -88,7 +91,7 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedI
     // every global operand of the prologue is requested up front: one memory latency, not three
 #pragma unroll
     for (int i = 0; i < MAX_CH4; ++i) {
-        const int c4 = tid + 256 * i;
+        const int c4 = tid + NT * i;
         const bool live = c4 < n4;
         v[i] = live ? *(const f32x4 *)(in.x + (size_t)c4 * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
         if (PRO == PRO_RMSNORM) {
@@ -123,7 +126,7 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(GemvBatch batch, FusedI
     }
 #pragma unroll
     for (int i = 0; i < MAX_CH4; ++i) {
-        const int c4 = tid + 256 * i;
+        const int c4 = tid + NT * i;
         const bool live = c4 < n4;
         f32x4 a = v[i];
         if (live) {
@@ -351,13 +354,25 @@ void launch_r(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *c
         waves += ((int)ws[i]->n + R - 1) / R;
     }
     batch.total_waves = waves;
-    // at most 8 workgroups per CU: beyond that the wavefronts stride over the row groups
-    const int wgs = (waves + 3) / 4;
-    const dim3 grid((unsigned)(wgs < cus * 8 ? wgs : cus * 8)), block(256);
     const size_t lds = (size_t)K + (size_t)(K >> 5) * 8 + 16;
-    if (R == 4) launch_k(ctx, gemv_fused_kernel<DT, 4, PRO, NCH, EPI_NONE>, grid, block, lds, batch, in, K, alpha, beta, FusedEpi{});
-    else if (R == 2) launch_k(ctx, gemv_fused_kernel<DT, 2, PRO, NCH, EPI_NONE>, grid, block, lds, batch, in, K, alpha, beta, FusedEpi{});
-    else launch_k(ctx, gemv_fused_kernel<DT, 1, PRO, NCH, EPI_NONE>, grid, block, lds, batch, in, K, alpha, beta, FusedEpi{});
+    if constexpr (PRO == PRO_QUANT) {
+        // The plain preparation runs in 1024-thread workgroups, the same 32 wavefronts per CU at most: a quarter of the
+        // workgroups re-read and re-quantize the activation, and fewer of them hit its few L2 lines at the same moment
+        // (q4, one row: 4096x4096 5.3 -> 4.6 us, 14336x4096 8.7 -> 7.8 us, 262144x2048 47 -> 45.8 us).
+        constexpr int WNT = 1024, WNCH = (NCH * 256 + WNT - 1) / WNT;
+        const int wg = (waves + WNT / 64 - 1) / (WNT / 64), cap = cus * 32 / (WNT / 64);
+        const dim3 wgrid((unsigned)(wg < cap ? wg : cap)), wblock(WNT);
+        if (R == 4) launch_k(ctx, gemv_fused_kernel<DT, 4, PRO_QUANT, WNCH, EPI_NONE, WNT>, wgrid, wblock, lds, batch, in, K, alpha, beta, FusedEpi{});
+        else if (R == 2) launch_k(ctx, gemv_fused_kernel<DT, 2, PRO_QUANT, WNCH, EPI_NONE, WNT>, wgrid, wblock, lds, batch, in, K, alpha, beta, FusedEpi{});
+        else launch_k(ctx, gemv_fused_kernel<DT, 1, PRO_QUANT, WNCH, EPI_NONE, WNT>, wgrid, wblock, lds, batch, in, K, alpha, beta, FusedEpi{});
+    } else {
+        // at most 8 workgroups per CU: beyond that the wavefronts stride over the row groups
+        const int wgs = (waves + 3) / 4;
+        const dim3 grid((unsigned)(wgs < cus * 8 ? wgs : cus * 8)), block(256);
+        if (R == 4) launch_k(ctx, gemv_fused_kernel<DT, 4, PRO, NCH, EPI_NONE>, grid, block, lds, batch, in, K, alpha, beta, FusedEpi{});
+        else if (R == 2) launch_k(ctx, gemv_fused_kernel<DT, 2, PRO, NCH, EPI_NONE>, grid, block, lds, batch, in, K, alpha, beta, FusedEpi{});
+        else launch_k(ctx, gemv_fused_kernel<DT, 1, PRO, NCH, EPI_NONE>, grid, block, lds, batch, in, K, alpha, beta, FusedEpi{});
+    }
 }
 
 template <int DT, int PRO>
