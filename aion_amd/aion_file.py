@@ -218,11 +218,12 @@ def _window(c):
 
 
 def _strings(buf):
-    """parse.zig:272-284."""
+    """parse.zig:272-284. aion keeps strings as raw bytes without validating them; bytes that are not UTF-8 survive here
+    as surrogate escapes (`s.encode("utf-8", "surrogateescape")` gives them back) instead of failing the parse."""
     c = _Cursor(buf, "strings")
     out = []
     for _ in range(c.u32()):
-        out.append(bytes(c.take(c.u32())).decode("utf-8"))
+        out.append(bytes(c.take(c.u32())).decode("utf-8", "surrogateescape"))
     c.done()
     return out
 

@@ -71,6 +71,11 @@ class Weight:
         self.backend._check(self.backend._lib.aionhip_weight_download(self.backend._ctx, self.ptr, out.ctypes.data, out.nbytes))
         return out
 
+    def drop_bf16(self):
+        """Releases the bf16 copy the bf16 GEMM mode keeps of this weight (rebuilt on its next bf16 call)."""
+        if self.ptr:
+            self.backend._lib.aionhip_weight_drop_bf16(self.backend._ctx, self.ptr)
+
     def free(self):
         if self.ptr:
             self.backend._lib.aionhip_weight_free(self.backend._ctx, self.ptr)
@@ -215,6 +220,20 @@ class HipBackend:
         p = C.c_void_p()
         self._check(self._lib.aionhip_program_end(self._ctx, C.byref(p)))
         return p
+
+    def program_abort(self):
+        self._check(self._lib.aionhip_program_abort(self._ctx))
+
+    def record_program(self, issue):
+        """Records the steps `issue()` makes into a program. If a step raises, the recording is dropped (the context is
+        left executing eagerly, not stuck in capture) and the error propagates."""
+        self.program_begin()
+        try:
+            issue()
+        except BaseException:
+            self._lib.aionhip_program_abort(self._ctx)
+            raise
+        return self.program_end()
 
     def program_execute(self, prog):
         self._check(self._lib.aionhip_program_execute(self._ctx, prog))

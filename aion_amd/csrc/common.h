@@ -219,7 +219,6 @@ constexpr int DPP_QUAD_XOR2 = 0x4E;     // quad_perm [2,3,0,1]
 constexpr int DPP_ROW_HALF_MIRROR = 0x141;
 constexpr int DPP_ROW_MIRROR = 0x140;
 
-// sum over the 64 lanes of a wavefront; every lane returns the total
 // The rotation of one RoPE pair with every product and the sum rounded on its own, as aion's CPU kernel computes it
 // (cpu/kernels/rope.zig:90-91, no fused multiply-add) - and so the same bits from every kernel that rotates.
 __device__ __forceinline__ void rope_rotate(float xl, float xh, float sn, float cs, float &yl, float &yh) {
@@ -228,6 +227,7 @@ __device__ __forceinline__ void rope_rotate(float xl, float xh, float sn, float 
     yh = xl * sn + xh * cs;
 }
 
+// sum over the 64 lanes of a wavefront; every lane returns the total
 __device__ __forceinline__ float wave_sum(float v) {
     v += dpp_f<DPP_QUAD_XOR1>(v);
     v += dpp_f<DPP_QUAD_XOR2>(v);
@@ -245,6 +245,35 @@ __device__ __forceinline__ float wave_max(float v) {
     v = fmaxf(v, __shfl_xor(v, 16, 64));
     v = fmaxf(v, __shfl_xor(v, 32, 64));
     return v;
+}
+
+// The int8 preparation of one 32-element activation block (aion cpu/kernels/matmul_q_i8.zig:187-203 quantizeABlock,
+// :227-264 prepareARow) held by 8 consecutive lanes, 4 values each: amax over the block; a zero block gives zero
+// codes and scale 0; else scale = amax / 127, inv = 127 / amax, code = clamp(round-half-away(v * inv), -127, 127).
+// Every lane of the 8 returns its four codes packed into `word`, the block scale and the plain sum of the 32 codes.
+// The one definition every kernel that prepares activations calls, so that they cannot drift apart.
+__device__ __forceinline__ void prepare_act_block8(float v0, float v1, float v2, float v3, int &word, float &scale, int &sum) {
+    float amax = fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3)));
+    amax = fmaxf(amax, dpp_f<DPP_QUAD_XOR1>(amax));
+    amax = fmaxf(amax, dpp_f<DPP_QUAD_XOR2>(amax));
+    amax = fmaxf(amax, dpp_f<DPP_ROW_HALF_MIRROR>(amax));
+    word = 0;
+    scale = 0.f;
+    int s = 0;
+    if (amax != 0.f) {
+        scale = amax / 127.f;
+        const float inv = 127.f / amax;
+        const int q0 = (int)fminf(127.f, fmaxf(-127.f, roundf(v0 * inv)));
+        const int q1 = (int)fminf(127.f, fmaxf(-127.f, roundf(v1 * inv)));
+        const int q2 = (int)fminf(127.f, fmaxf(-127.f, roundf(v2 * inv)));
+        const int q3 = (int)fminf(127.f, fmaxf(-127.f, roundf(v3 * inv)));
+        word = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
+        s = q0 + q1 + q2 + q3;
+    }
+    s += dpp_i<DPP_QUAD_XOR1>(s);
+    s += dpp_i<DPP_QUAD_XOR2>(s);
+    s += dpp_i<DPP_ROW_HALF_MIRROR>(s);
+    sum = s;
 }
 
 __device__ __forceinline__ int dot4_i8(int a, int b, int c) { return __builtin_amdgcn_sdot4(a, b, c, false); }

@@ -602,14 +602,24 @@ int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *cw, size_t m, const
     const size_t N = w->n, K = w->k;
     if ((((uintptr_t)a) & 3) != 0) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "gemm: A must be 4-byte aligned");
     if (!w->bf16) {
+        // The bf16 copy is built on first use and kept until aionhip_weight_drop_bf16 / aionhip_weight_free: N*K*2 bytes
+        // (about 4x a q4 weight). Not while a program is being recorded (it allocates), and the field is set only once
+        // the conversion launch has been accepted. A weight shared by several contexts must see its first bf16 call from
+        // one of them alone.
+        if (ctx->capturing)
+            return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "the bf16 copy of a weight must be built while a program is being recorded: run the steps once before recording");
         void *p = nullptr;
         HIP_TRY(ctx, hipMalloc(&p, N * K * 2));
-        w->bf16 = (unsigned short *)p;
         const size_t threads = N * (K / 8);
         const unsigned grid = (unsigned)((threads + 255) / 256);
-        if (w->dtype == AIONHIP_Q8_0) dequant_bf16_kernel<AIONHIP_Q8_0><<<dim3(grid), dim3(256), 0, ctx->stream>>>(w->qs, w->sc, w->bf16, N, K);
-        else dequant_bf16_kernel<AIONHIP_Q4_0><<<dim3(grid), dim3(256), 0, ctx->stream>>>(w->qs, w->sc, w->bf16, N, K);
-        LAUNCH_CHECK(ctx, "dequant_bf16");
+        if (w->dtype == AIONHIP_Q8_0) dequant_bf16_kernel<AIONHIP_Q8_0><<<dim3(grid), dim3(256), 0, ctx->stream>>>(w->qs, w->sc, (unsigned short *)p, N, K);
+        else dequant_bf16_kernel<AIONHIP_Q4_0><<<dim3(grid), dim3(256), 0, ctx->stream>>>(w->qs, w->sc, (unsigned short *)p, N, K);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) {
+            (void)hipFree(p);
+            return set_err(ctx, AIONHIP_EXECUTION_FAILED, "launch dequant_bf16: %s", hipGetErrorString(e));
+        }
+        w->bf16 = (unsigned short *)p;
     }
     int rc = ensure_scratch2(ctx, m * K * 2);
     if (rc) return rc;

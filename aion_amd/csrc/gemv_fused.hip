@@ -145,25 +145,9 @@ __global__ __launch_bounds__(NT) void gemv_fused_kernel(GemvBatch batch, FusedIn
             }
         }
         // 8 consecutive lanes share one 32-element block (c4 >> 3)
-        float amax = fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w)));
-        amax = fmaxf(amax, dpp_f<DPP_QUAD_XOR1>(amax));
-        amax = fmaxf(amax, dpp_f<DPP_QUAD_XOR2>(amax));
-        amax = fmaxf(amax, dpp_f<DPP_ROW_HALF_MIRROR>(amax));
-        int word = 0, s = 0;
-        float scale = 0.f;
-        if (amax != 0.f) {
-            scale = amax / 127.f;
-            const float inv = 127.f / amax;
-            const int q0 = (int)fminf(127.f, fmaxf(-127.f, roundf(a.x * inv)));
-            const int q1 = (int)fminf(127.f, fmaxf(-127.f, roundf(a.y * inv)));
-            const int q2 = (int)fminf(127.f, fmaxf(-127.f, roundf(a.z * inv)));
-            const int q3 = (int)fminf(127.f, fmaxf(-127.f, roundf(a.w * inv)));
-            word = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
-            s = q0 + q1 + q2 + q3;
-        }
-        s += dpp_i<DPP_QUAD_XOR1>(s);
-        s += dpp_i<DPP_QUAD_XOR2>(s);
-        s += dpp_i<DPP_ROW_HALF_MIRROR>(s);
+        int word, s;
+        float scale;
+        prepare_act_block8(a.x, a.y, a.z, a.w, word, scale, s);
         if (live) {
             s_aq[c4] = word;
             if ((c4 & 7) == 0) {
@@ -284,27 +268,11 @@ __global__ __launch_bounds__(NT) void gemv_fused_kernel(GemvBatch batch, FusedIn
             if ((gwave >> 2) & 1) {
                 __syncthreads();
                 if (tid < 8) {
-                    // the arithmetic of prepare_act_kernel (aion cpu/kernels/matmul_q_i8.zig:187-203), 8 lanes x 4 values
+                    // the shared block preparation (aion cpu/kernels/matmul_q_i8.zig:187-203), 8 lanes x 4 values
                     const float v0 = s_h[tid * 4], v1 = s_h[tid * 4 + 1], v2 = s_h[tid * 4 + 2], v3 = s_h[tid * 4 + 3];
-                    float amax = fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3)));
-                    amax = fmaxf(amax, dpp_f<DPP_QUAD_XOR1>(amax));
-                    amax = fmaxf(amax, dpp_f<DPP_QUAD_XOR2>(amax));
-                    amax = fmaxf(amax, dpp_f<DPP_ROW_HALF_MIRROR>(amax));
-                    int word = 0, sq = 0;
-                    float scale = 0.f;
-                    if (amax != 0.f) {
-                        scale = amax / 127.f;
-                        const float inv = 127.f / amax;
-                        const int q0 = (int)fminf(127.f, fmaxf(-127.f, roundf(v0 * inv)));
-                        const int q1 = (int)fminf(127.f, fmaxf(-127.f, roundf(v1 * inv)));
-                        const int q2 = (int)fminf(127.f, fmaxf(-127.f, roundf(v2 * inv)));
-                        const int q3 = (int)fminf(127.f, fmaxf(-127.f, roundf(v3 * inv)));
-                        word = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
-                        sq = q0 + q1 + q2 + q3;
-                    }
-                    sq += dpp_i<DPP_QUAD_XOR1>(sq);
-                    sq += dpp_i<DPP_QUAD_XOR2>(sq);
-                    sq += dpp_i<DPP_ROW_HALF_MIRROR>(sq);
+                    int word, sq;
+                    float scale;
+                    prepare_act_block8(v0, v1, v2, v3, word, scale, sq);
                     const int blk = gwave >> 3;                     // task = quant block of the down projection's activation
                     epi.act_q[blk * 8 + tid] = word;
                     if (tid == 0) {

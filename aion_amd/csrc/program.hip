@@ -61,6 +61,18 @@ int aionhip_program_end(aionhip_ctx *ctx, aionhip_program **out) {
     return AIONHIP_OK;
 }
 
+int aionhip_program_abort(aionhip_ctx *ctx) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (!ctx->capturing) return AIONHIP_OK;
+    ctx->capturing = false;
+    hipGraph_t graph = nullptr;
+    const hipError_t e = hipStreamEndCapture(ctx->stream, &graph);      // also when a step failed mid-recording
+    if (graph) (void)hipGraphDestroy(graph);
+    (void)hipGetLastError();                                            // an invalidated capture leaves a sticky error behind
+    if (e != hipSuccess && e != hipErrorStreamCaptureInvalidated) return set_err(ctx, AIONHIP_EXECUTION_FAILED, "hipStreamEndCapture: %s", hipGetErrorString(e));
+    return AIONHIP_OK;
+}
+
 int aionhip_program_execute(aionhip_ctx *ctx, aionhip_program *prog) {
     if (!ctx || !prog || !prog->exec) return AIONHIP_INVALID_ARGUMENT;
     if (ctx->capturing) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "program_execute: a recording is open");

@@ -131,25 +131,9 @@ __global__ __launch_bounds__(256) void prepare_act_kernel(const float *__restric
         v2 = aion_gate_gelu(v2, u[2]);
         v3 = aion_gate_gelu(v3, u[3]);
     }
-    float amax = fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3)));
-    amax = fmaxf(amax, dpp_f<DPP_QUAD_XOR1>(amax));
-    amax = fmaxf(amax, dpp_f<DPP_QUAD_XOR2>(amax));
-    amax = fmaxf(amax, dpp_f<DPP_ROW_HALF_MIRROR>(amax));
-    int word = 0, s = 0;
-    float scale = 0.f;
-    if (amax != 0.f) {
-        scale = amax / 127.f;
-        const float inv = 127.f / amax;
-        const int q0 = (int)fminf(127.f, fmaxf(-127.f, roundf(v0 * inv)));
-        const int q1 = (int)fminf(127.f, fmaxf(-127.f, roundf(v1 * inv)));
-        const int q2 = (int)fminf(127.f, fmaxf(-127.f, roundf(v2 * inv)));
-        const int q3 = (int)fminf(127.f, fmaxf(-127.f, roundf(v3 * inv)));
-        word = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
-        s = q0 + q1 + q2 + q3;
-    }
-    s += dpp_i<DPP_QUAD_XOR1>(s);
-    s += dpp_i<DPP_QUAD_XOR2>(s);
-    s += dpp_i<DPP_ROW_HALF_MIRROR>(s);
+    int word, s;
+    float scale;
+    prepare_act_block8(v0, v1, v2, v3, word, scale, s);
     if (live) {
         aq[(row * k + kb * QK) / 4 + sub] = word;
         if (sub == 0) {

@@ -186,6 +186,13 @@ void aionhip_weight_free(aionhip_ctx *ctx, aionhip_weight *w) {
     delete w;
 }
 
+void aionhip_weight_drop_bf16(aionhip_ctx *ctx, aionhip_weight *w) {
+    if (!w || !w->bf16) return;
+    if (ctx) (void)hipStreamSynchronize(ctx->stream);      // launches that read the copy may still be queued
+    (void)hipFree(w->bf16);
+    w->bf16 = nullptr;
+}
+
 size_t aionhip_weight_packed_bytes(const aionhip_weight *w) {
     if (!w) return 0;
     return w->n * (w->k / QK) * (w->dtype == AIONHIP_Q8_0 ? Q8_BYTES : Q4_BYTES);

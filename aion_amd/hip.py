@@ -48,6 +48,7 @@ _SIGS = {
     "aionhip_weight_upload": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p, C.POINTER(C.c_void_p)]),
     "aionhip_weight_from_device": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint64, C.POINTER(C.c_void_p)]),
     "aionhip_weight_free": (None, [C.c_void_p, C.c_void_p]),
+    "aionhip_weight_drop_bf16": (None, [C.c_void_p, C.c_void_p]),
     "aionhip_weight_packed_bytes": (C.c_size_t, [C.c_void_p]),
     "aionhip_weight_device_bytes": (C.c_size_t, [C.c_void_p]),
     "aionhip_weight_download": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
@@ -65,6 +66,7 @@ _SIGS = {
     "aionhip_step_add_i32": (C.c_int, [C.c_void_p] + [C.c_uint64] * 3 + [C.c_size_t]),
     "aionhip_program_begin": (C.c_int, [C.c_void_p]),
     "aionhip_program_end": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p)]),
+    "aionhip_program_abort": (C.c_int, [C.c_void_p]),
     "aionhip_program_execute": (C.c_int, [C.c_void_p, C.c_void_p]),
     "aionhip_program_node_count": (C.c_size_t, [C.c_void_p]),
     "aionhip_program_destroy": (None, [C.c_void_p, C.c_void_p]),

@@ -731,12 +731,13 @@ class PackageRunner:
             if self.one is None:
                 self.one = g.upload(np.ones(1, np.int32))
             tok_buf = plan.outputs[token_output][0]
-            g.program_begin()
-            self._issue(plan)
-            g._check(g._lib.aionhip_d2d(g._ctx, plan.inputs["tokens"][0].handle, 0, tok_buf.handle, 0, 4))
-            for kind in ("positions", "cache_write_index", "cache_visible_end"):
-                g.step_add_i32(plan.inputs[kind][0], plan.inputs[kind][0], self.one, 1)
-            self.program = g.program_end()
+
+            def issue():
+                self._issue(plan)
+                g._check(g._lib.aionhip_d2d(g._ctx, plan.inputs["tokens"][0].handle, 0, tok_buf.handle, 0, 4))
+                for kind in ("positions", "cache_write_index", "cache_visible_end"):
+                    g.step_add_i32(plan.inputs[kind][0], plan.inputs[kind][0], self.one, 1)
+            self.program = g.record_program(issue)
         self._token_output = token_output
 
     def decode_step(self, read_token=True):

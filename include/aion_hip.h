@@ -175,6 +175,11 @@ int aionhip_step_gate_matmul(aionhip_ctx *ctx, const aionhip_weight *b, size_t r
  * and exact). BF16_MFMA_ALWAYS: the bf16 kernel for every m > 8, whatever the shape. */
 typedef enum aionhip_gemm_mode { AIONHIP_GEMM_EXACT_I8 = 0, AIONHIP_GEMM_BF16_MFMA = 1, AIONHIP_GEMM_BF16_MFMA_ALWAYS = 2 } aionhip_gemm_mode;
 int aionhip_set_gemm_mode(aionhip_ctx *ctx, int mode);
+/* The bf16 kernel keeps a bf16 copy of every weight it has multiplied (n * k * 2 bytes - about four times a q4_0 weight -
+ * built on the first such call, never while a program is being recorded, released by aionhip_weight_free). This releases
+ * the copy of one weight early (it is rebuilt on the next bf16 call); aion's derived-weight reclamation
+ * (storage/derived.zig:1-17) is the counterpart. Waits for the context's stream. */
+void aionhip_weight_drop_bf16(aionhip_ctx *ctx, aionhip_weight *w);
 /* Name of the kernel the last matmul/attention step launched (the reference's tests assert
  * which kernel ran after a parity check, backend/gpu/test_gpu_backend.zig:1116-1162). */
 const char *aionhip_last_kernel(aionhip_ctx *ctx);
@@ -293,6 +298,9 @@ int aionhip_step_add_i32(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle a,
  * steps once eagerly first. Per-token inputs must live in device buffers the steps read. */
 int aionhip_program_begin(aionhip_ctx *ctx);
 int aionhip_program_end(aionhip_ctx *ctx, aionhip_program **out);
+/* Leaves a recording without a program (for a caller whose step failed between begin and end): the captured work is
+ * dropped and the context executes eagerly again. No-op when nothing is being recorded. */
+int aionhip_program_abort(aionhip_ctx *ctx);
 int aionhip_program_execute(aionhip_ctx *ctx, aionhip_program *prog);
 size_t aionhip_program_node_count(const aionhip_program *prog);
 void aionhip_program_destroy(aionhip_ctx *ctx, aionhip_program *prog);

@@ -169,3 +169,37 @@ def test_load_maps_the_file(tmp_path):
     table = pkg.tensors[pkg.values[pkg.nodes[0].inputs[0]].initializer]
     assert not table.data.flags.writeable
     assert np.array_equal(np.frombuffer(table.data, np.float32).reshape(embed.shape), embed)
+
+
+def test_byte_mutations_raise_only_package_errors():
+    # every mutated file either parses or is refused with PackageError - never another exception type (the string table is
+    # raw bytes in aion, parse.zig:272-284: bytes that are not UTF-8 must not fail the reader)
+    data, _ = make()
+    rng = np.random.default_rng(123)
+    # the structured part of the file: header, directory and every section but the bulk tensor payloads
+    n = struct.unpack_from("<I", data, 8)[0]
+    spans = [(0, 72 + n * 24)]
+    for i in range(n):
+        stype, _f, off, size = struct.unpack_from("<IIQQ", data, 72 + i * 24)
+        spans.append((off, min(size, 4096) if stype == 2 else size))
+    positions = np.concatenate([np.arange(o, o + s) for o, s in spans])
+    outcomes = {"ok": 0, "refused": 0}
+    for _ in range(3000):
+        m = bytearray(data)
+        for _k in range(int(rng.integers(1, 4))):
+            m[int(rng.choice(positions))] = int(rng.integers(0, 256))
+        try:
+            aion_file.parse(bytes(m))
+            outcomes["ok"] += 1
+        except aion_file.PackageError:
+            outcomes["refused"] += 1
+    assert outcomes["refused"] > 100 and outcomes["ok"] > 100, outcomes
+    # a string that is not UTF-8 survives as its bytes
+    sidx = [struct.unpack_from("<I", data, 72 + i * 24)[0] for i in range(n)].index(1)
+    soff = struct.unpack_from("<Q", data, 72 + sidx * 24 + 8)[0]
+    first_len = struct.unpack_from("<I", data, soff + 4)[0]
+    assert first_len > 0
+    m = bytearray(data)
+    m[soff + 8] = 0xFF
+    pkg = aion_file.parse(bytes(m))
+    assert pkg.strings[0].encode("utf-8", "surrogateescape") == bytes(m[soff + 8:soff + 8 + first_len])

@@ -77,9 +77,9 @@ def test_prefill_causal_gqa(gpu, orc, kind, tol, D, L, kernel):
 
 
 @pytest.mark.parametrize("kind,tol", [("f16", 2e-3), ("bf16", 1e-2)])
-@pytest.mark.parametrize("T,B", [(1024, 1), (4096, 8), (777, 3)])
+@pytest.mark.parametrize("T,B", [(1024, 1), (1024, 8), (4096, 1), (4096, 8), (16384, 1), (16384, 8), (777, 3)])
 def test_decode_split_k(gpu, orc, kind, tol, T, B):
-    # BASELINE config 4b shape family: 1 query token at position T-1, 8 q heads / 1 kv head, hd 256
+    # BASELINE config 4b, every (T, B) it names: 1 query token at position T-1, 8 q heads / 1 kv head, hd 256
     Hq, Hkv, D = 8, 1, 256
     say("decode", kind, T, B)
     (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(T + B, B, 1, T, Hq, Hkv, D, kind)

@@ -82,6 +82,14 @@ def test_device_quantizer_bytes_match_oracle(gpu, orc, dtype, axis):
     v[0:32, 0] = 0.0
     v[0, 0:32] = 0.0
     v.reshape(-1)[5] = 0.5            # large outlier
+    # a block whose codes depend on WHICH scale divides (q4: the f32 scale; q8: the f16-rounded one), by hand:
+    # max_abs = 7 * (1 + 2^-12) -> q4 codes 7, 2, -2, 0 for 2.5, -2.5, 0.5 (3, -3, 1 if the stored f16 scale 1.0 divided)
+    special = np.zeros(32, np.float32)
+    special[:4] = [7.0 + 7.0 / 4096.0, 2.5, -2.5, 0.5]
+    if axis == 0:
+        v[32:64, 3] = special
+    else:
+        v[3, 32:64] = special
     src = gpu.upload(v)
     dst = gpu.quantize_device(dtype, src, rows, cols, axis)
     got = gpu.download(dst, np.uint8)

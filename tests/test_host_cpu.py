@@ -46,6 +46,15 @@ def test_host_quantizer_reference_test_vector(orc):
     assert np.array_equal(got, orc.quantize(orc.Q8_0, vals.reshape(64, 5), 0))
 
 
+def test_host_q4_quantizer_divides_by_the_unrounded_scale():
+    # the hand-computed block of test_oracle_quant.py (max_abs = 7 * (1 + 2^-12): stored scale f16 1.0, codes from the f32 scale)
+    v = np.zeros((1, 32), np.float32)
+    v[0, :4] = [7.0 + 7.0 / 4096.0, 2.5, -2.5, 0.5]
+    want = bytes([0x00, 0x3C, 15 | (10 << 4), 6 | (8 << 4)] + [0x88] * 14)
+    assert be.quantize_blocks(be.Q4_0, v, 1).tobytes() == want
+    assert be.quantize_blocks(be.Q4_0, np.ascontiguousarray(v.T), 0).tobytes() == want
+
+
 def test_host_quantizer_chunked_calls_equal_whole():
     # api/context.zig:443-489 quantizes 16 MiB at a time through first_elem/first_block
     lib = hip.load_library()

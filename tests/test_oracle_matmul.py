@@ -171,3 +171,23 @@ def test_activation_quant_noise_floor_vs_f32a(orc):
     f32a = orc.matmul_q_f32a(orc.Q8_0, True, a, blocks, n)
     nmse = float(((i8 - f32a) ** 2).sum() / (f32a ** 2).sum())
     assert 1e-6 < nmse < 2e-4
+
+
+def test_prepare_a_hand_computed_ties_and_special_blocks(orc):
+    # aion cpu/kernels/matmul_q_i8.zig:187-203 on blocks whose codes follow by hand: exact ties (Zig @round is half away
+    # from zero), amax on a negative element, 127 / amax (not 1 / (amax / 127)), a zero block, a denormal amax whose
+    # inverse overflows (every nonzero element then clamps to +-127)
+    import act_cases as ac
+    a = np.concatenate([np.array(ac.TIE_BLOCK, np.float32), np.array(ac.HALF_BLOCK, np.float32),
+                        ac.block_kinds(np.random.default_rng(0))[3], np.zeros(32, np.float32),
+                        ac.block_kinds(np.random.default_rng(0))[4]]).reshape(1, -1)
+    aq, sc, sm = orc.prepare_a(a)
+    aq = aq.reshape(5, 32)
+    assert aq[0].tolist() == ac.TIE_CODES and sc[0, 0] == np.float32(1.0)
+    half = [-127] + [(k + 1) * (1 if k % 2 else -1) for k in range(31)]          # (2k+1)/2 -> k+1, sign kept
+    assert aq[1].tolist() == half and sc[0, 1] == np.float32(2.0)
+    assert aq[2, :len(ac.INV_CODES)].tolist() == ac.INV_CODES
+    assert not aq[3].any() and sc[0, 3] == 0.0
+    assert aq[4].tolist() == [127 * (-1 if t % 2 else 1) for t in range(32)]
+    assert sc[0, 4] == np.float32(5e-40) / np.float32(127) and sc[0, 4] > 0
+    assert sm[0].tolist() == aq.astype(np.int64).sum(axis=1).tolist()

@@ -132,6 +132,27 @@ def test_quantize_special_cases(orc):
     assert list(codes[:6]) == [7, 1, -1, 2, 3, -3]
 
 
+def test_q4_divides_by_the_unrounded_scale_hand_computed_block(orc):
+    # aion cpu/test_cpu_kernels.zig:490-523: q = round(v / scale) with scale = max_abs / 7 in f32, while the STORED scale is
+    # f16(scale). Block: max_abs = 7 * (1 + 2^-12), so scale = 1 + 2^-12 exactly and f16(scale) = 1.0 (half an f16 ulp at 1 is
+    # 2^-11). Then 2.5 / scale = 2.4994 -> 2, -2.5 -> -2, 0.5 / scale = 0.49988 -> 0; a quantizer that divided by the
+    # stored (rounded) scale would hit the exact ties 2.5, -2.5, 0.5 and give 3, -3, 1.
+    v = np.zeros((1, 32), np.float32)
+    v[0, :4] = [7.0 + 7.0 / 4096.0, 2.5, -2.5, 0.5]
+    assert float(v[0, 0]) == 7.0 + 7.0 / 4096.0 and np.float32(v[0, 0]) / np.float32(7) == np.float32(1 + 2.0 ** -12)
+    b = orc.quantize(orc.Q4_0, v, 1)
+    want = bytes([0x00, 0x3C,                     # f16(1.000244) = 1.0
+                  (7 + 8) | ((2 + 8) << 4),       # elements 0 (low nibble) and 1 (high nibble)
+                  (-2 + 8) | ((0 + 8) << 4)]      # elements 2 and 3
+                 + [0x88] * 14)
+    assert b.tobytes() == want
+    # the same block through the q8_0 quantizer, which DOES divide by the f16-rounded scale (storage/quantize.zig:83-103):
+    # absmax / 127 = 0.055131567 -> f16 0.055145264; 2.5 / that = 45.335 -> 45 either way, so pin it with the stored bits
+    b8 = orc.quantize(orc.Q8_0, v, 1)
+    s16 = np.array([np.float32(v[0, 0]) / np.float32(127)], np.float32).astype(np.float16)
+    assert b8[:2].tobytes() == s16.tobytes() and b8[2:3].view(np.int8)[0] == 127
+
+
 def test_quantize_rejects_bad_axis(orc):
     with pytest.raises(ValueError):
         orc.quantize(orc.Q8_0, np.zeros((33, 4), np.float32), 0)
