@@ -173,6 +173,10 @@ class HipBackend:
         fn = self._lib.aionhip_step_matmul_nt if weight.layout == ROWS_NK else self._lib.aionhip_step_matmul
         self._check(fn(self._ctx, weight.ptr, m, a_buf.handle + a_offset, lda, c_buf.handle + c_offset, ldc, alpha, beta))
 
+    def step_matmul_static(self, weight, a_buf, m, c_buf, lda=0, ldc=0, alpha=1.0, beta=0.0):
+        """step_matmul through the entry point that allocates nothing (prepared activation in the library's static array)."""
+        self._check(self._lib.aionhip_step_matmul_static(self._ctx, weight.ptr, m, a_buf.handle, lda, c_buf.handle, ldc, alpha, beta))
+
     def step_matmul_batch(self, weights, a_buf, m, c_bufs, lda=0, alpha=1.0, beta=0.0, c_offsets=None):
         n = len(weights)
         ws = (C.c_void_p * n)(*[w.ptr.value for w in weights])

@@ -41,6 +41,8 @@ struct aionhip_ctx {
     // second scratch for GEMM staging (dequantized weights / bf16 activations / split-K partials)
     void *scratch2 = nullptr;
     size_t scratch2_bytes = 0;
+    // this device's copy of the library's file-scope scratch array (ctx.hip), for the entry point that allocates nothing
+    void *static_scratch = nullptr;
     // attention with f32 queries: false = one MFMA pass on q rounded to the K/V element type (2e-3 class),
     // true = q and the probabilities as hi+lo parts (f32-level accuracy, about 1.4x the instructions)
     bool attn_precise = false;
@@ -109,6 +111,8 @@ struct aionhip_weight {
 int set_err(aionhip_ctx *ctx, int status, const char *fmt, ...);
 int ensure_scratch(aionhip_ctx *ctx, size_t bytes);
 int ensure_scratch2(aionhip_ctx *ctx, size_t bytes);
+// size of the file-scope device scratch array behind aionhip_step_matmul_static (prepared activations of one call)
+constexpr size_t STATIC_SCRATCH_BYTES = AIONHIP_STATIC_SCRATCH_BYTES;
 
 #define HIP_TRY(ctx, expr)                                                                          \
     do {                                                                                            \

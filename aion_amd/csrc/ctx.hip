@@ -5,7 +5,32 @@
 #include <algorithm>
 
 #include <cstring>
+#include <mutex>
 #include <new>
+
+// Scratch for aionhip_step_matmul_static, the entry point that may not allocate: one copy per GPU the library runs on,
+// held until the process ends. The name below is a host-side stand-in, not a device address: host code uses the
+// address hipGetSymbolAddress returns for the current device (kept per device in g_static_scratch), never the name.
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+static std::mutex g_static_scratch_mutex;
+static void *g_static_scratch[64];
+
+// the current device's address of the array; looked up once per device, with that device current
+static hipError_t static_scratch_address(int device, void **out) {
+    std::lock_guard<std::mutex> lock(g_static_scratch_mutex);
+    const bool cached = device >= 0 && device < 64;
+    if (cached && g_static_scratch[device]) {
+        *out = g_static_scratch[device];
+        return hipSuccess;
+    }
+    void *ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!ptr) return hipErrorInvalidSymbol;
+    if (cached) g_static_scratch[device] = ptr;
+    *out = ptr;
+    return hipSuccess;
+}
 
 int set_err(aionhip_ctx *ctx, int status, const char *fmt, ...) {
     if (ctx) {
@@ -138,6 +163,11 @@ int aionhip_create(int device, void *stream, aionhip_ctx **out) {
     }
     hipDeviceProp_t prop;
     if (hipGetDeviceProperties(&prop, device) == hipSuccess) ctx->cu_count = prop.multiProcessorCount;
+    if (static_scratch_address(device, &ctx->static_scratch) != hipSuccess) {
+        if (ctx->own_stream) (void)hipStreamDestroy(ctx->stream);
+        delete ctx;
+        return AIONHIP_EXECUTION_FAILED;
+    }
     *out = ctx;
     return AIONHIP_OK;
 }

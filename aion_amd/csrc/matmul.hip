@@ -41,12 +41,21 @@ int check_batch(aionhip_ctx *ctx, const char *what, size_t count, const aionhip_
     return AIONHIP_OK;
 }
 
-// every weight of `b` against the f32 rows at `a` (already materialised)
-int run_rows(aionhip_ctx *ctx, const Batch &b, size_t m, const float *a, size_t lda, float alpha, float beta) {
+// every weight of `b` against the f32 rows at `a` (already materialised). static_scratch: the prepared activation goes
+// to the library's file-scope device array and nothing on the way may allocate.
+int run_rows(aionhip_ctx *ctx, const Batch &b, size_t m, const float *a, size_t lda, float alpha, float beta, bool static_scratch = false) {
     if (m > 0x7FFFFFFFu) return set_err(ctx, AIONHIP_UNSUPPORTED, "matmul: m exceeds 2^31-1");
+    if (static_scratch) {
+        if (ctx->profiling) return set_err(ctx, AIONHIP_UNSUPPORTED, "matmul_static: not available while per-launch profiling is on (it creates events)");
+        if (m > GEMV_MAX_M && ctx->gemm_mode != AIONHIP_GEMM_EXACT_I8)
+            return set_err(ctx, AIONHIP_UNSUPPORTED, "matmul_static: more than %zu rows under a bf16 GEMM mode would allocate", GEMV_MAX_M);
+        if (prepared_act_bytes(m, b.k) > STATIC_SCRATCH_BYTES)
+            return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "matmul_static: the prepared activation of m=%zu, k=%zu needs %zu bytes, the static scratch holds %zu",
+                           m, b.k, prepared_act_bytes(m, b.k), STATIC_SCRATCH_BYTES);
+    }
     if (m == 1 && b.k <= FUSED_PAYS_K && ((uintptr_t)a & 15) == 0)
         return launch_gemv_fused(ctx, b.w, b.c, b.ldc, (int)b.count, PRO_QUANT, FusedIn{a, nullptr, nullptr, nullptr, 0.f}, alpha, beta);
-    if (m > GEMV_MAX_M && ctx->gemm_mode != AIONHIP_GEMM_EXACT_I8) {
+    if (m > GEMV_MAX_M && ctx->gemm_mode != AIONHIP_GEMM_EXACT_I8 && !static_scratch) {
         // the bf16 kernel where it is expected to win (or always, if so asked), the exact kernel (below) for the rest
         bool all_bf16 = true;
         if (ctx->gemm_mode == AIONHIP_GEMM_BF16_MFMA)
@@ -59,9 +68,9 @@ int run_rows(aionhip_ctx *ctx, const Batch &b, size_t m, const float *a, size_t 
             return AIONHIP_OK;
         }
     }
-    int rc = ensure_scratch(ctx, prepared_act_bytes(m, b.k));
+    int rc = static_scratch ? (int)AIONHIP_OK : ensure_scratch(ctx, prepared_act_bytes(m, b.k));
     if (rc) return rc;
-    PreparedAct act = prepared_act_carve(ctx->scratch, m, b.k);
+    PreparedAct act = prepared_act_carve(static_scratch ? ctx->static_scratch : ctx->scratch, m, b.k);
     rc = launch_prepare_act(ctx, a, lda, m, b.k, act);
     if (rc) return rc;
     if (m <= GEMV_MAX_M) return launch_gemv_batch(ctx, b.w, b.c, b.ldc, (int)b.count, (int)m, act, alpha, beta);
@@ -75,7 +84,7 @@ int run_rows(aionhip_ctx *ctx, const Batch &b, size_t m, const float *a, size_t 
 }
 
 int run_matmul(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, aionhip_handle a_h, size_t lda, aionhip_handle c_h, size_t ldc,
-               float alpha, float beta) {
+               float alpha, float beta, bool static_scratch = false) {
     if (m == 0) return AIONHIP_OK;
     if (!a_h || !c_h) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "matmul: null A or C");
     if (lda == 0) lda = w->k;
@@ -83,7 +92,7 @@ int run_matmul(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, aionhip_hand
     Batch b;
     int rc = check_batch(ctx, "matmul", 1, &w, &c_h, &ldc, b);
     if (rc) return rc;
-    return run_rows(ctx, b, m, (const float *)(uintptr_t)a_h, lda, alpha, beta);
+    return run_rows(ctx, b, m, (const float *)(uintptr_t)a_h, lda, alpha, beta, static_scratch);
 }
 
 }  // namespace
@@ -116,6 +125,13 @@ int aionhip_step_matmul_nt(aionhip_ctx *ctx, const aionhip_weight *b, size_t m, 
     // StepMatMulNT: B is q8_0 [N,K] with quant_axis 1 (runtime/executable.zig:211-223)
     if (b->layout != AIONHIP_ROWS_NK || b->dtype != AIONHIP_Q8_0) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "MatMulNT needs a q8_0 [N,K] weight (quant_axis 1)");
     return run_matmul(ctx, b, m, a, lda, c, ldc, alpha, beta);
+}
+
+int aionhip_step_matmul_static(aionhip_ctx *ctx, const aionhip_weight *b, size_t m, aionhip_handle a, size_t lda,
+                               aionhip_handle c, size_t ldc, float alpha, float beta) {
+    if (!ctx || !b) return AIONHIP_INVALID_ARGUMENT;
+    if (!ctx->static_scratch) return set_err(ctx, AIONHIP_EXECUTION_FAILED, "matmul_static: the context has no static scratch address");
+    return run_matmul(ctx, b, m, a, lda, c, ldc, alpha, beta, true);
 }
 
 int aionhip_step_rmsnorm_matmul(aionhip_ctx *ctx, size_t count, const aionhip_weight *const *bs, size_t rows, aionhip_handle x,

@@ -12,6 +12,7 @@ F32, F16, I8, Q4_0, Q8_0, I32, BF16 = 0, 1, 2, 3, 4, 5, 16
 ROWS_NK, KMAJOR_KN = 0, 1
 GEMM_EXACT_I8, GEMM_BF16_MFMA, GEMM_BF16_MFMA_ALWAYS = 0, 1, 2
 UNBOUNDED = 0xFFFFFFFF
+STATIC_SCRATCH_BYTES = 1 << 20     # AIONHIP_STATIC_SCRATCH_BYTES
 
 
 class AionHipError(RuntimeError):
@@ -54,6 +55,7 @@ _SIGS = {
     "aionhip_weight_download": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
     "aionhip_step_matmul": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint64, C.c_size_t, C.c_uint64, C.c_size_t, C.c_float, C.c_float]),
     "aionhip_step_matmul_nt": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint64, C.c_size_t, C.c_uint64, C.c_size_t, C.c_float, C.c_float]),
+    "aionhip_step_matmul_static": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint64, C.c_size_t, C.c_uint64, C.c_size_t, C.c_float, C.c_float]),
     "aionhip_step_matmul_batch": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_void_p), C.c_size_t, C.c_uint64, C.c_size_t, C.POINTER(C.c_uint64), C.POINTER(C.c_size_t), C.c_float, C.c_float]),
     "aionhip_step_rmsnorm_matmul": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_void_p), C.c_size_t, C.c_uint64, C.c_uint64, C.c_uint64, C.c_float, C.POINTER(C.c_uint64), C.POINTER(C.c_size_t), C.c_float, C.c_float]),
     "aionhip_step_rmsnorm_qkv_rope_append": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_float,

@@ -126,6 +126,19 @@ int aionhip_step_matmul(aionhip_ctx *ctx, const aionhip_weight *b, size_t m,
 int aionhip_step_matmul_nt(aionhip_ctx *ctx, const aionhip_weight *b, size_t m,
                            aionhip_handle a, size_t lda, aionhip_handle c, size_t ldc, float alpha, float beta);
 
+/* aionhip_step_matmul / aionhip_step_matmul_nt (by the weight's layout) for callers that cannot allocate: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc. No counterpart in aion. Same kernels and the
+ * same results as the two entry points above, but the prepared activation (int8 codes, block scales, block code
+ * sums: m * k + m * k / 32 * 8 bytes, each plane rounded up to 256) lives in a file-scope device array of
+ * AIONHIP_STATIC_SCRATCH_BYTES instead of the context's growable scratch, and the call makes no hipMalloc / hipFree or
+ * other allocating call. AIONHIP_INVALID_ARGUMENT when the prepared activation of (m, k) does not fit the array;
+ * AIONHIP_UNSUPPORTED for m > 8 under a bf16 GEMM mode (that path builds weight copies) and while per-launch
+ * profiling is on (it creates events). Each GPU holds one array, shared by every context on it and keeping the last
+ * call's contents: calls that overlap on one GPU (two contexts, two streams) race. */
+#define AIONHIP_STATIC_SCRATCH_BYTES ((size_t)1 << 20)
+int aionhip_step_matmul_static(aionhip_ctx *ctx, const aionhip_weight *b, size_t m,
+                               aionhip_handle a, size_t lda, aionhip_handle c, size_t ldc, float alpha, float beta);
+
 /* Several matmul steps that read the SAME activation (q/k/v, gate/up) as one call: the activation
  * is prepared once and, for m <= 8, all weights stream through one launch. aion keeps such
  * siblings as separate MatMul/MatMulNT steps (graph/opt/weight_layout.zig:72-115 re-lays but never
