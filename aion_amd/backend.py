@@ -146,6 +146,10 @@ class HipBackend:
             self._check(self._lib.aionhip_d2h(self._ctx, out.ctypes.data, buf.handle, offset, out.nbytes))
         return out
 
+    def copy(self, dst, src, nbytes, dst_offset=0, src_offset=0):
+        """DeviceMemory.copyD2D on the context's stream (asynchronous)."""
+        self._check(self._lib.aionhip_d2d(self._ctx, dst.handle, dst_offset, src.handle, src_offset, nbytes))
+
     def zeros(self, nbytes):
         buf = self.alloc(nbytes)
         self._check(self._lib.aionhip_memset(self._ctx, buf.handle, 0, 0, nbytes))

@@ -41,6 +41,9 @@ struct aionhip_ctx {
     // second scratch for GEMM staging (dequantized weights / bf16 activations / split-K partials)
     void *scratch2 = nullptr;
     size_t scratch2_bytes = 0;
+    // K-split GEMV: the words in which the partial sums of sibling K slices meet (all zero between launches)
+    void *ksplit = nullptr;
+    size_t ksplit_bytes = 0;
     // this device's copy of the library's file-scope scratch array (ctx.hip), for the entry point that allocates nothing
     void *static_scratch = nullptr;
     // attention with f32 queries: false = one MFMA pass on q rounded to the K/V element type (2e-3 class),
@@ -197,6 +200,9 @@ int launch_gate_gelu(aionhip_ctx *ctx, float *out, const float *a, const float *
 // device table f[i] = scale_factor * freq_step^i built with f32 multiplies in sequence (aion cpu/kernels/rope.zig:22-30)
 int rope_table(aionhip_ctx *ctx, int pairs, float freq_step, float scale_factor, const float **out);
 
+// one activation row against one weight with a long reduction axis: K cut into slices, one launch (gemv_ksplit.hip)
+bool gemv_ksplit_applies(const aionhip_ctx *ctx, const aionhip_weight *w, const float *x);
+int launch_gemv_ksplit(aionhip_ctx *ctx, const aionhip_weight *w, float *c, const float *x, float alpha, float beta);
 int launch_gemv(aionhip_ctx *ctx, const aionhip_weight *w, int m, PreparedAct act, float *c, size_t ldc, float alpha, float beta);
 int launch_gemv_batch(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count, int m,
                       PreparedAct act, float alpha, float beta);

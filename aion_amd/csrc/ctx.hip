@@ -184,6 +184,7 @@ void aionhip_destroy(aionhip_ctx *ctx) {
     for (auto &t : ctx->rope_tables) (void)hipFree(t.freq);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
     if (ctx->scratch2) (void)hipFree(ctx->scratch2);
+    if (ctx->ksplit) (void)hipFree(ctx->ksplit);
     if (ctx->own_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }

@@ -14,6 +14,8 @@
 // Two optional epilogues finish a decode block in the same launch (EPI_ROPE_APPEND, EPI_GATE_QUANT below).
 #include "common.h"
 
+#include <type_traits>
+
 namespace {
 
 // NCH = float4 activation chunks per thread (K <= 1024 * NCH). LDS is sized per launch:
@@ -324,15 +326,24 @@ void launch_r(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *c
     batch.total_waves = waves;
     const size_t lds = (size_t)K + (size_t)(K >> 5) * 8 + 16;
     if constexpr (PRO == PRO_QUANT) {
-        // The plain preparation runs in 1024-thread workgroups, the same 32 wavefronts per CU at most: a quarter of the
-        // workgroups re-read and re-quantize the activation, and fewer of them hit its few L2 lines at the same moment
-        // (q4, one row: 4096x4096 5.3 -> 4.6 us, 14336x4096 8.7 -> 7.8 us, 262144x2048 47 -> 45.8 us).
-        constexpr int WNT = 1024, WNCH = (NCH * 256 + WNT - 1) / WNT;
-        const int wg = (waves + WNT / 64 - 1) / (WNT / 64), cap = cus * 32 / (WNT / 64);
-        const dim3 wgrid((unsigned)(wg < cap ? wg : cap)), wblock(WNT);
-        if (R == 4) launch_k(ctx, gemv_fused_kernel<DT, 4, PRO_QUANT, WNCH, EPI_NONE, WNT>, wgrid, wblock, lds, batch, in, K, alpha, beta, FusedEpi{});
-        else if (R == 2) launch_k(ctx, gemv_fused_kernel<DT, 2, PRO_QUANT, WNCH, EPI_NONE, WNT>, wgrid, wblock, lds, batch, in, K, alpha, beta, FusedEpi{});
-        else launch_k(ctx, gemv_fused_kernel<DT, 1, PRO_QUANT, WNCH, EPI_NONE, WNT>, wgrid, wblock, lds, batch, in, K, alpha, beta, FusedEpi{});
+        // The plain preparation runs in wide workgroups (1024 threads: sixteen wavefronts share one preparation, and fewer
+        // workgroups hit the activation's few L2 lines at the same moment; q4, one row: 4096x4096 5.3 -> 4.6 us,
+        // 14336x4096 8.7 -> 7.8 us) on a grid capped at 32 wavefronts per CU, whose wavefronts stride over the row groups.
+        // A weight with many more row groups than that (a logits head) gets 512-thread workgroups and up to eight rounds of
+        // them before the striding starts: the hardware then deals workgroups out as CUs free up, which evens out the tail
+        // (262144x2048: 45.8 -> 44 us back to back, 46 -> 45 us between other kernels).
+        const bool many = waves > cus * 64;
+        const int nt = many ? 512 : 1024, rounds = many ? 8 : 1;
+        auto go = [&](auto nt_tag) {
+            constexpr int WNT = decltype(nt_tag)::value, WNCH = (NCH * 256 + WNT - 1) / WNT;
+            const int wg = (waves + WNT / 64 - 1) / (WNT / 64), cap = cus * 32 / (WNT / 64) * rounds;
+            const dim3 wgrid((unsigned)(wg < cap ? wg : cap)), wblock(WNT);
+            if (R == 4) launch_k(ctx, gemv_fused_kernel<DT, 4, PRO_QUANT, WNCH, EPI_NONE, WNT>, wgrid, wblock, lds, batch, in, K, alpha, beta, FusedEpi{});
+            else if (R == 2) launch_k(ctx, gemv_fused_kernel<DT, 2, PRO_QUANT, WNCH, EPI_NONE, WNT>, wgrid, wblock, lds, batch, in, K, alpha, beta, FusedEpi{});
+            else launch_k(ctx, gemv_fused_kernel<DT, 1, PRO_QUANT, WNCH, EPI_NONE, WNT>, wgrid, wblock, lds, batch, in, K, alpha, beta, FusedEpi{});
+        };
+        if (nt == 512) go(std::integral_constant<int, 512>{});
+        else go(std::integral_constant<int, 1024>{});
     } else {
         // at most 8 workgroups per CU: beyond that the wavefronts stride over the row groups
         const int wgs = (waves + 3) / 4;

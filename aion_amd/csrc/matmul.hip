@@ -55,6 +55,10 @@ int run_rows(aionhip_ctx *ctx, const Batch &b, size_t m, const float *a, size_t 
     }
     if (m == 1 && b.k <= FUSED_PAYS_K && ((uintptr_t)a & 15) == 0)
         return launch_gemv_fused(ctx, b.w, b.c, b.ldc, (int)b.count, PRO_QUANT, FusedIn{a, nullptr, nullptr, nullptr, 0.f}, alpha, beta);
+    // one row, one weight, long K: slices of K across workgroups, preparation inside, one launch (it keeps a growable buffer
+    // of its own, so not on the path that may not allocate)
+    if (m == 1 && b.count == 1 && !static_scratch && gemv_ksplit_applies(ctx, b.w[0], a))
+        return launch_gemv_ksplit(ctx, b.w[0], b.c[0], a, alpha, beta);
     if (m > GEMV_MAX_M && ctx->gemm_mode != AIONHIP_GEMM_EXACT_I8 && !static_scratch) {
         // the bf16 kernel where it is expected to win (or always, if so asked), the exact kernel (below) for the rest
         bool all_bf16 = true;

@@ -70,13 +70,18 @@ class _Plan:
 
 
 class PackageRunner:
-    def __init__(self, gpu, pkg, capacity, capacity_symbol="ctx", tokens_symbol="seq", fuse=True, growth=None):
+    def __init__(self, gpu, pkg, capacity, capacity_symbol="ctx", tokens_symbol="seq", fuse=True, growth=None, keep_residuals=False):
         """growth: None = the capacity is fixed and a run that needs more is an error. A dict with "numerator",
         "denominator" and optionally "max_capacity" = the sequence caches grow on the device when a run needs more
         rows, on the schedule of aion's session (api/loaded_model.zig:735-827: geometric steps, then a power of
         two and at least four times the old capacity, since every capacity is a set of plans of its own; rolling
-        caches use the factor 2/1 and are re-placed row by row)."""
+        caches use the factor 2/1 and are re-placed row by row).
+        keep_residuals: a residual add folded into a matmul's beta normally overwrites the residual in place, so that after a
+        run only the last layer's residual stream is left on the device. True = the sum goes to a buffer of its own (one
+        device copy of the residual first, then the same beta = 1 launch), which keeps every layer's input readable after
+        the run through `plans[s].values` - for inspecting a fused schedule node by node, not for speed."""
         self.gpu, self.pkg, self.capacity, self.fuse = gpu, pkg, int(capacity), fuse
+        self.keep_residuals = keep_residuals
         self.growth = growth
         self.cache_meta = {}        # input index -> (value id, retained history tokens, rows if the capacity is a constant else None)
         self.sym_ctx, self.sym_seq = capacity_symbol, tokens_symbol
@@ -432,8 +437,12 @@ class PackageRunner:
             gamma, beta = get(n0.inputs[1]), get(n0.inputs[2])
             if res is not None:
                 rv = vals[res]
-                emit(g.step_rmsnorm_geglu_matmul, wg.buf, wu.buf, wd.buf, x.buf, gamma.buf, n0.attrs["eps"], rv.buf, beta=1.0, beta_norm=beta.buf)
-                vals[nodes[add].output] = _Val("dev", rv.buf, rv.shape, "f32", owned=True)
+                acc = rv.buf
+                if self.keep_residuals:
+                    acc = new(rv.shape, "f32")
+                    emit(g.copy, acc, rv.buf, _count(rv.shape) * 4)
+                emit(g.step_rmsnorm_geglu_matmul, wg.buf, wu.buf, wd.buf, x.buf, gamma.buf, n0.attrs["eps"], acc, beta=1.0, beta_norm=beta.buf)
+                vals[nodes[add].output] = _Val("dev", acc, rv.shape, "f32", owned=True)
                 skip.update((mg, mu, un, mul, md, add))
             else:                                   # the down projection feeds something else (a norm): a buffer of its own
                 oshape = pkg.shape_of(nodes[md].output, sym)
@@ -450,8 +459,12 @@ class PackageRunner:
             res = residual_of(add, out_vid) if add is not None else None
             if res is not None:
                 rv = vals[res]
-                launch(rv.buf, 1.0)
-                vals[nodes[add].output] = _Val("dev", rv.buf, rv.shape, "f32", owned=True)
+                acc = rv.buf
+                if self.keep_residuals:
+                    acc = new(rv.shape, "f32")
+                    emit(g.copy, acc, rv.buf, _count(rv.shape) * 4)
+                launch(acc, 1.0)
+                vals[nodes[add].output] = _Val("dev", acc, rv.shape, "f32", owned=True)
                 skip.add(add)
             else:
                 out = new(shape, "f32")
@@ -497,8 +510,9 @@ class PackageRunner:
                 if res is not None and vals[res].buf is not x.buf:
                     # add(residual, norm(x)): the norm step's own residual operand, summed in place (the same two roundings)
                     rv = vals[res]
-                    emit(g.step_rmsnorm, rv.buf, x.buf, gamma.buf, rows, cols, a["eps"], beta=beta.buf, residual=rv.buf)
-                    vals[nodes[add].output] = _Val("dev", rv.buf, rv.shape, "f32", owned=True)
+                    acc = new(rv.shape, "f32") if self.keep_residuals else rv.buf      # out-of-place needs no copy here
+                    emit(g.step_rmsnorm, acc, x.buf, gamma.buf, rows, cols, a["eps"], beta=beta.buf, residual=rv.buf)
+                    vals[nodes[add].output] = _Val("dev", acc, rv.shape, "f32", owned=True)
                     skip.add(add)
                     continue
                 out = new(shape, "f32")

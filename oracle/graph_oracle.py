@@ -28,7 +28,7 @@ def _initializer(pkg, vid):
     shape = pkg.shape_of(vid, {})
     if t.quantized:
         return _Quant(t.scheme, t.quant_axis, shape, np.asarray(t.data))
-    return np.frombuffer(np.asarray(t.data).tobytes(), _NP[t.dtype]).reshape(shape).copy()
+    return np.asarray(t.data).view(_NP[t.dtype]).reshape(shape)        # a read-only view of the payload, no copy
 
 
 def _matmul(x, w, alpha, attn_threads):
@@ -107,9 +107,15 @@ def _start(pkg, feeds, rolling_inputs):
         vals[vid] = np.asarray(feeds[name])
         if name in rolling_inputs:
             rolling.add(vid)
-    for vid, v in enumerate(pkg.values):
-        if v.initializer is not None:
-            vals[vid] = _initializer(pkg, vid)
+    # initializers are immutable: materialised once per package object (a 2-billion-parameter package is evaluated many times)
+    inits = getattr(pkg, "_graph_oracle_initializers", None)
+    if inits is None:
+        inits = {vid: _initializer(pkg, vid) for vid, v in enumerate(pkg.values) if v.initializer is not None}
+        try:
+            pkg._graph_oracle_initializers = inits
+        except AttributeError:
+            pass
+    vals.update(inits)
     return vals, rolling
 
 
@@ -129,14 +135,19 @@ def run_graph(pkg, feeds, symbols, rolling_inputs=(), exact_attention=False, rou
     return {name: vals[vid] for name, vid in pkg.outputs}
 
 
-def check_nodes(pkg, feeds, symbols, device_values, rolling_inputs=(), threads=4):
+def check_nodes(pkg, feeds, symbols, device_values, rolling_inputs=(), threads=4, sample_rows_over=None, with_carried=False):
     """Every node on its own: evaluated here on the inputs THE DEVICE produced (device_values: value id -> array, read
     back after a node-by-node run) and compared with the device's output of that node. Unlike an end-to-end comparison
     this does not let one node's rounding be amplified by the next ones. A SequenceAppend is skipped (its cache operand
     is updated in place, the earlier contents are gone) and so is a node with an operand the device did not keep.
-    Returns [(node index, op, max|device - here| / rms(here))]."""
+    sample_rows_over: a MatMul whose output has more elements than this is evaluated on its first, middle and last
+    activation row only (rows never interact), and those rows are compared.
+    Returns [(node index, op, max|device - here| / rms(here))]; with_carried adds a fourth field: True when an operand
+    was not the device's but carried on this side from the last values the device did keep (a fused schedule folds
+    values into its neighbours: the node then checks the whole folded chain, roundings of the chain included)."""
     vals, rolling = _start(pkg, feeds, rolling_inputs)
     vals.update({vid: np.asarray(v) for vid, v in device_values.items()})
+    carried = set()
     report = []
     for i, n in enumerate(pkg.nodes):
         if n.op == "SequenceAppend":
@@ -146,15 +157,32 @@ def check_nodes(pkg, feeds, symbols, device_values, rolling_inputs=(), threads=4
         if any(v not in vals for v in n.inputs):
             continue
         ring = n.op == "Attention" and n.inputs[1] in rolling
-        out = _eval(pkg, n, [vals[v] for v in n.inputs], n.attrs, ring, False, False, threads)
+        ins = [vals[v] for v in n.inputs]
+        from_carried = any(v in carried for v in n.inputs)
+        rows = None
+        if (sample_rows_over is not None and n.op == "MatMul" and n.output in device_values and not isinstance(ins[0], _Quant)
+                and int(np.prod(pkg.shape_of(n.output, symbols))) > sample_rows_over):
+            m = int(np.prod(ins[0].shape[:-1]))
+            rows = sorted({0, m // 2, m - 1})
+            ins = [ins[0].reshape(m, ins[0].shape[-1])[rows]] + ins[1:]
+        out = _eval(pkg, n, ins, n.attrs, ring, False, False, threads)
         if isinstance(out, _Quant):
             vals[n.output] = out
+            continue
+        if rows is not None:
+            ref = np.asarray(out).astype(np.float64).reshape(len(rows), -1)
+            dev = np.asarray(device_values[n.output]).astype(np.float64).reshape(m, -1)[rows]
+            rms = float(np.sqrt((ref ** 2).mean())) + 1e-30
+            report.append((i, n.op, float(np.abs(dev - ref).max()) / rms) + ((from_carried,) if with_carried else ()))
             continue
         out = np.asarray(out).reshape(pkg.shape_of(n.output, symbols))
         if n.output in device_values:
             ref = out.astype(np.float64)
             rms = float(np.sqrt((ref ** 2).mean())) + 1e-30
-            report.append((i, n.op, float(np.abs(np.asarray(device_values[n.output]).astype(np.float64) - ref).max()) / rms))
+            report.append((i, n.op, float(np.abs(np.asarray(device_values[n.output]).astype(np.float64) - ref).max()) / rms)
+                          + ((from_carried,) if with_carried else ()))
         else:
             vals[n.output] = out          # a view or a value the device folded into a neighbour: carry this side's
+            if n.op not in _VIEWS or from_carried:
+                carried.add(n.output)
     return report

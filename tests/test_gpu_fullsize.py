@@ -1,9 +1,10 @@
 """BASELINE config 2's vocabulary-projection shape (N x K = 262144 x 2048) at full size, q4_0 [K,N] and q8_0 [N,K], batch 1 / 4 / 8,
 against the CPU oracle - and the persistent row-group loop of every one-row kernel variant on cheap shapes.
 
-On this shape the one-row kernel's grid is capped (8192 wavefronts) and each wavefront walks several row groups
-(`gwave += wave_stride`, new row addresses, new first loads); no smaller test shape enters that loop. The 2..4-row kernel runs
-its persistent grid and 5..8 rows run on the 16-row tile of the exact GEMM at a size no other test reaches.
+This shape is where the one-row kernel runs its largest grid (8192 workgroups), the 2..4-row kernel its persistent grid, and
+where 5..8 rows run on the 16-row tile of the exact GEMM at a size no other test reaches. The loop in which a wavefront
+walks several row groups (`gwave += wave_stride`, new row addresses, new first loads) starts beyond the grid caps: the
+second test enters it with every prologue variant on weights that are long but thin.
 Bar: max|err| <= 1e-5 * rms(ref) and the 2e-3 elementwise bound (floored), as for every exact-integer-dot kernel.
 """
 import sys
@@ -65,13 +66,13 @@ def test_config2_vocabulary_shape_batch_1_4_8(gpu, orc, tag, dtype, layout):
     w.free()
 
 
-# One row, K = 256, N = 70000: 17500 row groups of four against a grid capped at 8192 wavefronts, so every wavefront
-# takes the strided loop two or three times - with the plain preparation (1024-thread workgroups), the RMSNorm prologue
-# and the gelu-gate prologue (256-thread workgroups), and with two weights in one launch (a row group never straddles two
-# weights; the second weight starts mid-grid).
+# One row, K = 256, N = 300000 (+ 40003 in the same launch): 75000 row groups of four against a grid capped at 65536
+# wavefronts for the plain preparation (512-thread workgroups, eight rounds) and at 8192 for the RMSNorm and gelu-gate
+# prologues (256-thread workgroups), so wavefronts take the strided loop - once for some, nine times for others - and with
+# two weights in one launch a row group never straddles two weights (the second weight starts mid-grid).
 @pytest.mark.parametrize("tag,dtype,layout", [("q4", be.Q4_0, be.KMAJOR_KN), ("q8", be.Q8_0, be.ROWS_NK), ("q8", be.Q8_0, be.KMAJOR_KN)])
 def test_strided_row_group_loop_of_every_one_row_variant(gpu, orc, tag, dtype, layout):
-    n, n2, k = 70000, 40003, 256
+    n, n2, k = 300000, 40003, 256
     say("stride path", tag, layout)
     rng = np.random.default_rng(n + dtype + layout)
     made = []

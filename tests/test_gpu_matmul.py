@@ -179,20 +179,26 @@ def test_config2_decode_shapes(gpu, orc, dtype, layout, n, k):
     w.free()
 
 
-# One activation row against a long reduction axis: past K = 4096 the activation is prepared by a launch of its own
-# and the GEMV reads it from memory (a preparation inside every workgroup costs more there). Edges: the first K past
-# 4096, few rows, K that is not a multiple of the 64 chunks a wavefront covers per pass, alpha/beta.
+# One activation row against a long reduction axis: past K = 4096 the K axis is cut into slices across workgroups, each of
+# which prepares its own slice of the activation (gemv_ksplit_kernel); past 65536 columns or rows the activation is prepared
+# by a launch of its own and the GEMV reads it from memory. Edges: the first K past 4096, few rows and one row, K that is not
+# a multiple of the 64 chunks a wavefront covers per pass or of the slice count, the config-2 shape 4096 x 14336, alpha/beta.
 @pytest.mark.parametrize("dtype,layout", CASES)
-@pytest.mark.parametrize("n,k,kernel", [(5, 4128, "gemv"), (300, 16384, "gemv"), (70, 16416, "gemv"), (2050, 8224, "gemv"), (9000, 4096, "fused")])
+@pytest.mark.parametrize("n,k,kernel", [(5, 4128, "ksplit"), (300, 16384, "ksplit"), (70, 16416, "ksplit"), (2050, 8224, "ksplit"), (9000, 4096, "fused"),
+                                        (4096, 14336, "ksplit"), (1, 32768, "ksplit"), (33, 65568, "gemv"), (70000, 4128, "gemv")])
 def test_single_row_long_k(gpu, orc, dtype, layout, n, k, kernel):
     say("single row, long k", dtype, layout, n, k)
     blocks, w = make_weight(gpu, orc, dtype, layout, n, k, seed=n + k)
     a = np.random.default_rng(k).standard_normal((1, k)).astype(np.float32)
     got = gpu.matmul(w, a)
     q = "q8" if dtype == be.Q8_0 else "q4"
-    assert gpu.last_kernel() == ("gemv_%s_fused" % q if kernel == "fused" else "gemv_%s" % q)
+    assert gpu.last_kernel() == {"fused": "gemv_%s_fused", "ksplit": "gemv_%s_ksplit", "gemv": "gemv_%s"}[kernel] % q
     want = oracle_matmul(orc, dtype, layout, a, blocks, n)
     assert norm_err(got, want) < TOL and rms_err(got, want) < RMS_TOL
+    if kernel == "ksplit":
+        # the partial sums of the K slices meet along a fixed tree: the same bits on every run, whichever workgroup is last
+        for _ in range(3):
+            assert np.array_equal(gpu.matmul(w, a), got)
     c0 = np.random.default_rng(1).standard_normal((1, n)).astype(np.float32)
     got2 = gpu.matmul(w, a, alpha=0.5, beta=-2.0, c=c0)
     want2 = oracle_matmul(orc, dtype, layout, a, blocks, n, alpha=0.5, beta=-2.0, c=c0)

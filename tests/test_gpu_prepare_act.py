@@ -31,9 +31,9 @@ def identity(gpu, kind, n, k):
 
 
 # (rows, n, k, kernel that must have run): the one-row kernel with the preparation inside (256- and 1024-thread forms share
-# the code; K = 4096 fills all four chunks per thread), the separate preparation launch in front of the one-row kernel for
-# K > 4096, the 2..8-row kernel, the 16-row tile of the exact GEMM for 5..8 rows against a wide weight, the exact GEMM.
-PRODUCERS = [(1, 512, 512, "gemv_%s_fused"), (1, 4096, 4096, "gemv_%s_fused"), (1, 4160, 4160, "gemv_%s"),
+# the code; K = 4096 fills all four chunks per thread), the K-split one-row kernel for K > 4096 (each workgroup prepares its
+# slice), the 2..8-row kernel behind the separate preparation launch, the 16-row tile of the exact GEMM for 5..8 rows against a wide weight, the exact GEMM.
+PRODUCERS = [(1, 512, 512, "gemv_%s_fused"), (1, 4096, 4096, "gemv_%s_fused"), (1, 4160, 4160, "gemv_%s_ksplit"), (1, 600, 14336, "gemv_%s_ksplit"),
              (2, 512, 512, "gemv_%s"), (4, 1056, 1056, "gemv_%s"), (8, 512, 512, "gemv_%s"), (3, 96, 8192, "gemv_%s"),
              (6, 16384, 512, "gemv_%s"), (20, 512, 512, "gemm_i8_%s"), (130, 300, 1056, "gemm_i8_%s")]
 
