@@ -44,6 +44,9 @@ struct aionhip_ctx {
     // K-split GEMV: the words in which the partial sums of sibling K slices meet (all zero between launches)
     void *ksplit = nullptr;
     size_t ksplit_bytes = 0;
+    // argmax: one ticket per row (all zero between launches)
+    void *tickets = nullptr;
+    size_t tickets_bytes = 0;
     // this device's copy of the library's file-scope scratch array (ctx.hip), for the entry point that allocates nothing
     void *static_scratch = nullptr;
     // attention with f32 queries: false = one MFMA pass on q rounded to the K/V element type (2e-3 class),

@@ -185,6 +185,7 @@ void aionhip_destroy(aionhip_ctx *ctx) {
     if (ctx->scratch) (void)hipFree(ctx->scratch);
     if (ctx->scratch2) (void)hipFree(ctx->scratch2);
     if (ctx->ksplit) (void)hipFree(ctx->ksplit);
+    if (ctx->tickets) (void)hipFree(ctx->tickets);
     if (ctx->own_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }

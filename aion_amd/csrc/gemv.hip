@@ -125,9 +125,11 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemvBatch batch, const u32x4 
 // q4: the two 16-code halves of a block sit in separate LDS planes, so consecutive lanes read consecutive
 // 16 bytes of each. K ranges (kb0, kbn in quant blocks) let a long K run as several launches that each fit
 // LDS, beta = 1 after the first.
-constexpr size_t ROWS_LDS_CAP = 72 * 1024;
-template <int DT, int B, int LPR, int R>
-__global__ __launch_bounds__(256) void gemv_rows_kernel(GemvBatch batch, const u32x4 *__restrict__ aq, const float *__restrict__ a_scale,
+// NT threads per workgroup: 256, or 1024 when the rows' K range needs most of a CU's LDS (one workgroup per CU then, and
+// sixteen wavefronts rather than four to keep loads in flight).
+constexpr size_t ROWS_LDS_CAP = 72 * 1024, ROWS_LDS_CAP_WIDE = 158 * 1024;
+template <int DT, int B, int LPR, int R, int NT = 256>
+__global__ __launch_bounds__(NT) void gemv_rows_kernel(GemvBatch batch, const u32x4 *__restrict__ aq, const float *__restrict__ a_scale,
                                                         const int *__restrict__ a_sum, int K, int m, int kb0, int kbn, float alpha, float beta) {
     extern __shared__ __attribute__((aligned(16))) unsigned char s_rows[];
     constexpr bool Q8 = DT == AIONHIP_Q8_0;
@@ -142,42 +144,42 @@ __global__ __launch_bounds__(256) void gemv_rows_kernel(GemvBatch batch, const u
     // load-then-store round trips costs a memory latency per trip, which for a small N is most of the kernel)
     {
         const int per_row = 2 * kbn, total = B * per_row;
-        for (int base = 0; base < total; base += 256 * 8) {
+        for (int base = 0; base < total; base += NT * 8) {
             u32x4 v[8];
             int dsti[8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const int idx = min(base + tid + 256 * i, total - 1);
+                const int idx = min(base + tid + NT * i, total - 1);
                 const int b = idx / per_row, c = idx - b * per_row;
                 dsti[i] = b * per_row + (Q8 ? c : ((c & 1) ? kbn + (c >> 1) : (c >> 1)));
                 v[i] = aq[(size_t)min(b, m - 1) * a_chunks + 2 * kb0 + c];
             }
 #pragma unroll
             for (int i = 0; i < 8; ++i)
-                if (base + tid + 256 * i < total) s_a[dsti[i]] = v[i];
+                if (base + tid + NT * i < total) s_a[dsti[i]] = v[i];
         }
         const int total_s = B * kbn;
-        for (int base = 0; base < total_s; base += 256 * 4) {
+        for (int base = 0; base < total_s; base += NT * 4) {
             float sv[4];
             int iv[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int idx = min(base + tid + 256 * i, total_s - 1);
+                const int idx = min(base + tid + NT * i, total_s - 1);
                 const int b = idx / kbn, j = idx - b * kbn;
                 sv[i] = a_scale[(size_t)min(b, m - 1) * KB + kb0 + j];
                 iv[i] = a_sum[(size_t)min(b, m - 1) * KB + kb0 + j];
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                if (base + tid + 256 * i < total_s) { s_scale[base + tid + 256 * i] = sv[i]; s_sum[base + tid + 256 * i] = iv[i]; }
+                if (base + tid + NT * i < total_s) { s_scale[base + tid + NT * i] = sv[i]; s_sum[base + tid + NT * i] = iv[i]; }
         }
     }
     __syncthreads();
 
     const int chunks_row = Q8 ? (K >> 4) : KB;      // 16-byte weight chunks per full row
     const int ch0 = Q8 ? 2 * kb0 : kb0, nch = Q8 ? 2 * kbn : kbn;
-    const int wave_stride = gridDim.x * 4;
-    for (int gwave = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(tid >> 6); gwave < batch.total_waves; gwave += wave_stride) {
+    const int wave_stride = gridDim.x * (NT / 64);
+    for (int gwave = blockIdx.x * (NT / 64) + __builtin_amdgcn_readfirstlane(tid >> 6); gwave < batch.total_waves; gwave += wave_stride) {
         int si = 0;
 #pragma unroll
         for (int i = 1; i < 4; ++i)
@@ -325,29 +327,36 @@ int launch_rows(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const 
         waves += ((int)ws[i]->n + rpw - 1) / rpw;
     }
     batch.total_waves = waves;
-    // K slices that fit the LDS cap, as even as possible
+    // K slices that fit LDS, as even as possible: up to 72 KB per 256-thread workgroup (two or more workgroups per CU); a K
+    // that needs more runs in one pass of 1024-thread workgroups with most of the CU's LDS rather than as two launches
     const size_t per_block = (size_t)B * 40;
-    const int max_kbn = (int)(ROWS_LDS_CAP / per_block);
+    const bool wide = (size_t)KB * per_block > ROWS_LDS_CAP && (size_t)KB * per_block <= ROWS_LDS_CAP_WIDE;
+    const int max_kbn = (int)((wide ? ROWS_LDS_CAP_WIDE : ROWS_LDS_CAP) / per_block);
     const int slices = (KB + max_kbn - 1) / max_kbn;
     const int kbn_even = (KB + slices - 1) / slices;
     const auto *aq = (const u32x4 *)act.q;
     for (int s = 0, kb0 = 0; s < slices; ++s, kb0 += kbn_even) {
         const int kbn = min(kbn_even, KB - kb0);
         const size_t lds = (size_t)kbn * per_block;
-        const int per_cu = (int)min((size_t)8, (size_t)(160 * 1024) / (lds + 512));
-        const int wgs = (waves + 3) / 4;
-        const dim3 grid((unsigned)min(wgs, cus * max(per_cu, 1))), block(256);
+        const int nt = wide ? 1024 : 256;
+        const int per_cu = wide ? 1 : (int)min((size_t)8, (size_t)(160 * 1024) / (lds + 512));
+        const int wgs = (waves + nt / 64 - 1) / (nt / 64);
+        const dim3 grid((unsigned)min(wgs, cus * max(per_cu, 1))), block((unsigned)nt);
         const float b_eff = s == 0 ? beta : 1.f;
         auto go = [&](auto kern) {
             if (lds > 64 * 1024) {
-                hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ROWS_LDS_CAP);
+                hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(wide ? ROWS_LDS_CAP_WIDE : ROWS_LDS_CAP));
                 if (e != hipSuccess) return set_err(ctx, AIONHIP_EXECUTION_FAILED, "gemv rows: %s", hipGetErrorString(e));
             }
             launch_k(ctx, kern, grid, block, lds, batch, aq, act.scale, act.sum, K, m, kb0, kbn, alpha, b_eff);
             return (int)AIONHIP_OK;
         };
         int rc;
-        if (R == 4) rc = lpr == 16 ? go(gemv_rows_kernel<DT, B, 16, 4>) : lpr == 32 ? go(gemv_rows_kernel<DT, B, 32, 4>) : go(gemv_rows_kernel<DT, B, 64, 4>);
+        if (wide) {
+            if (R == 4) rc = lpr == 16 ? go(gemv_rows_kernel<DT, B, 16, 4, 1024>) : lpr == 32 ? go(gemv_rows_kernel<DT, B, 32, 4, 1024>) : go(gemv_rows_kernel<DT, B, 64, 4, 1024>);
+            else if (R == 2) rc = lpr == 16 ? go(gemv_rows_kernel<DT, B, 16, 2, 1024>) : lpr == 32 ? go(gemv_rows_kernel<DT, B, 32, 2, 1024>) : go(gemv_rows_kernel<DT, B, 64, 2, 1024>);
+            else rc = lpr == 16 ? go(gemv_rows_kernel<DT, B, 16, 1, 1024>) : lpr == 32 ? go(gemv_rows_kernel<DT, B, 32, 1, 1024>) : go(gemv_rows_kernel<DT, B, 64, 1, 1024>);
+        } else if (R == 4) rc = lpr == 16 ? go(gemv_rows_kernel<DT, B, 16, 4>) : lpr == 32 ? go(gemv_rows_kernel<DT, B, 32, 4>) : go(gemv_rows_kernel<DT, B, 64, 4>);
         else if (R == 2) rc = lpr == 16 ? go(gemv_rows_kernel<DT, B, 16, 2>) : lpr == 32 ? go(gemv_rows_kernel<DT, B, 32, 2>) : go(gemv_rows_kernel<DT, B, 64, 2>);
         else rc = lpr == 16 ? go(gemv_rows_kernel<DT, B, 16, 1>) : lpr == 32 ? go(gemv_rows_kernel<DT, B, 32, 1>) : go(gemv_rows_kernel<DT, B, 64, 1>);
         if (rc) return rc;

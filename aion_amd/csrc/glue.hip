@@ -324,9 +324,11 @@ __global__ void cache_grow_rolling_kernel(unsigned *__restrict__ dst, const unsi
     dst[i] = v;
 }
 
-// cpu/exec/argmax.zig:56-81: strict > keeps the first maximum. Two stages: ARGMAX_PARTS workgroups
-// per row each reduce a contiguous slice to (value, index), then one workgroup picks among them
-// (ties -> the smaller index, which is the first maximum).
+// cpu/exec/argmax.zig:56-81: strict > keeps the first maximum. ARGMAX_PARTS workgroups per row each reduce a contiguous
+// slice to (value, index); the workgroup that draws the row's last ticket then picks among the parts (ties -> the smaller
+// index, which is the first maximum) - one launch. The parts and the ticket are device-scope atomics and the ticket is
+// taken after the part's stores were acknowledged, so no device-scope fence is needed (on this GPU such a fence writes
+// back and invalidates an XCD's whole L2); the pick does not depend on which workgroup came last. Tickets return to zero.
 constexpr int ARGMAX_PARTS = 64;
 __device__ __forceinline__ void argmax_reduce_256(float &best, int &idx, float *bv, int *bi) {
     bv[threadIdx.x] = best;
@@ -345,10 +347,12 @@ __device__ __forceinline__ void argmax_reduce_256(float &best, int &idx, float *
     }
     best = bv[0];
     idx = bi[0];
+    __syncthreads();
 }
-__global__ __launch_bounds__(256) void argmax_part_kernel(float *__restrict__ pv, int *__restrict__ pi, const float *__restrict__ x, size_t n) {
+__global__ __launch_bounds__(256) void argmax_kernel(int *__restrict__ out, float *pv, int *pi, unsigned *tickets, const float *__restrict__ x, size_t n) {
     __shared__ float bv[256];
     __shared__ int bi[256];
+    __shared__ int s_last;
     const size_t row = blockIdx.y;
     const size_t per = (n + ARGMAX_PARTS - 1) / ARGMAX_PARTS;
     const size_t lo = blockIdx.x * per, hi = lo + per < n ? lo + per : n;
@@ -361,21 +365,24 @@ __global__ __launch_bounds__(256) void argmax_part_kernel(float *__restrict__ pv
     }
     argmax_reduce_256(best, idx, bv, bi);
     if (threadIdx.x == 0) {
-        pv[row * ARGMAX_PARTS + blockIdx.x] = best;
-        pi[row * ARGMAX_PARTS + blockIdx.x] = idx;
+        __hip_atomic_store(pv + row * ARGMAX_PARTS + blockIdx.x, best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(pi + row * ARGMAX_PARTS + blockIdx.x, idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+        s_last = __hip_atomic_fetch_add(tickets + row, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ARGMAX_PARTS - 1;
     }
-}
-__global__ __launch_bounds__(256) void argmax_final_kernel(int *__restrict__ out, const float *__restrict__ pv, const int *__restrict__ pi) {
-    __shared__ float bv[256];
-    __shared__ int bi[256];
-    float best = -INFINITY;
-    int idx = 0x7FFFFFFF;
+    __syncthreads();
+    if (!s_last) return;
+    best = -INFINITY;
+    idx = 0x7FFFFFFF;
     if (threadIdx.x < ARGMAX_PARTS) {
-        best = pv[blockIdx.x * ARGMAX_PARTS + threadIdx.x];
-        idx = pi[blockIdx.x * ARGMAX_PARTS + threadIdx.x];
+        best = __hip_atomic_load(pv + row * ARGMAX_PARTS + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        idx = __hip_atomic_load(pi + row * ARGMAX_PARTS + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     argmax_reduce_256(best, idx, bv, bi);
-    if (threadIdx.x == 0) out[blockIdx.x] = idx == 0x7FFFFFFF ? 0 : idx;
+    if (threadIdx.x == 0) {
+        out[row] = idx == 0x7FFFFFFF ? 0 : idx;
+        __hip_atomic_store(tickets + row, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 }
 
 inline unsigned grid_for(size_t n, unsigned block) { return (unsigned)((n + block - 1) / block); }
@@ -671,10 +678,23 @@ int aionhip_step_argmax(aionhip_ctx *ctx, aionhip_handle out_i32, aionhip_handle
     if (rows > 65535) return set_err(ctx, AIONHIP_UNSUPPORTED, "argmax: more than 65535 rows");
     int rc = ensure_scratch2(ctx, rows * ARGMAX_PARTS * 8);
     if (rc) return rc;
+    if (rows * sizeof(unsigned) > ctx->tickets_bytes) {
+        if (ctx->capturing)
+            return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "the argmax tickets must grow while a program is being recorded: run the steps once before recording");
+        if (ctx->tickets) {
+            HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
+            HIP_TRY(ctx, hipFree(ctx->tickets));
+            ctx->tickets = nullptr;
+            ctx->tickets_bytes = 0;
+        }
+        const size_t want = (rows * sizeof(unsigned) + 4095) & ~(size_t)4095;
+        HIP_TRY(ctx, hipMalloc(&ctx->tickets, want));
+        ctx->tickets_bytes = want;
+        HIP_TRY(ctx, hipMemsetAsync(ctx->tickets, 0, want, ctx->stream));          // never inside a recording
+    }
     float *pv = (float *)ctx->scratch2;
     int *pi = (int *)(pv + rows * ARGMAX_PARTS);
-    argmax_part_kernel<<<dim3(ARGMAX_PARTS, (unsigned)rows), dim3(256), 0, ctx->stream>>>(pv, pi, dp<const float>(x), n);
-    argmax_final_kernel<<<dim3((unsigned)rows), dim3(256), 0, ctx->stream>>>(dp<int>(out_i32), pv, pi);
+    argmax_kernel<<<dim3(ARGMAX_PARTS, (unsigned)rows), dim3(256), 0, ctx->stream>>>(dp<int>(out_i32), pv, pi, (unsigned *)ctx->tickets, dp<const float>(x), n);
     LAUNCH_CHECK(ctx, "argmax");
     return AIONHIP_OK;
 }

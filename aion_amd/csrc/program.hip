@@ -22,9 +22,39 @@ __global__ void add_i32_kernel(int *__restrict__ out, const int *__restrict__ a,
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) out[i] = a[i] + b[i];
 }
+struct AdvanceArgs {
+    int *counter[8];
+    int count;
+};
+// the loop state of a device-resident greedy decode in one launch: the produced token becomes the next input, the indices move on
+__global__ void advance_state_kernel(int *__restrict__ dst, const int *__restrict__ src, size_t n, AdvanceArgs a, int delta) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = src[i];
+    if (blockIdx.x == 0 && (int)threadIdx.x < a.count) *a.counter[threadIdx.x] += delta;
+}
 }  // namespace
 
 extern "C" {
+
+int aionhip_step_advance_state(aionhip_ctx *ctx, aionhip_handle dst_tokens, aionhip_handle src_tokens, size_t n_tokens,
+                               const aionhip_handle *counters, size_t n_counters, int delta) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (n_counters > 8 || (n_counters && !counters) || (n_tokens && (!dst_tokens || !src_tokens)))
+        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "advance_state: null operand or more than 8 counters");
+    if (!n_tokens && !n_counters) return AIONHIP_OK;
+    AdvanceArgs a{};
+    a.count = (int)n_counters;
+    for (size_t i = 0; i < n_counters; ++i) {
+        if (!counters[i] || (counters[i] & 3)) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "advance_state: null or misaligned counter");
+        for (size_t j = 0; j < i; ++j)
+            if (counters[j] == counters[i]) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "advance_state: a counter is listed twice");
+        a.counter[i] = (int *)(uintptr_t)counters[i];
+    }
+    const size_t blocks = n_tokens ? (n_tokens + 63) / 64 : 1;
+    advance_state_kernel<<<dim3((unsigned)blocks), dim3(64), 0, ctx->stream>>>((int *)(uintptr_t)dst_tokens, (const int *)(uintptr_t)src_tokens, n_tokens, a, delta);
+    LAUNCH_CHECK(ctx, "advance_state");
+    return AIONHIP_OK;
+}
 
 int aionhip_program_begin(aionhip_ctx *ctx) {
     if (!ctx) return AIONHIP_INVALID_ARGUMENT;

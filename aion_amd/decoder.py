@@ -211,10 +211,7 @@ class Decoder:
             def issue():
                 self._forward(1, b)
                 # advance the device-resident loop state: next id = argmax, positions/write index/kv length += 1
-                g._check(g._lib.aionhip_d2d(g._ctx, b["ids"].handle, 0, self.token.handle, 0, 4))
-                g.step_add_i32(b["positions"], b["positions"], self.one, 1)
-                g.step_add_i32(b["write_index"], b["write_index"], self.one, 1)
-                g.step_add_i32(b["kv_len"], b["kv_len"], self.one, 1)
+                g.step_advance_state(b["ids"], self.token, 1, [b["positions"], b["write_index"], b["kv_len"]])
             self.program = g.record_program(issue)
 
     def _set_decode_state(self, b, token, pos):

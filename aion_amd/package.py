@@ -748,9 +748,8 @@ class PackageRunner:
 
             def issue():
                 self._issue(plan)
-                g._check(g._lib.aionhip_d2d(g._ctx, plan.inputs["tokens"][0].handle, 0, tok_buf.handle, 0, 4))
-                for kind in ("positions", "cache_write_index", "cache_visible_end"):
-                    g.step_add_i32(plan.inputs[kind][0], plan.inputs[kind][0], self.one, 1)
+                g.step_advance_state(plan.inputs["tokens"][0], tok_buf, 1,
+                                     [plan.inputs[kind][0] for kind in ("positions", "cache_write_index", "cache_visible_end")])
             self.program = g.record_program(issue)
         self._token_output = token_output
 

@@ -326,9 +326,10 @@ def time_kernel(gpu, ws, x, y, m, name, iters=20):
     gpu.profile_start()
     for i in range(iters):
         gpu.step_matmul(ws[i % len(ws)], x, m, y)
-    prof = [ms for (nm, ms) in gpu.profile_stop() if nm.startswith(name)]
-    per = len(prof) // iters                      # a long K at several rows runs as more than one launch
-    calls = sorted(sum(prof[i * per:(i + 1) * per]) for i in range(iters))
+    prof = gpu.profile_stop()
+    assert any(nm.startswith(name) for nm, _ms in prof), (name, prof[:4])
+    per = len(prof) // iters                      # every launch of the call: the activation preparation and the GEMV(s)
+    calls = sorted(sum(ms for _nm, ms in prof[i * per:(i + 1) * per]) for i in range(iters))
     return calls[iters // 2]
 
 
@@ -346,7 +347,7 @@ def run_sweep(gpu, be, q4_blocks):
                 ms = time_kernel(gpu, ws, x, y, m, kname)
                 by = algorithmic_bytes(bb, n, k, m)
                 res["%s %dx%d b%d" % ("q4" if dtype == be.Q4_0 else "q8", n, k, m)] = {
-                    "kernel_us": round(ms * 1e3, 2), "GBps": round(by / (ms * 1e-3) / 1e9, 1),
+                    "kernels": gpu.last_kernel(), "kernel_us": round(ms * 1e3, 2), "GBps": round(by / (ms * 1e-3) / 1e9, 1),
                     "frac_hbm_peak": round(by / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 3)}
                 x.free(); y.free()
             for w in ws:

@@ -302,6 +302,12 @@ int aionhip_step_argmax(aionhip_ctx *ctx, aionhip_handle out_i32, aionhip_handle
  * the cache write index and kv lengths on the device between replays of a decode program */
 int aionhip_step_add_i32(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle a, aionhip_handle b, size_t n);
 
+/* The same bookkeeping as one launch (a decode step is bound by its launch count): dst_tokens[0..n_tokens) = src_tokens[...]
+ * (i32, the token the step produced becomes the next step's input; StepCopy, runtime/executable.zig) and delta is added to
+ * each of up to 8 distinct scalar i32 device values (positions, write index, visible end). */
+int aionhip_step_advance_state(aionhip_ctx *ctx, aionhip_handle dst_tokens, aionhip_handle src_tokens, size_t n_tokens,
+                               const aionhip_handle *counters, size_t n_counters, int delta);
+
 /* ---- programs: record a fixed step sequence once, replay it per token ----------------------
  * Session.execute(prog) (backend/backend.zig:42-44) runs aion's ExecutableProgram step list; the
  * WebGPU backend replays cached dispatch state because a decode program is identical every token
