@@ -345,7 +345,9 @@ void launch_r(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *c
         if (nt == 512) go(std::integral_constant<int, 512>{});
         else go(std::integral_constant<int, 1024>{});
     } else {
-        // at most 8 workgroups per CU: beyond that the wavefronts stride over the row groups
+        // at most 8 workgroups per CU: beyond that the wavefronts stride over the row groups (more rounds of workgroups,
+        // as for the plain preparation above, cost more here than they even out: every workgroup redoes the norm's
+        // reduction; 262144x2048 behind an RMSNorm: 50.8 us on this grid, 56.7 us on eight rounds)
         const int wgs = (waves + 3) / 4;
         const dim3 grid((unsigned)(wgs < cus * 8 ? wgs : cus * 8)), block(256);
         if (R == 4) launch_k(ctx, gemv_fused_kernel<DT, 4, PRO, NCH, EPI_NONE>, grid, block, lds, batch, in, K, alpha, beta, FusedEpi{});

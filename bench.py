@@ -20,7 +20,8 @@ The same JSON line carries the two other metrics BASELINE.json names, in a "seco
 its own: "prefill_gemm" (config 3's largest shape, M = 2048, N = 14336, K = 4096, q4: the exact int8 path and the bf16 MFMA
 path, TFLOP/s against the named MFMA peak, with the tolerance class of each) and "decode" (config 5: the 26-layer decoder,
 128-token prompt, greedy decode of 128 tokens at batch 1: tokens/s, ms/token, weight bytes streamed per second against the
-HBM peak), plus "sweep": config 2's q8 legs and batch 4 / 8 per shape. `--headline-only` skips the secondary object.
+HBM peak), plus "sweep": config 2's q8 legs and batch 4 / 8 per shape. `--headline-only` skips the secondary object (and
+with it every stream capture: the form to run under rocprofv3, which does not survive a capture in the traced process).
 `--extras gemm,attention,decoder[,decoder_eager,package,package_bench_shape,package_bench_shape_eager]` adds the full config-3 and
 config-4 tables, the decoder with its CPU-oracle leg, and the package runner in an "extras" object.
 """
@@ -69,8 +70,6 @@ def main():
     ap.add_argument("--sweep", action="store_true", help="(kept for compatibility: the sweep is part of the default run)")
     ap.add_argument("--headline-only", action="store_true", help="skip the secondary metrics (prefill GEMM, decode, sweep)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--launch-by-launch", action="store_true",
-                    help="time the K steps as individual launches instead of one recorded program (the form a kernel trace or counter run can attribute: rocprofv3 does not survive stream capture in the traced process)")
     ap.add_argument("--extras", default="", help="comma list of gemm,attention,decoder")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -108,33 +107,17 @@ def main():
     for i in range(args.warmup):
         step(i)
     gpu.sync()
-    # pass 1: exactly K steps between two stream events -> value. The K steps are recorded once as a program (the library's
-    # replay of a fixed step sequence, a HIP graph: what a decode loop on this backend runs) and the program is executed once
-    # inside the timed region; the same K steps issued launch by launch are timed right after it and reported beside it.
+    # pass 1: exactly K steps between two stream events -> value (launch by launch: a single execution of the same steps as one
+    # recorded program was measured too - 66-76 us per step from run to run against a steady 67-68 here - and not adopted)
     ev0, ev1 = gpu.event(), gpu.event()
-    total_ms, wall_ms, program_nodes = None, None, 0
-    if not args.launch_by_launch:
-        prog = gpu.record_program(lambda: [step(args.warmup + i) for i in range(args.steps)])
-        gpu.program_execute(prog)                       # untimed: the first execution of a program uploads it
-        gpu.sync()
-        gpu.record(ev0)
-        t_wall = time.perf_counter()
-        gpu.program_execute(prog)
-        gpu.record(ev1)
-        gpu.sync()
-        wall_ms = (time.perf_counter() - t_wall) * 1e3
-        total_ms = gpu.elapsed_ms(ev0, ev1)
-        program_nodes = int(gpu.program_node_count(prog))
-        gpu.program_destroy(prog)
-    t_wall = time.perf_counter()
     gpu.record(ev0)
+    t_wall = time.perf_counter()
     for i in range(args.steps):
         step(args.warmup + i)
     gpu.record(ev1)
     gpu.sync()
-    eager_ms = gpu.elapsed_ms(ev0, ev1)
-    if total_ms is None:
-        total_ms, wall_ms = eager_ms, (time.perf_counter() - t_wall) * 1e3
+    wall_ms = (time.perf_counter() - t_wall) * 1e3
+    total_ms = gpu.elapsed_ms(ev0, ev1)
     # pass 2: the same K steps again, every dispatch carrying its own start/stop events -> roofline
     # (kept apart from pass 1 because timed dispatches cannot be queued back to back)
     gpu.profile_start()
@@ -193,11 +176,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": "config 2, q4_0 decode GEMV batch 1 over 4096x4096, 14336x4096, 4096x14336, 262144x2048 (one step = the four GEMVs incl. activation int8 preparation)",
                    "device": info["arch"], "cu_count": info["cu_count"], "weight_sets_rotated": n_sets,
-                   "step_algorithmic_bytes": step_bytes, "wall_ms_per_step": round(wall_ms / args.steps, 5),
-                   "issued_as": ("one recorded program of %d steps (%d kernel nodes), executed once between the two events" % (args.steps, program_nodes))
-                                if program_nodes else "%d steps launch by launch" % args.steps,
-                   "launch_by_launch_ms_per_step": round(eager_ms / args.steps, 5),
-                   "launch_by_launch_GBps": round(step_bytes / (eager_ms / args.steps * 1e-3) / 1e9, 1)},
+                   "step_algorithmic_bytes": step_bytes, "wall_ms_per_step": round(wall_ms / args.steps, 5)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": round(sum(MEASURED_TRAFFIC[sh] for sh in SHAPES) / len(SHAPES)),
@@ -223,7 +202,7 @@ def main():
             w.free()
     for t in xs + ys:
         t.free()
-    if not args.headline_only and not args.launch_by_launch:
+    if not args.headline_only:
         out["secondary"] = {"prefill_gemm": run_gemm_headline(gpu, be), "decode": run_decode_headline(gpu, be),
                             "sweep": run_sweep(gpu, be, host_blocks)}
     if extras:
