@@ -43,7 +43,7 @@ CAL_ELEMS = 1 << 26   # the counter-calibration cast: 256 MiB read, 128 MiB writ
 # counter runs of this same command scaled by what the same counters read for the calibration cast
 # (factors 1.9998 and 1.0000); the summary with the commands is profiles/gemv_q4_decode_bench_kernel_stats_and_traffic.md.
 # Counters cannot be read from inside the process, so the figures are carried here.
-MEASURED_TRAFFIC = {(4096, 4096): 9.655e6, (14336, 4096): 33.294e6, (4096, 14336): 33.243e6, (262144, 2048): 303.189e6}
+MEASURED_TRAFFIC = {(4096, 4096): 9.655e6, (14336, 4096): 33.299e6, (4096, 14336): 33.879e6, (262144, 2048): 303.159e6}
 
 
 def algorithmic_bytes(dtype_bytes, n, k, batch):
