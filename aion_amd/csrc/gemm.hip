@@ -326,6 +326,9 @@ __global__ void act_bf16_kernel(const float *__restrict__ a, size_t lda, unsigne
 // of the load, so that the 16 consecutive rows of a fragment read hit 16 distinct bank groups.
 // Four LDS stages: the loads of K steps kt+1..kt+3 are in flight during the MFMAs of step kt - a
 // load round trip through L2 under this traffic takes about as long as two K steps of MFMAs.
+// The loads of a stage are issued in two parts, the weight rows with the first half of a K step's MFMAs and the
+// activation rows with the second half, one load per MFMA: issued back to back, the four wavefronts' loads queue
+// up in the CU's address unit and the wavefronts stall there with their MFMAs behind them (measured: 3-5 %).
 // The wavefront waits on its own loads by count (s_waitcnt vmcnt) and the stages are handed over
 // with a bare s_barrier: a fence would drain the younger stages' loads as well.
 // Tile order: workgroup ids go round-robin over the 8 XCDs, so id -> (xcd, slot) -> a contiguous
@@ -333,6 +336,30 @@ __global__ void act_bf16_kernel(const float *__restrict__ a, size_t lda, unsigne
 constexpr int G2_BK = 32, G2_ROW = 64, G2_BN = 256;
 using f32x16 = __attribute__((ext_vector_type(16))) float;
 
+
+// Instruction order of half a K step: two MFMAs first (the wait in front of them then covers only reads issued long
+// ago), then every LDS read of the next fragment with an MFMA behind it (so that they are back when the next half
+// starts), then the V global->LDS loads one per MFMA. The address unit of a CU takes about 16 cycles per 16-byte
+// wavefront load; four wavefronts issuing theirs back to back stall on its queue, with an MFMA between two loads they do not.
+template <int NMMA, int NFR, int V>
+__device__ __forceinline__ void sched_half() {
+    constexpr int REST = NMMA - 2 - NFR;                     // MFMAs left once the reads are placed
+    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+#pragma unroll
+    for (int i = 0; i < NFR; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        if (REST <= 0 ? i < V : i >= NFR - (V - REST) ) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // loads that find no MFMA of their own
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    }
+    if constexpr (REST > 0) {
+#pragma unroll
+        for (int i = 0; i < (V < REST ? V : REST); ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+        if constexpr (REST > V) __builtin_amdgcn_sched_group_barrier(0x008, REST - V, 0);
+    }
+}
 
 template <int WM, int NST, int WN>
 __global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const unsigned short *__restrict__ A, const unsigned short *__restrict__ W,
@@ -370,16 +397,18 @@ __global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const unsigned shor
     for (int i = 0; i < NB; ++i) gb[i] = W + (size_t)min(n0 + i * 64 + lrow, N - 1) * K + lchunk * 8;
     const int KT = K / G2_BK;
 
-    auto issue_loads = [&](int kt) {
+    auto issue_loads = [&](int kt, bool a_part, bool b_part) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the builtin exists in the device pass only
         unsigned char *stage = lds2 + (kt % NST) * STAGE + wave * 16 * G2_ROW;
         const size_t k = (size_t)min(kt, KT - 1) * G2_BK;   // past the end: a harmless repeat into a dead stage
+        if (a_part)
 #pragma unroll
-        for (int i = 0; i < NA; ++i)
-            __builtin_amdgcn_global_load_lds(ga[i] + k, (lds_void *)(stage + i * 64 * G2_ROW), 16, 0, 0);
+            for (int i = 0; i < NA; ++i)
+                __builtin_amdgcn_global_load_lds(ga[i] + k, (lds_void *)(stage + i * 64 * G2_ROW), 16, 0, 0);
+        if (b_part)
 #pragma unroll
-        for (int i = 0; i < NB; ++i)
-            __builtin_amdgcn_global_load_lds(gb[i] + k, (lds_void *)(stage + A_BYTES + i * 64 * G2_ROW), 16, 0, 0);
+            for (int i = 0; i < NB; ++i)
+                __builtin_amdgcn_global_load_lds(gb[i] + k, (lds_void *)(stage + A_BYTES + i * 64 * G2_ROW), 16, 0, 0);
 #endif
     };
 
@@ -409,57 +438,29 @@ __global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const unsigned shor
     };
     constexpr int NMMA = WM * WN, NFR = WM + WN;
 
+    // issue order: A0 B0 A1 B1 .. A(NST-2) | K step 0: B(NST-2), A(NST-1) | K step 1: B(NST-1), A(NST) | ...
 #pragma unroll
-    for (int i = 0; i < NST - 1; ++i) issue_loads(i);
-    __builtin_amdgcn_s_waitcnt(vmcnt_imm((NST - 2) * NL));   // stage 0 of this wavefront has landed
+    for (int i = 0; i < NST - 2; ++i) issue_loads(i, true, true);
+    issue_loads(NST - 2, true, false);
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm((NST - 3) * NL + NA));   // stage 0 of this wavefront has landed
     __builtin_amdgcn_s_barrier();                            // ... and everybody else's
     Frag f0, f1;
     read_frag(f0, 0, 0);
     for (int kt = 0; kt < KT; ++kt) {
         // sub-step 0 while the fragments of sub-step 1 are read
         read_frag(f1, kt, 1);
+        issue_loads(kt + NST - 2, false, true);
         mma(f0);
-        // two MFMAs first: the wait in front of them then covers only reads issued long ago; all
-        // reads of the next fragment follow early, so that they are back when the next sub-step starts
-        if constexpr (WM >= 2) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-#pragma unroll
-            for (int i = 0; i < NFR; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            }
-            __builtin_amdgcn_sched_group_barrier(0x008, NMMA - 2 - NFR, 0);
-        }
+        if constexpr (WM >= 2) sched_half<NMMA, NFR, NB>();
         // stage kt+1 landed (stage kt+2 may still be in flight); past this barrier nobody reads stage kt-1
         __builtin_amdgcn_s_waitcnt(vmcnt_imm((NST - 3) * NL));
         __builtin_amdgcn_s_barrier();
         // sub-step 1 while fragments 0 of the next K step are read, then the loads of stage kt+3
         // (an LDS-writing load may not move above an LDS read: reads first)
         read_frag(f0, kt + 1, 0);
-        issue_loads(kt + NST - 1);
+        issue_loads(kt + NST - 1, true, false);
         mma(f1);
-        if constexpr (WM == 4) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-#pragma unroll
-            for (int i = 0; i < NFR; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            }
-#pragma unroll
-            for (int i = 0; i < NL / 2; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            }
-            __builtin_amdgcn_sched_group_barrier(0x008, NMMA - 2 - NFR - NL / 2, 0);
-        } else if constexpr (WM == 2) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-#pragma unroll
-            for (int i = 0; i < NFR; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            }
-        }
+        if constexpr (WM >= 2) sched_half<NMMA, NFR, NA>();
     }
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));                // no LDS-writing load may outlive the workgroup
 
