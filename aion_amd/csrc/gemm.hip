@@ -361,20 +361,15 @@ __device__ __forceinline__ void sched_half() {
     }
 }
 
+// one workgroup tile: rows m0 .., columns n0 .. of C (N is the column bound of W and C as passed)
 template <int WM, int NST, int WN>
-__global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const unsigned short *__restrict__ A, const unsigned short *__restrict__ W,
-                                                             float *__restrict__ c, int M, int N, int K, size_t ldc, float alpha,
-                                                             float beta, int tiles_m, int tiles) {
-    extern __shared__ __attribute__((aligned(1024))) unsigned char lds2[];
+__device__ __forceinline__ void gemm_bf16_tile(unsigned char *lds2, const unsigned short *__restrict__ A, const unsigned short *__restrict__ W,
+                                               float *__restrict__ c, int M, int N, int K, size_t ldc, float alpha, float beta, int m0, int n0) {
     constexpr int BM2 = WM * 64;
     constexpr int BN2 = WN * 64;                             // 256 columns, or 192 for the last partial round of tiles
     constexpr int A_BYTES = BM2 * G2_ROW, B_BYTES = BN2 * G2_ROW, STAGE = A_BYTES + B_BYTES;
     constexpr int NA = WM, NB = WN;                          // wavefront loads (16 rows each) per stage
     constexpr int NL = NA + NB;
-    const int per_xcd = (int)gridDim.x >> 3;
-    const int t = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
-    if (t >= tiles) return;
-    const int m0 = (t % tiles_m) * BM2, n0 = (t / tiles_m) * BN2;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l31 = lane & 31, lh = lane >> 5;
     const int wrow = (wave >> 1) * (WM * 32), wcol = (wave & 1) * (WN * 32);
@@ -480,6 +475,45 @@ __global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const unsigned shor
                 *dst = beta == 0.f ? v : v + beta * *dst;
             }
         }
+}
+
+template <int WM, int NST, int WN>
+__global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const unsigned short *__restrict__ A, const unsigned short *__restrict__ W,
+                                                             float *__restrict__ c, int M, int N, int K, size_t ldc, float alpha,
+                                                             float beta, int tiles_m, int tiles) {
+    extern __shared__ __attribute__((aligned(1024))) unsigned char lds2[];
+    const int per_xcd = (int)gridDim.x >> 3;
+    const int t = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
+    if (t >= tiles) return;
+    gemm_bf16_tile<WM, NST, WN>(lds2, A, W, c, M, N, K, ldc, alpha, beta, (t % tiles_m) * (WM * 64), (t / tiles_m) * (WN * 64));
+}
+
+// 256-row tiles over N = tw * 256 + (a rest covered by tn tiles of 192 columns), ONE launch: the column tiles go
+// wide, wide, narrow, narrow, ... while both kinds last. A CU's first tile is then wide on half of the CUs and narrow on the
+// other half, the CUs that finish early pick up wide tiles next, and the epilogues (64 MB of f32 stores that would otherwise
+// hit the HBM from every CU at the same moment, with the matrix pipes idle) fall into the others' main loops.
+template <int NST>
+__global__ __launch_bounds__(256) void gemm_bf16_mixed_kernel(const unsigned short *__restrict__ A, const unsigned short *__restrict__ W,
+                                                              float *__restrict__ c, int M, int N, int K, size_t ldc, float alpha,
+                                                              float beta, int tiles_m, int tw, int tn) {
+    extern __shared__ __attribute__((aligned(1024))) unsigned char lds2[];
+    const int per_xcd = (int)gridDim.x >> 3;
+    const int t = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
+    if (t >= tiles_m * (tw + tn)) return;
+    const int cg = t / tiles_m, m0 = (t % tiles_m) * 256;
+    const int fb = min(tw, tn) >> 1;                         // whole blocks of wide, wide, narrow, narrow
+    bool wide;
+    int idx;
+    if (cg < 4 * fb) {
+        wide = (cg & 3) < 2;
+        idx = (cg >> 2) * 2 + (cg & 1);
+    } else {
+        const int rest = cg - 4 * fb, rest_wide = tw - 2 * fb;
+        wide = rest < rest_wide;
+        idx = 2 * fb + (wide ? rest : rest - rest_wide);
+    }
+    if (wide) gemm_bf16_tile<4, NST, 4>(lds2, A, W, c, M, N, K, ldc, alpha, beta, m0, idx * 256);
+    else gemm_bf16_tile<4, NST, 3>(lds2, A, W, c, M, N, K, ldc, alpha, beta, m0, tw * 256 + idx * 192);
 }
 
 template <int DT, int WM, int KC, bool SPLITK>
@@ -651,7 +685,7 @@ int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *cw, size_t m, const
                 if ((long)narrow * tm <= cus) { tn_wide = tn - rest; tn_narrow = narrow; }
             }
         }
-        static bool attr[4] = {false, false, false, false};
+        static bool attr[3] = {false, false, false};
         auto launch = [&](auto kernel, int idx, int lds, const unsigned short *wp, float *cp, size_t ncols, int tiles) -> int {
             if (!attr[idx]) {
                 HIP_TRY(ctx, hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
@@ -660,13 +694,20 @@ int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *cw, size_t m, const
             launch_k(ctx, kernel, dim3((unsigned)((tiles + 7) / 8 * 8)), dim3(256), lds, abf, wp, cp, (int)m, (int)ncols, (int)K, ldc, alpha, beta, tm, tiles);
             return AIONHIP_OK;
         };
-        const size_t wide_cols = tn_narrow ? (size_t)tn_wide * G2_BN : N;
-        if (wm == 4) rc = launch(gemm_bf16_wide_kernel<4, 4, 4>, 0, 4 * (256 + 256) * G2_ROW, w->bf16, c, wide_cols, tm * tn_wide);
-        else if (wm == 2) rc = launch(gemm_bf16_wide_kernel<2, 4, 4>, 1, 4 * (128 + 256) * G2_ROW, w->bf16, c, wide_cols, tm * tn_wide);
-        else rc = launch(gemm_bf16_wide_kernel<1, 4, 4>, 2, 4 * (64 + 256) * G2_ROW, w->bf16, c, wide_cols, tm * tn_wide);
-        if (rc) return rc;
-        if (tn_narrow)
-            rc = launch(gemm_bf16_wide_kernel<4, 4, 3>, 3, 4 * (256 + 192) * G2_ROW, w->bf16 + wide_cols * K, c + wide_cols, N - wide_cols, tm * tn_narrow);
+        if (tn_narrow) {
+            // both kinds of tiles in one launch, interleaved (gemm_bf16_mixed_kernel)
+            static bool attr_mixed = false;
+            constexpr int lds = 4 * (256 + 256) * G2_ROW;
+            if (!attr_mixed) {
+                HIP_TRY(ctx, hipFuncSetAttribute((const void *)gemm_bf16_mixed_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+                attr_mixed = true;
+            }
+            const int tiles = tm * (tn_wide + tn_narrow);
+            launch_k(ctx, gemm_bf16_mixed_kernel<4>, dim3((unsigned)((tiles + 7) / 8 * 8)), dim3(256), lds, abf, w->bf16, c, (int)m, (int)N, (int)K, ldc, alpha, beta,
+                     tm, tn_wide, tn_narrow);
+        } else if (wm == 4) rc = launch(gemm_bf16_wide_kernel<4, 4, 4>, 0, 4 * (256 + 256) * G2_ROW, w->bf16, c, N, tm * tn_wide);
+        else if (wm == 2) rc = launch(gemm_bf16_wide_kernel<2, 4, 4>, 1, 4 * (128 + 256) * G2_ROW, w->bf16, c, N, tm * tn_wide);
+        else rc = launch(gemm_bf16_wide_kernel<1, 4, 4>, 2, 4 * (64 + 256) * G2_ROW, w->bf16, c, N, tm * tn_wide);
         if (rc) return rc;
     }
     LAUNCH_CHECK(ctx, "gemm_bf16");
