@@ -120,8 +120,11 @@ def test_bf16_gemm_ragged_shapes(gpu, orc, dtype, layout, m, n, k):
         gpu.set_gemm_mode(be.GEMM_EXACT_I8)
 
 
+# (2048, 14336): 32 column tiles of 256 and 32 of 192 interleaved in one launch (wide, wide, narrow, narrow, ...);
+# (2048, 9092): 32 of 256 and 5 of 192 - two whole blocks of that pattern, then the rest of the wide tiles, then the last
+# narrow one, which also hangs over the last column. Rows from every 256-row tile, all columns.
 @pytest.mark.parametrize("dtype,layout", [(be.Q8_0, be.ROWS_NK), (be.Q4_0, be.KMAJOR_KN)])
-@pytest.mark.parametrize("m,n", [(512, 4096), (2048, 14336)])
+@pytest.mark.parametrize("m,n", [(512, 4096), (2048, 14336), (2048, 9092)])
 def test_config3_bf16_full_size_on_row_sample(gpu, orc, dtype, layout, m, n):
     k = 4096
     say("config3 bf16", dtype, m, n)
@@ -130,7 +133,7 @@ def test_config3_bf16_full_size_on_row_sample(gpu, orc, dtype, layout, m, n):
         blocks, w = make_weight(gpu, dtype, layout, n, k, seed=n + 1)
         a = bf16_round(np.random.default_rng(m + 1).standard_normal((m, k)).astype(np.float32))
         got = gpu.matmul(w, a)
-        rows = np.array([0, 17, 255, 256, m // 2, m - 1])
+        rows = np.unique(np.array([0, 17, 255, 256, m // 2, m - 1] + [t * 256 + 29 * (t + 1) for t in range(m // 256)]))
         f32a = orc.matmul_q_f32a(dtype, layout == be.ROWS_NK, np.ascontiguousarray(a[rows]), blocks, n, threads=8)
         r = rms_err(got[rows], f32a)
         say("  max|err|/rms vs f32-A dequant", r)
