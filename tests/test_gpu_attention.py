@@ -214,8 +214,8 @@ def test_prefill_config4_sizes(gpu, orc):
     # BASELINE config 4a at L = 1024 and 2048: 8 q heads / 1 kv head, head size 256, bf16, scale 1/16, causal;
     # every row against the f64 reference (1e-2: bf16 MFMA operands). L = 512 is 32 prefill workgroups (an
     # eighth of the CUs: 16-row split kernel); L = 1024 and 2048 run on the prefill kernel with the key range of
-    # every row tile cut into 4 and 2 segments that a merge pass folds. At L = 4096 the oracle is too slow,
-    # so the kernel is held to properties that do not depend on the size: V = const gives that const back (the
+    # every row tile cut into 4 and 2 segments that a merge pass folds. At L = 4096 the oracle is too slow for every row,
+    # so the kernel is held to a sample of 30 positions over the whole range and to properties that do not depend on the size: V = const gives that const back (the
     # probabilities of a row sum to one), and row 0 sees key 0 only.
     for L, kernel in ((512, "attn_flash_split"), (1024, "attn_prefill"), (2048, "attn_prefill")):
         say("prefill config 4 L%d" % L)
@@ -239,6 +239,14 @@ def test_prefill_config4_sizes(gpu, orc):
     # the last rows against the reference on the last 16 positions only (full key range)
     ref_tail = orc.attention_f64(qf[:, L - 16:], kf, vf, 1 / 16.0, positions=np.arange(L - 16, L, dtype=np.int32).reshape(1, 16))
     assert float(np.abs(got[:, L - 16:] - ref_tail).max()) < 1e-2
+    # and a sample of positions over the whole range against the reference: around the 128-row workgroup tiles (8 heads x 16
+    # positions each), around the middle of the key range, where a row tile's two key segments meet, and in between
+    idx = np.unique(np.array([1, 15, 16, 17, 63, 64, 200, 1000, 1023, 1024, 1025, 2040, 2047, 2048, 2049, 2111, 2112, 3000, 3071, 3072,
+                              4000, 4079, 4080] + list(range(777, 4096, 512))))
+    ref_s = orc.attention_f64(np.ascontiguousarray(qf[:, idx]), kf, vf, 1 / 16.0, positions=idx.astype(np.int32).reshape(1, -1))
+    err = float(np.abs(got[:, idx] - ref_s).max())
+    say("  L4096 sample of", idx.size, "positions: max err", err)
+    assert err < 1e-2
 
 
 @pytest.mark.parametrize("B,Lq,T,lens,kernel", [
