@@ -187,7 +187,7 @@ def main():
                          "kernel_us": {sh: round(us, 2) for sh, us in read_us.items()},
                          "GBps": round(step_bytes / (sum(read_us.values()) * 1e-6) / 1e9, 1),
                          "gemv_rate_over_plain_read_rate": round(sum(read_us.values()) / (avg_launch_ms * 1e3 * len(SHAPES)), 3),
-                         "note": "stream_read_kernel: 16-byte non-temporal loads only, cold data, same byte count per launch"}},
+                         "note": "stream_read_kernel: reads only (one contiguous 4 KiB piece per wavefront, 16-byte non-temporal loads), cold data, same byte count per launch"}},
     }
 
     out["config"]["arithmetic"] = "int8 activations x int4 weights, exact i32 block dots (v_dot4_i32_i8), f32 scale-accumulate"
