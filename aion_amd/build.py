@@ -8,7 +8,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libaion_hip.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-SOURCES = ["ctx.hip", "quant.hip", "weights.hip", "gemv.hip", "gemv_fused.hip", "gemv_ksplit.hip", "gemm.hip", "matmul.hip", "attention.hip", "glue.hip", "program.hip"]
+SOURCES = ["ctx.hip", "quant.hip", "weights.hip", "gemv.hip", "gemv_fused.hip", "gemv_ksplit.hip", "gemm.hip", "matmul.hip", "attention.hip", "attention_prefill.hip", "glue.hip", "program.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-result",
     # hipcc -O3 may otherwise form packed-f32 instructions, which have given wrong results on this pool
@@ -19,9 +19,14 @@ FLAGS = [
 ]
 
 
+# per-file additions: the prefill attention kernel keeps MFMA results in vector registers (its softmax reads the scores
+# where the MFMA wrote them; with the default form every score passes through an accumulation-register copy)
+EXTRA_FLAGS = {"attention_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
+
 def _compile(src):
     obj = os.path.join(CSRC, src[:-4] + ".o")
-    cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [HIPCC, *FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     err = "\n".join(l for l in r.stderr.splitlines() if noise not in l)

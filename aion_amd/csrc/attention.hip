@@ -14,122 +14,17 @@
 //       attn_merge_kernel (the flash-decoding split of cpu/exec/attention.zig:879-962).
 //     per-wavefront mode - a workgroup is four 16-row tiles, each wavefront walks its own key range; used
 //       for many query rows only when the hi+lo precise mode is on (see attn_prefill_kernel otherwise).
-// attn_prefill_kernel - many query rows: 128 rows per workgroup, K/V tiles shared through LDS, 32x32x16 MFMA
-//   (described at the kernel).
+// attn_prefill_kernel (attention_prefill.hip) - many query rows: 128 rows per workgroup, K/V tiles shared through LDS,
+//   32x32x16 MFMA (described at the kernel).
 // attn_generic_kernel - any head size / f32 K,V: one wavefront per query row, scores staged in
 //   global scratch. Slow; it exists so that every shape the op allows has a GPU path.
 //
 // Softmax uses exp2 on (s - m) * log2(e); aion's CPU path uses a 4th-order polynomial exp
 // (cpu/kernels/fast_math.zig:79-92, rel. err 4e-5), so results agree to ~1e-4, not bitwise.
-#include "common.h"
-
-#include <climits>
-#include <type_traits>
+#include "attention_common.h"
 
 namespace {
-
-using f16x8 = __attribute__((ext_vector_type(8))) _Float16;
-using bf16x8 = __attribute__((ext_vector_type(8))) __bf16;
-
-constexpr float LOG2E = 1.4426950408889634f;
-constexpr int TILE_KEYS = 32;
-
-struct AttnArgs {
-    const void *q, *k, *v;
-    float *out;
-    const int *positions, *kv_lengths;
-    float *partial;
-    int B, L, T, Hq, Hkv, groups, rows_total, row_tiles, nseg;
-    int ring;      // rolling caches: T (logical key t lives in row t % T); 0: row t is key t
-    int q_dtype, kv_dtype;
-    float scale, soft_cap;
-    unsigned win_left, win_right, win_chunk;
-};
-
-__device__ __forceinline__ unsigned short f32_to_bf16_bits(float x) {
-    unsigned u = __float_as_uint(x);
-    u += 0x7FFFu + ((u >> 16) & 1u);
-    return (unsigned short)(u >> 16);
-}
-__device__ __forceinline__ float bf16_bits_to_f32(unsigned short b) { return __uint_as_float((unsigned)b << 16); }
-
-template <int KV>
-__device__ __forceinline__ unsigned short to_half_bits(float x) {
-    if (KV == AIONHIP_F16) return __half_as_ushort(__float2half_rn(x));
-    return f32_to_bf16_bits(x);
-}
-template <int KV>
-__device__ __forceinline__ float from_half_bits(unsigned short b) {
-    if (KV == AIONHIP_F16) return __half2float(__ushort_as_half(b));
-    return bf16_bits_to_f32(b);
-}
-// two f32 -> one 32-bit word of two halves (RNE), low half first
-using f32x2 = __attribute__((ext_vector_type(2))) float;
-using bf16x2 = __attribute__((ext_vector_type(2))) __bf16;
-template <int KV>
-__device__ __forceinline__ unsigned pack2(float a, float b) {
-    if (KV == AIONHIP_F16) {
-        const __half2 h = __floats2half2_rn(a, b);
-        return *reinterpret_cast<const unsigned *>(&h);
-    }
-    // one v_cvt_pk_bf16_f32 (round to nearest even) instead of integer rounding per element
-    return __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2{a, b}, bf16x2));
-}
-template <int KV>
-__device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
-    if (KV == AIONHIP_F16)
-        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-}
-
-__device__ __forceinline__ float load_scalar(const void *p, int dtype, size_t i) {
-    if (dtype == AIONHIP_F32) return ((const float *)p)[i];
-    if (dtype == AIONHIP_F16) return __half2float(((const __half *)p)[i]);
-    return bf16_bits_to_f32(((const unsigned short *)p)[i]);
-}
-
-// AttentionWindow.keys (aion graph/graph.zig:160-167)
-__device__ __forceinline__ void window_keys(unsigned left, unsigned right, unsigned chunk, int pos, int kv_end, int &lo, int &hi) {
-    const long anchor = chunk > 0 ? (long)(pos / (int)chunk) * (int)chunk : pos;
-    const long span = chunk > 0 ? chunk : 1;
-    const long l = anchor - (anchor < (long)left ? anchor : (long)left);
-    long h = right == 0xFFFFFFFFu ? (long)INT_MAX : anchor + span + (long)right;
-    if (h > kv_end) h = kv_end;
-    lo = (int)l;
-    hi = (int)h;
-}
-
-// Rolling caches (aion storage/cache.zig:202-207, cpu/exec/attention.zig:1072-1075, 1150-1152): the cache length may
-// exceed the capacity, keys older than length - capacity are gone, and key t is read from row t % capacity.
-__device__ __forceinline__ int phys_key(int ring, int t) { return ring ? (int)((unsigned)t % (unsigned)ring) : t; }
-// The same for the keys of one tile, whose first key key0 is uniform: one modulo per tile (base), then an add and
-// a conditional subtract per key. Valid while a tile is no longer than the ring (the launcher sees to that).
-struct TileMap {
-    int key0, base, wrap;
-    __device__ __forceinline__ TileMap(int ring, int k0) : key0(k0), base(ring ? (int)((unsigned)k0 % (unsigned)ring) : k0), wrap(ring ? ring : INT_MAX) {}
-    __device__ __forceinline__ int row(int key) const {
-        const int r = base + (key - key0);
-        return r >= wrap ? r - wrap : r;
-    }
-};
-__device__ __forceinline__ int clip_kv_end(int ring, int t_cap, int kv_end_raw) {
-    return ring ? max(0, kv_end_raw) : max(0, min(kv_end_raw, t_cap));
-}
-__device__ __forceinline__ void clip_to_ring(int ring, int kv_end, int &lo, int &hi) {
-    if (ring) lo = max(lo, kv_end - ring);
-    if (hi < lo) hi = lo;
-}
-
-__device__ __forceinline__ int wave_min_i(int v) {
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) v = min(v, __shfl_xor(v, o, 64));
-    return v;
-}
-__device__ __forceinline__ int wave_max_i(int v) {
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) v = max(v, __shfl_xor(v, o, 64));
-    return v;
-}
+using namespace attn;
 
 // NW = wavefronts per workgroup: 4 in prefill mode, 8 in split mode (a decode over a short cache
 // is one workgroup whose eight wavefronts take one 32-key tile each)
@@ -521,580 +416,6 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
     }
 }
 
-// ------------------------------------------------------------------------------------------------
-// attn_prefill_kernel - many query rows (prefill), q already in the K/V element type or f32 (rounded).
-//   A workgroup owns 128 query rows of one (batch, kv head) - position-major, GQA head fastest - and
-//   walks the 32-key tiles of the union of their intervals once; K and V tiles are loaded by the whole
-//   workgroup and shared through LDS (double-buffered, one barrier per tile), so a K/V byte fetched
-//   from L2 feeds 128 rows instead of 16. Each wavefront owns 32 rows and works in the transposed
-//   form on v_mfma_f32_32x32x16:
-//       S^T[32 keys x 32 rows]  = K_tile[32 x D] . Q^T[D x 32]       A = K rows from LDS (16 B reads)
-//       O^T[D x 32 rows]       += V^T[D x 32 keys] . P^T[32 x 32]    A = V^T rows from LDS (8 B reads)
-//   so every accumulator, the running max and the running sum of a lane belong to ONE query row.
-//   V is transposed once per tile by the loading threads (two keys packed per 32-bit store into
-//   V^T[dv][key], row stride 72 B: stores and operand reads are bank-conflict-free); the k index of
-//   the second product is permuted (slot s of lane half h <-> key (s/4)*8 + 4h + s%4 of a 16-key step)
-//   so that the probabilities feed the MFMA straight from the S accumulators without a shuffle.
-constexpr int PF_ROWS = 128, PF_TK = 64, PF_VROW = 136;
-constexpr float PF_LAZY = 8.f;
-#ifndef PF_AHEAD
-#define PF_AHEAD 3
-#endif
-#ifndef PF_FLASH_BELOW
-#define PF_FLASH_BELOW 8   // prompts whose 128-row workgroups would fill under 1/PF_FLASH_BELOW of the CUs run on the 16-row split kernel
-#endif
-#ifndef PF_SEG_TILES
-#define PF_SEG_TILES 4     // fewest 64-key tiles a key segment of the prefill kernel is worth
-#endif
-#ifndef PF_PIPE_D
-#define PF_PIPE_D 256      // head sizes from here on run the software-pipelined tile loop
-#endif
-using f32x16 = __attribute__((ext_vector_type(16))) float;
-using u32x2 = __attribute__((ext_vector_type(2))) unsigned int;
-
-template <int D>
-struct PrefillCfg {
-    static constexpr int KROW = D * 2;                              // unpadded (filled by LDS-writing loads), chunk slots swizzled
-    static constexpr int K_BYTES = PF_TK * KROW;
-    static constexpr int V_BYTES = D * PF_VROW;
-    static constexpr int STAGE = K_BYTES + V_BYTES;
-    static constexpr int LDS_BYTES = 2 * STAGE + 64;
-};
-
-template <int KV>
-__device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
-    if (KV == AIONHIP_F16)
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-}
-
-template <int KV, int D, bool CAP, bool RING = false>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
-    const int ring = RING ? a.ring : 0;
-    extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
-    using Cfg = PrefillCfg<D>;
-    constexpr int KK = D / 16;          // k-steps of the first product
-    constexpr int NJ = D / 32;          // 32-wide dv tiles of the second product
-    constexpr int CPK = D / 8;          // 16-byte chunks per key row
-    constexpr int NKI = PF_TK * Cfg::KROW / 1024 / 4;   // K loads (1 KiB each) per wavefront per tile
-    constexpr int KEYS_PER_KI = 1024 / Cfg::KROW;       // keys covered by one K load
-    constexpr int V_ITEMS = (PF_TK / 2) * CPK;          // V (key pair, chunk) items per tile
-    constexpr int NVL = V_ITEMS / 256;
-    static_assert(NKI >= 1 && NVL >= 1, "head size below 64 is not handled here");
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int l31 = lane & 31, lh = lane >> 5;
-    const int unit = blockIdx.y, b = unit / a.Hkv, hk = unit % a.Hkv;
-
-    // ---- this lane's query row (lanes l and l+32 share it)
-    // row tiles in descending order: under a causal mask the last rows see the most keys, and workgroups are
-    // dispatched in index order - the long ones start first and the short ones fill the gaps at the end
-    const int r = ((int)gridDim.x - 1 - (int)blockIdx.x) * PF_ROWS + wave * 32 + l31;
-    const bool row_ok = r < a.rows_total;
-    const int li = row_ok ? r / a.groups : 0, gi = row_ok ? r % a.groups : 0;
-    const int hq = hk * a.groups + gi;
-    const int kv_end_raw = a.kv_lengths ? a.kv_lengths[b] : a.T;
-    const int pos_raw = (row_ok && a.positions) ? a.positions[(size_t)b * a.L + li] : li;
-    const size_t qbase = (((size_t)b * a.L + li) * a.Hq + hq) * D;
-
-    // Q^T operand: lane (row l31, half lh) holds d = 16*kk + 8*lh .. +7 for every kk
-    u32x4 qf[KK];
-    if (a.q_dtype == KV) {
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) qf[kk] = *(const u32x4 *)((const unsigned short *)a.q + qbase + kk * 16 + lh * 8);
-    } else if (a.q_dtype == AIONHIP_F32 && (((uintptr_t)a.q) & 15) == 0) {
-        // f32 queries (aion's decode graphs: f32 q over an f16 cache): 16-byte loads, all requested before the first is converted
-        f32x4 x0[KK], x1[KK];
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-            const f32x4 *qp = (const f32x4 *)((const float *)a.q + qbase + kk * 16 + lh * 8);
-            x0[kk] = qp[0];
-            x1[kk] = qp[1];
-        }
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk)
-            qf[kk] = u32x4{pack2<KV>(x0[kk].x, x0[kk].y), pack2<KV>(x0[kk].z, x0[kk].w), pack2<KV>(x1[kk].x, x1[kk].y), pack2<KV>(x1[kk].z, x1[kk].w)};
-    } else {
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-            float x[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) x[j] = load_scalar(a.q, a.q_dtype, qbase + kk * 16 + lh * 8 + j);
-            qf[kk] = u32x4{pack2<KV>(x[0], x[1]), pack2<KV>(x[2], x[3]), pack2<KV>(x[4], x[5]), pack2<KV>(x[6], x[7])};
-        }
-    }
-    if (!row_ok) {
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) qf[kk] = u32x4{0u, 0u, 0u, 0u};
-    }
-
-    const int kv_end = clip_kv_end(ring, a.T, kv_end_raw);
-    int lo = 0, hi = 0;
-    if (row_ok) {
-        window_keys(a.win_left, a.win_right, a.win_chunk, max(pos_raw, 0), kv_end, lo, hi);
-        clip_to_ring(ring, kv_end, lo, hi);
-    }
-    const bool live = hi > lo;
-    // wavefront: union (which tiles it computes) and intersection (which tiles need no mask)
-    const int w_lo = wave_min_i(live ? lo : INT_MAX), w_hi = wave_max_i(live ? hi : 0);
-    const int w_lo_max = wave_max_i(live ? lo : INT_MAX), w_hi_min = wave_min_i(live ? hi : 0);
-    // workgroup union through LDS
-    int *s_rng = (int *)(lds + 2 * Cfg::STAGE);
-    if (lane == 0) { s_rng[wave] = w_lo; s_rng[4 + wave] = w_hi; }
-    __syncthreads();
-    const int g_lo = min(min(s_rng[0], s_rng[1]), min(s_rng[2], s_rng[3]));
-    const int g_hi = max(max(s_rng[4], s_rng[5]), max(s_rng[6], s_rng[7]));
-    // key segments (a.nseg > 1: few row tiles on many CUs): workgroup z takes the z-th part of the union's tiles and
-    // leaves its unnormalized accumulators, reference maximum and sum in the partial buffer for attn_merge_kernel
-    const int nseg = a.nseg, seg = blockIdx.z;
-    int t_begin = g_lo / PF_TK, t_end = (g_hi + PF_TK - 1) / PF_TK;
-    bool nothing = g_hi <= g_lo;
-    if (nseg > 1 && !nothing) {
-        const int per = (t_end - t_begin + nseg - 1) / nseg;
-        t_begin += seg * per;
-        t_end = min(t_end, t_begin + per);
-        nothing = t_begin >= t_end;
-    }
-    float *part = nullptr;
-    if (nseg > 1) part = a.partial + ((size_t)(unit * a.row_tiles + (r >> 4)) * nseg + seg) * (16 * D + 32);
-    if (nothing) {                                      // nothing visible to any row: zeros / an empty partial
-        if (row_ok) {
-            float *o = nseg > 1 ? part + (r & 15) * D : a.out + qbase;
-            for (int d = lh * (D / 2); d < (lh + 1) * (D / 2); d += 4) *(f32x4 *)(o + d) = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (nseg > 1 && lh == 0) {
-                part[16 * D + (r & 15)] = -INFINITY;
-                part[16 * D + 16 + (r & 15)] = 0.f;
-            }
-        }
-        return;
-    }
-
-    const unsigned short *kp = (const unsigned short *)a.k;
-    const unsigned short *vp = (const unsigned short *)a.v;
-    const size_t kv_row = (size_t)a.Hkv * D;
-    const size_t kv_base = ((size_t)b * a.T * a.Hkv + hk) * D;
-    const int key_clamp_hi = g_hi - 1;
-
-    // ---- cooperative tile loads. K: global -> LDS directly, 1 KiB per instruction; the 16-byte chunk c of key k
-    // sits at slot c ^ swz(k), swz = k & 15 (k >> 1 & 7 for 128-byte rows), so that the 16 consecutive keys of
-    // an operand read hit 16 distinct bank groups. V: registers now, transposed stores after this tile's MFMAs.
-    // Keys outside the union are read from a clamped in-range key (masked scores / exact-zero probabilities).
-    const int k_key_in = (lane * 16) / Cfg::KROW, k_slot = ((lane * 16) % Cfg::KROW) / 16;
-    auto load_k = [&](int t, unsigned char *st) {
-#if defined(__HIP_DEVICE_COMPILE__)   // the builtin exists in the device pass only
-        const int key0 = t * PF_TK;
-        const TileMap tm(ring, key0);
-#pragma unroll
-        for (int i = 0; i < NKI; ++i) {
-            const int key = (wave * NKI + i) * KEYS_PER_KI + k_key_in;
-            const int swz = CPK >= 16 ? (key & 15) : ((key >> 1) & 7);
-            const int kabs = tm.row(min(max(key0 + key, g_lo), key_clamp_hi));
-            __builtin_amdgcn_global_load_lds(kp + kv_base + (size_t)kabs * kv_row + (k_slot ^ swz) * 8,
-                                             (lds_void *)(st + (wave * NKI + i) * 1024), 16, 0, 0);
-        }
-#endif
-    };
-    u32x4 vreg[NVL][2];
-    auto load_v = [&](int t) {
-        const int key0 = t * PF_TK;
-        const TileMap tm(ring, key0);
-#pragma unroll
-        for (int i = 0; i < NVL; ++i) {
-            const int id = tid + 256 * i, pair = (id & 15) + 16 * (id / (16 * CPK)), c = (id >> 4) % CPK;
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const int kabs = tm.row(min(max(key0 + pair * 2 + h, g_lo), key_clamp_hi));
-                vreg[i][h] = *(const u32x4 *)(vp + kv_base + (size_t)kabs * kv_row + c * 8);
-            }
-        }
-    };
-    auto store_v = [&](unsigned char *st) {
-#pragma unroll
-        for (int i = 0; i < NVL; ++i) {
-            const int id = tid + 256 * i, pair = (id & 15) + 16 * (id / (16 * CPK)), c = (id >> 4) % CPK;
-            unsigned char *vt = st + Cfg::K_BYTES + (c * 8) * PF_VROW + pair * 4;
-            const u32x4 x = vreg[i][0], y = vreg[i][1];
-            const unsigned xs[4] = {x.x, x.y, x.z, x.w}, ys[4] = {y.x, y.y, y.z, y.w};
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                *(unsigned *)(vt + (2 * w) * PF_VROW) = (xs[w] & 0xFFFFu) | (ys[w] << 16);
-                *(unsigned *)(vt + (2 * w + 1) * PF_VROW) = (xs[w] >> 16) | (ys[w] & 0xFFFF0000u);
-            }
-        }
-    };
-
-    f32x16 acc[NJ];
-#pragma unroll
-    for (int j = 0; j < NJ; ++j)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[j][i] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;
-    const float cap_inv = CAP ? 1.f / a.soft_cap : 0.f;
-
-    if constexpr (D < PF_PIPE_D) {
-    load_k(t_begin, lds);
-    load_v(t_begin);
-    store_v(lds);
-    __syncthreads();                                               // also waits for the K loads (fence)
-
-    // operand addresses: K row (kb*32 + l31) at slot (2*kk + lh) ^ swz(row); V^T row (j*32 + l31), keys of step s2
-    const int k_swz = CPK >= 16 ? (l31 & 15) : ((l31 >> 1) & 7);
-    const int k_row = l31 * Cfg::KROW;
-    const int v_off = Cfg::K_BYTES + l31 * PF_VROW + lh * 8;        // + j * 32 rows + s2 * 32 bytes (+16 for the second 4 keys)
-    for (int t = t_begin; t < t_end; ++t) {
-        const unsigned char *st = lds + ((t - t_begin) & 1) * Cfg::STAGE;
-        unsigned char *nx = lds + ((t - t_begin + 1) & 1) * Cfg::STAGE;
-        const bool more = t + 1 < t_end;
-        if (more) {
-            load_k(t + 1, nx);
-            load_v(t + 1);
-        }
-        const int key0 = t * PF_TK;
-        // Every wavefront computes every tile of the workgroup's union, also one that none of its own rows sees
-        // (all of its scores are then masked and it adds exact zeros): the wavefronts meet at the barrier below
-        // anyway, and a branch around the MFMAs makes the compiler carry the accumulators in vector registers
-        // and copy all of them to and from the accumulation registers on every tile.
-        {
-            // -- S^T = K . Q^T for the two 32-key halves (two independent accumulation chains)
-            f32x16 s[2];
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) s[kb][i] = 0.f;
-#pragma unroll
-            for (int kk = 0; kk < KK; ++kk) {
-                const int slot = ((2 * kk + lh) ^ k_swz) * 16;
-                const u32x4 k0 = *(const u32x4 *)(st + k_row + slot);
-                const u32x4 k1 = *(const u32x4 *)(st + 32 * Cfg::KROW + k_row + slot);
-                s[0] = mfma32<KV>(k0, qf[kk], s[0]);
-                s[1] = mfma32<KV>(k1, qf[kk], s[1]);
-            }
-            // issue order: the LDS reads run PF_AHEAD k-steps ahead of the MFMAs that consume them (left alone the
-            // compiler issues each read right before its MFMA, which then waits out the whole LDS latency)
-            __builtin_amdgcn_sched_group_barrier(0x100, 2 * PF_AHEAD, 0);
-#pragma unroll
-            for (int kk = 0; kk < KK - PF_AHEAD; ++kk) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-            }
-            __builtin_amdgcn_sched_group_barrier(0x008, 2 * PF_AHEAD, 0);
-            // -- lane holds keys key0 + kb*32 + (i/4)*8 + lh*4 + i%4 of row l31
-            float x[32];
-            const bool full = key0 >= w_lo_max && key0 + PF_TK <= w_hi_min;   // every key visible to every row
-#pragma unroll
-            for (int i = 0; i < 32; ++i) {
-                float v = s[i >> 4][i & 15] * a.scale;
-                if (CAP) v = a.soft_cap * tanhf(v * cap_inv);
-                x[i] = v;
-            }
-            if (!full) {                                                      // wavefront-uniform
-                const int kbase = key0 + lh * 4;
-#pragma unroll
-                for (int i = 0; i < 32; ++i) {
-                    const int key = kbase + (i >> 4) * 32 + ((i >> 2) & 3) * 8 + (i & 3);
-                    x[i] = (key >= lo && key < hi) ? x[i] : -INFINITY;
-                }
-            }
-            float mx = x[0];
-#pragma unroll
-            for (int i = 1; i < 32; ++i) mx = fmaxf(mx, x[i]);
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            // the reference maximum only moves when the tile's maximum exceeds it by more than PF_LAZY:
-            // probabilities stay below e^PF_LAZY (exact in the f32 sums, fine in the 16-bit operand) and the
-            // 2*D-register rescale of the accumulators becomes rare after the first tiles
-            const float m_new = mx > m_run + PF_LAZY ? mx : m_run;
-            float alpha = 1.f, rowsum = 0.f;
-            if (m_new > -INFINITY) {
-                alpha = m_run > -INFINITY ? __builtin_amdgcn_exp2f((m_run - m_new) * LOG2E) : 1.f;
-                const float mneg = -m_new * LOG2E;
-#pragma unroll
-                for (int i = 0; i < 32; ++i) {
-                    x[i] = __builtin_amdgcn_exp2f(fmaf(x[i], LOG2E, mneg));      // exp2(-inf) = 0 for masked keys
-                    rowsum += x[i];
-                }
-            } else {
-#pragma unroll
-                for (int i = 0; i < 32; ++i) x[i] = 0.f;
-            }
-            rowsum += __shfl_xor(rowsum, 32, 64);
-            l_run = l_run * alpha + rowsum;
-            m_run = m_new;
-            // P^T operand of 16-key step s2: slots 0..7 <- accumulator elements 8*s2 .. 8*s2+7
-            u32x4 pf[4];
-#pragma unroll
-            for (int s2 = 0; s2 < 4; ++s2)
-                pf[s2] = u32x4{pack2<KV>(x[8 * s2], x[8 * s2 + 1]), pack2<KV>(x[8 * s2 + 2], x[8 * s2 + 3]),
-                               pack2<KV>(x[8 * s2 + 4], x[8 * s2 + 5]), pack2<KV>(x[8 * s2 + 6], x[8 * s2 + 7])};
-            // -- O^T += V^T . P^T
-            if (__any(alpha != 1.f)) {              // wavefront-uniform and rare: must stay a branch, not a select
-                // The accumulators live in accumulation registers for the MFMAs. Written as plain C++ the multiply
-                // makes the compiler keep them in vector registers around this branch and copy all of them back and
-                // forth on the common path (several hundred moves per key tile). So: read, scale and write back each
-                // one here, with the register class pinned. The s_nops cover the waits between an MFMA result and
-                // its read, and between the write-back and the next MFMA, which the compiler cannot see in here.
-                asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory");
-#pragma unroll
-                for (int j = 0; j < NJ; ++j)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        float tmp;
-                        asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 1\n\tv_accvgpr_write_b32 %0, %1"
-                                     : "+a"(acc[j][i]), "=&v"(tmp) : "v"(alpha));
-                    }
-                asm volatile("s_nop 7" ::: "memory");
-            }
-            // key step outermost: consecutive MFMAs go to different accumulators
-#pragma unroll
-            for (int s2 = 0; s2 < 4; ++s2)
-#pragma unroll
-                for (int j = 0; j < NJ; ++j) {
-                    const unsigned char *vrow = st + v_off + j * 32 * PF_VROW + s2 * 32;
-                    const u32x2 va = *(const u32x2 *)(vrow), vb = *(const u32x2 *)(vrow + 16);
-                    acc[j] = mfma32<KV>(u32x4{va.x, va.y, vb.x, vb.y}, pf[s2], acc[j]);
-                }
-            __builtin_amdgcn_sched_group_barrier(0x100, 2 * PF_AHEAD, 1);
-#pragma unroll
-            for (int i = 0; i < 4 * NJ - 2 * PF_AHEAD; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 1);
-            }
-            __builtin_amdgcn_sched_group_barrier(0x008, 2 * PF_AHEAD, 1);
-        }
-        if (more) store_v(nx);
-        __syncthreads();                                           // also waits for this wavefront's K loads (fence)
-    }
-
-    } else {
-    // operand addresses: K row (kb*32 + l31) at slot (2*kk + lh) ^ swz(row); V^T row (j*32 + l31), keys of step s2
-    const int k_swz = CPK >= 16 ? (l31 & 15) : ((l31 >> 1) & 7);
-    const int k_row = l31 * Cfg::KROW;
-    const int v_off = Cfg::K_BYTES + l31 * PF_VROW + lh * 8;        // + j * 32 rows + s2 * 32 bytes (+16 for the second 4 keys)
-
-    // Head size 256 and up (below, the serial loop above is faster: fewer MFMAs per tile to hide anything behind).
-    // The loop is software-pipelined over the key tiles: iteration t computes S_t = K_t . Q^T, then the softmax of
-    // S_t (vector ALU) TOGETHER WITH O += V_(t-1)^T . P_(t-1) (matrix pipe) - one wavefront per SIMD has nobody else
-    // to fill the matrix pipe while it computes exponentials, so it has to overlap the two itself. P_(t-1) and the
-    // running statistics of tile t-1 are consistent with the accumulators; the rescale by alpha_t follows the product.
-    // LDS: K_t sits in stage t&1 (requested an iteration ahead), V_t is requested into registers in iteration t-1,
-    // transposed into stage t&1 at the top of iteration t and consumed in iteration t+1: one barrier per tile.
-    f32x16 sc[2];
-    u32x4 pf[4] = {};
-    auto tile_qk = [&](const unsigned char *st) __attribute__((always_inline)) {
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) sc[kb][i] = 0.f;
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-            const int slot = ((2 * kk + lh) ^ k_swz) * 16;
-            const u32x4 k0 = *(const u32x4 *)(st + k_row + slot);
-            const u32x4 k1 = *(const u32x4 *)(st + 32 * Cfg::KROW + k_row + slot);
-            sc[0] = mfma32<KV>(k0, qf[kk], sc[0]);
-            sc[1] = mfma32<KV>(k1, qf[kk], sc[1]);
-        }
-    };
-    // scaled (capped, masked) scores of the tile: lane holds keys key0 + kb*32 + (i/4)*8 + lh*4 + i%4 of row l31.
-    // No branch in this kernel may contain an MFMA on the output accumulators (the compiler would then carry them in
-    // vector registers and copy all of them to and from the accumulation registers on every tile), so the one
-    // wavefront-uniform branch of a tile - mask or no mask - sits here, around vector instructions only.
-    float x[32];
-    auto tile_scores = [&](int key0) __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < 32; ++i) {
-            float v = sc[i >> 4][i & 15] * a.scale;
-            if (CAP) v = a.soft_cap * tanhf(v * cap_inv);
-            x[i] = v;
-        }
-        const bool full = key0 >= w_lo_max && key0 + PF_TK <= w_hi_min;   // every key visible to every row
-        if (!full) {
-            // key = key0 + 4*lh + c_i is visible iff lo <= key < hi, i.e. (unsigned)(c_i - lo_rel) < span
-            const int lo_rel = lo - (key0 + lh * 4);
-            const unsigned span = (unsigned)(hi - lo);
-#pragma unroll
-            for (int i = 0; i < 32; ++i) {
-                const int c = (i >> 4) * 32 + ((i >> 2) & 3) * 8 + (i & 3);
-                x[i] = (unsigned)(c - lo_rel) < span ? x[i] : -INFINITY;
-            }
-        }
-    };
-    // softmax of x -> pf (next iteration's P^T operand), interleaved with the product of the previous tile
-    auto tile_softmax_pv = [&](auto with_pv_c, const unsigned char *vst) __attribute__((always_inline)) {
-        constexpr bool WITH_PV = decltype(with_pv_c)::value;
-        // The softmax is cut into 32 units of a few vector instructions, and the product of the previous tile into its
-        // NM MFMAs; unit group k is issued right behind MFMA k and a scheduling barrier keeps the pairs in this order
-        // (left to itself the compiler issues the whole softmax first and the MFMAs behind it). The V^T operand of
-        // MFMA k + PV_AHEAD is requested behind MFMA k.
-        //   units 0..7    partial maxima of four scores each (two chains)
-        //   unit  8       row maximum across the two lane halves, new reference maximum, alpha, exponent offset
-        //   units 9..24   two exponentials each, partial sums (two chains)
-        //   units 25..28  the four P^T operands of the next product
-        //   unit  29      row sum across the lane halves, running sum and maximum
-        constexpr int NM = 4 * NJ, UPM = 32 / NM, PV_AHEAD = NM >= 16 ? 4 : 2;
-        float mxp[2] = {-INFINITY, -INFINITY}, rs[2] = {0.f, 0.f};
-        float m_new = m_run, alpha = 1.f, mneg = 0.f;
-        u32x4 pn[4];
-        auto unit = [&](int u) __attribute__((always_inline)) {
-            if (u < 8) {
-                mxp[u & 1] = fmaxf(fmaxf(mxp[u & 1], fmaxf(x[4 * u], x[4 * u + 1])), fmaxf(x[4 * u + 2], x[4 * u + 3]));
-            } else if (u == 8) {
-                float mx = fmaxf(mxp[0], mxp[1]);
-                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                // the reference maximum only moves when the tile's maximum exceeds it by more than PF_LAZY:
-                // probabilities stay below e^PF_LAZY (exact in the f32 sums, fine in the 16-bit operand) and the
-                // 2*D-register rescale of the accumulators becomes rare after the first tiles
-                m_new = mx > m_run + PF_LAZY ? mx : m_run;
-                // branch-free: with nothing visible so far (m_new = -inf) the exponent's offset is 0 and every
-                // masked score still gives exp2(-inf) = 0
-                alpha = m_run > -INFINITY ? __builtin_amdgcn_exp2f((m_run - m_new) * LOG2E) : 1.f;
-                mneg = m_new > -INFINITY ? -m_new * LOG2E : 0.f;
-            } else if (u < 25) {
-                const int i0 = 2 * (u - 9);
-                x[i0] = __builtin_amdgcn_exp2f(fmaf(x[i0], LOG2E, mneg));
-                x[i0 + 1] = __builtin_amdgcn_exp2f(fmaf(x[i0 + 1], LOG2E, mneg));
-                rs[0] += x[i0];
-                rs[1] += x[i0 + 1];
-            } else if (u < 29) {
-                const int s2 = u - 25;
-                // P^T operand of 16-key step s2: slots 0..7 <- accumulator elements 8*s2 .. 8*s2+7
-                pn[s2] = u32x4{pack2<KV>(x[8 * s2], x[8 * s2 + 1]), pack2<KV>(x[8 * s2 + 2], x[8 * s2 + 3]),
-                               pack2<KV>(x[8 * s2 + 4], x[8 * s2 + 5]), pack2<KV>(x[8 * s2 + 6], x[8 * s2 + 7])};
-            } else if (u == 29) {
-                float rowsum = rs[0] + rs[1];
-                rowsum += __shfl_xor(rowsum, 32, 64);
-                l_run = l_run * alpha + rowsum;
-                m_run = m_new;
-            }
-        };
-        if (WITH_PV) {
-            // -- O^T += V^T . P^T of the previous tile; key step outermost: consecutive MFMAs go to different accumulators
-            auto v_operand = [&](int idx) __attribute__((always_inline)) {
-                const unsigned char *vrow = vst + v_off + (idx % NJ) * 32 * PF_VROW + (idx / NJ) * 32;
-                const u32x2 va = *(const u32x2 *)(vrow), vb = *(const u32x2 *)(vrow + 16);
-                return u32x4{va.x, va.y, vb.x, vb.y};
-            };
-            u32x4 vop[PV_AHEAD];
-#pragma unroll
-            for (int k = 0; k < PV_AHEAD; ++k) vop[k] = v_operand(k);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int k = 0; k < NM; ++k) {
-                acc[k % NJ] = mfma32<KV>(vop[k % PV_AHEAD], pf[k / NJ], acc[k % NJ]);
-                if (k + PV_AHEAD < NM) vop[k % PV_AHEAD] = v_operand(k + PV_AHEAD);
-#pragma unroll
-                for (int u = k * UPM; u < (k + 1) * UPM; ++u) unit(u);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        } else {
-#pragma unroll
-            for (int u = 0; u < 30; ++u) unit(u);
-        }
-        if (__any(alpha != 1.f)) {              // wavefront-uniform and rare: must stay a branch, not a select
-            // The accumulators live in accumulation registers for the MFMAs. Written as plain C++ the multiply
-            // makes the compiler keep them in vector registers around this branch and copy all of them back and
-            // forth on the common path (several hundred moves per key tile). So: read, scale and write back each
-            // one here, with the register class pinned. The s_nops cover the waits between an MFMA result and
-            // its read, and between the write-back and the next MFMA, which the compiler cannot see in here.
-            asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory");
-#pragma unroll
-            for (int j = 0; j < NJ; ++j)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    float tmp;
-                    asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 1\n\tv_accvgpr_write_b32 %0, %1"
-                                 : "+a"(acc[j][i]), "=&v"(tmp) : "v"(alpha));
-                }
-            asm volatile("s_nop 7" ::: "memory");
-        }
-#pragma unroll
-        for (int s2 = 0; s2 < 4; ++s2) pf[s2] = pn[s2];
-    };
-    auto pin_acc = [&]() __attribute__((always_inline)) {
-#pragma unroll
-        for (int j = 0; j < NJ; ++j)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) asm volatile("" : "+a"(acc[j][i]));
-    };
-    using yes = std::integral_constant<bool, true>;
-    using no = std::integral_constant<bool, false>;
-
-    // one tile's front half: V_t to LDS for the next iteration's product, requests for tile t+1, S_t
-    auto tile_front = [&](int t) __attribute__((always_inline)) {
-        unsigned char *st = lds + ((t - t_begin) & 1) * Cfg::STAGE;
-        unsigned char *other = lds + ((t - t_begin + 1) & 1) * Cfg::STAGE;
-        store_v(st);
-        // unconditional (a branch would split the block): past the end the last tile is requested once more, into
-        // the stage and the registers that nobody reads again
-        const int tn = min(t + 1, t_end - 1);
-        load_k(tn, other);
-        load_v(tn);
-        tile_qk(st);
-        // issue order: the LDS reads run PF_AHEAD k-steps ahead of the MFMAs that consume them (left alone the
-        // compiler issues each read right before its MFMA, which then waits out the whole LDS latency)
-        __builtin_amdgcn_sched_group_barrier(0x100, 2 * PF_AHEAD, 0);
-#pragma unroll
-        for (int kk = 0; kk < KK - PF_AHEAD; ++kk) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, 2 * PF_AHEAD, 0);
-        tile_scores(t * PF_TK);
-    };
-
-    load_k(t_begin, lds);
-    load_v(t_begin);
-    __syncthreads();                                               // K of the first tile has landed (fence)
-    // first tile, peeled: there is no previous product to overlap with
-    tile_front(t_begin);
-    tile_softmax_pv(no{}, lds);
-    __syncthreads();
-    for (int t = t_begin + 1; t < t_end; ++t) {
-        // the accumulators are declared to sit in accumulation registers here and after the front half: without
-        // these two pins the register allocator parks them in vector registers while S_t is computed and copies all
-        // of them back for the product (2 x D/2 moves per tile)
-        pin_acc();
-        tile_front(t);
-        pin_acc();
-        tile_softmax_pv(yes{}, lds + ((t - t_begin + 1) & 1) * Cfg::STAGE);
-        __syncthreads();                                           // also waits for this wavefront's K loads (fence)
-    }
-    {   // the last tile's product
-        const unsigned char *vst = lds + ((t_end - 1 - t_begin) & 1) * Cfg::STAGE;
-        constexpr int NM = 4 * NJ, PV_AHEAD = 4;
-        auto v_operand = [&](int idx) __attribute__((always_inline)) {
-            const unsigned char *vrow = vst + v_off + (idx % NJ) * 32 * PF_VROW + (idx / NJ) * 32;
-            const u32x2 va = *(const u32x2 *)(vrow), vb = *(const u32x2 *)(vrow + 16);
-            return u32x4{va.x, va.y, vb.x, vb.y};
-        };
-        u32x4 vop[PV_AHEAD];
-#pragma unroll
-        for (int k = 0; k < PV_AHEAD; ++k) vop[k] = v_operand(k);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int k = 0; k < NM; ++k) {
-            acc[k % NJ] = mfma32<KV>(vop[k % PV_AHEAD], pf[k / NJ], acc[k % NJ]);
-            if (k + PV_AHEAD < NM) vop[k % PV_AHEAD] = v_operand(k + PV_AHEAD);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    }
-    }
-
-    if (row_ok) {
-        const float inv = nseg > 1 ? 1.f : (l_run > 0.f ? 1.f / l_run : 0.f);          // empty interval -> zeros
-        float *o = nseg > 1 ? part + (r & 15) * D : a.out + qbase;
-        if (nseg > 1 && lh == 0) {
-            part[16 * D + (r & 15)] = m_run;
-            part[16 * D + 16 + (r & 15)] = l_run;
-        }
-#pragma unroll
-        for (int j = 0; j < NJ; ++j)
-#pragma unroll
-            for (int q4 = 0; q4 < 4; ++q4) {
-                const f32x4 v = f32x4{acc[j][q4 * 4], acc[j][q4 * 4 + 1], acc[j][q4 * 4 + 2], acc[j][q4 * 4 + 3]} * inv;
-                *(f32x4 *)(o + j * 32 + q4 * 8 + lh * 4) = v;
-            }
-    }
-}
-
 // log-sum-exp merge of the key segments: one workgroup per (row tile, 16-wide dv slice, unit).
 // Thread = (segment group of 4, row of 16, 4 consecutive dv): it folds every fourth segment with all
 // of a round's loads in flight at once, then the four groups fold through LDS.
@@ -1167,53 +488,6 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnArgs a) {
     }
 }
 
-// The same merge for many rows and few segments (the prefill kernel's key segments): one thread per (row, four
-// consecutive dv), so that a wavefront reads whole contiguous rows of every segment's accumulators.
-template <int D>
-__global__ __launch_bounds__(256) void attn_merge_rows_kernel(AttnArgs a) {
-    constexpr int WSTRIDE = 16 * D + 32;
-    constexpr int TPR = D / 4, RPB = 256 / TPR;          // threads per row, rows per workgroup
-    constexpr int UN = 4;
-    const int unit = blockIdx.y, b = unit / a.Hkv, hk = unit % a.Hkv;
-    const int rr = blockIdx.x * RPB + (int)threadIdx.x / TPR, dv = ((int)threadIdx.x % TPR) * 4;
-    if (rr >= a.rows_total) return;
-    const int rt = rr >> 4, row = rr & 15;
-    const float *base = a.partial + (size_t)(unit * a.row_tiles + rt) * a.nseg * WSTRIDE;
-    float m_all = -INFINITY, l_all = 0.f;
-    f32x4 o = f32x4{0.f, 0.f, 0.f, 0.f};
-    for (int s0 = 0; s0 < a.nseg; s0 += UN) {
-        float ms[UN], ls[UN];
-        f32x4 os[UN];
-#pragma unroll
-        for (int u = 0; u < UN; ++u) {
-            const float *p = base + (size_t)min(s0 + u, a.nseg - 1) * WSTRIDE;      // clamped: every load is unconditional
-            ms[u] = p[16 * D + row];
-            ls[u] = p[16 * D + 16 + row];
-            os[u] = *(const f32x4 *)(p + row * D + dv);
-        }
-        float m_new = m_all;
-#pragma unroll
-        for (int u = 0; u < UN; ++u)
-            if (s0 + u < a.nseg) m_new = fmaxf(m_new, ms[u]);
-        if (m_new > -INFINITY) {
-            const float f0 = m_all > -INFINITY ? exp2f((m_all - m_new) * LOG2E) : 0.f;
-            o *= f0;
-            l_all *= f0;
-#pragma unroll
-            for (int u = 0; u < UN; ++u) {
-                const bool live = s0 + u < a.nseg && ms[u] > -INFINITY;
-                const float f = live ? exp2f((ms[u] - m_new) * LOG2E) : 0.f;
-                o += os[u] * f;
-                l_all += ls[u] * f;
-            }
-            m_all = m_new;
-        }
-    }
-    const int l2 = rr / a.groups, g3 = rr % a.groups;
-    const float inv = l_all > 0.f ? 1.f / l_all : 0.f;
-    *(f32x4 *)(a.out + (((size_t)b * a.L + l2) * a.Hq + hk * a.groups + g3) * D + dv) = o * inv;
-}
-
 // One wavefront per query row; any head sizes and element types. scores: [rows][T] f32 scratch.
 __global__ __launch_bounds__(256) void attn_generic_kernel(AttnArgs a, int d_k, int d_v, float *scores) {
     const int lane = threadIdx.x & 63;
@@ -1279,7 +553,8 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
     // (measured: one batch, one kv head, up to ~1024 positions x 8 heads): 16-row tiles spread the K/V reads
     // over many CUs, which outweighs re-reading K/V per row tile from L2.
     const int cus0 = ctx->cu_count > 0 ? ctx->cu_count : 256;
-    const bool split = a.rows_total <= 64 || (!HILO && (long)units * ((a.rows_total + PF_ROWS - 1) / PF_ROWS) * PF_FLASH_BELOW <= cus0);
+    const bool split = a.rows_total <= 64 || (!HILO && (long)units * ((a.rows_total + PF_ROWS - 1) / PF_ROWS) * PF_FLASH_BELOW <= cus0) ||
+                       (!HILO && !prefill_takes(a, D));      // e.g. a softmax scale that is not positive: the 16-row kernel takes any
     if (split) {
         // key segments: one 32-key tile per wavefront while that leaves the device under-filled,
         // more tiles per wavefront beyond one workgroup per CU (its LDS tiles fill a CU)
@@ -1310,41 +585,7 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
         }
         LAUNCH_CHECK(ctx, "attn_flash_split");
     } else if (!HILO) {
-        using PCfg = PrefillCfg<D>;
-        // No more workgroups than CUs: the key range of every row tile is cut into segments (at least
-        // PF_SEG_TILES tiles each) and the partial results are merged, as in the decode path. Measured at 8 heads
-        // x head size 256: L = 4096 (256 workgroups) 167 -> 136 us with two segments, L = 3072 125 -> 90 us.
-        const int wgs = units * ((a.rows_total + PF_ROWS - 1) / PF_ROWS);
-        const int key_tiles = (a.T + PF_TK - 1) / PF_TK;
-        int want = cus0 / max(wgs, 1);
-        if (want < 2 && wgs <= cus0) want = 2;      // one round of workgroups: two segments even out what a causal mask skews
-        int nseg = max(1, min(min(want, key_tiles / PF_SEG_TILES), 16));
-        a.nseg = nseg;
-        if (nseg > 1) {
-            const size_t bytes = (size_t)units * a.row_tiles * nseg * (16 * D + 32) * sizeof(float);
-            int rc = ensure_scratch2(ctx, bytes);
-            if (rc) return rc;
-            a.partial = (float *)ctx->scratch2;
-        }
-        static bool attr_pf[2] = {false, false};
-        const bool cap = a.soft_cap > 0.f;
-        const void *fn = cap ? (const void *)attn_prefill_kernel<KV, D, true, RING> : (const void *)attn_prefill_kernel<KV, D, false, RING>;
-        if (!attr_pf[cap]) {
-            HIP_TRY(ctx, hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, PCfg::LDS_BYTES));
-            attr_pf[cap] = true;
-        }
-        {
-            ProfScope scope(ctx, "attn_prefill");
-            const dim3 grid((unsigned)((a.rows_total + PF_ROWS - 1) / PF_ROWS), (unsigned)units, (unsigned)nseg);
-            if (cap) launch_k(ctx, attn_prefill_kernel<KV, D, true, RING>, grid, dim3(256), PCfg::LDS_BYTES, a);
-            else launch_k(ctx, attn_prefill_kernel<KV, D, false, RING>, grid, dim3(256), PCfg::LDS_BYTES, a);
-        }
-        if (nseg > 1) {
-            ProfScope scope(ctx, "attn_merge");
-            constexpr int RPB = 256 / (D / 4);
-            launch_k(ctx, attn_merge_rows_kernel<D>, dim3((unsigned)((a.rows_total + RPB - 1) / RPB), (unsigned)units), dim3(256), 0, a);
-        }
-        LAUNCH_CHECK(ctx, "attn_prefill");
+        return launch_prefill(ctx, a, D);
     } else {
         a.nseg = 1;
         static bool attr_prefill = false;

@@ -88,7 +88,7 @@ int rope_table(aionhip_ctx *ctx, int pairs, float freq_step, float scale_factor,
             return AIONHIP_OK;
         }
     if (ctx->capturing)
-        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "a RoPE table must be built while a program is being recorded: run the steps once before recording");
+        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "a RoPE table cannot be built while a program is being recorded: run the steps once before recording");
     std::vector<float> host((size_t)(pairs > 0 ? pairs : 1));
     float f = scale_factor;
     for (int i = 0; i < pairs; ++i) {

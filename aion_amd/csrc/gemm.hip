@@ -642,7 +642,7 @@ int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *cw, size_t m, const
         // the conversion launch has been accepted. A weight shared by several contexts must see its first bf16 call from
         // one of them alone.
         if (ctx->capturing)
-            return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "the bf16 copy of a weight must be built while a program is being recorded: run the steps once before recording");
+            return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "the bf16 copy of a weight cannot be built while a program is being recorded: run the steps once before recording");
         void *p = nullptr;
         HIP_TRY(ctx, hipMalloc(&p, N * K * 2));
         const size_t threads = N * (K / 8);
