@@ -94,6 +94,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
     constexpr int CPK = D / 8;          // 16-byte chunks per key row
     constexpr int NKI = PF_TK * Cfg::KROW / 1024 / 4;   // K loads (1 KiB each) per wavefront per tile
     constexpr int KEYS_PER_KI = 1024 / Cfg::KROW;       // keys covered by one K load
+    (void)KEYS_PER_KI;                                  // (the loads are in the device pass only)
     constexpr int V_ITEMS = (PF_TK / 2) * CPK;          // V (key pair, chunk) items per tile
     constexpr int NVL = V_ITEMS / 256;
     static_assert(NKI >= 1 && NVL >= 1, "head size below 64 is not handled here");
@@ -196,6 +197,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
     // an operand read hit 16 distinct bank groups. V: registers now, transposed stores after this tile's MFMAs.
     // Keys outside the union are read from a clamped in-range key (masked scores / exact-zero probabilities).
     const int k_key_in = (lane * 16) / Cfg::KROW, k_slot = ((lane * 16) % Cfg::KROW) / 16;
+    (void)k_key_in; (void)k_slot;
     auto load_k = [&](int t, unsigned char *st) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the builtin exists in the device pass only
         const int key0 = t * PF_TK;
@@ -405,6 +407,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
     // lane offset: a clamp and a 24-bit multiply-add per load. Keys outside the union are read from a clamped in-range key.
     const unsigned row_bytes = (unsigned)kv_row * 2u;
     const int ld_key = lane / CPK, ld_slot = lane % CPK;
+    (void)ld_key; (void)ld_slot;                          // used in the device pass only
     struct TileSrc {
         const unsigned char *base;    // uniform
         int rbase, rel_lo, rel_hi;    // uniform: first row of the tile (rolling caches), clamp bounds relative to the tile

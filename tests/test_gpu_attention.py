@@ -76,6 +76,28 @@ def test_prefill_causal_gqa(gpu, orc, kind, tol, D, L, kernel):
     assert float(np.abs(got - blocked).max()) < tol
 
 
+def test_prefill_head_256_stale_tail_odd_lengths_and_scales(gpu, orc):
+    """The head-size-256 prefill loop reads whole 64-key tiles by address arithmetic on a uniform tile base and takes
+    the row maximum before the softmax scale: a cache longer than the lengths in use whose tail holds NaN patterns,
+    lengths that end inside a tile, a large scale (scores far apart: the lazy reference maximum moves often), and a
+    scale that is not positive, which the 16-row kernel takes instead."""
+    B, L, T, Hq, Hkv, D = 2, 300, 1000, 8, 2, 256
+    (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(77, B, L, T, Hq, Hkv, D, "f16")
+    ends = np.array([911, 333], np.int32)
+    pos = np.stack([np.arange(e - L, e, dtype=np.int32) for e in ends])
+    for b in range(B):
+        k[b, ends[b]:] = np.nan
+        v[b, ends[b]:] = np.nan
+    # (the queries are rounded to f16 for the MFMA: the error of a score grows with the scale, hence the second bar)
+    for scale, kernel, tol in ((1 / 16.0, "attn_prefill", 2e-3), (0.25, "attn_prefill", 8e-3), (-0.05, "attn_flash_split", 2e-3)):
+        got = run_attention(gpu, q, k, v, scale, qd, kd, positions=pos, kv_lengths=ends)
+        assert gpu.last_kernel() == kernel
+        ref = orc.attention_f64(qf, kf, vf, scale, positions=pos, kv_lengths=ends)
+        err = float(np.abs(got - ref).max())
+        say("  scale", scale, "max err", err)
+        assert np.isfinite(got).all() and err < tol
+
+
 @pytest.mark.parametrize("kind,tol", [("f16", 2e-3), ("bf16", 1e-2)])
 @pytest.mark.parametrize("T,B", [(1024, 1), (1024, 8), (4096, 1), (4096, 8), (16384, 1), (16384, 8), (777, 3)])
 def test_decode_split_k(gpu, orc, kind, tol, T, B):
