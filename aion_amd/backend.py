@@ -126,6 +126,16 @@ class HipBackend:
         self._check(self._lib.aionhip_alloc(self._ctx, nbytes, alignment, C.byref(h)))
         return DeviceBuffer(self, h.value, nbytes)
 
+    def trim(self):
+        """Gives the blocks the context's pool has cached back to the device (waits for the stream)."""
+        self._check(self._lib.aionhip_trim(self._ctx))
+
+    def memory_stats(self):
+        """(bytes handed out by alloc and not yet freed, bytes of freed blocks the pool keeps for reuse)"""
+        live, cached = C.c_uint64(), C.c_uint64()
+        self._check(self._lib.aionhip_memory_stats(self._ctx, C.byref(live), C.byref(cached)))
+        return live.value, cached.value
+
     def upload(self, array):
         a = np.ascontiguousarray(array)
         buf = self.alloc(max(a.nbytes, 1))

@@ -8,6 +8,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "../../include/aion_hip.h"
@@ -35,6 +36,13 @@ struct aionhip_ctx {
     const char *last_kernel = "";
     int gemm_mode = AIONHIP_GEMM_EXACT_I8;
     int cu_count = 0;
+    // Device memory pool behind aionhip_alloc / aionhip_free. A freed block of up to POOL_MAX_BLOCK bytes is kept under
+    // its size class and handed out again to the next request of that class: everything this context does runs on one
+    // stream, so the reuse is ordered behind the last use without the device-wide wait a hipFree implies.
+    static constexpr size_t POOL_MAX_BLOCK = (size_t)64 << 20;
+    std::unordered_map<void *, size_t> pool_live;                  // block -> bytes of its size class
+    std::unordered_map<size_t, std::vector<void *>> pool_free;     // size class -> cached blocks
+    size_t pool_live_bytes = 0, pool_cached_bytes = 0;
     // prepared-activation scratch (int8 codes, per-block f32 scale, per-block code sum)
     void *scratch = nullptr;
     size_t scratch_bytes = 0;

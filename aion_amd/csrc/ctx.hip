@@ -172,6 +172,8 @@ int aionhip_create(int device, void *stream, aionhip_ctx **out) {
     return AIONHIP_OK;
 }
 
+static void pool_release_cached(aionhip_ctx *ctx);
+
 void aionhip_destroy(aionhip_ctx *ctx) {
     if (!ctx) return;
     (void)hipSetDevice(ctx->device);
@@ -186,6 +188,7 @@ void aionhip_destroy(aionhip_ctx *ctx) {
     if (ctx->scratch2) (void)hipFree(ctx->scratch2);
     if (ctx->ksplit) (void)hipFree(ctx->ksplit);
     if (ctx->tickets) (void)hipFree(ctx->tickets);
+    pool_release_cached(ctx);
     if (ctx->own_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }
@@ -221,26 +224,100 @@ int aionhip_device_info(aionhip_ctx *ctx, int *cu_count, int *wave_size, uint64_
     return AIONHIP_OK;
 }
 
+// Size classes of the pool: multiples of an eighth of the power of two below the request (at least 256 bytes), so a
+// block is at most 12.5 % larger than asked for and requests that differ a little share a class.
+static size_t pool_class(size_t bytes) {
+    if (bytes < 256) return 256;
+    size_t p2 = 256;
+    while (p2 <= bytes / 2) p2 <<= 1;                      // largest power of two <= bytes
+    const size_t step = p2 / 8 < 256 ? 256 : p2 / 8;
+    return (bytes + step - 1) / step * step;
+}
+
+static void pool_release_cached(aionhip_ctx *ctx) {
+    if (ctx->pool_cached_bytes == 0) return;
+    (void)hipStreamSynchronize(ctx->stream);               // cached blocks may still be read by work in flight
+    for (auto &kv : ctx->pool_free)
+        for (void *p : kv.second) (void)hipFree(p);
+    ctx->pool_free.clear();
+    ctx->pool_cached_bytes = 0;
+}
+
 int aionhip_alloc(aionhip_ctx *ctx, size_t bytes, size_t alignment, aionhip_handle *out) {
     if (!ctx || !out) return AIONHIP_INVALID_ARGUMENT;
     *out = 0;
-    if (alignment > 256 && (alignment & (alignment - 1)) != 0) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "alignment %zu is not a power of two", alignment);
+    if (alignment > 1 && (alignment & (alignment - 1)) != 0) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "alignment %zu is not a power of two", alignment);
+    const size_t cls = pool_class(bytes);
     void *p = nullptr;
-    // hipMalloc returns 256-byte aligned memory; larger alignments are met by over-allocation only
-    // up to 4 KiB pages, which hipMalloc also satisfies.
-    HIP_TRY(ctx, hipMalloc(&p, bytes ? bytes : 1));
-    if (alignment > 1 && ((uintptr_t)p % alignment) != 0) {
-        (void)hipFree(p);
-        return set_err(ctx, AIONHIP_UNSUPPORTED, "cannot satisfy alignment %zu", alignment);
+    auto it = ctx->pool_free.find(cls);
+    if (it != ctx->pool_free.end()) {
+        // a cached block of this class that also meets the alignment (hipMalloc aligns to 256 bytes and in practice to pages)
+        auto &v = it->second;
+        for (size_t i = v.size(); i-- > 0;) {
+            if (alignment <= 1 || ((uintptr_t)v[i] % alignment) == 0) {
+                p = v[i];
+                v.erase(v.begin() + (long)i);
+                ctx->pool_cached_bytes -= cls;
+                break;
+            }
+        }
+        if (v.empty()) ctx->pool_free.erase(it);
     }
+    if (!p) {
+        hipError_t e = hipMalloc(&p, cls);
+        if (e == hipErrorOutOfMemory && ctx->pool_cached_bytes) {      // give the cached blocks back and try once more
+            (void)hipGetLastError();
+            pool_release_cached(ctx);
+            e = hipMalloc(&p, cls);
+        }
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return set_err(ctx, e == hipErrorOutOfMemory ? AIONHIP_OUT_OF_MEMORY : AIONHIP_EXECUTION_FAILED, "hipMalloc(%zu): %s", cls, hipGetErrorString(e));
+        }
+        if (alignment > 1 && ((uintptr_t)p % alignment) != 0) {
+            (void)hipFree(p);
+            return set_err(ctx, AIONHIP_UNSUPPORTED, "cannot satisfy alignment %zu", alignment);
+        }
+    }
+    ctx->pool_live[p] = cls;
+    ctx->pool_live_bytes += cls;
     *out = (aionhip_handle)(uintptr_t)p;
     return AIONHIP_OK;
 }
 
 void aionhip_free(aionhip_ctx *ctx, aionhip_handle h) {
     if (!ctx || !h) return;
-    (void)hipStreamSynchronize(ctx->stream);
-    (void)hipFree((void *)(uintptr_t)h);
+    void *p = (void *)(uintptr_t)h;
+    auto it = ctx->pool_live.find(p);
+    if (it == ctx->pool_live.end()) {                      // not from aionhip_alloc of this context: plain release
+        (void)hipStreamSynchronize(ctx->stream);
+        (void)hipFree(p);
+        return;
+    }
+    const size_t cls = it->second;
+    ctx->pool_live.erase(it);
+    ctx->pool_live_bytes -= cls;
+    if (cls <= aionhip_ctx::POOL_MAX_BLOCK) {
+        ctx->pool_free[cls].push_back(p);
+        ctx->pool_cached_bytes += cls;
+    } else {
+        (void)hipStreamSynchronize(ctx->stream);
+        (void)hipFree(p);
+    }
+}
+
+int aionhip_trim(aionhip_ctx *ctx) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (ctx->capturing) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "trim waits for the stream and cannot be recorded into a program");
+    pool_release_cached(ctx);
+    return AIONHIP_OK;
+}
+
+int aionhip_memory_stats(aionhip_ctx *ctx, uint64_t *live_bytes, uint64_t *cached_bytes) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (live_bytes) *live_bytes = (uint64_t)ctx->pool_live_bytes;
+    if (cached_bytes) *cached_bytes = (uint64_t)ctx->pool_cached_bytes;
+    return AIONHIP_OK;
 }
 
 int aionhip_h2d(aionhip_ctx *ctx, aionhip_handle dst, size_t dst_offset, const void *src, size_t bytes) {

@@ -40,6 +40,8 @@ _SIGS = {
     "aionhip_device_info": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_uint64), C.c_char_p, C.c_size_t]),
     "aionhip_alloc": (C.c_int, [C.c_void_p, C.c_size_t, C.c_size_t, C.POINTER(C.c_uint64)]),
     "aionhip_free": (None, [C.c_void_p, C.c_uint64]),
+    "aionhip_trim": (C.c_int, [C.c_void_p]),
+    "aionhip_memory_stats": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "aionhip_h2d": (C.c_int, [C.c_void_p, C.c_uint64, C.c_size_t, C.c_void_p, C.c_size_t]),
     "aionhip_d2h": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64, C.c_size_t, C.c_size_t]),
     "aionhip_d2d": (C.c_int, [C.c_void_p, C.c_uint64, C.c_size_t, C.c_uint64, C.c_size_t, C.c_size_t]),

@@ -75,8 +75,16 @@ int aionhip_device_info(aionhip_ctx *ctx, int *cu_count, int *wave_size, uint64_
 
 /* ---- DeviceMemory.VTable (runtime/device_memory.zig:36-108); memory model = discrete,
  *      maxBindingBytes = unbounded (tensors are never chunked, storage/layout.zig:22-39) ------ */
+/* alloc / free go through a pool kept by the context: a freed block of up to 64 MiB stays with the context under its size
+ * class (at most 12.5 % above the request) and serves the next request of that class, in stream order, without the
+ * device-wide wait of a hipFree (aion's WebGPU backend keeps grow-only pooled device buffers the same way,
+ * backend/gpu/context.zig:80-110; its activations live in planned workspace slots, graph/program/workspace.zig:1-60).
+ * An allocation that fails for lack of memory releases the cached blocks and is tried once more. */
 int aionhip_alloc(aionhip_ctx *ctx, size_t bytes, size_t alignment, aionhip_handle *out);
 void aionhip_free(aionhip_ctx *ctx, aionhip_handle h);
+/* gives the cached blocks back to the device (waits for the stream); bytes handed out / bytes cached by the pool */
+int aionhip_trim(aionhip_ctx *ctx);
+int aionhip_memory_stats(aionhip_ctx *ctx, uint64_t *live_bytes, uint64_t *cached_bytes);
 int aionhip_h2d(aionhip_ctx *ctx, aionhip_handle dst, size_t dst_offset, const void *src, size_t bytes);
 int aionhip_d2h(aionhip_ctx *ctx, void *dst, aionhip_handle src, size_t src_offset, size_t bytes);
 int aionhip_d2d(aionhip_ctx *ctx, aionhip_handle dst, size_t dst_offset, aionhip_handle src, size_t src_offset, size_t bytes);

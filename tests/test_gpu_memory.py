@@ -1,0 +1,66 @@
+"""Device memory behind the DeviceMemory interface (aion runtime/device_memory.zig:36-108): the context's pool.
+A freed block serves the next request of its size class in stream order; nothing the pool does may change what a
+buffer holds while it is live."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def test_freed_blocks_are_reused_by_size_class(gpu):
+    gpu.trim()
+    live0, cached0 = gpu.memory_stats()
+    assert cached0 == 0
+    a = gpu.alloc(1000)
+    live1, _ = gpu.memory_stats()
+    assert live1 - live0 == 1024                     # classes below 2 KiB are multiples of 256 bytes
+    h = a.handle
+    a.free()
+    assert gpu.memory_stats() == (live0, 1024)
+    b = gpu.alloc(900)                               # same class: the cached block comes back
+    assert b.handle == h and gpu.memory_stats() == (live0 + 1024, 0)
+    c = gpu.alloc(5000)                              # another class: a block of its own
+    assert c.handle != h
+    live2, _ = gpu.memory_stats()
+    assert 5000 <= live2 - live0 - 1024 <= 5000 * 1.125 + 256
+    b.free(); c.free()
+    _, cached = gpu.memory_stats()
+    assert cached == live2 - live0
+    gpu.trim()
+    assert gpu.memory_stats() == (live0, 0)
+
+
+def test_reuse_is_ordered_behind_the_last_use(gpu):
+    """A block is freed while work that reads it is still in the stream, and handed out again at once: the new owner's
+    writes are enqueued behind that work, so the copy made from the old contents is intact."""
+    n = 1 << 20
+    src = np.arange(n, dtype=np.float32)
+    a = gpu.upload(src)
+    dst = gpu.alloc(n * 4)
+    gpu._check(gpu._lib.aionhip_d2d(gpu._ctx, dst.handle, 0, a.handle, 0, n * 4))      # reads `a`, asynchronous
+    h = a.handle
+    a.free()
+    b = gpu.alloc(n * 4)
+    assert b.handle == h
+    gpu._check(gpu._lib.aionhip_memset(gpu._ctx, b.handle, 0, 0, n * 4))                  # overwrites the block
+    assert np.array_equal(dst.numpy(np.float32, (n,)), src)
+    assert not gpu.download(b, np.float32, (n,)).any()
+    b.free(); dst.free()
+
+
+def test_large_blocks_alignment_and_foreign_handles(gpu):
+    gpu.trim()
+    live0, _ = gpu.memory_stats()
+    big = gpu.alloc((64 << 20) + 4096)               # above the pool's block limit: released on free, not cached
+    big.free()
+    assert gpu.memory_stats() == (live0, 0)
+    al = gpu.alloc(3000, alignment=4096)
+    assert al.handle % 4096 == 0
+    h = al.handle
+    al.free()
+    again = gpu.alloc(3000, alignment=4096)
+    assert again.handle == h                         # the cached block meets the alignment: it is the one handed out
+    again.free()
+    with pytest.raises(Exception):
+        gpu.alloc(100, alignment=48)                 # not a power of two
+    gpu.trim()
