@@ -20,7 +20,8 @@ The same JSON line carries the two other metrics BASELINE.json names, in a "seco
 its own: "prefill_gemm" (config 3's largest shape, M = 2048, N = 14336, K = 4096, q4: the exact int8 path and the bf16 MFMA
 path, TFLOP/s against the named MFMA peak, with the tolerance class of each) and "decode" (config 5: the 26-layer decoder,
 128-token prompt, greedy decode of 128 tokens at batch 1: tokens/s, ms/token, weight bytes streamed per second against the
-HBM peak), plus "sweep": config 2's q8 legs and batch 4 / 8 per shape. `--headline-only` skips the secondary object (and
+HBM peak), plus "sweep": config 2's q8 legs and batch 4 / 8 per shape, and "attention": config 4's longest prompt and
+largest decode shape. `--headline-only` skips the secondary object (and
 with it every stream capture: the form to run under rocprofv3, which does not survive a capture in the traced process).
 `--extras gemm,attention,decoder[,decoder_eager,package,package_bench_shape,package_bench_shape_eager]` adds the full config-3 and
 config-4 tables, the decoder with its CPU-oracle leg, and the package runner in an "extras" object.
@@ -204,7 +205,7 @@ def main():
         t.free()
     if not args.headline_only:
         out["secondary"] = {"prefill_gemm": run_gemm_headline(gpu, be), "decode": run_decode_headline(gpu, be),
-                            "sweep": run_sweep(gpu, be, host_blocks)}
+                            "sweep": run_sweep(gpu, be, host_blocks), "attention": run_attention_headline(gpu, be)}
     if extras:
         out["extras"] = {}
         if "gemm" in extras:
@@ -398,7 +399,7 @@ def _bf16_bits(x):
     return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
 
 
-def run_attention(gpu, be):
+def run_attention(gpu, be, prefill=(1024, 2048, 4096), decode=((1024, 1), (1024, 8), (4096, 1), (4096, 8), (16384, 1), (16384, 8))):
     """BASELINE config 4: 8 q heads / 1 kv head, head_dim 256, bf16 Q/K/V, scale 1/16, causal."""
     res = {}
     rng = np.random.default_rng(4)
@@ -421,7 +422,7 @@ def run_attention(gpu, be):
         per_call = sorted(sum(kernels[i * per:(i + 1) * per]) for i in range(iters))
         return per_call[iters // 2]
 
-    for L in (1024, 2048, 4096):
+    for L in prefill:
         q = gpu.upload(_bf16_bits(rng.standard_normal((1, L, Hq, D))))
         k = gpu.upload(_bf16_bits(rng.standard_normal((1, L, Hkv, D))))
         v = gpu.upload(_bf16_bits(rng.standard_normal((1, L, Hkv, D))))
@@ -435,8 +436,8 @@ def run_attention(gpu, be):
                                   "kernel": gpu.last_kernel()}
         for t in (q, k, v, o):
             t.free()
-    for T in (1024, 4096, 16384):
-        for B in (1, 8):
+    for T, B in decode:
+        if True:
             q = gpu.upload(_bf16_bits(rng.standard_normal((B, 1, Hq, D))))
             k = gpu.upload(_bf16_bits(rng.standard_normal((B, T, Hkv, D))))
             v = gpu.upload(_bf16_bits(rng.standard_normal((B, T, Hkv, D))))
@@ -450,6 +451,24 @@ def run_attention(gpu, be):
             for t in (q, k, v, o, pos, kl):
                 t.free()
     return res
+
+
+def run_attention_headline(gpu, be):
+    """Config 4 in the default line: the longest prompt and the largest decode shape of the table `--extras attention`
+    prints in full, each with its roofline block."""
+    full = run_attention(gpu, be, prefill=(4096,), decode=((16384, 8),))
+    pf, dc = full["prefill L4096"], full["decode T16384 B8"]
+    return {
+        "workload": "config 4: 8 q heads / 1 kv head, head size 256, bf16 Q/K/V, scale 1/16, causal",
+        "prefill_L4096": {"kernel_ms": pf["kernel_ms"], "TFLOPs": pf["TFLOPs"],
+                          "note": "tile kernel + merge of its two key segments; flop = 4 Hq D L (L + 1) / 2",
+                          "roofline": {"bound": "mfma", "achieved": pf["TFLOPs"], "peak": MFMA_PEAK["bf16"], "unit": "TFLOP/s",
+                                       "frac": pf["frac_mfma_peak"], "traffic": None, "peak_named": "dense bf16 MFMA"}},
+        "decode_T16384_B8": {"kernel_us": dc["kernel_us"],
+                             "note": "split-K kernel + merge; bytes = K and V of the cache once, queries and outputs",
+                             "roofline": {"bound": "hbm", "achieved": dc["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                                          "frac": dc["frac_hbm_peak"], "traffic": None}},
+    }
 
 
 def run_decoder_eager(gpu, be, steps=8):
