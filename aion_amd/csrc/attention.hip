@@ -26,6 +26,15 @@
 namespace {
 using namespace attn;
 
+using u32x2 = __attribute__((ext_vector_type(2))) unsigned int;
+template <int I, int E, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (I < E) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, E>(f);
+    }
+}
+
 // NW = wavefronts per workgroup: 4 in prefill mode, 8 in split mode (a decode over a short cache
 // is one workgroup whose eight wavefronts take one 32-key tile each)
 template <int D, int NW>
@@ -189,8 +198,10 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
     // K (MFMA operand layout, registers) of a tile is requested one tile ahead, right after the S MFMAs
     // have released the registers. V goes global -> LDS directly (global_load_lds_dwordx4, 1 KiB per
     // instruction) into this wavefront's tile, requested as soon as the previous tile's gathers are done.
-    // Tile layout: key row of D*2 bytes, 16-byte chunk c of key k at slot c ^ (2 * ((k >> 2) & 3)): the
-    // four key groups of a gather then read distinct banks. Keys outside the union interval are read from
+    // Tile layout: key row of D*2 bytes, 16-byte chunk c of key k at slot c ^ (2 * ((k >> 2) & 3)) ^ (8 * (k & 1)) (the
+    // last term for rows of 256 bytes and more; 128-byte rows alternate bank halves by themselves): the sixteen keys
+    // one transposing read of the second product covers (four key groups x four keys) then fall on eight distinct
+    // 32-byte bank ranges, two keys each - 512 bytes in the two passes they need anyway. Keys outside the union interval are read from
     // a clamped in-range key instead (their probabilities are exact zeros, and the cache tail may hold
     // anything, so the value must only be finite).
     constexpr int NVI = TILE_KEYS * D * 2 / 1024;
@@ -238,7 +249,7 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
             const int key = i * KEYS_PER_VI + v_key_in;
             // (key >> 2) & 3 does not depend on the lane while an instruction covers at most four keys
             const int grp = KEYS_PER_VI <= 4 ? ((i * KEYS_PER_VI) >> 2) & 3 : (key >> 2) & 3;
-            const int chunk = v_slot ^ (2 * grp);
+            const int chunk = v_slot ^ (2 * grp) ^ (D >= 128 ? 8 * (key & 1) : 0);
             const int kabs = tm.row(min(max(key0 + key, uni_lo), v_hi_key));
             if (near)
                 __builtin_amdgcn_global_load_lds(vb8 + (__umul24((unsigned)kabs, row_bytes) + (unsigned)chunk * 16u), (lds_void *)(vs + i * 1024), 16, 0, 0);
@@ -251,6 +262,10 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
         if (near) load_v_as(t, std::true_type{});
         else load_v_as(t, std::false_type{});
     };
+    // V^T operand addresses (second product): lane = 16*g + 4*r + q reads key 4g+r (and 16+4g+r), dv 16*mt + 4q .. +3
+    const int tr_r = (lane >> 2) & 3, tr_q = lane & 3;
+    const unsigned v_rowaddr = (unsigned)(size_t)(lds_void *)vs + (unsigned)((4 * g + tr_r) * Cfg::ROW_BYTES + (tr_q & 1) * 8);
+    const unsigned v_slot_l = (unsigned)(((tr_q >> 1) ^ (2 * g) ^ (D >= 128 ? 8 * (tr_r & 1) : 0)) << 4);
     if (t_begin < t_end) {
         load_k(t_begin);
         load_v(t_begin);
@@ -332,26 +347,33 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
 
         // -- O^T += V^T . P^T ; operand slot j of lane group g is key g*4+j (j<4) / 16+g*4+j-4
         const bool rescale = __any(alpha != 1.f);     // wavefront-uniform: skip 4*MT multiplies when no row's max moved
-        // element (key, dv) sits at key*ROW + ((dv/8) ^ 2g)*16 + (dv%8)*2; (key >> 2) & 3 == g for all 8 keys of a lane
-        const unsigned char *vcol = vs + (n & 7) * 2;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            unsigned short e[8];
-            const int coff = ((mt * 2 + (n >> 3)) ^ (2 * g)) * 16;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int key = j < 4 ? g * 4 + j : 16 + g * 4 + (j - 4);
-                e[j] = *(const unsigned short *)(vcol + key * Cfg::ROW_BYTES + coff);
-            }
-            const u32x4 vf = u32x4{(unsigned)e[0] | ((unsigned)e[1] << 16), (unsigned)e[2] | ((unsigned)e[3] << 16),
-                                   (unsigned)e[4] | ((unsigned)e[5] << 16), (unsigned)e[6] | ((unsigned)e[7] << 16)};
+        // The V^T operand of a 16-dv tile comes by two transposing LDS reads (ds_read_b64_tr_b16: within 16 lanes, lane
+        // 4r+q supplies the address of 4 consecutive dv of key r, lane i receives keys 0..3 of dv i): keys 4g+r and
+        // 16+4g+r of row-major V, dv 16*mt + 4q .. +3, which is the slot order above. Written as assembly and waited for
+        // by count: as a builtin the compiler would wait for every load in flight - the next tile's K - before the first.
+        constexpr int VA = 2;                                        // operands requested ahead
+        u32x4 vop[VA];
+        auto v_operand = [&](auto mt_c) __attribute__((always_inline)) {
+            constexpr int mt = decltype(mt_c)::value;
+            const unsigned addr = v_rowaddr + (v_slot_l ^ (unsigned)(mt << 5));
+            u32x2 a0, a1;
+            asm volatile("ds_read_b64_tr_b16 %0, %2\n\tds_read_b64_tr_b16 %1, %2 offset:%3"
+                         : "=&v"(a0), "=&v"(a1) : "v"(addr), "n"(16 * Cfg::ROW_BYTES) : "memory");
+            return u32x4{a0.x, a0.y, a1.x, a1.y};
+        };
+        static_for<0, VA>([&](auto mc) __attribute__((always_inline)) { vop[decltype(mc)::value] = v_operand(mc); });
+        static_for<0, MT>([&](auto mc) __attribute__((always_inline)) {
+            constexpr int mt = decltype(mc)::value;
+            constexpr int later = MT - 1 - mt < VA - 1 ? MT - 1 - mt : VA - 1;
+            asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(vop[mt % VA]) : "n"(2 * later));
             f32x4 c = acc[mt];
             if (rescale) c *= alpha;
-            c = mfma16<KV>(vf, pf, c);
-            if (HILO) c = mfma16<KV>(vf, pf_lo, c);
+            c = mfma16<KV>(vop[mt % VA], pf, c);
+            if (HILO) c = mfma16<KV>(vop[mt % VA], pf_lo, c);
             acc[mt] = c;
-        }
-        if (more) load_v(t + t_step);      // the gathers above are complete: their values fed the MFMAs
+            if constexpr (mt + VA < MT) vop[mt % VA] = v_operand(std::integral_constant<int, mt + VA>{});
+        });
+        if (more) load_v(t + t_step);      // the operand reads above are complete: each was waited for before its MFMA
     }
 
     if (!SPLIT) {
