@@ -32,7 +32,7 @@ constexpr float PF_LAZY = 8.f;
 #define PF_SEG_TILES 4     // fewest 64-key tiles a key segment of the prefill kernel is worth
 #endif
 #ifndef PF_PIPE_D
-#define PF_PIPE_D 256      // head sizes from here on run the software-pipelined tile loop
+#define PF_PIPE_D 128      // head sizes from here on run the software-pipelined tile loop
 #endif
 using f32x16 = __attribute__((ext_vector_type(16))) float;
 using u32x2 = __attribute__((ext_vector_type(2))) unsigned int;
@@ -371,7 +371,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
     }
 
     } else {
-    // Head size 256 and up (below, the serial loop above is faster: fewer MFMAs per tile to hide anything behind).
+    // Head sizes 128 and up (64 keeps the serial loop above: its key rows have 8 chunks, too few for the swizzles here).
+    // At head size 128 the kernel needs under 256 registers and half the LDS, so two workgroups share a CU and the
+    // softmax of one runs beside the MFMAs of the other as well.
     // The loop is software-pipelined over the key tiles: iteration t computes S_t = K_t . Q^T, then the softmax of
     // S_t (vector ALU) TOGETHER WITH O += V_(t-1)^T . P_(t-1) (matrix pipe) - one wavefront per SIMD has nobody else
     // to fill the matrix pipe while it computes exponentials, so it has to overlap the two itself. P_(t-1) and the
