@@ -545,10 +545,14 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
         float m_new = m_run, alpha = 1.f, mneg = 0.f;
         auto unit = [&](int u) __attribute__((always_inline)) {
             if (u < 8) {
-                // v_max3_f32 by hand: fmaxf on MFMA results first canonicalizes every input (one more instruction per score)
+                // v_max3_f32 by hand: fmaxf on MFMA results first canonicalizes every input (one more instruction per score).
+                // The compiler does not see that this assembly reads MFMA results, so the wait states a vector read of
+                // them needs behind the last MFMA of S_t (ten for an 8-pass MFMA) are put here, once per tile; the
+                // other units follow behind these.
+                if (u == 0) asm volatile("s_nop 7\n\ts_nop 3" ::: "memory");
                 float t;
-                asm("v_max3_f32 %0, %1, %2, %3" : "=v"(t) : "v"(mxp[u & 1]), "v"(sc[u >> 2][(4 * u) & 15]), "v"(sc[u >> 2][(4 * u + 1) & 15]));
-                asm("v_max3_f32 %0, %1, %2, %3" : "=v"(mxp[u & 1]) : "v"(t), "v"(sc[u >> 2][(4 * u + 2) & 15]), "v"(sc[u >> 2][(4 * u + 3) & 15]));
+                asm volatile("v_max3_f32 %0, %1, %2, %3" : "=v"(t) : "v"(mxp[u & 1]), "v"(sc[u >> 2][(4 * u) & 15]), "v"(sc[u >> 2][(4 * u + 1) & 15]));
+                asm volatile("v_max3_f32 %0, %1, %2, %3" : "=v"(mxp[u & 1]) : "v"(t), "v"(sc[u >> 2][(4 * u + 2) & 15]), "v"(sc[u >> 2][(4 * u + 3) & 15]));
             } else if (u == 8) {
                 const float mx = other_half_max(fmaxf(mxp[0], mxp[1])) * qscale;
                 // the reference maximum only moves when the tile's maximum exceeds it by more than PF_LAZY:
