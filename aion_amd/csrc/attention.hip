@@ -26,15 +26,6 @@
 namespace {
 using namespace attn;
 
-using u32x2 = __attribute__((ext_vector_type(2))) unsigned int;
-template <int I, int E, class F>
-__device__ __forceinline__ void static_for(F &&f) {
-    if constexpr (I < E) {
-        f(std::integral_constant<int, I>{});
-        static_for<I + 1, E>(f);
-    }
-}
-
 // NW = wavefronts per workgroup: 4 in prefill mode, 8 in split mode (a decode over a short cache
 // is one workgroup whose eight wavefronts take one 32-key tile each)
 template <int D, int NW>

@@ -112,6 +112,17 @@ __device__ __forceinline__ int wave_max_i(int v) {
     return v;
 }
 
+using u32x2 = __attribute__((ext_vector_type(2))) unsigned int;
+// f(integral_constant<int, I>) for I in [I0, E): a loop whose index is a constant expression in the body (immediate
+// operands of assembly, if constexpr)
+template <int I, int E, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (I < E) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, E>(f);
+    }
+}
+
 // ---- prefill kernel (attention_prefill.hip): 128 query rows per workgroup, 64-key tiles
 constexpr int PF_ROWS = 128, PF_TK = 64;
 #ifndef PF_FLASH_BELOW

@@ -35,20 +35,12 @@ constexpr float PF_LAZY = 8.f;
 #define PF_PIPE_D 128      // head sizes from here on run the software-pipelined tile loop
 #endif
 using f32x16 = __attribute__((ext_vector_type(16))) float;
-using u32x2 = __attribute__((ext_vector_type(2))) unsigned int;
 
 using v4s16 = __attribute__((ext_vector_type(4))) short;
 typedef __attribute__((address_space(3))) v4s16 lds_v4s16;
 // Softmax units of the pipelined prefill loop (46 of them, see there) dealt out behind the nm MFMAs of the product by
 // issue cost: unit u goes behind MFMA k when the cost of units 0..u first exceeds k/nm of the total. Returns the first
 // unit that does NOT go behind MFMAs 0..k-1.
-template <int I, int E, class F>
-__device__ __forceinline__ void static_for(F &&f) {
-    if constexpr (I < E) {
-        f(std::integral_constant<int, I>{});
-        static_for<I + 1, E>(f);
-    }
-}
 constexpr int pf_unit_cost(int u) { return u < 8 ? 2 : (u == 8 ? 12 : (u < 41 ? 5 : (u < 45 ? 8 : 4))); }
 constexpr int pf_unit_end(int k, int nm) {
     int total = 0;
