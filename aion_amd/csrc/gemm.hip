@@ -685,7 +685,9 @@ int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *cw, size_t m, const
                 if ((long)narrow * tm <= cus) { tn_wide = tn - rest; tn_narrow = narrow; }
             }
         }
-        static bool attr[3] = {false, false, false};
+        // 64-row tiles that still leave CUs idle (few tokens against a narrow weight): 128 columns instead of 256, twice the workgroups
+        const bool half_cols = wm == 1 && (long)tm1 * tn < cus;
+        static bool attr[4] = {false, false, false, false};
         auto launch = [&](auto kernel, int idx, int lds, const unsigned short *wp, float *cp, size_t ncols, int tiles) -> int {
             if (!attr[idx]) {
                 HIP_TRY(ctx, hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
@@ -707,6 +709,7 @@ int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *cw, size_t m, const
                      tm, tn_wide, tn_narrow);
         } else if (wm == 4) rc = launch(gemm_bf16_wide_kernel<4, 4, 4>, 0, 4 * (256 + 256) * G2_ROW, w->bf16, c, N, tm * tn_wide);
         else if (wm == 2) rc = launch(gemm_bf16_wide_kernel<2, 4, 4>, 1, 4 * (128 + 256) * G2_ROW, w->bf16, c, N, tm * tn_wide);
+        else if (half_cols) rc = launch(gemm_bf16_wide_kernel<1, 4, 2>, 3, 4 * (64 + 128) * G2_ROW, w->bf16, c, N, tm * (int)((N + 127) / 128));
         else rc = launch(gemm_bf16_wide_kernel<1, 4, 4>, 2, 4 * (64 + 256) * G2_ROW, w->bf16, c, N, tm * tn_wide);
         if (rc) return rc;
     }
