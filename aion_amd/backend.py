@@ -230,11 +230,16 @@ class HipBackend:
     def step_add_i32(self, out, a, b, n):
         self._check(self._lib.aionhip_step_add_i32(self._ctx, out.handle, a.handle, b.handle, n))
 
-    def step_advance_state(self, dst_tokens, src_tokens, n_tokens, counters, delta=1):
-        """One launch: dst_tokens <- src_tokens (i32) and delta added to every scalar i32 buffer in `counters`."""
+    def step_advance_state(self, dst_tokens, src_tokens, n_tokens, counters, delta=1, log=None, log_index=None, log_capacity=0):
+        """One launch: dst_tokens <- src_tokens (i32) and delta added to every scalar i32 buffer in `counters`; with `log`,
+        the tokens also go to log[*log_index ..] (the index is read before the counters move and may be one of them)."""
         n = len(counters)
         arr = (C.c_uint64 * max(n, 1))(*[c.handle for c in counters])
-        self._check(self._lib.aionhip_step_advance_state(self._ctx, dst_tokens.handle, src_tokens.handle, n_tokens, arr, n, delta))
+        if log is None:
+            self._check(self._lib.aionhip_step_advance_state(self._ctx, dst_tokens.handle, src_tokens.handle, n_tokens, arr, n, delta))
+        else:
+            self._check(self._lib.aionhip_step_advance_state_log(self._ctx, dst_tokens.handle, src_tokens.handle, n_tokens, arr, n, delta,
+                                                                 log.handle, log_index.handle, log_capacity))
 
     # ---- programs (HIP graph replay of a recorded step sequence)
     def program_begin(self):

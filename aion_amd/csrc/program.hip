@@ -27,9 +27,19 @@ struct AdvanceArgs {
     int count;
 };
 // the loop state of a device-resident greedy decode in one launch: the produced token becomes the next input, the indices move on
-__global__ void advance_state_kernel(int *__restrict__ dst, const int *__restrict__ src, size_t n, AdvanceArgs a, int delta) {
+// log (optional, n <= 64 so that one wavefront does everything): log[*log_index + i] = src[i], *log_index read before any
+// counter moves (it may be one of them: the position a token was produced at)
+__global__ void advance_state_kernel(int *__restrict__ dst, const int *__restrict__ src, size_t n, AdvanceArgs a, int delta,
+                                     int *__restrict__ log, const int *__restrict__ log_index, int log_capacity) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) dst[i] = src[i];
+    int at = -1;
+    if (log) at = *log_index;
+    if (i < n) {
+        const int t = src[i];
+        dst[i] = t;
+        if (log && at >= 0 && (long)at + (long)i < (long)log_capacity) log[(size_t)at + i] = t;
+    }
+    __builtin_amdgcn_s_waitcnt(0);                  // the index has been read before a counter that may alias it moves
     if (blockIdx.x == 0 && (int)threadIdx.x < a.count) *a.counter[threadIdx.x] += delta;
 }
 }  // namespace
@@ -38,7 +48,15 @@ extern "C" {
 
 int aionhip_step_advance_state(aionhip_ctx *ctx, aionhip_handle dst_tokens, aionhip_handle src_tokens, size_t n_tokens,
                                const aionhip_handle *counters, size_t n_counters, int delta) {
+    return aionhip_step_advance_state_log(ctx, dst_tokens, src_tokens, n_tokens, counters, n_counters, delta, 0, 0, 0);
+}
+
+int aionhip_step_advance_state_log(aionhip_ctx *ctx, aionhip_handle dst_tokens, aionhip_handle src_tokens, size_t n_tokens,
+                                   const aionhip_handle *counters, size_t n_counters, int delta,
+                                   aionhip_handle log, aionhip_handle log_index, size_t log_capacity) {
     if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (log && (!log_index || (log & 3) || (log_index & 3) || n_tokens > 64 || log_capacity > 0x7FFFFFFFu))
+        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "advance_state: a token log needs an aligned index, at most 64 tokens per step and a capacity below 2^31");
     if (n_counters > 8 || (n_counters && !counters) || (n_tokens && (!dst_tokens || !src_tokens)))
         return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "advance_state: null operand or more than 8 counters");
     if (!n_tokens && !n_counters) return AIONHIP_OK;
@@ -51,7 +69,8 @@ int aionhip_step_advance_state(aionhip_ctx *ctx, aionhip_handle dst_tokens, aion
         a.counter[i] = (int *)(uintptr_t)counters[i];
     }
     const size_t blocks = n_tokens ? (n_tokens + 63) / 64 : 1;
-    advance_state_kernel<<<dim3((unsigned)blocks), dim3(64), 0, ctx->stream>>>((int *)(uintptr_t)dst_tokens, (const int *)(uintptr_t)src_tokens, n_tokens, a, delta);
+    advance_state_kernel<<<dim3((unsigned)blocks), dim3(64), 0, ctx->stream>>>((int *)(uintptr_t)dst_tokens, (const int *)(uintptr_t)src_tokens, n_tokens, a, delta,
+                                                                                    (int *)(uintptr_t)log, (const int *)(uintptr_t)log_index, (int)log_capacity);
     LAUNCH_CHECK(ctx, "advance_state");
     return AIONHIP_OK;
 }

@@ -119,6 +119,7 @@ class Decoder:
         self.one = gpu.upload(np.ones(1, np.int32))
         self.logits = gpu.alloc(cfg.vocab * 4)
         self.token = gpu.alloc(4)
+        self.history = gpu.alloc(cfg.max_seq * 4)       # token produced at each position (decode program's log)
         self.state = {}        # S -> activation buffers
         self.program = None
         self.pos = 0
@@ -210,8 +211,10 @@ class Decoder:
 
             def issue():
                 self._forward(1, b)
-                # advance the device-resident loop state: next id = argmax, positions/write index/kv length += 1
-                g.step_advance_state(b["ids"], self.token, 1, [b["positions"], b["write_index"], b["kv_len"]])
+                # advance the device-resident loop state: next id = argmax, positions/write index/kv length += 1; the token
+                # is also logged at the position it was produced at, so that a run of steps needs no read-back per step
+                g.step_advance_state(b["ids"], self.token, 1, [b["positions"], b["write_index"], b["kv_len"]],
+                                     log=self.history, log_index=b["positions"], log_capacity=self.cfg.max_seq)
             self.program = g.record_program(issue)
 
     def _set_decode_state(self, b, token, pos):
@@ -230,6 +233,17 @@ class Decoder:
         if read_token:
             return int(self.gpu.download(self.token, np.int32, (1,))[0])
         return None
+
+    def decode_run(self, n):
+        """Replays the decode program n times back to back (nothing is read back in between: the loop state and the token
+        log live on the device) and returns the n tokens."""
+        if self.pos + n > self.cfg.max_seq:
+            raise ValueError("cache capacity exhausted")
+        start = self.pos
+        for _ in range(n):
+            self.gpu.program_execute(self.program)
+        self.pos += n
+        return self.gpu.download(self.history, np.int32, (n,), offset=start * 4)
 
     def decode_step_eager(self, token):
         """The same step without a program (used by tests to check the replayed graph)."""
@@ -251,5 +265,5 @@ class Decoder:
         for bufs in self.state.values():
             for t in bufs.values():
                 t.free()
-        for t in (self.embed, self.gamma, self.one, self.logits, self.token):
+        for t in (self.embed, self.gamma, self.one, self.logits, self.token, self.history):
             t.free()

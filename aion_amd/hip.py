@@ -69,6 +69,8 @@ _SIGS = {
     "aionhip_step_rope_append": (C.c_int, [C.c_void_p] + [C.c_uint64] * 8 + [C.c_size_t] * 6 + [C.c_float] * 3),
     "aionhip_step_add_i32": (C.c_int, [C.c_void_p] + [C.c_uint64] * 3 + [C.c_size_t]),
     "aionhip_step_advance_state": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64, C.c_size_t, C.POINTER(C.c_uint64), C.c_size_t, C.c_int]),
+    "aionhip_step_advance_state_log": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64, C.c_size_t, C.POINTER(C.c_uint64), C.c_size_t, C.c_int,
+                                                 C.c_uint64, C.c_uint64, C.c_size_t]),
     "aionhip_program_begin": (C.c_int, [C.c_void_p]),
     "aionhip_program_end": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p)]),
     "aionhip_program_abort": (C.c_int, [C.c_void_p]),

@@ -315,6 +315,13 @@ int aionhip_step_add_i32(aionhip_ctx *ctx, aionhip_handle out, aionhip_handle a,
  * each of up to 8 distinct scalar i32 device values (positions, write index, visible end). */
 int aionhip_step_advance_state(aionhip_ctx *ctx, aionhip_handle dst_tokens, aionhip_handle src_tokens, size_t n_tokens,
                                const aionhip_handle *counters, size_t n_counters, int delta);
+/* The same, and the tokens are also written to log[*log_index .. + n_tokens) (i32; *log_index is a device scalar read
+ * before the counters move and may be one of them, e.g. the position; writes past log_capacity are dropped; at most 64
+ * tokens per step): a device-resident greedy loop then needs no read-back per step, the host collects the tokens when it
+ * wants them (aion's sessions keep the loop state on the device the same way, api/loaded_model.zig:735-827). */
+int aionhip_step_advance_state_log(aionhip_ctx *ctx, aionhip_handle dst_tokens, aionhip_handle src_tokens, size_t n_tokens,
+                                   const aionhip_handle *counters, size_t n_counters, int delta,
+                                   aionhip_handle log, aionhip_handle log_index, size_t log_capacity);
 
 /* ---- programs: record a fixed step sequence once, replay it per token ----------------------
  * Session.execute(prog) (backend/backend.zig:42-44) runs aion's ExecutableProgram step list; the

@@ -121,3 +121,23 @@ def test_recorded_program_replays_equal_eager_steps(gpu, orc):
             assert np.array_equal(la, lb), step       # same kernels, same inputs: bit-identical
     finally:
         a.close(); b.close()
+
+
+def test_decode_run_without_read_back_gives_the_same_tokens(gpu, orc):
+    """A run of program replays with the loop state and the token log on the device (nothing read back between steps)
+    against the same generation with a read-back after every step; then a second run continues where the first stopped."""
+    cfg = DecoderConfig(wdtype=be.Q4_0, **SMALL)
+    w = SyntheticWeights(cfg, 5)
+    a, b = Decoder(gpu, cfg, w), Decoder(gpu, cfg, w)
+    try:
+        prompt = np.random.default_rng(2).integers(0, cfg.vocab, 7).astype(np.int32)
+        ta, tb = a.prefill(prompt), b.prefill(prompt)
+        assert ta == tb
+        a.begin_decode(ta)
+        b.begin_decode(tb)
+        want = [b.decode_step() for _ in range(11)]
+        got = list(a.decode_run(6)) + list(a.decode_run(5))
+        assert got == want
+    finally:
+        a.close(); b.close()
+

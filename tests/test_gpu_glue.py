@@ -410,3 +410,23 @@ def test_unary_and_binary_steps(gpu, orc):
     assert np.array_equal(gpu.download(ab, np.float32, a.shape), a * a)
     for t in (xb, ob, ab, outb, bad):
         t.free()
+
+
+def test_advance_state_logs_tokens_at_a_device_index(gpu):
+    """advance_state with a token log: the tokens land at the index the counter held BEFORE the step moved it (the index
+    may be one of the counters), writes past the capacity are dropped, and the plain entry point is unchanged."""
+    ids, tok = gpu.upload(np.array([0], np.int32)), gpu.upload(np.array([41], np.int32))
+    pos, end = gpu.upload(np.array([3], np.int32)), gpu.upload(np.array([4], np.int32))
+    log = gpu.upload(np.full(6, -1, np.int32))
+    for step in range(4):                                   # positions 3, 4, 5 fit the log of 6, position 6 does not
+        gpu.write(tok, np.array([41 + step], np.int32))
+        gpu.step_advance_state(ids, tok, 1, [pos, end], log=log, log_index=pos, log_capacity=6)
+    assert list(gpu.download(log, np.int32, (6,))) == [-1, -1, -1, 41, 42, 43]
+    assert int(gpu.download(ids, np.int32, (1,))[0]) == 44
+    assert int(gpu.download(pos, np.int32, (1,))[0]) == 7 and int(gpu.download(end, np.int32, (1,))[0]) == 8
+    gpu.step_advance_state(ids, tok, 1, [pos])              # no log
+    assert int(gpu.download(pos, np.int32, (1,))[0]) == 8
+    assert list(gpu.download(log, np.int32, (6,))) == [-1, -1, -1, 41, 42, 43]
+    for t in (ids, tok, pos, end, log):
+        t.free()
+
