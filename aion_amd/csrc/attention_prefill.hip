@@ -51,6 +51,15 @@ constexpr int pf_unit_end(int k, int nm) {
     while (u < 46 && (run + pf_unit_cost(u)) * nm <= total * k) run += pf_unit_cost(u++);
     return u;
 }
+// A key segment's partial result for one 16-row tile: [16][D] accumulators, then the rows' reference maxima and sums.
+// Over a bf16 cache the accumulators are stored as f16 (the probabilities of the second product carry 8 bits, the f16
+// accumulators 11), each row scaled by a power of two so that any bf16 value range fits, with that scale as a third
+// per-row float; the values of a row stand in the order the lanes hold them (position j*32 + h*16 + q*4 + i holds dv
+// j*32 + q*8 + h*4 + i), 32 contiguous bytes per lane and dv tile. Half the bytes written by the tile kernel and read
+// by the merge: both are bound by the bytes they move (the workgroups of a round all store at the same time).
+constexpr bool pf_half_partials(int kv) { return kv == AIONHIP_BF16; }
+constexpr int pf_partial_bytes(int d, bool half) { return half ? 32 * d + 192 : 64 * d + 128; }
+
 template <int D>
 struct PrefillCfg {
     static constexpr int KROW = D * 2;                              // unpadded (filled by LDS-writing loads), chunk slots swizzled
@@ -164,15 +173,24 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
         t_end = min(t_end, t_begin + per);
         nothing = t_begin >= t_end;
     }
-    float *part = nullptr;
-    if (nseg > 1) part = a.partial + ((size_t)(unit * a.row_tiles + (r >> 4)) * nseg + seg) * (16 * D + 32);
+    constexpr bool HP = pf_half_partials(KV);
+    constexpr int PART_BYTES = pf_partial_bytes(D, HP);
+    unsigned char *part = nullptr;
+    if (nseg > 1) part = (unsigned char *)a.partial + ((size_t)(unit * a.row_tiles + (r >> 4)) * nseg + seg) * PART_BYTES;
+    float *part_stats = (float *)(part + (HP ? 32 * D : 64 * D));          // [16] maxima, [16] sums, (f16 form) [16] scales
     if (nothing) {                                      // nothing visible to any row: zeros / an empty partial
         if (row_ok) {
-            float *o = nseg > 1 ? part + (r & 15) * D : a.out + qbase;
-            for (int d = lh * (D / 2); d < (lh + 1) * (D / 2); d += 4) *(f32x4 *)(o + d) = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (HP && nseg > 1) {
+                unsigned char *o = part + (r & 15) * (D * 2) + lh * D;
+                for (int d = 0; d < D; d += 16) *(u32x4 *)(o + d) = u32x4{0u, 0u, 0u, 0u};
+            } else {
+                float *o = nseg > 1 ? (float *)part + (r & 15) * D : a.out + qbase;
+                for (int d = lh * (D / 2); d < (lh + 1) * (D / 2); d += 4) *(f32x4 *)(o + d) = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
             if (nseg > 1 && lh == 0) {
-                part[16 * D + (r & 15)] = -INFINITY;
-                part[16 * D + 16 + (r & 15)] = 0.f;
+                part_stats[r & 15] = -INFINITY;
+                part_stats[16 + (r & 15)] = 0.f;
+                if (HP) part_stats[32 + (r & 15)] = 1.f;
             }
         }
         return;
@@ -637,12 +655,40 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
     }
     }
 
-    if (row_ok) {
+    if (HP && nseg > 1) {
+        // f16 accumulators under a per-row power of two: 2^e <= max|acc| < 2^(e+1) (e clamped so that its inverse is a
+        // normal number; a row of zeros takes 1)
+        float amax = 0.f;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(acc[j][i]));
+        amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+        unsigned e = (__float_as_uint(amax) >> 23) & 0xFFu;
+        e = e == 0u ? 127u : min(e, 253u);
+        const float down = __uint_as_float((254u - e) << 23);
+        if (row_ok) {
+            if (lh == 0) {
+                part_stats[r & 15] = m_run;
+                part_stats[16 + (r & 15)] = l_run;
+                part_stats[32 + (r & 15)] = __uint_as_float(e << 23);
+            }
+            unsigned char *o = part + (r & 15) * (D * 2) + lh * 32;
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                unsigned w[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) w[i] = pack2<AIONHIP_F16>(acc[j][2 * i] * down, acc[j][2 * i + 1] * down);
+                *(u32x4 *)(o + j * 64) = u32x4{w[0], w[1], w[2], w[3]};
+                *(u32x4 *)(o + j * 64 + 16) = u32x4{w[4], w[5], w[6], w[7]};
+            }
+        }
+    } else if (row_ok) {
         const float inv = nseg > 1 ? 1.f : (l_run > 0.f ? 1.f / l_run : 0.f);          // empty interval -> zeros
-        float *o = nseg > 1 ? part + (r & 15) * D : a.out + qbase;
+        float *o = nseg > 1 ? (float *)part + (r & 15) * D : a.out + qbase;
         if (nseg > 1 && lh == 0) {
-            part[16 * D + (r & 15)] = m_run;
-            part[16 * D + 16 + (r & 15)] = l_run;
+            part_stats[r & 15] = m_run;
+            part_stats[16 + (r & 15)] = l_run;
         }
 #pragma unroll
         for (int j = 0; j < NJ; ++j)
@@ -656,16 +702,20 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
 
 // The same merge for many rows and few segments (the prefill kernel's key segments): one thread per (row, four
 // consecutive dv), so that a wavefront reads whole contiguous rows of every segment's accumulators.
-template <int D>
+__device__ __forceinline__ float half_bits_to_float(unsigned bits) { return (float)__builtin_bit_cast(_Float16, (unsigned short)bits); }
+
+template <int D, bool HP>
 __global__ __launch_bounds__(256) void attn_merge_rows_kernel(AttnArgs a) {
-    constexpr int WSTRIDE = 16 * D + 32;
+    constexpr int PART_BYTES = pf_partial_bytes(D, HP);
     constexpr int TPR = D / 4, RPB = 256 / TPR;          // threads per row, rows per workgroup
     constexpr int UN = 4;
     const int unit = blockIdx.y, b = unit / a.Hkv, hk = unit % a.Hkv;
     const int rr = blockIdx.x * RPB + (int)threadIdx.x / TPR, dv = ((int)threadIdx.x % TPR) * 4;
     if (rr >= a.rows_total) return;
     const int rt = rr >> 4, row = rr & 15;
-    const float *base = a.partial + (size_t)(unit * a.row_tiles + rt) * a.nseg * WSTRIDE;
+    const unsigned char *base = (const unsigned char *)a.partial + (size_t)(unit * a.row_tiles + rt) * a.nseg * PART_BYTES;
+    // f16 form: where dv .. dv+3 stand in the row (the order the tile kernel's lanes hold them)
+    const int pos = (dv & ~31) + ((dv >> 2) & 1) * 16 + ((dv >> 3) & 3) * 4;
     float m_all = -INFINITY, l_all = 0.f;
     f32x4 o = f32x4{0.f, 0.f, 0.f, 0.f};
     for (int s0 = 0; s0 < a.nseg; s0 += UN) {
@@ -673,10 +723,19 @@ __global__ __launch_bounds__(256) void attn_merge_rows_kernel(AttnArgs a) {
         f32x4 os[UN];
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
-            const float *p = base + (size_t)min(s0 + u, a.nseg - 1) * WSTRIDE;      // clamped: every load is unconditional
-            ms[u] = p[16 * D + row];
-            ls[u] = p[16 * D + 16 + row];
-            os[u] = *(const f32x4 *)(p + row * D + dv);
+            const unsigned char *p = base + (size_t)min(s0 + u, a.nseg - 1) * PART_BYTES;      // clamped: every load is unconditional
+            const float *st = (const float *)(p + (HP ? 32 * D : 64 * D));
+            ms[u] = st[row];
+            ls[u] = st[16 + row];
+            if (HP) {
+                const u32x2 h = *(const u32x2 *)(p + (row * D + pos) * 2);
+                const float sc = st[32 + row];
+                const unsigned w0 = h.x, w1 = h.y;
+                os[u] = f32x4{half_bits_to_float(w0 & 0xFFFFu), half_bits_to_float(w0 >> 16), half_bits_to_float(w1 & 0xFFFFu),
+                              half_bits_to_float(w1 >> 16)} * sc;
+            } else {
+                os[u] = *(const f32x4 *)((const float *)p + row * D + dv);
+            }
         }
         float m_new = m_all;
 #pragma unroll
@@ -716,7 +775,7 @@ int launch_prefill_t(aionhip_ctx *ctx, AttnArgs &a) {
     int nseg = max(1, min(min(want, key_tiles / PF_SEG_TILES), 16));
     a.nseg = nseg;
     if (nseg > 1) {
-        const size_t bytes = (size_t)units * a.row_tiles * nseg * (16 * D + 32) * sizeof(float);
+        const size_t bytes = (size_t)units * a.row_tiles * nseg * pf_partial_bytes(D, pf_half_partials(KV));
         int rc = ensure_scratch2(ctx, bytes);
         if (rc) return rc;
         a.partial = (float *)ctx->scratch2;
@@ -737,7 +796,7 @@ int launch_prefill_t(aionhip_ctx *ctx, AttnArgs &a) {
     if (nseg > 1) {
         ProfScope scope(ctx, "attn_merge");
         constexpr int RPB = 256 / (D / 4);
-        launch_k(ctx, attn_merge_rows_kernel<D>, dim3((unsigned)((a.rows_total + RPB - 1) / RPB), (unsigned)units), dim3(256), 0, a);
+        launch_k(ctx, attn_merge_rows_kernel<D, pf_half_partials(KV)>, dim3((unsigned)((a.rows_total + RPB - 1) / RPB), (unsigned)units), dim3(256), 0, a);
     }
     LAUNCH_CHECK(ctx, "attn_prefill");
     return AIONHIP_OK;
