@@ -47,6 +47,28 @@ CAL_ELEMS = 1 << 26   # the counter-calibration cast: 256 MiB read, 128 MiB writ
 MEASURED_TRAFFIC = {(4096, 4096): 9.655e6, (14336, 4096): 33.299e6, (4096, 14336): 33.879e6, (262144, 2048): 303.159e6}
 
 
+SETTLE_MS = 80.0
+
+
+def settle(gpu, fn, ms=SETTLE_MS):
+    """Untimed load ahead of a measurement: `ms` milliseconds of the same calls, queued with no gap before what is timed.
+    From idle the device needs 15-50 ms of a workload before its clocks settle (on one box: the four-GEMV step 70-73 us for
+    the first 100 steps, 65.4 after 250; the bf16 GEMM 238-281 us for its first 20 launches, 220 after 100; prefill attention
+    at L = 4096 105-112 us for its first 100 launches, 89 after 400), and what a decoder or a prompt sees is the settled rate. Returns the
+    number of calls made."""
+    ev0, ev1 = gpu.event(), gpu.event()
+    gpu.record(ev0)
+    for i in range(4):
+        fn(i)
+    gpu.record(ev1)
+    gpu.sync()
+    per = max(gpu.elapsed_ms(ev0, ev1) / 4, 1e-3)
+    n = int(ms / per) + 1
+    for i in range(n):
+        fn(4 + i)
+    return 4 + n
+
+
 def algorithmic_bytes(dtype_bytes, n, k, batch):
     return n * k // 32 * dtype_bytes + batch * (k + n) * 4
 
@@ -105,6 +127,7 @@ def main():
         for j in range(len(SHAPES)):
             gpu.step_matmul(ws[j], xs[j], batch, ys[j])
 
+    settled = settle(gpu, step)          # device conditioning, reported in config; then the W warm-up steps as asked
     for i in range(args.warmup):
         step(i)
     gpu.sync()
@@ -177,7 +200,10 @@ def main():
         "data": "synthetic",
         "config": {"workload": "config 2, q4_0 decode GEMV batch 1 over 4096x4096, 14336x4096, 4096x14336, 262144x2048 (one step = the four GEMVs incl. activation int8 preparation)",
                    "device": info["arch"], "cu_count": info["cu_count"], "weight_sets_rotated": n_sets,
-                   "step_algorithmic_bytes": step_bytes, "wall_ms_per_step": round(wall_ms / args.steps, 5)},
+                   "step_algorithmic_bytes": step_bytes, "wall_ms_per_step": round(wall_ms / args.steps, 5),
+                   "settling": "%d untimed steps (%.0f ms) ahead of the warm-up steps, and the same %.0f ms of load ahead of every "
+                               "secondary figure: the first 15-50 ms of a workload after idle run 5-25 %% slower while the clocks settle"
+                               % (settled, SETTLE_MS, SETTLE_MS)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": round(sum(MEASURED_TRAFFIC[sh] for sh in SHAPES) / len(SHAPES)),
@@ -269,16 +295,15 @@ def run_gemm_headline(gpu, be):
              "observed 1e-6. The parity path, not the throughput path: both operands carry a scale per 32-block, so every 16x16x32 "
              "MFMA is followed by 12 VALU instructions of rescaling, which bounds it near 15 % of the int8 peak")):
         gpu.set_gemm_mode(mode)
-        for _ in range(3):
-            gpu.step_matmul(w, x, m, y)
-        gpu.sync()
+        gpu.step_matmul(w, x, m, y)          # first call: the bf16 copy of the weight
+        settle(gpu, lambda i: gpu.step_matmul(w, x, m, y))
         gpu.profile_start()
-        for _ in range(10):
+        for _ in range(20):
             gpu.step_matmul(w, x, m, y)
         prof = [ms for (nm, ms) in gpu.profile_stop() if nm == kname]
-        ms = sum(prof) / 10
+        ms = sum(prof) / 20
         tf = 2.0 * m * n * k / (ms * 1e-3) / 1e12
-        res[key] = {"kernel_ms": round(ms, 4), "launches_per_call": len(prof) // 10, "TFLOPs": round(tf, 1), "note": note,
+        res[key] = {"kernel_ms": round(ms, 4), "launches_per_call": len(prof) // 20, "TFLOPs": round(tf, 1), "note": note,
                     "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_PEAK[peak], "unit": "TFLOP/s",
                                  "frac": round(tf / MFMA_PEAK[peak], 4), "traffic": None, "peak_named": "dense " + peak + " MFMA"}}
     gpu.set_gemm_mode(be.GEMM_EXACT_I8)
@@ -418,10 +443,8 @@ def run_attention(gpu, be, prefill=(1024, 2048, 4096), decode=((1024, 1), (1024,
     Hq, Hkv, D = 8, 1, 256
 
     def timed(name, shape, bufs, pos=None, kl=None, iters=10):
-        for _ in range(2):
-            gpu.step_attention(bufs[3], bufs[0], bufs[1], bufs[2], shape, 1 / 16.0, q_dtype=be.BF16, kv_dtype=be.BF16,
-                               query_positions=pos, kv_lengths=kl)
-        gpu.sync()
+        settle(gpu, lambda i: gpu.step_attention(bufs[3], bufs[0], bufs[1], bufs[2], shape, 1 / 16.0, q_dtype=be.BF16, kv_dtype=be.BF16,
+                                                 query_positions=pos, kv_lengths=kl))
         gpu.profile_start()
         for _ in range(iters):
             gpu.step_attention(bufs[3], bufs[0], bufs[1], bufs[2], shape, 1 / 16.0, q_dtype=be.BF16, kv_dtype=be.BF16,
