@@ -429,7 +429,7 @@ __device__ __forceinline__ void gemm_bf16_tile(unsigned char *lds2, const unsign
         for (int mi = 0; mi < WM; ++mi)
 #pragma unroll
             for (int ni = 0; ni < WN; ++ni)
-                acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, f.a[mi]), __builtin_bit_cast(bf16x8, f.b[ni]), acc[mi][ni], 0, 0, 0);
+                acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, f.b[ni]), __builtin_bit_cast(bf16x8, f.a[mi]), acc[mi][ni], 0, 0, 0);
     };
     constexpr int NMMA = WM * WN, NFR = WM + WN;
 
@@ -459,22 +459,33 @@ __device__ __forceinline__ void gemm_bf16_tile(unsigned char *lds2, const unsign
     }
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));                // no LDS-writing load may outlive the workgroup
 
-    // 32x32 accumulator layout: element i of lane l is row (i / 4) * 8 + (l / 32) * 4 + i % 4, column l % 32
+    // The products are taken transposed (weight fragment as the first operand): element i of lane l then belongs to output
+    // row l % 32 (a token) and column (i / 4) * 8 + (l / 32) * 4 + i % 4, so every four accumulator elements are four
+    // consecutive floats of a C row - 16-byte stores, a quarter of the store instructions of a lane-per-column layout.
+    const bool vec_ok = (((uintptr_t)c | (ldc * sizeof(float))) & 15) == 0;
 #pragma unroll
-    for (int mi = 0; mi < WM; ++mi)
+    for (int mi = 0; mi < WM; ++mi) {
+        const int row = m0 + wrow + mi * 32 + l31;
+        if (row >= M) continue;
+        float *crow = c + (size_t)row * ldc;
 #pragma unroll
-        for (int ni = 0; ni < WN; ++ni) {
-            const int col = n0 + wcol + ni * 32 + l31;
-            if (col >= N) continue;
+        for (int ni = 0; ni < WN; ++ni)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int row = m0 + wrow + mi * 32 + (i >> 2) * 8 + lh * 4 + (i & 3);
-                if (row >= M) continue;
-                float *dst = c + (size_t)row * ldc + col;
-                const float v = alpha * acc[mi][ni][i];
-                *dst = beta == 0.f ? v : v + beta * *dst;
+            for (int g = 0; g < 4; ++g) {
+                const int col = n0 + wcol + ni * 32 + g * 8 + lh * 4;
+                if (col >= N) continue;
+                f32x4 v = f32x4{acc[mi][ni][g * 4], acc[mi][ni][g * 4 + 1], acc[mi][ni][g * 4 + 2], acc[mi][ni][g * 4 + 3]} * alpha;
+                if (vec_ok && col + 3 < N) {
+                    if (beta != 0.f) v += *(const f32x4 *)(crow + col) * beta;
+                    *(f32x4 *)(crow + col) = v;
+                } else {
+                    const float e[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        if (col + t < N) crow[col + t] = beta == 0.f ? e[t] : e[t] + beta * crow[col + t];
+                }
             }
-        }
+    }
 }
 
 template <int WM, int NST, int WN>
