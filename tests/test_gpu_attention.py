@@ -148,6 +148,32 @@ def test_windows_prefill_and_decode(gpu, orc, window):
     assert float(np.abs(got1 - ref1).max()) < 2e-3
 
 
+def test_prefill_bf16_key_segments_empty_segments_and_value_range(gpu, orc):
+    """Over a bf16 cache the key segments of the prefill kernel leave f16 partial accumulators under a per-row power-of-two
+    scale. A sliding window leaves whole segments of a row tile without a visible key (empty partial results beside live
+    ones), a short cache length cuts the last segments, and values of magnitude 2^100 and 2^-100 (exact in bf16) lie far
+    outside what f16 holds without the scale."""
+    B, L, Hq, Hkv, D = 1, 1024, 8, 1, 128
+    (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(77, B, L, L, Hq, Hkv, D, "bf16")
+    pos = np.arange(L, dtype=np.int32).reshape(1, L)
+    for window, lens in (((100, 0, 0), None), (be.CAUSAL, np.array([700], np.int32)), ((16, 0, 64), None)):
+        say("bf16 key segments", window, lens)
+        got = run_attention(gpu, q, k, v, 1 / math.sqrt(D), qd, kd, window=window, positions=pos, kv_lengths=lens)
+        assert gpu.last_kernel() == "attn_prefill"
+        ref = orc.attention_f64(qf, kf, vf, 1 / math.sqrt(D), window=window, positions=pos, kv_lengths=lens)
+        err = float(np.abs(got - ref).max())
+        say("  max err", err)
+        assert np.isfinite(got).all() and err < 1e-2
+    ref = orc.attention_f64(qf, kf, vf, 1 / math.sqrt(D))
+    for e in (100, -100):
+        vb, vbf = to_bf16(vf * np.float32(2.0 ** e))
+        got = run_attention(gpu, q, k, vb, 1 / math.sqrt(D), qd, kd)
+        assert gpu.last_kernel() == "attn_prefill"
+        err = float(np.abs(got * np.float32(2.0 ** -e) - ref).max())
+        say("  values x 2^%d: max err" % e, err)
+        assert np.isfinite(got).all() and err < 1e-2
+
+
 def test_soft_cap(gpu, orc):
     (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(13, 1, 40, 40, 8, 1, 64, "f16")
     # logits of std ~24 before the cap: the flash kernel feeds q to the MFMA in the K/V element
