@@ -409,9 +409,8 @@ def run_gemm(gpu, be):
                 y = gpu.alloc(m * n * 4)
                 for mode, kname, peak in ((be.GEMM_BF16_MFMA_ALWAYS, "gemm_bf16", "bf16"), (be.GEMM_EXACT_I8, "gemm_i8_" + tag, "int8")):
                     gpu.set_gemm_mode(mode)
-                    for _ in range(2):
-                        gpu.step_matmul(w, x, m, y)
-                    gpu.sync()
+                    gpu.step_matmul(w, x, m, y)
+                    settle(gpu, lambda i: gpu.step_matmul(w, x, m, y), 40.0)
                     gpu.profile_start()
                     t0 = time.perf_counter()
                     for _ in range(10):
