@@ -267,21 +267,34 @@ __global__ __launch_bounds__(256, KC == 4 || SPLITK ? 2 : 1) void gemm_i8_lds_ke
 }
 
 // ------------------------------------------------------------------------------------ bf16 MFMA
+constexpr int G2_TILE_K = 32;                                // k extent of a block of the tiled bf16 operands = the kernel's K step
 __device__ __forceinline__ unsigned short bf16_rne(float x) {
     unsigned u = __float_as_uint(x);
     u += 0x7FFFu + ((u >> 16) & 1u);
     return (unsigned short)(u >> 16);
 }
 
-// device row layout -> bf16 [N][K]: value = code * f32(f16 scale), rounded to bf16
+// Both bf16 operands of the MFMA kernel are private copies, laid out for its loads: 16 rows x 32 k (1 KiB) per block, blocks
+// k-major within a group of 16 rows - [rows / 16][K / 32][16][32]. One LDS-writing load of a wavefront (16 rows x 64 bytes
+// of one K step) is then 1 KiB of consecutive memory, eight whole 128-byte lines, where a row-major operand gives the L2
+// sixteen 64-byte requests, which it serves at the rate of 128-byte ones. Rows are padded to a multiple of 16 with zeros.
+__device__ __forceinline__ size_t bf16_tiled_index(size_t row, size_t k0, size_t K) {
+    return (((row >> 4) * (K / G2_TILE_K) + k0 / G2_TILE_K) * 16 + (row & 15)) * G2_TILE_K + (k0 % G2_TILE_K);
+}
+
+// device row layout -> bf16 tiled copy: value = code * f32(f16 scale), rounded to bf16
 template <int DT>
 __global__ void dequant_bf16_kernel(const uint8_t *__restrict__ qs, const __half *__restrict__ sc, unsigned short *__restrict__ out,
                                     size_t N, size_t K) {
     // one thread per 8 consecutive k of one row
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const size_t per_row = K / 8;
-    if (i >= N * per_row) return;
+    const size_t per_row = K / 8, rows = (N + 15) & ~(size_t)15;
+    if (i >= rows * per_row) return;
     const size_t n = i / per_row, k0 = (i % per_row) * 8;
+    if (n >= N) {
+        *(u32x4 *)(out + bf16_tiled_index(n, k0, K)) = u32x4{0u, 0u, 0u, 0u};
+        return;
+    }
     const float s = __half2float(sc[n * (K / QK) + k0 / QK]);
     int code[8];
     if (DT == AIONHIP_Q8_0) {
@@ -301,21 +314,25 @@ __global__ void dequant_bf16_kernel(const uint8_t *__restrict__ qs, const __half
     o.y = (unsigned)bf16_rne((float)code[2] * s) | ((unsigned)bf16_rne((float)code[3] * s) << 16);
     o.z = (unsigned)bf16_rne((float)code[4] * s) | ((unsigned)bf16_rne((float)code[5] * s) << 16);
     o.w = (unsigned)bf16_rne((float)code[6] * s) | ((unsigned)bf16_rne((float)code[7] * s) << 16);
-    *(u32x4 *)(out + n * K + k0) = o;
+    *(u32x4 *)(out + bf16_tiled_index(n, k0, K)) = o;
 }
 
 __global__ void act_bf16_kernel(const float *__restrict__ a, size_t lda, unsigned short *__restrict__ out, size_t M, size_t K) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const size_t per_row = K / 8;
-    if (i >= M * per_row) return;
+    const size_t per_row = K / 8, rows = (M + 15) & ~(size_t)15;
+    if (i >= rows * per_row) return;
     const size_t m = i / per_row, k0 = (i % per_row) * 8;
+    if (m >= M) {
+        *(u32x4 *)(out + bf16_tiled_index(m, k0, K)) = u32x4{0u, 0u, 0u, 0u};
+        return;
+    }
     const float *p = a + m * lda + k0;
     u32x4 o;
     o.x = (unsigned)bf16_rne(p[0]) | ((unsigned)bf16_rne(p[1]) << 16);
     o.y = (unsigned)bf16_rne(p[2]) | ((unsigned)bf16_rne(p[3]) << 16);
     o.z = (unsigned)bf16_rne(p[4]) | ((unsigned)bf16_rne(p[5]) << 16);
     o.w = (unsigned)bf16_rne(p[6]) | ((unsigned)bf16_rne(p[7]) << 16);
-    *(u32x4 *)(out + m * K + k0) = o;
+    *(u32x4 *)(out + bf16_tiled_index(m, k0, K)) = o;
 }
 
 // ---- wide-tile kernel: workgroup tile (WM*64) x 256, K step 32, v_mfma_f32_32x32x16_bf16.
@@ -334,6 +351,7 @@ __global__ void act_bf16_kernel(const float *__restrict__ a, size_t lda, unsigne
 // Tile order: workgroup ids go round-robin over the 8 XCDs, so id -> (xcd, slot) -> a contiguous
 // run of tiles per XCD, M fastest: the workgroups that share a weight column tile run on one L2.
 constexpr int G2_BK = 32, G2_ROW = 64, G2_BN = 256;
+static_assert(G2_BK == G2_TILE_K, "a block of the tiled operands is one K step");
 using f32x16 = __attribute__((ext_vector_type(16))) float;
 
 
@@ -383,19 +401,21 @@ __device__ __forceinline__ void gemm_bf16_tile(unsigned char *lds2, const unsign
             for (int i = 0; i < 16; ++i) acc[mi][ni][i] = 0.f;
 
     // load i of this wavefront covers tile rows i*64 + wave*16 .. +16; lane -> (row lane>>2, slot lane&3)
-    const int lrow = wave * 16 + (lane >> 2);
-    const int lchunk = (lane & 3) ^ ((lrow >> 2) & 3);
+    // (operands in the tiled layout: the wavefront's 16 rows of a K step are one 1 KiB block; within it lane -> row
+    // lane >> 2, chunk (lane & 3) ^ ((lane >> 4) & 3), the swizzle the fragment reads undo)
+    const int KT = K / G2_BK;
+    const int in_block = (lane >> 2) * G2_BK + (((lane & 3) ^ ((lane >> 4) & 3)) * 8);
+    const int a_blocks = (M + 15) >> 4, w_blocks = (N + 15) >> 4;
     const unsigned short *ga[NA], *gb[NB];
 #pragma unroll
-    for (int i = 0; i < NA; ++i) ga[i] = A + (size_t)min(m0 + i * 64 + lrow, M - 1) * K + lchunk * 8;
+    for (int i = 0; i < NA; ++i) ga[i] = A + (size_t)min((m0 >> 4) + i * 4 + wave, a_blocks - 1) * KT * (16 * G2_BK) + in_block;
 #pragma unroll
-    for (int i = 0; i < NB; ++i) gb[i] = W + (size_t)min(n0 + i * 64 + lrow, N - 1) * K + lchunk * 8;
-    const int KT = K / G2_BK;
+    for (int i = 0; i < NB; ++i) gb[i] = W + (size_t)min((n0 >> 4) + i * 4 + wave, w_blocks - 1) * KT * (16 * G2_BK) + in_block;
 
     auto issue_loads = [&](int kt, bool a_part, bool b_part) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the builtin exists in the device pass only
         unsigned char *stage = lds2 + (kt % NST) * STAGE + wave * 16 * G2_ROW;
-        const size_t k = (size_t)min(kt, KT - 1) * G2_BK;   // past the end: a harmless repeat into a dead stage
+        const size_t k = (size_t)min(kt, KT - 1) * (16 * G2_BK);   // the next block of the row group; past the end: a harmless repeat into a dead stage
         if (a_part)
 #pragma unroll
             for (int i = 0; i < NA; ++i)
@@ -655,8 +675,9 @@ int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *cw, size_t m, const
         if (ctx->capturing)
             return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "the bf16 copy of a weight cannot be built while a program is being recorded: run the steps once before recording");
         void *p = nullptr;
-        HIP_TRY(ctx, hipMalloc(&p, N * K * 2));
-        const size_t threads = N * (K / 8);
+        const size_t rows_padded = (N + 15) & ~(size_t)15;
+        HIP_TRY(ctx, hipMalloc(&p, rows_padded * K * 2));
+        const size_t threads = rows_padded * (K / 8);
         const unsigned grid = (unsigned)((threads + 255) / 256);
         if (w->dtype == AIONHIP_Q8_0) dequant_bf16_kernel<AIONHIP_Q8_0><<<dim3(grid), dim3(256), 0, ctx->stream>>>(w->qs, w->sc, (unsigned short *)p, N, K);
         else dequant_bf16_kernel<AIONHIP_Q4_0><<<dim3(grid), dim3(256), 0, ctx->stream>>>(w->qs, w->sc, (unsigned short *)p, N, K);
@@ -667,11 +688,12 @@ int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *cw, size_t m, const
         }
         w->bf16 = (unsigned short *)p;
     }
-    int rc = ensure_scratch2(ctx, m * K * 2);
+    const size_t m_padded = (m + 15) & ~(size_t)15;
+    int rc = ensure_scratch2(ctx, m_padded * K * 2);
     if (rc) return rc;
     unsigned short *abf = (unsigned short *)ctx->scratch2;
     {
-        const size_t threads = m * (K / 8);
+        const size_t threads = m_padded * (K / 8);
         ProfScope scope(ctx, "act_bf16");
         launch_k(ctx, act_bf16_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, a, lda, abf, m, K);
         LAUNCH_CHECK(ctx, "act_bf16");
