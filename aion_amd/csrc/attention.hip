@@ -226,6 +226,7 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
     const int v_key_in = (lane * 16) / (D * 2);                      // key of this lane within one V load
     const int v_slot = ((lane * 16) % (D * 2)) / 16;                 // its 16-byte slot within the key row
     const int v_hi_key = max(uni_hi - 1, 0);
+    (void)NVI; (void)KEYS_PER_VI; (void)vb8; (void)v_key_in; (void)v_slot; (void)v_hi_key;   // (used by the V loads, which exist in the device pass only)
     auto load_k = [&](int t) __attribute__((always_inline)) {
         if (near) load_k_as(t, std::true_type{});
         else load_k_as(t, std::false_type{});
