@@ -70,6 +70,8 @@ class _Plan:
 
 
 class PackageRunner:
+    LOG_TOKENS = 4096                      # tokens decode_run leaves on the device between two read-backs
+
     def __init__(self, gpu, pkg, capacity, capacity_symbol="ctx", tokens_symbol="seq", fuse=True, growth=None, keep_residuals=False):
         """growth: None = the capacity is fixed and a run that needs more is an error. A dict with "numerator",
         "denominator" and optionally "max_capacity" = the sequence caches grow on the device when a run needs more
@@ -91,6 +93,7 @@ class PackageRunner:
         self.plans = {}             # new tokens per run -> _Plan
         self.program = None
         self.one = None
+        self.log = self.log_at = None      # device token log of decode_run and its counter
         self.uses = {}
         for i, n in enumerate(pkg.nodes):
             for v in n.inputs:
@@ -652,11 +655,13 @@ class PackageRunner:
         return {name: self.gpu.download(buf, np_t[dt], shape) for name, (buf, shape, dt) in plan.outputs.items() if name in want}
 
     # ---- cache growth
-    def _required(self, s):
-        """Rows the caches must hold for a run of s tokens at self.pos (api/loaded_model/sequence_cache.zig:45-51)."""
+    def _required(self, s, pos=None):
+        """Rows the caches must hold for a run of s tokens at position pos (self.pos if not given;
+        api/loaded_model/sequence_cache.zig:45-51)."""
+        pos = self.pos if pos is None else pos
         need = 0
         for idx, (_vid, retained, fixed_rows) in self.cache_meta.items():
-            rows = (min(self.pos, retained) if retained else self.pos) + s
+            rows = (min(pos, retained) if retained else pos) + s
             if fixed_rows is None:
                 need = max(need, rows)
             elif rows > fixed_rows:             # a cache of constant shape (a local layer's ring): nothing to grow
@@ -746,10 +751,17 @@ class PackageRunner:
                 self.one = g.upload(np.ones(1, np.int32))
             tok_buf = plan.outputs[token_output][0]
 
+            if self.log is None:
+                # the tokens a run of replays produces, logged on the device at a counter of their own (decode_run reads them
+                # once per run; the counter is one more value the state-advance launch moves)
+                self.log = g.alloc(self.LOG_TOKENS * 4)
+                self.log_at = g.upload(np.zeros(1, np.int32))
+
             def issue():
                 self._issue(plan)
                 g.step_advance_state(plan.inputs["tokens"][0], tok_buf, 1,
-                                     [plan.inputs[kind][0] for kind in ("positions", "cache_write_index", "cache_visible_end")])
+                                     [plan.inputs[kind][0] for kind in ("positions", "cache_write_index", "cache_visible_end")] + [self.log_at],
+                                     log=self.log, log_index=self.log_at, log_capacity=self.LOG_TOKENS)
             self.program = g.record_program(issue)
         self._token_output = token_output
 
@@ -768,6 +780,28 @@ class PackageRunner:
             return int(self.gpu.download(buf, np.int32, shape).reshape(-1)[-1])
         return None
 
+    def decode_run(self, n):
+        """n replays of the decode program with nothing read back in between: the produced tokens are logged on the device
+        and collected once per stretch of replays (a stretch ends where the caches have to grow, or the log is full)."""
+        out = []
+        while n > 0:
+            if self._required(1) > self.capacity:
+                if self.growth is None:
+                    raise ValueError("cache capacity exhausted")
+                token = int(self.gpu.download(self.plans[1].inputs["tokens"][0], np.int32, (1,))[0])
+                self._grow(self._required(1))
+                self.begin_decode(token, self._token_output)
+            c = 1                                # single-token runs that fit the caches as they are
+            while c < min(n, self.LOG_TOKENS) and self._required(1, self.pos + c) <= self.capacity:
+                c += 1
+            self.gpu.write(self.log_at, np.zeros(1, np.int32))
+            for _ in range(c):
+                self.gpu.program_execute(self.program)
+            self.pos += c
+            out.extend(int(t) for t in self.gpu.download(self.log, np.int32, (c,)))
+            n -= c
+        return out
+
     def reset(self):
         self.pos = 0
 
@@ -784,4 +818,6 @@ class PackageRunner:
             b.free()
         if self.one is not None:
             self.one.free()
-        self.plans, self.consts, self.caches, self.one = {}, {}, {}, None
+        if self.log is not None:
+            self.log.free(); self.log_at.free()
+        self.plans, self.consts, self.caches, self.one, self.log, self.log_at = {}, {}, {}, None, None, None

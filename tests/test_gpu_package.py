@@ -222,6 +222,32 @@ def test_growing_caches_match_preallocated_ones(gpu):
         grow.close(); full.close()
 
 
+def test_decode_run_logs_tokens_on_the_device_across_cache_growth(gpu):
+    """decode_run: replays back to back with the produced tokens logged on the device (a counter of their own beside the
+    loop state) against the same generation one read-back per step; the run crosses a growth of the caches (32 -> 128)
+    and a second run goes on where the first stopped."""
+    cfg = DecoderConfig(wdtype=be.Q4_0, **SMALL)
+    weights = SyntheticWeights(cfg, 23)
+    d = dict(layers=cfg.layers, hidden=cfg.hidden, heads=cfg.heads, kv_heads=cfg.kv_heads, head_dim=cfg.head_dim, ffn=cfg.ffn,
+             vocab=cfg.vocab, eps=cfg.eps, rope_base=cfg.rope_base, wdtype="q4_0")
+    pkg = aion_file.parse(aion_writer.build_decoder_package(d, weights.blocks, weights.embed(), growable=True))
+    logged = PackageRunner(gpu, pkg, capacity=32, growth=dict(numerator=2, denominator=1, max_capacity=128))
+    stepped = PackageRunner(gpu, pkg, capacity=128)
+    try:
+        prompt = np.random.default_rng(6).integers(0, cfg.vocab, 9).astype(np.int32)
+        a, b = logged.run(prompt, want=("next_token",)), stepped.run(prompt, want=("next_token",))
+        tok = int(b["next_token"][0, -1])
+        assert int(a["next_token"][0, -1]) == tok
+        logged.begin_decode(tok); stepped.begin_decode(tok)
+        want = [stepped.decode_step() for _ in range(70)]
+        got = logged.decode_run(40) + logged.decode_run(30)
+        assert logged.capacity == 128 and logged.pos == stepped.pos == 79
+        assert got == want
+        assert logged.decode_step() == stepped.decode_step()       # a single step after the runs: the loop state is where it should be
+    finally:
+        logged.close(); stepped.close()
+
+
 def test_rolling_caches_grow_for_a_long_run(gpu):
     """A ring of 64 rows (12 retained) asked to take a 60-token run needs 12 + 60 rows: it grows to 256 with its
     retained rows re-placed (storage/manager/grow.zig:107-150), and the session goes on as one that had 256 rows all
