@@ -118,7 +118,7 @@ struct aionhip_weight {
     uint8_t *qs = nullptr;
     __half *sc = nullptr;
     size_t qs_bytes = 0, sc_bytes = 0;
-    // lazily built by the bf16 MFMA GEMM: the weight dequantized to bf16 [n][k]
+    // lazily built by the bf16 MFMA GEMM: the weight dequantized to bf16, [n / 16][k / 32][16][32] (n padded to 16 with zeros)
     unsigned short *bf16 = nullptr;
 };
 

@@ -196,7 +196,7 @@ int aionhip_step_gate_matmul(aionhip_ctx *ctx, const aionhip_weight *b, size_t r
  * and exact). BF16_MFMA_ALWAYS: the bf16 kernel for every m > 8, whatever the shape. */
 typedef enum aionhip_gemm_mode { AIONHIP_GEMM_EXACT_I8 = 0, AIONHIP_GEMM_BF16_MFMA = 1, AIONHIP_GEMM_BF16_MFMA_ALWAYS = 2 } aionhip_gemm_mode;
 int aionhip_set_gemm_mode(aionhip_ctx *ctx, int mode);
-/* The bf16 kernel keeps a bf16 copy of every weight it has multiplied (n * k * 2 bytes - about four times a q4_0 weight -
+/* The bf16 kernel keeps a bf16 copy of every weight it has multiplied (n rounded up to 16, times k * 2 bytes - about four times a q4_0 weight -
  * built on the first such call, never while a program is being recorded, released by aionhip_weight_free). This releases
  * the copy of one weight early (it is rebuilt on the next bf16 call); aion's derived-weight reclamation
  * (storage/derived.zig:1-17) is the counterpart. Waits for the context's stream. */
