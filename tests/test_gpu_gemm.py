@@ -145,6 +145,34 @@ def test_config3_bf16_full_size_on_row_sample(gpu, orc, dtype, layout, m, n):
         gpu.set_gemm_mode(be.GEMM_EXACT_I8)
 
 
+@pytest.mark.parametrize("ldc,c_offset", [(520, 0), (524, 0), (521, 0), (528, 3)])
+def test_bf16_gemm_alpha_beta_and_output_strides(gpu, orc, ldc, c_offset):
+    """The bf16 kernel's epilogue: 16-byte stores where the output rows allow them (row pitch and base 16-byte aligned),
+    single floats otherwise (odd pitch, a base that is only 4-byte aligned), alpha and beta in both, the columns between
+    n and the pitch untouched. Checked against the same kernel's plain product: C' = alpha * (A W^T) + beta * C."""
+    say("bf16 alpha/beta", ldc, c_offset)
+    m, n, k = 300, 520, 1024
+    gpu.set_gemm_mode(be.GEMM_BF16_MFMA_ALWAYS)
+    try:
+        blocks, w = make_weight(gpu, be.Q4_0, be.KMAJOR_KN, n, k, seed=31)
+        rng = np.random.default_rng(32)
+        a = rng.standard_normal((m, k)).astype(np.float32)
+        c0 = rng.standard_normal(m * ldc + c_offset).astype(np.float32)
+        plain = gpu.matmul(w, a)
+        assert gpu.last_kernel() == "gemm_bf16"
+        a_buf, c_buf = gpu.upload(a), gpu.upload(c0)
+        gpu.step_matmul(w, a_buf, m, c_buf, ldc=ldc, alpha=0.5, beta=2.0, c_offset=c_offset * 4)
+        got = gpu.download(c_buf, np.float32, (m * ldc + c_offset,))
+        assert np.array_equal(got[:c_offset], c0[:c_offset])
+        got2, old2 = got[c_offset:].reshape(m, ldc), c0[c_offset:].reshape(m, ldc)
+        want = 0.5 * plain + 2.0 * old2[:, :n]
+        assert float(np.abs(got2[:, :n] - want).max()) <= 1e-5 * float(np.abs(want).max())
+        assert np.array_equal(got2[:, n:], old2[:, n:])
+        a_buf.free(); c_buf.free(); w.free()
+    finally:
+        gpu.set_gemm_mode(be.GEMM_EXACT_I8)
+
+
 def test_bf16_mode_runs_the_bf16_kernel_only_where_it_pays(gpu, orc):
     """In bf16 mode a shape the bf16 kernel is not expected to win (few rows: it streams a 2-byte copy of the weight
     through 256-column tiles) stays on the exact kernel - same numbers as the exact mode - and a large one moves."""
