@@ -574,7 +574,9 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
         // more tiles per wavefront beyond one workgroup per CU (its LDS tiles fill a CU)
         const int cus = ctx->cu_count > 0 ? ctx->cu_count : 256;
         const int tiles = (a.T + TILE_KEYS - 1) / TILE_KEYS;
-        int nseg = (cus + units * a.row_tiles - 1) / (units * a.row_tiles);
+        // (as many segments as keep the workgroups within one per CU: a second, partial round of workgroups plus the merge
+        // launch costs more than CUs left idle - 192 row tiles in two segments each took 26 us, in one 13)
+        int nseg = cus / (units * a.row_tiles);
         nseg = max(1, min(nseg, (tiles + SPLIT_NW - 1) / SPLIT_NW));
         nseg = min(nseg, 256);
         a.nseg = nseg;
