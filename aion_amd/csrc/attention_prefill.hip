@@ -31,6 +31,9 @@ constexpr float PF_LAZY = 8.f;
 #ifndef PF_SEG_TILES
 #define PF_SEG_TILES 4     // fewest 64-key tiles a key segment of the prefill kernel is worth
 #endif
+#ifndef PF_TWO_SEG_BELOW_TENTHS
+#define PF_TWO_SEG_BELOW_TENTHS 12   // row tiles up to 1.2 x the CUs: two key segments per tile
+#endif
 #ifndef PF_PIPE_D
 #define PF_PIPE_D 128      // head sizes from here on run the software-pipelined tile loop
 #endif
@@ -772,6 +775,11 @@ int launch_prefill_t(aionhip_ctx *ctx, AttnArgs &a) {
     const int key_tiles = (a.T + PF_TK - 1) / PF_TK;
     int want = cus0 / max(wgs, 1);
     if (want < 2 && wgs <= cus0) want = 2;      // one round of workgroups: two segments even out what a causal mask skews
+    // Between one and two rounds the longest row tile alone takes as long as two average ones (under a causal mask a tile's
+    // work grows with its index): the device is busy wgs / (2 * CUs) of the time. Two segments halve the longest piece;
+    // they pay while that gain exceeds the merge pass (measured at 8 heads x head size 256: 260 workgroups 109 -> 94 us, 288
+    // 122 -> 116, 320 the same, 352 and more slower).
+    if (want < 2 && (long)wgs * 10 < (long)cus0 * PF_TWO_SEG_BELOW_TENTHS) want = 2;
     int nseg = max(1, min(min(want, key_tiles / PF_SEG_TILES), 16));
     a.nseg = nseg;
     if (nseg > 1) {

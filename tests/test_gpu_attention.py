@@ -295,6 +295,18 @@ def test_prefill_config4_sizes(gpu, orc):
     err = float(np.abs(got[:, idx] - ref_s).max())
     say("  L4096 sample of", idx.size, "positions: max err", err)
     assert err < 1e-2
+    # just past one workgroup per CU (260 row tiles on 256 CUs): two key segments per row tile again, because the longest
+    # row tile alone would take as long as two average ones
+    L = 4160
+    say("prefill config 4 L4160 sample")
+    (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(47, 1, L, L, 8, 1, 256, "bf16")
+    got = run_attention(gpu, q, k, v, 1 / 16.0, qd, kd)
+    assert gpu.last_kernel() == "attn_prefill"
+    idx = np.array([0, 1, 16, 1000, 2079, 2080, 2081, 3000, 4095, 4096, 4144, 4159])
+    ref_s = orc.attention_f64(np.ascontiguousarray(qf[:, idx]), kf, vf, 1 / 16.0, positions=idx.astype(np.int32).reshape(1, -1))
+    err = float(np.abs(got[:, idx] - ref_s).max())
+    say("  L4160 sample of", idx.size, "positions: max err", err)
+    assert err < 1e-2
 
 
 @pytest.mark.parametrize("B,Lq,T,lens,kernel", [
