@@ -629,10 +629,13 @@ bool gemm_bf16_pays(const aionhip_ctx *ctx, size_t m, size_t n, size_t k) {
     pick_i8_shape(ctx, m, n, k, &per_block);
     const float blocks = (float)(k / 32);
     const float exact_us = per_block * blocks + 5.f + (float)m * (float)k * 4.f / 2.0e6f;       // + the int8 preparation of A
-    const float copy_us = (float)n * (float)k * 2.f / 4.0e6f;                                  // weight bytes at ~4 TB/s
+    // (constants fitted to both kernels' times over six weight shapes x 65..1024 rows, q4: the choice costs 0.3 % over
+    // always taking the faster one; always exact would cost 36 %, always bf16 17 %)
+    const float copy_us = (float)n * (float)k * 2.f / 3.0e6f;                                  // weight bytes at ~3 TB/s
     const float flop_us = 2.f * (float)m * (float)n * (float)k / 9.0e8f;                        // ~900 TFLOP/s
-    const float chain_us = blocks * 0.27f;                                                       // one workgroup's K loop
-    const float bf16_us = fmaxf(fmaxf(copy_us, flop_us), chain_us) + 15.f;
+    const float chain_us = blocks * 0.24f;                                                       // one workgroup's K loop
+    const float act_us = (float)m * (float)k * 6.f / 4.0e6f;                                     // the bf16 rounding of A
+    const float bf16_us = fmaxf(fmaxf(copy_us, flop_us), chain_us) + act_us;
     return bf16_us < exact_us;
 }
 
