@@ -423,7 +423,15 @@ int launch_gemv_batch(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *
     // 5..8 rows against a wide, short weight (a logits head at batch 8): the 16-row MFMA tile of the LDS-staged int8
     // GEMM beats the lane-per-row kernel, whose LDS traffic grows with the rows (262144 x 2048, 8 rows: 77 against
     // 104 us for q4, 110 against 142 us for q8). Long K or few columns leave that kernel's grid too sparse.
-    if (count == 1 && m >= 5 && ws[0]->n >= 16384 && ws[0]->k >= 256 && ws[0]->k <= 4096) {
+    // q8 (twice the weight bytes per row: the lane-per-row kernel leaves its latency floor later) moves there from two
+    // rows on once the weight has some 12k columns - 14336 x 4096: 22 -> 20 us at 4 rows, 26.6 -> 20.3 at 8;
+    // 16384 x 2048: 15 -> 13.7 at 2-4 rows - but not against the largest weights, which the lane-per-row kernel
+    // streams faster at 2-4 rows (65536 x 4096: 58-64 against 70 us).
+    const size_t n = ws[0]->n, k = ws[0]->k;
+    const bool q8w = ws[0]->dtype == AIONHIP_Q8_0;
+    const bool tile16 = (m >= 5 && n >= 16384) || (q8w && m >= 2 && n >= 12288 && n * k <= ((size_t)1 << 27)) ||
+                        (q8w && m >= 5 && n >= 8192 && k <= 2048);
+    if (count == 1 && tile16 && k >= 256 && k <= 4096) {
         const int rc = launch_gemm_i8_few_rows(ctx, ws[0], (size_t)m, act, cs[0], ldcs[0], alpha, beta);
         if (rc) return rc;
         LAUNCH_CHECK(ctx, name);
