@@ -57,6 +57,8 @@ struct aionhip_ctx {
     size_t tickets_bytes = 0;
     // this device's copy of the library's file-scope scratch array (ctx.hip), for the entry point that allocates nothing
     void *static_scratch = nullptr;
+    // true while that entry point runs: no launcher may take a path that needs scratch of its own
+    bool no_scratch_paths = false;
     // attention with f32 queries: false = one MFMA pass on q rounded to the K/V element type (2e-3 class),
     // true = q and the probabilities as hi+lo parts (f32-level accuracy, about 1.4x the instructions)
     bool attn_precise = false;

@@ -45,7 +45,7 @@ template <int KC> struct GiCfg { static constexpr int ROW = KC * 32 + 16; };   /
 template <int DT, int WM, int KC, bool SPLITK>
 __global__ __launch_bounds__(256, KC == 4 || SPLITK ? 2 : 1) void gemm_i8_lds_kernel(GemmSegs segs,
                                                           const int8_t *__restrict__ aq, const float *__restrict__ a_scale,
-                                                          int M, int K, float alpha, float beta) {
+                                                          int M, int K, float alpha, float beta, float *__restrict__ partial, int partial_ld) {
     constexpr bool Q8 = DT == AIONHIP_Q8_0;
     static_assert(!SPLITK || KC == 8, "split K: two blocks per wavefront per step");
     constexpr int BM3 = (SPLITK ? 16 : 32) * WM, BN3 = SPLITK ? 64 : 128, ROW = GiCfg<KC>::ROW;
@@ -154,12 +154,24 @@ __global__ __launch_bounds__(256, KC == 4 || SPLITK ? 2 : 1) void gemm_i8_lds_ke
         for (int i = 0; i < NWS; ++i) ws_l[tid + 256 * i] = kb0 + (tid + 256 * i) % KC < KB ? __half2float(rws[i]) : 0.f;
     };
 
-    load_stage(0);
-    store_stage(lds3, 0);
+    // K slices (grid z, few workgroups against a long K): slice z takes its share of the K steps and leaves raw sums in
+    // `partial` [z][M][partial_ld] for gemm_i8_slices_kernel, which adds the slices in their order
+    const int kt_per = (KT + (int)gridDim.z - 1) / (int)gridDim.z;
+    const int kt_lo = (int)blockIdx.z * kt_per, kt_hi = min(KT, kt_lo + kt_per);
+    if (partial) {
+        partial += (size_t)blockIdx.z * M * partial_ld + (size_t)blockIdx.x * BN3;
+        c = partial - n0;                                // column n0 + j of this tile -> partial column blockIdx.x * BN3 + j
+        alpha = 1.f;
+        beta = 0.f;
+    }
+    const size_t ldo = partial ? (size_t)partial_ld : ldc;
+    const int n_hi = partial ? n0 + BN3 : N;            // (a partial tile is written whole: its padding columns are sums over clamped rows, never read)
+    load_stage(kt_lo);
+    store_stage(lds3, kt_lo);
     __syncthreads();
-    for (int kt = 0; kt < KT; ++kt) {
-        const unsigned char *st = lds3 + (kt & 1) * STAGE;
-        const bool more = kt + 1 < KT;
+    for (int kt = kt_lo; kt < kt_hi; ++kt) {
+        const unsigned char *st = lds3 + ((kt - kt_lo) & 1) * STAGE;
+        const bool more = kt + 1 < kt_hi;
         if (more) load_stage(kt + 1);
         const float *as_l = (const float *)(st + A_BYTES + B_BYTES), *ws_l = (const float *)(st + A_BYTES + B_BYTES + AS_BYTES);
         float wsc[4][KCW];
@@ -219,7 +231,7 @@ __global__ __launch_bounds__(256, KC == 4 || SPLITK ? 2 : 1) void gemm_i8_lds_ke
 #pragma unroll
             for (int ni = 0; ni < 4; ++ni) dprev[ni] = dcur[ni];
         }
-        if (more) store_stage(lds3 + ((kt + 1) & 1) * STAGE, kt + 1);
+        if (more) store_stage(lds3 + ((kt + 1 - kt_lo) & 1) * STAGE, kt + 1);
         __syncthreads();
     }
 
@@ -241,8 +253,8 @@ __global__ __launch_bounds__(256, KC == 4 || SPLITK ? 2 : 1) void gemm_i8_lds_ke
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int row = m0 + mi * 16 + g * 4 + i;
-                if (row >= M || col >= N) continue;
-                float *dst = c + (size_t)row * ldc + col;
+                if (row >= M || col >= n_hi) continue;
+                float *dst = c + (size_t)row * ldo + col;
                 const float v = alpha * sum[i];
                 *dst = beta == 0.f ? v : v + beta * *dst;
             }
@@ -258,8 +270,8 @@ __global__ __launch_bounds__(256, KC == 4 || SPLITK ? 2 : 1) void gemm_i8_lds_ke
 #pragma unroll
             for (int ni = 0; ni < 4; ++ni) {
                 const int col = n0 + wn0 + ni * 16 + r;
-                if (col >= N) continue;
-                float *dst = c + (size_t)row * ldc + col;
+                if (col >= n_hi) continue;
+                float *dst = c + (size_t)row * ldo + col;
                 const float v = alpha * acc[mi][ni][i];
                 *dst = beta == 0.f ? v : v + beta * *dst;
             }
@@ -547,6 +559,55 @@ __global__ __launch_bounds__(256) void gemm_bf16_mixed_kernel(const unsigned sho
     else gemm_bf16_tile<4, NST, 3>(lds2, A, W, c, M, N, K, ldc, alpha, beta, m0, tw * 256 + idx * 192);
 }
 
+// Tile choice by a small cost model fitted to measurements on one MI355X (q4, K = 2048..8192, 24..2048
+// rows): a lone workgroup of each shape costs `us_per_block` per quant block of K; workgroups beyond one
+// per CU overlap by the factor `overlap` (two resident per CU hide each other's staging).
+struct GiShape { int wm; bool split; float us_per_block, overlap; };
+constexpr GiShape GI_SHAPES[6] = {
+    {4, false, 0.81f, 1.40f}, {2, false, 0.44f, 1.25f}, {1, false, 0.284f, 1.55f},
+    {4, true, 0.253f, 1.45f}, {2, true, 0.164f, 1.50f}, {1, true, 0.121f, 1.85f},
+};
+// The K slices of gemm_i8_lds_kernel folded in slice order: C = alpha * (p[0] + p[1] + ...) + beta * C, one thread per
+// (row, four columns of a tile).
+__global__ __launch_bounds__(256) void gemm_i8_slices_kernel(GemmSegs segs, const float *__restrict__ partial, int M, int slices, int partial_ld,
+                                                             int bn, float alpha, float beta) {
+    const int quads = partial_ld >> 2;
+    const size_t id = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (id >= (size_t)M * quads) return;
+    const int row = (int)(id / quads), pc = (int)(id % quads) * 4, tile = pc / bn;
+    int si = 0;
+#pragma unroll
+    for (int i = 1; i < 4; ++i)
+        if (i < segs.count && tile >= segs.first_tile[i]) si = i;
+    const int col = pc - segs.first_tile[si] * bn;
+    if (col >= segs.n[si]) return;
+    f32x4 sum = *(const f32x4 *)(partial + (size_t)row * partial_ld + pc);
+    for (int z = 1; z < slices; ++z) sum += *(const f32x4 *)(partial + ((size_t)z * M + row) * partial_ld + pc);
+    float *dst = segs.c[si] + (size_t)row * segs.ldc[si] + col;
+    const float e[4] = {sum.x, sum.y, sum.z, sum.w};
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+        if (col + t < segs.n[si]) dst[t] = beta == 0.f ? alpha * e[t] : alpha * e[t] + beta * dst[t];
+}
+
+// How many K slices a launch of `wgs` workgroups (each able to overlap `overlap` to a CU, `us_per_block` per quant block of a
+// lone one) over `kt` K steps of `blocks` quant blocks is cut into. Slices pay when the modelled time with them, the
+// launch that adds them up included, is under three quarters of the time without (measured: 4096 x 14336 at 16 rows
+// 52 -> 22 us in 7 slices, 2048 x 8192 33 -> 15 us, 4096 x 4096 20 -> 15 us; K = 2048 never: the second launch costs what
+// the slices save).
+inline int i8_k_slices(const aionhip_ctx *ctx, float wgs, float overlap, int kt, float us_per_block, float blocks) {
+    const float cus = (float)(ctx->cu_count > 0 ? ctx->cu_count : 256);
+    const float rounds = wgs / (cus * overlap);
+    if (ctx->no_scratch_paths || rounds >= 0.75f || kt < 8) return 1;
+    int s = (int)(1.f / rounds + 0.5f);
+    s = s < kt / 4 ? s : kt / 4;                          // at least four K steps per slice
+    s = s > 8 ? 8 : s;
+    if (s < 2) return 1;
+    const float alone = us_per_block * blocks;
+    const float sliced = alone / (float)s * (rounds * (float)s > 1.f ? rounds * (float)s : 1.f) + 4.f;
+    return sliced < 0.75f * alone ? s : 1;
+}
+
 template <int DT, int WM, int KC, bool SPLITK>
 int launch_i8_lds(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count, size_t m, PreparedAct act,
                   float alpha, float beta) {
@@ -571,19 +632,30 @@ int launch_i8_lds(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *cons
         segs.first_tile[i] = tiles;
         tiles += (int)((ws[i]->n + BN3 - 1) / BN3);
     }
-    const dim3 grid((unsigned)tiles, (unsigned)((m + BM3 - 1) / BM3));
-    launch_k(ctx, gemm_i8_lds_kernel<DT, WM, KC, SPLITK>, grid, dim3(256), LDS, segs, act.q, act.scale, (int)m, (int)ws[0]->k, alpha, beta);
+    const int m_tiles = (int)((m + BM3 - 1) / BM3), kt = (int)(((ws[0]->k >> 5) + KC - 1) / KC);
+    // Few workgroups against a long K (a short prompt or a batch of 9..64 rows on a narrow weight): the K steps are cut into
+    // slices across more workgroups and a second, small launch adds the slices in order - the same sums in the same
+    // order per slice, the slices in a fixed order, so the result does not depend on timing.
+    constexpr GiShape SHAPE = GI_SHAPES[(SPLITK ? 3 : 0) + (WM == 4 ? 0 : WM == 2 ? 1 : 2)];
+    static_assert(SHAPE.wm == WM && SHAPE.split == SPLITK, "shape table order");
+    int slices = i8_k_slices(ctx, (float)tiles * (float)m_tiles, SHAPE.overlap, kt, SHAPE.us_per_block, (float)(ws[0]->k >> 5));
+    while (slices > 1 && (kt + slices - 1) / slices * (slices - 1) >= kt) --slices;      // no empty slice
+    float *partial = nullptr;
+    const int partial_ld = tiles * BN3;
+    if (slices > 1) {
+        const int rc = ensure_scratch2(ctx, (size_t)slices * m * partial_ld * sizeof(float));
+        if (rc) return rc;
+        partial = (float *)ctx->scratch2;
+    }
+    const dim3 grid((unsigned)tiles, (unsigned)m_tiles, (unsigned)slices);
+    launch_k(ctx, gemm_i8_lds_kernel<DT, WM, KC, SPLITK>, grid, dim3(256), LDS, segs, act.q, act.scale, (int)m, (int)ws[0]->k, alpha, beta, partial, partial_ld);
+    if (slices > 1) {
+        const size_t threads = m * (size_t)(partial_ld >> 2);
+        launch_k(ctx, gemm_i8_slices_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, segs, partial, (int)m, slices, partial_ld, BN3, alpha, beta);
+    }
     return AIONHIP_OK;
 }
 
-// Tile choice by a small cost model fitted to measurements on one MI355X (q4, K = 2048..8192, 24..2048
-// rows): a lone workgroup of each shape costs `us_per_block` per quant block of K; workgroups beyond one
-// per CU overlap by the factor `overlap` (two resident per CU hide each other's staging).
-struct GiShape { int wm; bool split; float us_per_block, overlap; };
-constexpr GiShape GI_SHAPES[6] = {
-    {4, false, 0.81f, 1.40f}, {2, false, 0.44f, 1.25f}, {1, false, 0.284f, 1.55f},
-    {4, true, 0.253f, 1.45f}, {2, true, 0.164f, 1.50f}, {1, true, 0.121f, 1.85f},
-};
 // the cheapest shape for m rows against an n x k weight and its modelled time per quant block of K
 int pick_i8_shape(const aionhip_ctx *ctx, size_t m, size_t n, size_t k, float *us_per_block) {
     const float cus = (float)(ctx->cu_count > 0 ? ctx->cu_count : 256);
@@ -626,9 +698,17 @@ int launch_i8_lds_pick(aionhip_ctx *ctx, const aionhip_weight *const *ws, float 
 // Modelled times in microseconds, constants fitted to a sweep of 9..512 rows over four weight shapes.
 bool gemm_bf16_pays(const aionhip_ctx *ctx, size_t m, size_t n, size_t k) {
     float per_block = 0.f;
-    pick_i8_shape(ctx, m, n, k, &per_block);
+    const GiShape &g = GI_SHAPES[pick_i8_shape(ctx, m, n, k, &per_block)];
     const float blocks = (float)(k / 32);
-    const float exact_us = per_block * blocks + 5.f + (float)m * (float)k * 4.f / 2.0e6f;       // + the int8 preparation of A
+    // (the exact kernel cuts a long K into slices across workgroups when its grid is sparse)
+    const size_t bm = (size_t)(g.split ? 16 : 32) * g.wm, bn = g.split ? 64 : 128;
+    const float wgs = (float)(((m + bm - 1) / bm) * ((n + bn - 1) / bn));
+    const int kc = g.split ? 8 : 4;                      // (the launcher's KC per shape)
+    const int slices = i8_k_slices(ctx, wgs, g.overlap, (int)((k / 32 + kc - 1) / kc), g.us_per_block, blocks);
+    const float cus = (float)(ctx->cu_count > 0 ? ctx->cu_count : 256);
+    const float rounds = wgs * (float)slices / (cus * g.overlap);
+    const float kernel_us = slices > 1 ? g.us_per_block * blocks / (float)slices * (rounds > 1.f ? rounds : 1.f) + 4.f : per_block * blocks;
+    const float exact_us = kernel_us + 5.f + (float)m * (float)k * 4.f / 2.0e6f;               // + the int8 preparation of A
     // (constants fitted to both kernels' times over six weight shapes x 65..1024 rows, q4: the choice costs 0.3 % over
     // always taking the faster one; always exact would cost 36 %, always bf16 17 %)
     const float copy_us = (float)n * (float)k * 2.f / 3.0e6f;                                  // weight bytes at ~3 TB/s

@@ -135,7 +135,10 @@ int aionhip_step_matmul_static(aionhip_ctx *ctx, const aionhip_weight *b, size_t
                                aionhip_handle c, size_t ldc, float alpha, float beta) {
     if (!ctx || !b) return AIONHIP_INVALID_ARGUMENT;
     if (!ctx->static_scratch) return set_err(ctx, AIONHIP_EXECUTION_FAILED, "matmul_static: the context has no static scratch address");
-    return run_matmul(ctx, b, m, a, lda, c, ldc, alpha, beta, true);
+    ctx->no_scratch_paths = true;
+    const int rc = run_matmul(ctx, b, m, a, lda, c, ldc, alpha, beta, true);
+    ctx->no_scratch_paths = false;
+    return rc;
 }
 
 int aionhip_step_rmsnorm_matmul(aionhip_ctx *ctx, size_t count, const aionhip_weight *const *bs, size_t rows, aionhip_handle x,

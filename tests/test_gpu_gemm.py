@@ -145,6 +145,43 @@ def test_config3_bf16_full_size_on_row_sample(gpu, orc, dtype, layout, m, n):
         gpu.set_gemm_mode(be.GEMM_EXACT_I8)
 
 
+@pytest.mark.parametrize("dtype,layout", CASES)
+def test_exact_gemm_k_slices(gpu, orc, dtype, layout):
+    """Few workgroups against a long K: the exact kernel cuts the K steps into slices across workgroups (grid z) and a
+    second launch adds the slices in order. Parity as for every exact kernel, alpha / beta / row pitch through the second
+    launch, the same bits on a second run (nothing depends on which slice finishes first), and sibling weights that share
+    the launch."""
+    say("k slices", dtype, layout)
+    m, n, k = 24, 520, 8192
+    gpu.set_gemm_mode(be.GEMM_EXACT_I8)
+    blocks, w = make_weight(gpu, dtype, layout, n, k, seed=41)
+    blocks2, w2 = make_weight(gpu, dtype, layout, 200, k, seed=42)
+    rng = np.random.default_rng(43)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    a_buf = gpu.upload(a)
+    ldc = 524
+    c0 = rng.standard_normal((m, ldc)).astype(np.float32)
+    c_buf = gpu.upload(c0)
+    gpu.profile_start()
+    gpu.step_matmul(w, a_buf, m, c_buf, ldc=ldc, alpha=0.5, beta=2.0)
+    prof = gpu.profile_stop()
+    assert [nm for nm, _ in prof if nm.startswith("gemm_i8")] == [prof[-1][0]] * 2        # the sliced kernel and the fold
+    got = gpu.download(c_buf, np.float32, (m, ldc))
+    want = oracle_i8(orc, dtype, layout, a, blocks, n, alpha=0.5, beta=2.0, c=np.ascontiguousarray(c0[:, :n]))
+    assert norm_err(got[:, :n], want) < 2e-3 and rms_err(got[:, :n], want) < 1e-5
+    assert np.array_equal(got[:, n:], c0[:, n:])
+    first = gpu.matmul(w, a)
+    assert np.array_equal(first.view(np.uint32), gpu.matmul(w, a).view(np.uint32))
+    c1, c2 = gpu.alloc(m * n * 4), gpu.alloc(m * 200 * 4)
+    gpu.step_matmul_batch([w, w2], a_buf, m, [c1, c2])
+    got1, got2 = gpu.download(c1, np.float32, (m, n)), gpu.download(c2, np.float32, (m, 200))
+    assert rms_err(got1, oracle_i8(orc, dtype, layout, a, blocks, n)) < 1e-5
+    assert rms_err(got2, oracle_i8(orc, dtype, layout, a, blocks2, 200)) < 1e-5
+    for t in (a_buf, c_buf, c1, c2):
+        t.free()
+    w.free(); w2.free()
+
+
 @pytest.mark.parametrize("ldc,c_offset", [(520, 0), (524, 0), (521, 0), (528, 3)])
 def test_bf16_gemm_alpha_beta_and_output_strides(gpu, orc, ldc, c_offset):
     """The bf16 kernel's epilogue: 16-byte stores where the output rows allow them (row pitch and base 16-byte aligned),

@@ -1,8 +1,10 @@
 """aionhip_step_matmul_static - the matmul step for callers that cannot allocate - against aionhip_step_matmul /
-aionhip_step_matmul_nt on the same operands, through the C ABI. Where both run the same kernel the bar is bit equality; one row
-against K > 4096 runs the K-split kernel in the allocating entry point (it keeps a growable buffer) and the separate
-preparation + one-row kernel in the static one: the same int8 codes and block dots, another order of the f32 additions,
-held to max|diff| <= 1e-5 * rms like every exact-integer-dot kernel against the oracle.
+aionhip_step_matmul_nt on the same operands, through the C ABI. Where both run the same kernel the same way the bar is bit
+equality. Two cases differ in the order of their f32 additions only - the same int8 codes and block dots - and are held to
+max|diff| <= 1e-5 * rms like every exact-integer-dot kernel against the oracle: one row against K > 4096 runs the K-split
+kernel in the allocating entry point (it keeps a growable buffer) and the separate preparation + one-row kernel in the
+static one; and the exact GEMM cuts a long K into slices across workgroups when its grid is sparse, through a buffer of
+partial sums that the static entry point may not take.
 
 Every call on a GPU shares one static device array that keeps the last call's contents: the calls come in pairs, the second
 with a smaller input than the first (fewer rows, shorter K), so stale bytes of the first call lie right behind the second
@@ -42,7 +44,7 @@ def both(gpu, w, a, alpha=1.0, beta=0.0, c0=None):
         outs.append(gpu.download(c_buf, np.float32, (m, w.n)))
         c_buf.free()
     a_buf.free()
-    return outs[0], outs[1], kernels[0] == kernels[1]
+    return outs[0], outs[1], kernels[0] == kernels[1] and not kernels[0].startswith("gemm_i8")
 
 
 def same(want, got, same_kernel):
@@ -64,7 +66,7 @@ def test_static_entry_point_equals_the_allocating_one_on_two_calls_in_a_row(gpu,
             w = make(gpu, dtype, layout, n, k, seed=n + k)
             a = rng.standard_normal((m, k)).astype(np.float32)
             want, got, same_kernel = both(gpu, w, a)
-            assert same_kernel == (not (m == 1 and k > 4096))
+            assert same_kernel == (not (m == 1 and k > 4096) and m <= 8)
             assert same(want, got, same_kernel), (m, n, k)
             ref = orc.matmul_nt_q8(a, w.download(), n, threads=8) if layout == be.ROWS_NK else orc.matmul_q_packed(dtype, a, w.download(), n, threads=8)
             assert float(np.abs(got - ref).max()) <= 1e-5 * float(np.sqrt((ref.astype(np.float64) ** 2).mean()))
