@@ -567,7 +567,11 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
     // (measured: one batch, one kv head, up to ~1024 positions x 8 heads): 16-row tiles spread the K/V reads
     // over many CUs, which outweighs re-reading K/V per row tile from L2.
     const int cus0 = ctx->cu_count > 0 ? ctx->cu_count : 256;
-    const bool split = a.rows_total <= 64 || (!HILO && (long)units * ((a.rows_total + PF_ROWS - 1) / PF_ROWS) * PF_FLASH_BELOW <= cus0) ||
+    // (the smaller the head, the longer the 16-row kernel stays ahead: per key it re-reads less. Crossovers measured over
+    // five head layouts x L = 128 .. 2048: about 80 / 40 / 32 workgroups of the 128-row kernel at head size 64 / 128 / 256)
+    const long pf_wgs = (long)units * ((a.rows_total + PF_ROWS - 1) / PF_ROWS);
+    const long pf_min = D <= 64 ? (long)cus0 * 5 / (2 * PF_FLASH_BELOW) : D <= 128 ? (long)cus0 * 5 / (4 * PF_FLASH_BELOW) : (long)cus0 / PF_FLASH_BELOW;
+    const bool split = a.rows_total <= 64 || (!HILO && pf_wgs <= pf_min) ||
                        (!HILO && !prefill_takes(a, D));      // e.g. a softmax scale that is not positive: the 16-row kernel takes any
     if (split) {
         // key segments: one 32-key tile per wavefront while that leaves the device under-filled,

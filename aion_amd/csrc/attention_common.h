@@ -126,7 +126,7 @@ __device__ __forceinline__ void static_for(F &&f) {
 // ---- prefill kernel (attention_prefill.hip): 128 query rows per workgroup, 64-key tiles
 constexpr int PF_ROWS = 128, PF_TK = 64;
 #ifndef PF_FLASH_BELOW
-#define PF_FLASH_BELOW 8   // prompts whose 128-row workgroups would fill under 1/PF_FLASH_BELOW of the CUs run on the 16-row split kernel
+#define PF_FLASH_BELOW 8   // prompts whose 128-row workgroups would fill under 1/PF_FLASH_BELOW of the CUs (head size 256; more at smaller heads) run on the 16-row split kernel
 #endif
 // whether the prefill kernel takes this call (head size 64, 128 or 256; K/V f16 or bf16; not the hi+lo precise mode)
 bool prefill_takes(const AttnArgs &a, int d);

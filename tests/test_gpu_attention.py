@@ -57,11 +57,13 @@ def make_qkv(seed, B, L, T, Hq, Hkv, D, kind):
     return (qb, kb, vb, be.BF16, be.BF16), (qf, kf, vf)
 
 
-# A prompt whose 128-row workgroups would leave three quarters of the CUs idle runs on the 16-row split kernel;
-# L = 150 (2 x 2 units x 5 workgroups) is such a prompt, L = 560 (2 x 2 x 18) is not.
+# A prompt with few 128-row workgroups runs on the 16-row split kernel (up to about 80 / 40 / 32 of them at head size
+# 64 / 128 / 256: the smaller the head, the longer the 16-row kernel stays ahead). L = 150 (2 x 2 units x 5 workgroups) is
+# such a prompt at every head size, L = 560 (2 x 2 x 18 = 72) at head size 64 only, L = 1100 (140) at none.
 @pytest.mark.parametrize("kind,tol", [("f16", 2e-3), ("bf16", 1e-2)])
-@pytest.mark.parametrize("D", [64, 128, 256])
-@pytest.mark.parametrize("L,kernel", [(150, "attn_flash_split"), (560, "attn_prefill")])
+@pytest.mark.parametrize("D,L,kernel", [(64, 150, "attn_flash_split"), (128, 150, "attn_flash_split"), (256, 150, "attn_flash_split"),
+                                        (64, 560, "attn_flash_split"), (128, 560, "attn_prefill"), (256, 560, "attn_prefill"),
+                                        (64, 1100, "attn_prefill")])
 def test_prefill_causal_gqa(gpu, orc, kind, tol, D, L, kernel):
     B, Hq, Hkv = 2, 8, 2
     say("prefill", kind, D, L)
