@@ -777,14 +777,14 @@ int launch_prefill_t(aionhip_ctx *ctx, AttnArgs &a) {
     // two segments for balance only pay from 32 key tiles on (8 kv heads x 4 query heads each, L = 1024: 26 us in one
     // segment, 35 in two; one kv head x 8, L = 2048: 40 against 33).
     const int seg_tiles = D > 128 ? PF_SEG_TILES : 2 * PF_SEG_TILES;
-    const bool balance_pays = key_tiles >= (D > 128 ? 16 : 32);
+    const bool balance_pays = key_tiles >= (D > 128 ? 40 : 32);     // (head size 256, 2 kv heads x 8, L = 2048, 32 key tiles: 63 us in one segment, 78 in two)
     int want = cus0 / max(wgs, 1);
     if (want < 2 && wgs <= cus0 && balance_pays) want = 2;      // one round of workgroups: two segments even out what a causal mask skews
     // Between one and two rounds the longest row tile alone takes as long as two average ones (under a causal mask a tile's
     // work grows with its index): the device is busy wgs / (2 * CUs) of the time. Two segments halve the longest piece;
     // they pay while that gain exceeds the merge pass (measured at 8 heads x head size 256: 260 workgroups 109 -> 94 us, 288
     // 122 -> 116, 320 the same, 352 and more slower).
-    if (want < 2 && D > 128 && (long)wgs * 10 < (long)cus0 * PF_TWO_SEG_BELOW_TENTHS) want = 2;
+    if (want < 2 && D > 128 && wgs > cus0 && balance_pays && (long)wgs * 10 < (long)cus0 * PF_TWO_SEG_BELOW_TENTHS) want = 2;
     int nseg = max(1, min(min(want, key_tiles / seg_tiles), 16));
     a.nseg = nseg;
     if (nseg > 1) {
