@@ -41,6 +41,18 @@ int check_batch(aionhip_ctx *ctx, const char *what, size_t count, const aionhip_
     return AIONHIP_OK;
 }
 
+// One row: the kernel that prepares the activation in every workgroup. Up to FUSED_PAYS_K always; up to FUSED_MAX_K where
+// the outputs are many enough for the weight stream to hide the longer prologue (from 16384 outputs on it measures 8-30 %
+// ahead of both the K slices and preparation + GEMV: q4 8192 -> 28672 at 23.2 against 25.3 us, q8 8192 -> 32768 at 46 against 65),
+// up to a GiB of weights (q8 8192 -> 131072, 1.14 GB, measures 207 against 175 us the other way).
+static bool fused_row_pays(const Batch &b) {
+    if (b.k <= FUSED_PAYS_K) return true;
+    size_t n = 0;
+    for (size_t i = 0; i < b.count; ++i) n += b.w[i]->n;
+    const size_t bytes = n * (b.k / 32) * (b.w[0]->dtype == AIONHIP_Q8_0 ? 34 : 18);
+    return b.k <= FUSED_MAX_K && n >= 16384 && bytes <= ((size_t)1 << 30);
+}
+
 // every weight of `b` against the f32 rows at `a` (already materialised). static_scratch: the prepared activation goes
 // to the library's file-scope device array and nothing on the way may allocate.
 int run_rows(aionhip_ctx *ctx, const Batch &b, size_t m, const float *a, size_t lda, float alpha, float beta, bool static_scratch = false) {
@@ -53,7 +65,7 @@ int run_rows(aionhip_ctx *ctx, const Batch &b, size_t m, const float *a, size_t 
             return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "matmul_static: the prepared activation of m=%zu, k=%zu needs %zu bytes, the static scratch holds %zu",
                            m, b.k, prepared_act_bytes(m, b.k), STATIC_SCRATCH_BYTES);
     }
-    if (m == 1 && b.k <= FUSED_PAYS_K && ((uintptr_t)a & 15) == 0)
+    if (m == 1 && fused_row_pays(b) && ((uintptr_t)a & 15) == 0)
         return launch_gemv_fused(ctx, b.w, b.c, b.ldc, (int)b.count, PRO_QUANT, FusedIn{a, nullptr, nullptr, nullptr, 0.f}, alpha, beta);
     // one row, one weight, long K: slices of K across workgroups, preparation inside, one launch (it keeps a growable buffer
     // of its own, so not on the path that may not allocate)
@@ -152,7 +164,7 @@ int aionhip_step_rmsnorm_matmul(aionhip_ctx *ctx, size_t count, const aionhip_we
     if (!x || !gamma) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "rmsnorm_matmul: null x or gamma");
     if (!(eps > 0.f) || !(eps < INFINITY)) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "rmsnorm_matmul: eps must be positive and finite");
     const float *xp = (const float *)(uintptr_t)x, *gp = (const float *)(uintptr_t)gamma, *bp = (const float *)(uintptr_t)beta_norm;
-    if (rows == 1 && b.k <= FUSED_PAYS_K && ((x | gamma | beta_norm) & 15) == 0)
+    if (rows == 1 && fused_row_pays(b) && ((x | gamma | beta_norm) & 15) == 0)
         return launch_gemv_fused(ctx, b.w, b.c, b.ldc, (int)b.count, PRO_RMSNORM, FusedIn{xp, nullptr, gp, bp, eps}, alpha, beta);
     // several rows: the norm runs as its own kernel into scratch, then the ordinary routing
     const size_t act_bytes = (prepared_act_bytes(rows, b.k) + 255) & ~(size_t)255;
@@ -228,7 +240,7 @@ int aionhip_step_gate_matmul(aionhip_ctx *ctx, const aionhip_weight *w, size_t r
     if (rc) return rc;
     if (!gate || !up || ((gate | up) & 3)) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "gate_matmul: null or misaligned gate/up");
     const float *gp = (const float *)(uintptr_t)gate, *up_p = (const float *)(uintptr_t)up;
-    if (rows == 1 && b.k <= FUSED_PAYS_K && ((gate | up) & 15) == 0)
+    if (rows == 1 && fused_row_pays(b) && ((gate | up) & 15) == 0)
         return launch_gemv_fused(ctx, b.w, b.c, b.ldc, 1, PRO_GATE, FusedIn{gp, up_p, nullptr, nullptr, 0.f}, alpha, beta);
     if (rows <= GEMV_MAX_M) {
         // gate and activation preparation in one small launch, then the GEMV on the prepared rows

@@ -181,11 +181,13 @@ def test_config2_decode_shapes(gpu, orc, dtype, layout, n, k):
 
 # One activation row against a long reduction axis: past K = 4096 the K axis is cut into slices across workgroups, each of
 # which prepares its own slice of the activation (gemv_ksplit_kernel); past 65536 columns or rows the activation is prepared
-# by a launch of its own and the GEMV reads it from memory. Edges: the first K past 4096, few rows and one row, K that is not
+# by a launch of its own and the GEMV reads it from memory. Up to K = 8192 a weight of 16384 or more outputs stays on the
+# kernel that prepares the whole activation in every workgroup (the weight stream hides the prologue). Edges: the first K past 4096, few rows and one row, K that is not
 # a multiple of the 64 chunks a wavefront covers per pass or of the slice count, the config-2 shape 4096 x 14336, alpha/beta.
 @pytest.mark.parametrize("dtype,layout", CASES)
 @pytest.mark.parametrize("n,k,kernel", [(5, 4128, "ksplit"), (300, 16384, "ksplit"), (70, 16416, "ksplit"), (2050, 8224, "ksplit"), (9000, 4096, "fused"),
-                                        (4096, 14336, "ksplit"), (1, 32768, "ksplit"), (33, 65568, "gemv"), (70000, 4128, "gemv")])
+                                        (4096, 14336, "ksplit"), (1, 32768, "ksplit"), (33, 65568, "gemv"), (70000, 4128, "fused"),
+                                        (16390, 8192, "fused"), (16376, 8192, "ksplit"), (66000, 8224, "gemv")])
 def test_single_row_long_k(gpu, orc, dtype, layout, n, k, kernel):
     say("single row, long k", dtype, layout, n, k)
     blocks, w = make_weight(gpu, orc, dtype, layout, n, k, seed=n + k)
@@ -386,3 +388,39 @@ def test_rmsnorm_matmul_and_gate_matmul_match_the_separate_steps(gpu, orc, dtype
     for t in (xb, gb, c1, c2, gtb, upb, cres, g8, u8, c8):
         t.free()
     w1.free(); w2.free(); w3.free()
+
+
+# K between 4096 and 8192 with 16384 or more outputs in the call: one row keeps the fused kernels (eight activation chunks
+# per thread), with the RMSNorm and the gate prologues as well; the outputs of two sibling weights count together.
+@pytest.mark.parametrize("dtype,layout", CASES)
+def test_fused_prologues_at_k_up_to_8192_with_many_outputs(gpu, orc, dtype, layout):
+    rng = np.random.default_rng(11 + dtype)
+    k, n1, n2 = 6176, 9000, 7400
+    b1, w1 = make_weight(gpu, orc, dtype, layout, n1, k, seed=1)
+    b2, w2 = make_weight(gpu, orc, dtype, layout, n2, k, seed=2)
+    x = rng.standard_normal((1, k)).astype(np.float32)
+    gamma = (1 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    xb, gb = gpu.upload(x), gpu.upload(gamma)
+    c1, c2 = gpu.alloc(n1 * 4), gpu.alloc(n2 * 4)
+    gpu.step_rmsnorm_matmul([w1, w2], xb, gb, 1, [c1, c2], 1e-6)
+    assert gpu.last_kernel().endswith("_rmsnorm")
+    h = orc.rmsnorm(x, gamma, 1e-6)
+    assert rms_err(gpu.download(c1, np.float32, (1, n1)), oracle_matmul(orc, dtype, layout, h, b1, n1)) < 3e-3
+    assert rms_err(gpu.download(c2, np.float32, (1, n2)), oracle_matmul(orc, dtype, layout, h, b2, n2)) < 3e-3
+    gpu.step_rmsnorm_matmul([w1], xb, gb, 1, [c1], 1e-6)           # 9000 outputs alone: norm kernel, then the K slices
+    assert not gpu.last_kernel().endswith("_rmsnorm")
+    assert rms_err(gpu.download(c1, np.float32, (1, n1)), oracle_matmul(orc, dtype, layout, h, b1, n1)) < 3e-3
+    w1.free(); w2.free()
+    n3 = 16384
+    b3, w3 = make_weight(gpu, orc, dtype, layout, n3, 8192, seed=3)
+    gate = (rng.standard_normal((1, 8192)) * 2).astype(np.float32)
+    up = rng.standard_normal((1, 8192)).astype(np.float32)
+    res0 = rng.standard_normal((1, n3)).astype(np.float32)
+    g8, u8, c3 = gpu.upload(gate), gpu.upload(up), gpu.upload(res0)
+    gpu.step_gate_matmul(w3, g8, u8, 1, c3, beta=1.0)
+    assert gpu.last_kernel().endswith("_gate")
+    want = oracle_matmul(orc, dtype, layout, orc.gate_gelu(gate, up).reshape(1, 8192), b3, n3, beta=1.0, c=res0)
+    assert rms_err(gpu.download(c3, np.float32, (1, n3)), want) < 3e-3
+    for t in (xb, gb, c1, c2, g8, u8, c3):
+        t.free()
+    w3.free()
