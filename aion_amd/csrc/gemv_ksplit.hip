@@ -27,7 +27,8 @@ constexpr int KSPLIT_MAX_S = 8;
 // round trip of the activation slice. NCH: float4 activation chunks per thread (the slice has at most 4 * NT * NCH floats).
 template <int DT, int R, int NT, int NCH, int CPL>
 __global__ __launch_bounds__(NT) void gemv_ksplit_kernel(const u32x4 *__restrict__ qs, const __half *__restrict__ sc, float *__restrict__ c,
-                                                         const float *__restrict__ x, unsigned long long *meet, int N, int K, int kbs, int S, float alpha, float beta) {
+                                                         const float *__restrict__ x, unsigned long long *meet, int N, int K, int kbs, int S, int groups, int interleave,
+                                                         float alpha, float beta) {
     extern __shared__ __attribute__((aligned(16))) unsigned char s_mem[];
     constexpr bool Q8 = DT == AIONHIP_Q8_0;
     constexpr int WPB = NT / 64;                            // wavefronts per workgroup
@@ -37,7 +38,19 @@ __global__ __launch_bounds__(NT) void gemv_ksplit_kernel(const u32x4 *__restrict
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int g = blockIdx.x, s = blockIdx.y;
+    // workgroup -> (row group, slice). Slice-major (all row groups of slice 0 first) is the faster order in general. Where
+    // the row pitch is a multiple of 8 KiB, a slice is the same 2 KiB column range of every row, and a dispatch order that
+    // works through one slice at a time keeps hitting the same quarter of the memory channels; there the slices alternate from
+    // one workgroup to the next, rotated every 8 / S row groups so that one XCD (every eighth workgroup) sees all of them.
+    const int b_lin = blockIdx.x;
+    int g, s;
+    if (interleave) {
+        g = b_lin / S;
+        s = (b_lin % S + g / (S >= 8 ? 1 : 8 / S)) % S;
+    } else {
+        g = b_lin % groups;
+        s = b_lin / groups;
+    }
     const int KB = K >> 5, kb0 = s * kbs, kbn = min(kbs, KB - kb0);
     const int gw = g * WPB + wave;                          // this wavefront's row group
     const int row0 = gw * R;
@@ -161,13 +174,19 @@ __global__ __launch_bounds__(NT) void gemv_ksplit_kernel(const u32x4 *__restrict
 template <int DT, int R, int NT, int CPL>
 void launch_s(aionhip_ctx *ctx, const aionhip_weight *w, float *c, const float *x, unsigned long long *meet, int groups, int kbs, int S,
               float alpha, float beta) {
-    const dim3 grid((unsigned)groups, (unsigned)S), block(NT);
+    const dim3 grid((unsigned)groups * (unsigned)S), block(NT);
+    // Bytes from one weight row to the next. Near 4, 8 or 32 KiB the slices alternate in dispatch order (measured over N =
+    // 2048 ... 14336: 8 KiB from 4096 rows on, q8 8192 x 8192 19.4 -> 14.2 us, q4 8192 x 16384 20.2 -> 15.0; 4 KiB from 8192 rows
+    // on, q4 8192 x 8192 9.3 -> 8.1; 32 KiB 3-25 %; 12, 16, 20, 24 KiB and every other pitch are 3-10 % better slice by slice).
+    const size_t pitch = w->dtype == AIONHIP_Q8_0 ? w->k : w->k / 2;
+    auto near = [&](size_t p) { return pitch + 128 >= p && pitch <= p + 128; };
+    const int interleave = S > 1 && ((near(8192) && w->n >= 4096) || (near(4096) && w->n >= 8192) || near(32768)) ? 1 : 0;
     const size_t lds = (size_t)kbs * 40 + 16;
     const int n = (int)w->n, k = (int)w->k;
     const int per_pass = NT / 8;                            // quant blocks one pass of the workgroup prepares
-    if (kbs <= per_pass) launch_k(ctx, gemv_ksplit_kernel<DT, R, NT, 1, CPL>, grid, block, lds, (const u32x4 *)w->qs, w->sc, c, x, meet, n, k, kbs, S, alpha, beta);
-    else if (kbs <= 2 * per_pass) launch_k(ctx, gemv_ksplit_kernel<DT, R, NT, 2, CPL>, grid, block, lds, (const u32x4 *)w->qs, w->sc, c, x, meet, n, k, kbs, S, alpha, beta);
-    else launch_k(ctx, gemv_ksplit_kernel<DT, R, NT, 4, CPL>, grid, block, lds, (const u32x4 *)w->qs, w->sc, c, x, meet, n, k, kbs, S, alpha, beta);
+    if (kbs <= per_pass) launch_k(ctx, gemv_ksplit_kernel<DT, R, NT, 1, CPL>, grid, block, lds, (const u32x4 *)w->qs, w->sc, c, x, meet, n, k, kbs, S, groups, interleave, alpha, beta);
+    else if (kbs <= 2 * per_pass) launch_k(ctx, gemv_ksplit_kernel<DT, R, NT, 2, CPL>, grid, block, lds, (const u32x4 *)w->qs, w->sc, c, x, meet, n, k, kbs, S, groups, interleave, alpha, beta);
+    else launch_k(ctx, gemv_ksplit_kernel<DT, R, NT, 4, CPL>, grid, block, lds, (const u32x4 *)w->qs, w->sc, c, x, meet, n, k, kbs, S, groups, interleave, alpha, beta);
 }
 
 template <int DT, int R, int NT>

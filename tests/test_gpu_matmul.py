@@ -184,10 +184,13 @@ def test_config2_decode_shapes(gpu, orc, dtype, layout, n, k):
 # by a launch of its own and the GEMV reads it from memory. Up to K = 8192 a weight of 16384 or more outputs stays on the
 # kernel that prepares the whole activation in every workgroup (the weight stream hides the prologue). Edges: the first K past 4096, few rows and one row, K that is not
 # a multiple of the 64 chunks a wavefront covers per pass or of the slice count, the config-2 shape 4096 x 14336, alpha/beta.
+# The last four: row pitches of 4, 8 and 32 KiB, where the workgroups take the slices in alternating instead of slice-major
+# order (q8 8192 and 32768, q4 8192 and 16384).
 @pytest.mark.parametrize("dtype,layout", CASES)
 @pytest.mark.parametrize("n,k,kernel", [(5, 4128, "ksplit"), (300, 16384, "ksplit"), (70, 16416, "ksplit"), (2050, 8224, "ksplit"), (9000, 4096, "fused"),
                                         (4096, 14336, "ksplit"), (1, 32768, "ksplit"), (33, 65568, "gemv"), (70000, 4128, "fused"),
-                                        (16390, 8192, "fused"), (16376, 8192, "ksplit"), (66000, 8224, "gemv")])
+                                        (16390, 8192, "fused"), (16376, 8192, "ksplit"), (66000, 8224, "gemv"),
+                                        (4100, 8192, "ksplit"), (8200, 8192, "ksplit"), (4100, 16384, "ksplit"), (40, 32768, "ksplit")])
 def test_single_row_long_k(gpu, orc, dtype, layout, n, k, kernel):
     say("single row, long k", dtype, layout, n, k)
     blocks, w = make_weight(gpu, orc, dtype, layout, n, k, seed=n + k)
@@ -205,6 +208,19 @@ def test_single_row_long_k(gpu, orc, dtype, layout, n, k, kernel):
     got2 = gpu.matmul(w, a, alpha=0.5, beta=-2.0, c=c0)
     want2 = oracle_matmul(orc, dtype, layout, a, blocks, n, alpha=0.5, beta=-2.0, c=c0)
     assert norm_err(got2, want2) < TOL and rms_err(got2, want2) < RMS_TOL
+    w.free()
+
+
+def test_single_row_q4_eight_alternating_slices(gpu, orc):
+    # q4 at K = 65536: eight slices over a row pitch of 32 KiB, taken in alternating order
+    n, k = 24, 65536
+    blocks, w = make_weight(gpu, orc, be.Q4_0, be.KMAJOR_KN, n, k, seed=5)
+    a = np.random.default_rng(5).standard_normal((1, k)).astype(np.float32)
+    got = gpu.matmul(w, a)
+    assert gpu.last_kernel() == "gemv_q4_ksplit"
+    want = oracle_matmul(orc, be.Q4_0, be.KMAJOR_KN, a, blocks, n)
+    assert norm_err(got, want) < TOL and rms_err(got, want) < RMS_TOL
+    assert np.array_equal(gpu.matmul(w, a), got)
     w.free()
 
 
