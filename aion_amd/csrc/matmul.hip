@@ -53,6 +53,21 @@ static bool fused_row_pays(const Batch &b) {
     return b.k <= FUSED_MAX_K && n >= 16384 && bytes <= ((size_t)1 << 30);
 }
 
+// Prepared rows against the weights of `b`: the GEMV kernels up to eight rows, except five to eight rows over a K past 4096,
+// where the GEMV walks K with all eight accumulator sets live and falls far behind the exact GEMM's 16-row tile (q8
+// 14336 x 8192 at 8 rows: 80 against 33 us, q4 65 against 29; the two meet at K = 4096 ... 5120); the GEMM beyond eight rows.
+static int launch_prepared_rows(aionhip_ctx *ctx, const Batch &b, size_t m, PreparedAct act, float alpha, float beta) {
+    if (m <= GEMV_MAX_M && !(m >= 5 && b.k > FUSED_PAYS_K))
+        return launch_gemv_batch(ctx, b.w, b.c, b.ldc, (int)b.count, (int)m, act, alpha, beta);
+    // sibling weights (q/k/v, gate/up) share one launch, four at a time
+    for (size_t i = 0; i < b.count; i += 4) {
+        const size_t cnt = b.count - i < 4 ? b.count - i : 4;
+        const int rc = launch_gemm_i8_batch(ctx, b.w + i, b.c + i, b.ldc + i, (int)cnt, m, act, alpha, beta);
+        if (rc) return rc;
+    }
+    return AIONHIP_OK;
+}
+
 // every weight of `b` against the f32 rows at `a` (already materialised). static_scratch: the prepared activation goes
 // to the library's file-scope device array and nothing on the way may allocate.
 int run_rows(aionhip_ctx *ctx, const Batch &b, size_t m, const float *a, size_t lda, float alpha, float beta, bool static_scratch = false) {
@@ -89,14 +104,7 @@ int run_rows(aionhip_ctx *ctx, const Batch &b, size_t m, const float *a, size_t 
     PreparedAct act = prepared_act_carve(static_scratch ? ctx->static_scratch : ctx->scratch, m, b.k);
     rc = launch_prepare_act(ctx, a, lda, m, b.k, act);
     if (rc) return rc;
-    if (m <= GEMV_MAX_M) return launch_gemv_batch(ctx, b.w, b.c, b.ldc, (int)b.count, (int)m, act, alpha, beta);
-    // sibling weights (q/k/v, gate/up) share one launch, four at a time
-    for (size_t i = 0; i < b.count; i += 4) {
-        const size_t cnt = b.count - i < 4 ? b.count - i : 4;
-        rc = launch_gemm_i8_batch(ctx, b.w + i, b.c + i, b.ldc + i, (int)cnt, m, act, alpha, beta);
-        if (rc) return rc;
-    }
-    return AIONHIP_OK;
+    return launch_prepared_rows(ctx, b, m, act, alpha, beta);
 }
 
 int run_matmul(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, aionhip_handle a_h, size_t lda, aionhip_handle c_h, size_t ldc,
@@ -249,7 +257,7 @@ int aionhip_step_gate_matmul(aionhip_ctx *ctx, const aionhip_weight *w, size_t r
         PreparedAct act = prepared_act_carve(ctx->scratch, rows, b.k);
         rc = launch_prepare_gate(ctx, gp, up_p, rows, b.k, act);
         if (rc) return rc;
-        return launch_gemv_batch(ctx, b.w, b.c, b.ldc, 1, (int)rows, act, alpha, beta);
+        return launch_prepared_rows(ctx, b, rows, act, alpha, beta);
     }
     const size_t act_bytes = (prepared_act_bytes(rows, b.k) + 255) & ~(size_t)255;
     rc = ensure_scratch(ctx, act_bytes + rows * b.k * sizeof(float));

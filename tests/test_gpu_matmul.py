@@ -289,12 +289,14 @@ def test_exact_gemm_shapes_and_edges(gpu, orc, dtype, layout, m, n, k):
 
 
 # 2..8 activation rows (gemv_rows_kernel): row counts that fill a 2-, 4- or 8-row instance only partly, N that is
-# not a multiple of the rows a wavefront works on, K of one LDS pass and K long enough to run as several K-range
-# launches (14336 at 8 rows), alpha/beta on a pre-filled C. The last three shapes (5..8 rows, at least 16384 columns,
-# K up to 4096) run on the 16-row tile of the LDS-staged MFMA kernel instead: ragged N, K of one and of many steps.
+# not a multiple of the rows a wavefront works on, K of one LDS pass, K that needs most of a CU's LDS (16384 at 4 rows) and K
+# long enough to run as several K-range launches (32768 at 3 rows), alpha/beta on a pre-filled C. Three shapes (5..8 rows, at
+# least 16384 columns, K up to 4096) run on the 16-row tile of the LDS-staged MFMA kernel instead: ragged N, K of one and of
+# many steps. Five to eight rows over a K past 4096 take the exact GEMM (its 16-row tile is far ahead there).
 @pytest.mark.parametrize("dtype,layout", CASES)
 @pytest.mark.parametrize("m,n,k", [(2, 70, 96), (3, 1001, 1056), (5, 333, 2048), (8, 1030, 14336), (7, 4100, 7200), (4, 9000, 512),
-                                   (5, 16390, 256), (8, 20001, 2048), (6, 16384, 4096)])
+                                   (5, 16390, 256), (8, 20001, 2048), (6, 16384, 4096), (4, 1030, 16384), (3, 300, 32768),
+                                   (5, 70, 4128), (8, 14336, 8192)])
 def test_decode_gemv_two_to_eight_rows(gpu, orc, dtype, layout, m, n, k):
     say("gemv rows", dtype, layout, m, n, k)
     blocks, w = make_weight(gpu, orc, dtype, layout, n, k, seed=m * 31 + n + k, std=0.05)
@@ -302,7 +304,7 @@ def test_decode_gemv_two_to_eight_rows(gpu, orc, dtype, layout, m, n, k):
     a = rng.standard_normal((m, k)).astype(np.float32)
     c0 = rng.standard_normal((m, n)).astype(np.float32)
     got = gpu.matmul(w, a)
-    assert gpu.last_kernel() == ("gemv_q8" if dtype == be.Q8_0 else "gemv_q4")
+    assert gpu.last_kernel() == ("gemm_i8_" if m >= 5 and k > 4096 else "gemv_") + ("q8" if dtype == be.Q8_0 else "q4")
     want = oracle_matmul(orc, dtype, layout, a, blocks, n)
     assert norm_err(got, want) < TOL and rms_err(got, want) < RMS_TOL
     got2 = gpu.matmul(w, a, alpha=-1.5, beta=0.25, c=c0)
@@ -361,7 +363,7 @@ def test_single_row_fused_kernel_equals_prepared_path(gpu, orc, dtype, layout):
 
 
 @pytest.mark.parametrize("dtype,layout", CASES)
-@pytest.mark.parametrize("rows", [1, 3])
+@pytest.mark.parametrize("rows", [1, 3, 6])
 def test_rmsnorm_matmul_and_gate_matmul_match_the_separate_steps(gpu, orc, dtype, layout, rows):
     say("fused steps", dtype, layout, rows)
     rng = np.random.default_rng(rows + dtype)
