@@ -45,8 +45,11 @@ int check_batch(aionhip_ctx *ctx, const char *what, size_t count, const aionhip_
 // the outputs are many enough for the weight stream to hide the longer prologue (from 16384 outputs on it measures 8-30 %
 // ahead of both the K slices and preparation + GEMV: q4 8192 -> 28672 at 23.2 against 25.3 us, q8 8192 -> 32768 at 46 against 65),
 // up to a GiB of weights (q8 8192 -> 131072, 1.14 GB, measures 207 against 175 us the other way).
+// Sibling weights in one call have no K-slice form: up to FUSED_MAX_K they stay here as well, one launch against preparation +
+// GEMV (q/k/v of 5120 -> 5120 + 2 x 1024, q4: 6.5 against 10.2 us; 8192 -> 8192 + 2 x 1024: 11.0 against 18.2).
 static bool fused_row_pays(const Batch &b) {
     if (b.k <= FUSED_PAYS_K) return true;
+    if (b.count > 1 && b.k <= FUSED_MAX_K) return true;
     size_t n = 0;
     for (size_t i = 0; i < b.count; ++i) n += b.w[i]->n;
     const size_t bytes = n * (b.k / 32) * (b.w[0]->dtype == AIONHIP_Q8_0 ? 34 : 18);

@@ -439,6 +439,14 @@ def test_fused_prologues_at_k_up_to_8192_with_many_outputs(gpu, orc, dtype, layo
     assert gpu.last_kernel().endswith("_gate")
     want = oracle_matmul(orc, dtype, layout, orc.gate_gelu(gate, up).reshape(1, 8192), b3, n3, beta=1.0, c=res0)
     assert rms_err(gpu.download(c3, np.float32, (1, n3)), want) < 3e-3
-    for t in (xb, gb, c1, c2, g8, u8, c3):
+    # sibling weights in one call stay on the fused kernel whatever their size (there is no K-slice form for them)
+    b4, w4 = make_weight(gpu, orc, dtype, layout, 300, k, seed=4)
+    b5, w5 = make_weight(gpu, orc, dtype, layout, 72, k, seed=5)
+    c4, c5 = gpu.alloc(300 * 4), gpu.alloc(72 * 4)
+    gpu.step_matmul_batch([w4, w5], xb, 1, [c4, c5])
+    assert gpu.last_kernel().endswith("_fused")
+    assert rms_err(gpu.download(c4, np.float32, (1, 300)), oracle_matmul(orc, dtype, layout, x, b4, 300)) < RMS_TOL
+    assert rms_err(gpu.download(c5, np.float32, (1, 72)), oracle_matmul(orc, dtype, layout, x, b5, 72)) < RMS_TOL
+    for t in (xb, gb, c1, c2, g8, u8, c3, c4, c5):
         t.free()
-    w3.free()
+    w3.free(); w4.free(); w5.free()
