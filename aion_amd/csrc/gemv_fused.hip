@@ -416,10 +416,12 @@ int launch_gemv_fused_geglu(aionhip_ctx *ctx, const aionhip_weight *gate, const 
     const size_t k = gate->k;
     if (q8) {
         if (k <= 2048) launch_geglu<AIONHIP_Q8_0, 2>(ctx, gate, up, in, out);
-        else launch_geglu<AIONHIP_Q8_0, 4>(ctx, gate, up, in, out);
+        else if (k <= 4096) launch_geglu<AIONHIP_Q8_0, 4>(ctx, gate, up, in, out);
+        else launch_geglu<AIONHIP_Q8_0, 8>(ctx, gate, up, in, out);
     } else {
         if (k <= 2048) launch_geglu<AIONHIP_Q4_0, 2>(ctx, gate, up, in, out);
-        else launch_geglu<AIONHIP_Q4_0, 4>(ctx, gate, up, in, out);
+        else if (k <= 4096) launch_geglu<AIONHIP_Q4_0, 4>(ctx, gate, up, in, out);
+        else launch_geglu<AIONHIP_Q4_0, 8>(ctx, gate, up, in, out);
     }
     LAUNCH_CHECK(ctx, name);
     return AIONHIP_OK;
@@ -432,10 +434,12 @@ int launch_gemv_fused_rope(aionhip_ctx *ctx, const aionhip_weight *const *ws, fl
     const size_t k = ws[0]->k;
     if (q8) {
         if (k <= 2048) launch_rope<AIONHIP_Q8_0, 2>(ctx, ws, q_out, in, epi);
-        else launch_rope<AIONHIP_Q8_0, 4>(ctx, ws, q_out, in, epi);
+        else if (k <= 4096) launch_rope<AIONHIP_Q8_0, 4>(ctx, ws, q_out, in, epi);
+        else launch_rope<AIONHIP_Q8_0, 8>(ctx, ws, q_out, in, epi);
     } else {
         if (k <= 2048) launch_rope<AIONHIP_Q4_0, 2>(ctx, ws, q_out, in, epi);
-        else launch_rope<AIONHIP_Q4_0, 4>(ctx, ws, q_out, in, epi);
+        else if (k <= 4096) launch_rope<AIONHIP_Q4_0, 4>(ctx, ws, q_out, in, epi);
+        else launch_rope<AIONHIP_Q4_0, 8>(ctx, ws, q_out, in, epi);
     }
     LAUNCH_CHECK(ctx, name);
     return AIONHIP_OK;

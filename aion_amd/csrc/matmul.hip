@@ -205,8 +205,8 @@ int aionhip_step_rmsnorm_qkv_rope_append(aionhip_ctx *ctx, const aionhip_weight 
     if (d == 0 || d % 8 != 0 || d > 65528 || h_q == 0 || h_kv == 0 || wq->n != h_q * d || wk->n != h_kv * d || wv->n != h_kv * d)
         return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "qkv_rope_append: weight rows must be heads x head size, head size a multiple of 8");
     // one token of one sequence, short enough K for the in-kernel prologue: anything else takes the separate steps
-    if (wq->k > FUSED_PAYS_K || ((x | gamma | beta_norm) & 15) || (q_out & 3) || ((k_cache | v_cache) & 1) || t_cap == 0 || t_cap > 0x7FFFFFFFu)
-        return set_err(ctx, AIONHIP_UNSUPPORTED, "qkv_rope_append: needs k <= %zu, 16-byte aligned x/gamma/beta and a cache of 1..2^31-1 tokens", FUSED_PAYS_K);
+    if (wq->k > FUSED_MAX_K || ((x | gamma | beta_norm) & 15) || (q_out & 3) || ((k_cache | v_cache) & 1) || t_cap == 0 || t_cap > 0x7FFFFFFFu)
+        return set_err(ctx, AIONHIP_UNSUPPORTED, "qkv_rope_append: needs k <= %zu, 16-byte aligned x/gamma/beta and a cache of 1..2^31-1 tokens", FUSED_MAX_K);
     const size_t half = d / 2;
     size_t rope_pairs = (size_t)floorf(rope_proportion * (float)half);
     if (rope_pairs > half) rope_pairs = half;
@@ -229,8 +229,8 @@ int aionhip_step_rmsnorm_geglu_matmul(aionhip_ctx *ctx, const aionhip_weight *w_
     if (w_gate->k != w_up->k || w_gate->n != w_up->n || w_gate->dtype != w_up->dtype || w_down->k != w_gate->n)
         return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "geglu_matmul: gate and up must match, down must take their outputs");
     if (c & 3) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "geglu_matmul: C not 4-byte aligned");
-    if (w_gate->k > FUSED_PAYS_K || w_gate->n % 32 != 0 || ((x | gamma | beta_norm) & 15))
-        return set_err(ctx, AIONHIP_UNSUPPORTED, "geglu_matmul: needs k <= %zu, a hidden size that is a multiple of 32 and 16-byte aligned x/gamma/beta", FUSED_PAYS_K);
+    if (w_gate->k > FUSED_MAX_K || w_gate->n % 32 != 0 || ((x | gamma | beta_norm) & 15))
+        return set_err(ctx, AIONHIP_UNSUPPORTED, "geglu_matmul: needs k <= %zu, a hidden size that is a multiple of 32 and 16-byte aligned x/gamma/beta", FUSED_MAX_K);
     int rc = ensure_scratch(ctx, prepared_act_bytes(1, w_down->k));
     if (rc) return rc;
     PreparedAct act = prepared_act_carve(ctx->scratch, 1, w_down->k);

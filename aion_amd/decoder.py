@@ -147,7 +147,7 @@ class Decoder:
         scale = 1.0 / math.sqrt(c.head_dim)
         for l in range(c.layers):
             p = "l%d." % l
-            if s == 1 and c.hidden <= 4096 and c.head_dim % 8 == 0:
+            if s == 1 and c.hidden <= 8192 and c.head_dim % 8 == 0:
                 # one new token: RMSNorm -> MatMul q, k, v -> RoPE1D(q), RoPE1D(k) -> f16 -> append, one launch
                 g.step_rmsnorm_qkv_rope_append(self.w[p + "wq"], self.w[p + "wk"], self.w[p + "wv"], b["x"], self.gamma, c.eps,
                                                b["qr"], self.kc[l], self.vc[l], b["positions"], b["write_index"],
@@ -164,7 +164,7 @@ class Decoder:
                              query_positions=b["positions"], kv_lengths=b["kv_len"])
             # MatMul o with beta = 1: x = x + att @ Wo (the residual add rides on the matmul's beta)
             g.step_matmul(self.w[p + "wo"], b["att"], s, b["x"], beta=1.0)
-            if s == 1 and c.hidden <= 4096 and c.ffn % 32 == 0:
+            if s == 1 and c.hidden <= 8192 and c.ffn % 32 == 0:
                 # one row: RMSNorm -> MatMul gate, up -> gate(gelu) -> MatMul down (beta = 1), two launches
                 g.step_rmsnorm_geglu_matmul(self.w[p + "wgate"], self.w[p + "wup"], self.w[p + "wdown"], b["x"], self.gamma, c.eps,
                                             b["x"], beta=1.0)

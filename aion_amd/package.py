@@ -263,7 +263,7 @@ class PackageRunner:
                 return False
             n0 = nodes[i]
             x = get(n0.inputs[0])
-            if x.shape[0] != 1 or x.shape[-1] > 4096:
+            if x.shape[0] != 1 or x.shape[-1] > 8192:
                 return False
             chains = {}
             for m in mms:
@@ -411,7 +411,7 @@ class PackageRunner:
                 return False
             n0 = nodes[i]
             x = get(n0.inputs[0])
-            if _count(x.shape[:-1]) != 1 or x.shape[-1] > 4096:
+            if _count(x.shape[:-1]) != 1 or x.shape[-1] > 8192:
                 return False
             ge = [m for m in mms if sole_user(nodes[m].output, "Unary") is not None]
             if len(ge) != 1:

@@ -162,7 +162,7 @@ int aionhip_step_matmul_batch(aionhip_ctx *ctx, size_t count, const aionhip_weig
  * (StepSequenceAppend, cpu/exec/sequence_append.zig:12-104), as one launch. q_out receives the rotated
  * query [h_q, d] f32; the caches are [t_cap, h_kv, d] f16 (batch 1). Same arithmetic as the separate steps
  * (aionhip_step_rmsnorm_matmul + aionhip_step_rope_append); rolling = 1: the caches are rings, as in
- * aionhip_step_append_f16. AIONHIP_UNSUPPORTED when the shape does not qualify (k above 4096, misaligned
+ * aionhip_step_append_f16. AIONHIP_UNSUPPORTED when the shape does not qualify (k above 8192, misaligned
  * operands): the caller then issues the separate steps. */
 int aionhip_step_rmsnorm_qkv_rope_append(aionhip_ctx *ctx, const aionhip_weight *wq, const aionhip_weight *wk, const aionhip_weight *wv,
                                          aionhip_handle x, aionhip_handle gamma, aionhip_handle beta_norm, float eps,
@@ -173,7 +173,7 @@ int aionhip_step_rmsnorm_qkv_rope_append(aionhip_ctx *ctx, const aionhip_weight 
  * gate(gelu_tanh) * up (cpu/exec/elementwise.zig:25-37) -> int8 activation preparation -> down matmul,
  * C[1, n_down] = alpha * (...) + beta * C, in two launches; the gate / up / gated rows never reach memory.
  * Same arithmetic as aionhip_step_rmsnorm_matmul + aionhip_step_gate_matmul. AIONHIP_UNSUPPORTED when the
- * shape does not qualify (k above 4096, hidden size not a multiple of 32, misaligned operands). */
+ * shape does not qualify (k above 8192, hidden size not a multiple of 32, misaligned operands). */
 int aionhip_step_rmsnorm_geglu_matmul(aionhip_ctx *ctx, const aionhip_weight *w_gate, const aionhip_weight *w_up, const aionhip_weight *w_down,
                                       aionhip_handle x, aionhip_handle gamma, aionhip_handle beta_norm, float eps,
                                       aionhip_handle c, float alpha, float beta);

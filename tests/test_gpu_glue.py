@@ -231,7 +231,7 @@ def test_headnorm_rope_append_equals_the_separate_steps(gpu, orc, B, S, T, Hq, H
 
 
 @pytest.mark.parametrize("dtype", ["q4", "q8"])
-@pytest.mark.parametrize("D,Hq,Hkv,K", [(256, 8, 1, 2048), (64, 4, 2, 512)])
+@pytest.mark.parametrize("D,Hq,Hkv,K", [(256, 8, 1, 2048), (64, 4, 2, 512), (128, 8, 2, 5120), (64, 16, 4, 8192)])
 def test_qkv_rope_append_fusion_equals_the_separate_steps(gpu, orc, dtype, D, Hq, Hkv, K):
     """RMSNorm -> q/k/v matmuls -> RoPE -> f16 append in one launch against the same steps issued one by one
     (and through them against the oracle, which the separate steps are tested against)."""
@@ -283,7 +283,7 @@ def test_qkv_rope_append_fusion_equals_the_separate_steps(gpu, orc, dtype, D, Hq
 
 
 @pytest.mark.parametrize("dtype", ["q4", "q8"])
-@pytest.mark.parametrize("K,F", [(2048, 8192), (256, 96), (4096, 1024)])
+@pytest.mark.parametrize("K,F", [(2048, 8192), (256, 96), (4096, 1024), (5120, 1024), (8192, 2048)])
 def test_geglu_fusion_equals_the_separate_steps(gpu, orc, dtype, K, F):
     """RMSNorm -> gate/up matmuls -> gelu gate -> int8 preparation -> down matmul in two launches against the
     separate steps: the prepared codes are the same integers, so the result is the same up to f32 summation order."""
