@@ -365,7 +365,8 @@ def time_kernel(gpu, ws, x, y, m, name, iters=20):
     for i in range(iters):
         gpu.step_matmul(ws[i % len(ws)], x, m, y)
     prof = gpu.profile_stop()
-    assert any(nm.startswith(name) for nm, _ms in prof), (name, prof[:4])
+    names = (name,) if isinstance(name, str) else tuple(name)
+    assert any(nm.startswith(names) for nm, _ms in prof), (name, prof[:4])
     per = len(prof) // iters                      # every launch of the call: the activation preparation and the GEMV(s)
     calls = sorted(sum(ms for _nm, ms in prof[i * per:(i + 1) * per]) for i in range(iters))
     return calls[iters // 2]
@@ -382,7 +383,8 @@ def run_sweep(gpu, be, q4_blocks):
             for m in (1, 4, 8):
                 x = gpu.upload(rng.standard_normal((m, k)).astype(np.float32))
                 y = gpu.alloc(m * n * 4)
-                ms = time_kernel(gpu, ws, x, y, m, kname)
+                # five to eight rows over a K past 4096 run on the exact GEMM's 16-row tile, everything else on a GEMV kernel
+                ms = time_kernel(gpu, ws, x, y, m, (kname, "gemm_i8_" + kname[-2:]) if m >= 5 and k > 4096 else kname)
                 by = algorithmic_bytes(bb, n, k, m)
                 res["%s %dx%d b%d" % ("q4" if dtype == be.Q4_0 else "q8", n, k, m)] = {
                     "kernels": gpu.last_kernel(), "kernel_us": round(ms * 1e3, 2), "GBps": round(by / (ms * 1e-3) / 1e9, 1),
