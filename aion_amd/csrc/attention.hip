@@ -571,8 +571,28 @@ int launch_flash(aionhip_ctx *ctx, AttnArgs &a) {
     // five head layouts x L = 128 .. 2048: about 80 / 40 / 32 workgroups of the 128-row kernel at head size 64 / 128 / 256)
     const long pf_wgs = (long)units * ((a.rows_total + PF_ROWS - 1) / PF_ROWS);
     const long pf_min = D <= 64 ? (long)cus0 * 5 / (2 * PF_FLASH_BELOW) : D <= 128 ? (long)cus0 * 5 / (4 * PF_FLASH_BELOW) : (long)cus0 / PF_FLASH_BELOW;
-    const bool split = a.rows_total <= 64 || (!HILO && pf_wgs <= pf_min) ||
-                       (!HILO && !prefill_takes(a, D));      // e.g. a softmax scale that is not positive: the 16-row kernel takes any
+    bool split = a.rows_total <= 64 || (!HILO && pf_wgs <= pf_min) ||
+                 (!HILO && !prefill_takes(a, D));      // e.g. a softmax scale that is not positive: the 16-row kernel takes any
+    // A chunk of queries over a cache at least four times its length (chunked prompts, speculative batches): the crossover
+    // above was measured on prompts over their own keys, where few rows mean few keys. Here the keys dominate, and the 128-row
+    // kernel, which can cut them into up to 16 segments, is weighed against the 16-row kernel by what both measured over
+    // 1 ... 1024 queries x 1024 ... 16384 keys at head sizes 128 and 256: the 16-row kernel 13 us + 0.56 us per 32-key tile a
+    // workgroup walks (head size 256; in proportion below), the 128-row kernel 16 us + 1.9 us per 64-key tile (1.2 at head
+    // size 128, 0.85 at 64; 0.7 of that while half the CUs stay free). 8 heads x 256, 256 queries over 16384 keys: 159 -> 46 us.
+    if (!HILO && a.rows_total > 64 && pf_wgs <= pf_min && prefill_takes(a, D) && (long)a.T >= 4L * a.L && a.win_left >= (unsigned)a.T) {
+        const float ds = (float)D / 256.f;
+        const long wgs16 = (long)units * a.row_tiles;
+        const int tiles32 = (a.T + TILE_KEYS - 1) / TILE_KEYS;
+        const long nseg_s = max(1L, min((long)cus0 / max(wgs16, 1L), (long)(tiles32 + SPLIT_NW - 1) / SPLIT_NW));
+        const long rounds_s = (wgs16 * nseg_s + cus0 - 1) / cus0;
+        const float split_us = (nseg_s > 1 ? 13.f : 10.f) + (float)((tiles32 + nseg_s - 1) / nseg_s) * 0.56f * ds * (float)rounds_s;
+        const int tiles64 = (a.T + PF_TK - 1) / PF_TK;
+        const long nseg_p = max(1L, min(min((long)cus0 / max(pf_wgs, 1L), (long)tiles64 / (D > 128 ? 4 : 8)), 16L));
+        const long rounds_p = (pf_wgs * nseg_p + cus0 - 1) / cus0;
+        const float per_tile = (0.5f + 1.4f * ds) * (pf_wgs * nseg_p * 2 <= cus0 ? 0.7f : 1.f);
+        const float prefill_us = (nseg_p > 1 ? 16.f : 12.f) + (float)((tiles64 + nseg_p - 1) / nseg_p) * per_tile * (float)rounds_p;
+        if (prefill_us < split_us) split = false;
+    }
     if (split) {
         // key segments: one 32-key tile per wavefront while that leaves the device under-filled,
         // more tiles per wavefront beyond one workgroup per CU (its LDS tiles fill a CU)

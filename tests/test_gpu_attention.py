@@ -332,6 +332,27 @@ def test_prefill_chunk_with_positions_over_a_longer_cache(gpu, orc, B, Lq, T, le
     assert float(np.abs(got - ref).max()) < 2e-3
 
 
+# A chunk of queries over a cache at least four times its length: with enough keys the 128-row kernel (keys cut into
+# segments, partial results merged) takes over from the 16-row kernel well below the row count at which it takes a prompt
+# over its own keys. 80 queries x 8 heads over 4096 keys at head size 256 -> 128-row kernel; 24 queries over the same cache
+# stay on the 16-row kernel. The second sequence sees 1500 keys only (segments with nothing visible must contribute nothing).
+@pytest.mark.parametrize("kind,tol", [("f16", 2e-3), ("bf16", 1e-2)])
+@pytest.mark.parametrize("Lq,kernel", [(80, "attn_prefill"), (24, "attn_flash_split")])
+def test_query_chunk_over_a_long_cache(gpu, orc, kind, tol, Lq, kernel):
+    B, T, Hq, Hkv, D = 2, 4096, 8, 1, 256
+    say("chunk over a long cache", kind, Lq)
+    (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(Lq, B, Lq, T, Hq, Hkv, D, kind)
+    pos = np.tile(np.arange(T - Lq, T, dtype=np.int32), (B, 1))
+    lens = np.array([T, 1500], np.int32)
+    got = run_attention(gpu, q, k, v, 1 / math.sqrt(D), qd, kd, positions=pos, kv_lengths=lens)
+    assert gpu.last_kernel() == kernel
+    ref = orc.attention_f64(qf, kf, vf, 1 / math.sqrt(D), positions=pos, kv_lengths=lens)
+    assert np.isfinite(got).all()
+    err = float(np.abs(got - ref).max())
+    say("  max err", err)
+    assert err < tol
+
+
 def ring_of(linear, T):
     """The last T steps of a linear history [B, end, H, D], each at row t % T."""
     end = linear.shape[1]
