@@ -787,20 +787,40 @@ int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *cw, size_t m, const
         const int tn = (int)((N + G2_BN - 1) / G2_BN);
         // tallest tile that still gives every CU a workgroup; 64-row tiles when even 128-row ones leave half idle
         const int tm4 = (int)((m + 255) / 256), tm2 = (int)((m + 127) / 128), tm1 = (int)((m + 63) / 64);
-        const int wm = (long)tm4 * tn >= cus ? 4 : ((long)tm2 * tn * 2 > cus ? 2 : 1);
-        const int tm = wm == 4 ? tm4 : (wm == 2 ? tm2 : tm1);
-        // Whole rounds of 256-column tiles first; if the columns left over would make a partial round, they are
-        // covered with 192-column tiles when those fit one round (3/4 of the time of a round of full tiles).
+        int wm = (long)tm4 * tn >= cus ? 4 : ((long)tm2 * tn * 2 > cus ? 2 : 1);
+        // 256-row tiles come 256 or 192 columns wide (a 192-column tile takes 3/4 of the time). Three covers of N are weighed
+        // by their rounds: whole rounds of wide tiles with the columns left over in one round of narrow ones; wide tiles only;
+        // narrow tiles only (N = 11008 at 2048 rows: 58 narrow column tiles are two rounds of 3/4 where 32 wide + 15 narrow are
+        // 1 + 3/4). Narrow tiles only also replace 128-row tiles that would need two half-time rounds where one round of
+        // 256 x 192 tiles covers N (N = 5120 ... 6144 at 2048 rows).
         int tn_wide = tn, tn_narrow = 0;
-        if (wm == 4) {
-            const int per_round = cus / tm;                     // column tiles per round
+        const int all_narrow = (int)((N + 191) / 192);
+        if (wm == 2 && (long)tm4 * all_narrow <= cus && (long)tm2 * tn > cus) {
+            wm = 4;
+            tn_wide = 0;
+            tn_narrow = all_narrow;
+        } else if (wm == 4) {
+            const int per_round = cus / tm4;                    // column tiles per round
             const int rest = per_round > 0 ? tn % per_round : 0;
-            if (per_round > 0 && rest > 0 && tn > per_round) {
-                const size_t cols_left = N - (size_t)(tn - rest) * G2_BN;
-                const int narrow = (int)((cols_left + 191) / 192);
-                if ((long)narrow * tm <= cus) { tn_wide = tn - rest; tn_narrow = narrow; }
+            if (per_round > 0) {
+                float best = (float)((tn + per_round - 1) / per_round);            // wide tiles only
+                if (rest > 0 && tn > per_round) {
+                    const size_t cols_left = N - (size_t)(tn - rest) * G2_BN;
+                    const int narrow = (int)((cols_left + 191) / 192);
+                    if ((long)narrow * tm4 <= cus && (float)((tn - rest) / per_round) + 0.75f <= best) {
+                        best = (float)((tn - rest) / per_round) + 0.75f;
+                        tn_wide = tn - rest;
+                        tn_narrow = narrow;
+                    }
+                }
+                const float narrow_only = 0.75f * (float)((all_narrow + per_round - 1) / per_round);
+                if (narrow_only < best) {
+                    tn_wide = 0;
+                    tn_narrow = all_narrow;
+                }
             }
         }
+        const int tm = wm == 4 ? tm4 : (wm == 2 ? tm2 : tm1);
         // 64-row tiles that still leave CUs idle (few tokens against a narrow weight): 128 columns instead of 256, twice the workgroups
         const bool half_cols = wm == 1 && (long)tm1 * tn < cus;
         static bool attr[4] = {false, false, false, false};
