@@ -787,7 +787,7 @@ int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *cw, size_t m, const
         const int tn = (int)((N + G2_BN - 1) / G2_BN);
         // tallest tile that still gives every CU a workgroup; 64-row tiles when even 128-row ones leave half idle
         const int tm4 = (int)((m + 255) / 256), tm2 = (int)((m + 127) / 128), tm1 = (int)((m + 63) / 64);
-        int wm = (long)tm4 * tn >= cus ? 4 : ((long)tm2 * tn * 2 > cus ? 2 : 1);
+        int wm = (long)tm4 * tn >= cus ? 4 : ((long)tm2 * tn * 2 > cus && (long)tm1 * tn > cus ? 2 : 1);   // (64-row tiles while they fit one round)
         // 256-row tiles come 256 or 192 columns wide (a 192-column tile takes 3/4 of the time). Three covers of N are weighed
         // by their rounds: whole rounds of wide tiles with the columns left over in one round of narrow ones; wide tiles only;
         // narrow tiles only (N = 11008 at 2048 rows: 58 narrow column tiles are two rounds of 3/4 where 32 wide + 15 narrow are
