@@ -420,7 +420,7 @@ __global__ __launch_bounds__(SPLIT ? SPLIT_NW * 64 : 256) void attn_flash_kernel
                 const float inv = l_all > 0.f ? 1.f / l_all : 0.f;
                 *(f32x4 *)(a.out + (((size_t)b * a.L + l2) * a.Hq + hk * a.groups + g2) * D + col) = o * inv;
             }
-        } else {
+        } else if (rt * 16 + row < a.rows_total) {        // (rows past the last query row are padding: nobody reads them)
             *(f32x4 *)(a.partial + pslot + row * D + col) = o;
             if (col == 0) {
                 a.partial[pslot + 16 * D + row] = m_all;
@@ -445,6 +445,9 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnArgs a) {
     const int tid = threadIdx.x, q4 = tid & 3, row = (tid >> 2) & 15, sg = tid >> 6;
     const float *base = a.partial + (size_t)(unit * a.row_tiles + rt) * a.nseg * WSTRIDE;
     const int dv = slice * MERGE_DV + q4 * 4;
+    // padding rows of the last tile were never stored: their threads read the tile's last real row instead (the same lines
+    // its own threads fetch) and drop the result below
+    const int row_ld = min(row, min(16, a.rows_total - rt * 16) - 1);
     float m_loc = -INFINITY, l_loc = 0.f;
     f32x4 o_loc = f32x4{0.f, 0.f, 0.f, 0.f};
     for (int s0 = sg; s0 < a.nseg; s0 += MERGE_SG * MERGE_UNROLL) {
@@ -454,9 +457,9 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnArgs a) {
         for (int u = 0; u < MERGE_UNROLL; ++u) {
             const int sidx = min(s0 + u * MERGE_SG, a.nseg - 1);      // clamped: every load is unconditional
             const float *p = base + (size_t)sidx * WSTRIDE;
-            ms[u] = p[16 * D + row];
-            ls[u] = p[16 * D + 16 + row];
-            os[u] = *(const f32x4 *)(p + row * D + dv);
+            ms[u] = p[16 * D + row_ld];
+            ls[u] = p[16 * D + 16 + row_ld];
+            os[u] = *(const f32x4 *)(p + row_ld * D + dv);
         }
         float m_new = m_loc;
 #pragma unroll
