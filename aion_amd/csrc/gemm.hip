@@ -815,8 +815,17 @@ int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *cw, size_t m, const
                 }
                 const float narrow_only = 0.75f * (float)((all_narrow + per_round - 1) / per_round);
                 if (narrow_only < best) {
+                    best = narrow_only;
                     tn_wide = 0;
                     tn_narrow = all_narrow;
+                }
+                // barely more 256-row tiles than CUs: two half-time rounds of 128-row tiles beat a second round of tall ones
+                // (1300 rows x 11008 columns: 258 tall tiles, 139 us; 473 of 128 rows, 115 us; a third, nearly empty half round
+                // costs more than it saves: 516 tiles of 128 rows took 166 against 145 us)
+                if (best > 1.f && (long)tm2 * tn <= 2L * cus) {
+                    wm = 2;
+                    tn_wide = tn;
+                    tn_narrow = 0;
                 }
             }
         }

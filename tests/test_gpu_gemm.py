@@ -124,9 +124,10 @@ def test_bf16_gemm_ragged_shapes(gpu, orc, dtype, layout, m, n, k):
 # (2048, 13000): 32 of 256 and 26 of 192 - thirteen whole blocks of that pattern, then the rest of the wide tiles; the last
 # narrow tile hangs over the last column. (2048, 9092): 48 tiles of 192 only (two rounds of 3/4 beat one wide round plus a
 # narrow one), the last one hanging over; (2048, 5120): 27 tiles of 192 in one round instead of two rounds of 128-row tiles.
+# (1300, 11008): 258 tiles of 256 rows would need a second round, so 473 tiles of 128 rows run in two half-time rounds.
 # Rows from every 256-row tile, all columns.
 @pytest.mark.parametrize("dtype,layout", [(be.Q8_0, be.ROWS_NK), (be.Q4_0, be.KMAJOR_KN)])
-@pytest.mark.parametrize("m,n", [(512, 4096), (2048, 14336), (2048, 9092), (2048, 13000), (2048, 5120)])
+@pytest.mark.parametrize("m,n", [(512, 4096), (2048, 14336), (2048, 9092), (2048, 13000), (2048, 5120), (1300, 11008)])
 def test_config3_bf16_full_size_on_row_sample(gpu, orc, dtype, layout, m, n):
     k = 4096
     say("config3 bf16", dtype, m, n)
