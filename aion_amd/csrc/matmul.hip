@@ -253,8 +253,11 @@ int aionhip_step_gate_matmul(aionhip_ctx *ctx, const aionhip_weight *w, size_t r
     const float *gp = (const float *)(uintptr_t)gate, *up_p = (const float *)(uintptr_t)up;
     if (rows == 1 && fused_row_pays(b) && ((gate | up) & 15) == 0)
         return launch_gemv_fused(ctx, b.w, b.c, b.ldc, 1, PRO_GATE, FusedIn{gp, up_p, nullptr, nullptr, 0.f}, alpha, beta);
-    if (rows <= GEMV_MAX_M) {
-        // gate and activation preparation in one small launch, then the GEMV on the prepared rows
+    // more rows, on the exact kernels (always, or where the bf16 kernel would not pay): the same two launches, the GEMM last
+    const bool bf16_route = rows > GEMV_MAX_M && (ctx->gemm_mode == AIONHIP_GEMM_BF16_MFMA_ALWAYS ||
+                                                  (ctx->gemm_mode == AIONHIP_GEMM_BF16_MFMA && gemm_bf16_pays(ctx, rows, b.w[0]->n, b.k)));
+    if (!bf16_route && rows <= 0x7FFFFFFFu) {
+        // gate and activation preparation in one small launch, then the GEMV (or GEMM) on the prepared rows
         rc = ensure_scratch(ctx, prepared_act_bytes(rows, b.k));
         if (rc) return rc;
         PreparedAct act = prepared_act_carve(ctx->scratch, rows, b.k);

@@ -363,7 +363,7 @@ def test_single_row_fused_kernel_equals_prepared_path(gpu, orc, dtype, layout):
 
 
 @pytest.mark.parametrize("dtype,layout", CASES)
-@pytest.mark.parametrize("rows", [1, 3, 6])
+@pytest.mark.parametrize("rows", [1, 3, 6, 40])
 def test_rmsnorm_matmul_and_gate_matmul_match_the_separate_steps(gpu, orc, dtype, layout, rows):
     say("fused steps", dtype, layout, rows)
     rng = np.random.default_rng(rows + dtype)
