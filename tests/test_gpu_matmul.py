@@ -378,6 +378,15 @@ def test_rmsnorm_matmul_and_gate_matmul_match_the_separate_steps(gpu, orc, dtype
     if rows == 1:
         assert gpu.last_kernel().endswith("_rmsnorm")
     got1, got2 = gpu.download(c1, np.float32, (rows, n1)), gpu.download(c2, np.float32, (rows, n2))
+    if rows > 1:
+        # several rows: the step is the norm step followed by the matmul step on the normalised rows, so the same bits come out
+        hb, d1, d2 = gpu.alloc(rows * k * 4), gpu.alloc(rows * n1 * 4), gpu.alloc(rows * n2 * 4)
+        gpu.step_rmsnorm(hb, xb, gb, rows, k, 1e-6)
+        gpu.step_matmul_batch([w1, w2], hb, rows, [d1, d2])
+        assert np.array_equal(gpu.download(d1, np.float32, (rows, n1)), got1)
+        assert np.array_equal(gpu.download(d2, np.float32, (rows, n2)), got2)
+        for t in (hb, d1, d2):
+            t.free()
     h = orc.rmsnorm(x, gamma, 1e-6)
     want1, want2 = oracle_matmul(orc, dtype, layout, h, b1, n1), oracle_matmul(orc, dtype, layout, h, b2, n2)
     # the norm's sum of squares is reduced in a different order than on the CPU: an activation on a
