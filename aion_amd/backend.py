@@ -227,6 +227,40 @@ class HipBackend:
             self._ctx, w_gate.ptr, w_up.ptr, w_down.ptr, x.handle, gamma.handle, beta_norm.handle if beta_norm is not None else 0, eps,
             c_buf.handle, alpha, beta))
 
+    # ---- a run of decoder blocks as one launch (one new token of one sequence)
+    def decoder_stack_create(self, layers, hidden, heads, kv_heads, head_dim, ffn, t_cap, eps1, eps2, attn_scale, rope_base=10000.0,
+                             rope_scale=1.0, rope_proportion=1.0, soft_cap=0.0, window=CAUSAL, rolling=False):
+        """layers: one dict per block with the weights wq, wk, wv, wo, w_gate, w_up, w_down (Weight), norm1_gamma, norm2_gamma,
+        k_cache, v_cache (DeviceBuffer) and optionally norm1_beta, norm2_beta. Raises AionHipError(UNSUPPORTED) for shapes the
+        one-launch form does not take."""
+        desc = hip.DecoderStackDesc(len(layers), hidden, heads, kv_heads, head_dim, ffn, t_cap, eps1, eps2, rope_base, rope_scale,
+                                    rope_proportion, attn_scale, soft_cap, window[0], window[1], window[2], 1 if rolling else 0)
+        arr = (hip.DecoderStackLayer * len(layers))()
+        for i, l in enumerate(layers):
+            for name in ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down"):
+                setattr(arr[i], name, l[name].ptr)
+            for name in ("norm1_gamma", "norm1_beta", "norm2_gamma", "norm2_beta", "k_cache", "v_cache"):
+                buf = l.get(name)
+                setattr(arr[i], name, buf.handle if buf is not None else 0)
+        st = C.c_void_p()
+        self._check(self._lib.aionhip_decoder_stack_create(self._ctx, C.byref(desc), arr, C.byref(st)))
+        return st
+
+    def decoder_stack_destroy(self, stack):
+        self._lib.aionhip_decoder_stack_destroy(self._ctx, stack)
+
+    def step_decoder_stack(self, stack, x_in, x_out, positions, write_index, kv_lengths):
+        self._check(self._lib.aionhip_step_decoder_stack(self._ctx, stack, x_in.handle, x_out.handle, positions.handle, write_index.handle,
+                                                         kv_lengths.handle))
+
+    def decoder_stack_status(self, stack):
+        """Waits for the stream; raises AionHipError(EXECUTION_FAILED) if a launch of the stack gave up waiting since the last call."""
+        failed = C.c_int(0)
+        self._check(self._lib.aionhip_decoder_stack_status(self._ctx, stack, C.byref(failed)))
+
+    def decoder_stack_set_poll_budget(self, stack, milliseconds):
+        self._check(self._lib.aionhip_decoder_stack_set_poll_budget(self._ctx, stack, float(milliseconds)))
+
     def step_add_i32(self, out, a, b, n):
         self._check(self._lib.aionhip_step_add_i32(self._ctx, out.handle, a.handle, b.handle, n))
 
@@ -266,6 +300,10 @@ class HipBackend:
 
     def program_execute(self, prog):
         self._check(self._lib.aionhip_program_execute(self._ctx, prog))
+
+    def program_is_current(self, prog):
+        """False once a work buffer the program's launches address has been replaced by a larger one: record it again."""
+        return bool(self._lib.aionhip_program_is_current(self._ctx, prog))
 
     def program_node_count(self, prog):
         return self._lib.aionhip_program_node_count(prog)

@@ -55,6 +55,9 @@ struct aionhip_ctx {
     // argmax: one ticket per row (all zero between launches)
     void *tickets = nullptr;
     size_t tickets_bytes = 0;
+    // moves on whenever one of the four buffers above is replaced by a larger one: a program recorded before that holds
+    // the old address and may not run any more
+    uint64_t buffer_generation = 0;
     // this device's copy of the library's file-scope scratch array (ctx.hip), for the entry point that allocates nothing
     void *static_scratch = nullptr;
     // true while that entry point runs: no launcher may take a path that needs scratch of its own
@@ -125,6 +128,8 @@ struct aionhip_weight {
 };
 
 int set_err(aionhip_ctx *ctx, int status, const char *fmt, ...);
+int dev_malloc(aionhip_ctx *ctx, void **out, size_t bytes, const char *what);
+int grow_work_buffer(aionhip_ctx *ctx, void **buf, size_t *have, size_t bytes, bool zeroed, const char *what);
 int ensure_scratch(aionhip_ctx *ctx, size_t bytes);
 int ensure_scratch2(aionhip_ctx *ctx, size_t bytes);
 // size of the file-scope device scratch array behind aionhip_step_matmul_static (prepared activations of one call)

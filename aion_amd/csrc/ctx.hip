@@ -44,25 +44,51 @@ int set_err(aionhip_ctx *ctx, int status, const char *fmt, ...) {
     return status;
 }
 
-static int grow(aionhip_ctx *ctx, void **buf, size_t *have, size_t bytes) {
+static void pool_release_cached(aionhip_ctx *ctx);
+
+// Every internal device allocation goes through here: when the device is out of memory the pool's cached blocks are
+// given back and the request is tried once more (not while a program is being recorded: releasing waits for the stream).
+int dev_malloc(aionhip_ctx *ctx, void **out, size_t bytes, const char *what) {
+    *out = nullptr;
+    hipError_t e = hipMalloc(out, bytes);
+    if (e == hipErrorOutOfMemory && ctx->pool_cached_bytes && !ctx->capturing) {
+        (void)hipGetLastError();
+        pool_release_cached(ctx);
+        e = hipMalloc(out, bytes);
+    }
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        *out = nullptr;
+        return set_err(ctx, e == hipErrorOutOfMemory ? AIONHIP_OUT_OF_MEMORY : AIONHIP_EXECUTION_FAILED, "hipMalloc(%zu) for %s: %s", bytes, what, hipGetErrorString(e));
+    }
+    return AIONHIP_OK;
+}
+
+// Context-owned work buffers (prepared activations, GEMM staging, K-split meeting words, argmax tickets) grow by
+// replacement. A recorded program holds the old address in its launches, so every replacement moves the context's
+// buffer generation on and aionhip_program_execute refuses a program recorded under an earlier one.
+int grow_work_buffer(aionhip_ctx *ctx, void **buf, size_t *have, size_t bytes, bool zeroed, const char *what) {
     if (bytes <= *have) return AIONHIP_OK;
     if (ctx->capturing)
-        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "scratch must grow to %zu bytes while a program is being recorded: run the steps once before recording", bytes);
+        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "%s must grow to %zu bytes while a program is being recorded: run the steps once before recording", what, bytes);
     if (*buf) {
         // earlier launches may still read the old buffer
         HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
         HIP_TRY(ctx, hipFree(*buf));
         *buf = nullptr;
         *have = 0;
+        ctx->buffer_generation++;
     }
     size_t want = bytes + bytes / 4;
-    want = (want + 255) & ~(size_t)255;
-    HIP_TRY(ctx, hipMalloc(buf, want));
+    want = (want + 4095) & ~(size_t)4095;
+    int rc = dev_malloc(ctx, buf, want, what);
+    if (rc) return rc;
     *have = want;
+    if (zeroed) HIP_TRY(ctx, hipMemsetAsync(*buf, 0, want, ctx->stream));          // never inside a recording (checked above)
     return AIONHIP_OK;
 }
-int ensure_scratch(aionhip_ctx *ctx, size_t bytes) { return grow(ctx, &ctx->scratch, &ctx->scratch_bytes, bytes); }
-int ensure_scratch2(aionhip_ctx *ctx, size_t bytes) { return grow(ctx, &ctx->scratch2, &ctx->scratch2_bytes, bytes); }
+int ensure_scratch(aionhip_ctx *ctx, size_t bytes) { return grow_work_buffer(ctx, &ctx->scratch, &ctx->scratch_bytes, bytes, false, "scratch"); }
+int ensure_scratch2(aionhip_ctx *ctx, size_t bytes) { return grow_work_buffer(ctx, &ctx->scratch2, &ctx->scratch2_bytes, bytes, false, "GEMM staging"); }
 
 static hipEvent_t take_event(aionhip_ctx *ctx) {
     if (!ctx->event_pool.empty()) {
@@ -96,7 +122,8 @@ int rope_table(aionhip_ctx *ctx, int pairs, float freq_step, float scale_factor,
         f *= freq_step;
     }
     void *dev = nullptr;
-    HIP_TRY(ctx, hipMalloc(&dev, host.size() * sizeof(float)));
+    const int rc = dev_malloc(ctx, &dev, host.size() * sizeof(float), "RoPE table");
+    if (rc) return rc;
     hipError_t e = hipMemcpyAsync(dev, host.data(), host.size() * sizeof(float), hipMemcpyHostToDevice, ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess) {
@@ -172,8 +199,6 @@ int aionhip_create(int device, void *stream, aionhip_ctx **out) {
     return AIONHIP_OK;
 }
 
-static void pool_release_cached(aionhip_ctx *ctx);
-
 void aionhip_destroy(aionhip_ctx *ctx) {
     if (!ctx) return;
     (void)hipSetDevice(ctx->device);
@@ -228,6 +253,7 @@ int aionhip_device_info(aionhip_ctx *ctx, int *cu_count, int *wave_size, uint64_
 // block is at most 12.5 % larger than asked for and requests that differ a little share a class.
 static size_t pool_class(size_t bytes) {
     if (bytes < 256) return 256;
+    if (bytes > aionhip_ctx::POOL_MAX_BLOCK) return (bytes + 255) & ~(size_t)255;      // never cached: no class to share, no padding to pay
     size_t p2 = 256;
     while (p2 <= bytes / 2) p2 <<= 1;                      // largest power of two <= bytes
     const size_t step = p2 / 8 < 256 ? 256 : p2 / 8;
@@ -264,16 +290,8 @@ int aionhip_alloc(aionhip_ctx *ctx, size_t bytes, size_t alignment, aionhip_hand
         if (v.empty()) ctx->pool_free.erase(it);
     }
     if (!p) {
-        hipError_t e = hipMalloc(&p, cls);
-        if (e == hipErrorOutOfMemory && ctx->pool_cached_bytes) {      // give the cached blocks back and try once more
-            (void)hipGetLastError();
-            pool_release_cached(ctx);
-            e = hipMalloc(&p, cls);
-        }
-        if (e != hipSuccess) {
-            (void)hipGetLastError();
-            return set_err(ctx, e == hipErrorOutOfMemory ? AIONHIP_OUT_OF_MEMORY : AIONHIP_EXECUTION_FAILED, "hipMalloc(%zu): %s", cls, hipGetErrorString(e));
-        }
+        const int rc = dev_malloc(ctx, &p, cls, "aionhip_alloc");
+        if (rc) return rc;
         if (alignment > 1 && ((uintptr_t)p % alignment) != 0) {
             (void)hipFree(p);
             return set_err(ctx, AIONHIP_UNSUPPORTED, "cannot satisfy alignment %zu", alignment);

@@ -226,19 +226,10 @@ int launch_gemv_ksplit(aionhip_ctx *ctx, const aionhip_weight *w, float *c, cons
     if ((S & (S - 1)) != 0 || S > KSPLIT_MAX_S || (long)kbs * (S - 1) >= KB || nch > 256 || kbs > NT / 2)
         return set_err(ctx, AIONHIP_UNSUPPORTED, "gemv ksplit: k = %zu does not cut into %d slices of at most %d blocks", w->k, S, max_kbs);
     const size_t need = (size_t)(S > 1 ? S - 1 : 1) * N * sizeof(unsigned long long);
-    if (need > ctx->ksplit_bytes) {
-        if (ctx->capturing)
-            return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "the K-split buffer must grow to %zu bytes while a program is being recorded: run the steps once before recording", need);
-        if (ctx->ksplit) {
-            HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
-            HIP_TRY(ctx, hipFree(ctx->ksplit));
-            ctx->ksplit = nullptr;
-            ctx->ksplit_bytes = 0;
-        }
-        const size_t want = (need + need / 4 + 255) & ~(size_t)255;
-        HIP_TRY(ctx, hipMalloc(&ctx->ksplit, want));
-        ctx->ksplit_bytes = want;
-        HIP_TRY(ctx, hipMemsetAsync(ctx->ksplit, 0, want, ctx->stream));          // every meeting word starts empty (never inside a recording)
+    {
+        // every meeting word starts empty and is left empty by the launch that used it
+        const int rc = grow_work_buffer(ctx, &ctx->ksplit, &ctx->ksplit_bytes, need, true, "the K-split buffer");
+        if (rc) return rc;
     }
     unsigned long long *meet = (unsigned long long *)ctx->ksplit;
     ProfScope scope(ctx, name);

@@ -678,20 +678,8 @@ int aionhip_step_argmax(aionhip_ctx *ctx, aionhip_handle out_i32, aionhip_handle
     if (rows > 65535) return set_err(ctx, AIONHIP_UNSUPPORTED, "argmax: more than 65535 rows");
     int rc = ensure_scratch2(ctx, rows * ARGMAX_PARTS * 8);
     if (rc) return rc;
-    if (rows * sizeof(unsigned) > ctx->tickets_bytes) {
-        if (ctx->capturing)
-            return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "the argmax tickets must grow while a program is being recorded: run the steps once before recording");
-        if (ctx->tickets) {
-            HIP_TRY(ctx, hipStreamSynchronize(ctx->stream));
-            HIP_TRY(ctx, hipFree(ctx->tickets));
-            ctx->tickets = nullptr;
-            ctx->tickets_bytes = 0;
-        }
-        const size_t want = (rows * sizeof(unsigned) + 4095) & ~(size_t)4095;
-        HIP_TRY(ctx, hipMalloc(&ctx->tickets, want));
-        ctx->tickets_bytes = want;
-        HIP_TRY(ctx, hipMemsetAsync(ctx->tickets, 0, want, ctx->stream));          // never inside a recording
-    }
+    rc = grow_work_buffer(ctx, &ctx->tickets, &ctx->tickets_bytes, rows * sizeof(unsigned), true, "the argmax tickets");
+    if (rc) return rc;
     float *pv = (float *)ctx->scratch2;
     int *pi = (int *)(pv + rows * ARGMAX_PARTS);
     argmax_kernel<<<dim3(ARGMAX_PARTS, (unsigned)rows), dim3(256), 0, ctx->stream>>>(dp<int>(out_i32), pv, pi, (unsigned *)ctx->tickets, dp<const float>(x), n);

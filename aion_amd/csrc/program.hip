@@ -15,6 +15,7 @@ struct aionhip_program {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     size_t nodes = 0;
+    uint64_t buffer_generation = 0;     // the context's work-buffer generation the launches were recorded under
 };
 
 namespace {
@@ -99,6 +100,7 @@ int aionhip_program_end(aionhip_ctx *ctx, aionhip_program **out) {
         return set_err(ctx, AIONHIP_OUT_OF_MEMORY, "host allocation failed");
     }
     p->graph = graph;
+    p->buffer_generation = ctx->buffer_generation;
     (void)hipGraphGetNodes(graph, nullptr, &p->nodes);
     e = hipGraphInstantiate(&p->exec, graph, nullptr, nullptr, 0);
     if (e != hipSuccess) {
@@ -125,11 +127,18 @@ int aionhip_program_abort(aionhip_ctx *ctx) {
 int aionhip_program_execute(aionhip_ctx *ctx, aionhip_program *prog) {
     if (!ctx || !prog || !prog->exec) return AIONHIP_INVALID_ARGUMENT;
     if (ctx->capturing) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "program_execute: a recording is open");
+    if (prog->buffer_generation != ctx->buffer_generation)
+        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "program_execute: stale program - a work buffer of the context was replaced by a larger one after this program "
+                                                      "was recorded (a later step needed more scratch); re-record it");
     HIP_TRY(ctx, hipGraphLaunch(prog->exec, ctx->stream));
     return AIONHIP_OK;
 }
 
 size_t aionhip_program_node_count(const aionhip_program *prog) { return prog ? prog->nodes : 0; }
+
+int aionhip_program_is_current(const aionhip_ctx *ctx, const aionhip_program *prog) {
+    return ctx && prog && prog->exec && prog->buffer_generation == ctx->buffer_generation ? 1 : 0;
+}
 
 void aionhip_program_destroy(aionhip_ctx *ctx, aionhip_program *prog) {
     if (!prog) return;

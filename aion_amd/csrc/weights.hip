@@ -121,10 +121,10 @@ int alloc_weight(aionhip_ctx *ctx, int dtype, int layout, size_t n, size_t k, ai
     // one allocation: quants first (16-byte aligned rows since k % 32 == 0), scales after
     const size_t qs_padded = (w->qs_bytes + 255) & ~(size_t)255;
     void *p = nullptr;
-    hipError_t e = hipMalloc(&p, qs_padded + w->sc_bytes + 256);  // slack: kernels may read one 16-byte chunk of a clamped row
-    if (e != hipSuccess) {
+    const int rc = dev_malloc(ctx, &p, qs_padded + w->sc_bytes + 256, "a weight");  // slack: kernels may read one 16-byte chunk of a clamped row
+    if (rc) {
         delete w;
-        return set_err(ctx, e == hipErrorOutOfMemory ? AIONHIP_OUT_OF_MEMORY : AIONHIP_EXECUTION_FAILED, "hipMalloc weight: %s", hipGetErrorString(e));
+        return rc;
     }
     w->qs = (uint8_t *)p;
     w->sc = (__half *)((uint8_t *)p + qs_padded);
@@ -165,7 +165,8 @@ int aionhip_weight_upload(aionhip_ctx *ctx, int dtype, int layout, size_t n, siz
     const size_t ld = ld_blocks ? ld_blocks : n;
     const size_t bytes = (layout == AIONHIP_KMAJOR_KN ? ((KB - 1) * ld + n) : n * KB) * bb;
     void *staging = nullptr;
-    HIP_TRY(ctx, hipMalloc(&staging, bytes));
+    rc = dev_malloc(ctx, &staging, bytes, "weight upload staging");
+    if (rc) return rc;
     hipError_t e = hipMemcpyAsync(staging, host_blocks, bytes, hipMemcpyHostToDevice, ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess) {
@@ -204,8 +205,9 @@ int aionhip_weight_download(aionhip_ctx *ctx, const aionhip_weight *w, void *hos
     const size_t want = aionhip_weight_packed_bytes(w);
     if (bytes != want) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "download: buffer is %zu bytes, packed form is %zu", bytes, want);
     void *staging = nullptr;
-    HIP_TRY(ctx, hipMalloc(&staging, want));
-    int rc = run_relay<true>(ctx, w, (uint8_t *)staging, w->n);
+    int rc = dev_malloc(ctx, &staging, want, "weight download staging");
+    if (rc) return rc;
+    rc = run_relay<true>(ctx, w, (uint8_t *)staging, w->n);
     if (rc == AIONHIP_OK) {
         hipError_t e = hipMemcpyAsync(host_blocks, staging, want, hipMemcpyDeviceToHost, ctx->stream);
         if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);

@@ -28,6 +28,17 @@ class Attention(C.Structure):
                 ("window_left", C.c_uint32), ("window_right", C.c_uint32), ("window_chunk", C.c_uint32), ("rolling", C.c_uint32)]
 
 
+class DecoderStackLayer(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in ("wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down")] + \
+               [(n, C.c_uint64) for n in ("norm1_gamma", "norm1_beta", "norm2_gamma", "norm2_beta", "k_cache", "v_cache")]
+
+
+class DecoderStackDesc(C.Structure):
+    _fields_ = [(n, C.c_size_t) for n in ("layers", "hidden", "heads", "kv_heads", "head_dim", "ffn", "t_cap")] + \
+               [(n, C.c_float) for n in ("eps1", "eps2", "rope_base", "rope_scale", "rope_proportion", "attn_scale", "attn_logits_soft_cap")] + \
+               [("window_left", C.c_uint32), ("window_right", C.c_uint32), ("window_chunk", C.c_uint32), ("rolling", C.c_int)]
+
+
 _SIGS = {
     # name: (restype, argtypes)
     "aionhip_create": (C.c_int, [C.c_int, C.c_void_p, C.POINTER(C.c_void_p)]),
@@ -71,11 +82,18 @@ _SIGS = {
     "aionhip_step_advance_state": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64, C.c_size_t, C.POINTER(C.c_uint64), C.c_size_t, C.c_int]),
     "aionhip_step_advance_state_log": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64, C.c_size_t, C.POINTER(C.c_uint64), C.c_size_t, C.c_int,
                                                  C.c_uint64, C.c_uint64, C.c_size_t]),
+    "aionhip_decoder_stack_create": (C.c_int, [C.c_void_p, C.POINTER(DecoderStackDesc), C.POINTER(DecoderStackLayer), C.POINTER(C.c_void_p)]),
+    "aionhip_decoder_stack_destroy": (None, [C.c_void_p, C.c_void_p]),
+    "aionhip_step_decoder_stack": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64]),
+    "aionhip_decoder_stack_status": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(C.c_int)]),
+    "aionhip_decoder_stack_set_poll_budget": (C.c_int, [C.c_void_p, C.c_void_p, C.c_double]),
+    "aionhip_decoder_stack_set_stamps": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64]),
     "aionhip_program_begin": (C.c_int, [C.c_void_p]),
     "aionhip_program_end": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p)]),
     "aionhip_program_abort": (C.c_int, [C.c_void_p]),
     "aionhip_program_execute": (C.c_int, [C.c_void_p, C.c_void_p]),
     "aionhip_program_node_count": (C.c_size_t, [C.c_void_p]),
+    "aionhip_program_is_current": (C.c_int, [C.c_void_p, C.c_void_p]),
     "aionhip_program_destroy": (None, [C.c_void_p, C.c_void_p]),
     "aionhip_set_attention_precise": (C.c_int, [C.c_void_p, C.c_int]),
     "aionhip_set_gemm_mode": (C.c_int, [C.c_void_p, C.c_int]),

@@ -743,6 +743,10 @@ class PackageRunner:
         g = self.gpu
         plan = self._plan(1)
         self._write_inputs(plan, np.array([first_token], np.int32), self.pos)
+        if self.program is not None and not g.program_is_current(self.program):
+            # a larger run since the recording made the context replace a work buffer the program's launches address
+            g.program_destroy(self.program)
+            self.program = None
         if self.program is None:
             self._issue(plan)                    # eager once: scratch buffers reach their final size
             g.sync()

@@ -323,13 +323,61 @@ int aionhip_step_advance_state_log(aionhip_ctx *ctx, aionhip_handle dst_tokens, 
                                    const aionhip_handle *counters, size_t n_counters, int delta,
                                    aionhip_handle log, aionhip_handle log_index, size_t log_capacity);
 
+/* ---- a whole run of decoder blocks for ONE new token of ONE sequence, as one launch ----------
+ * Session.execute receives the whole ExecutableProgram (backend/backend.zig:42-44); a decoder's program repeats
+ * one block per layer (src/bench/models.zig:433-536): RMSNorm -> MatMul q,k,v -> RoPE1D(q,k) -> Cast f16 +
+ * SequenceAppend(k,v) -> Attention -> MatMul o, beta = 1 (residual) -> RMSNorm -> MatMul gate,up -> gate(gelu) ->
+ * MatMul down, beta = 1. aionhip_step_decoder_stack runs `layers` such blocks in one cooperative launch of one
+ * workgroup per CU; between the phases of a block the small activation vectors travel through device memory as
+ * self-validating words, so no step boundary costs a dispatch. Same arithmetic per output as the separate steps
+ * (aionhip_step_rmsnorm_qkv_rope_append, aionhip_step_attention, aionhip_step_matmul, aionhip_step_rmsnorm_geglu_matmul).
+ * create returns AIONHIP_UNSUPPORTED for shapes outside its limits (head size 128 or 256, hidden and heads x head
+ * size up to 8192, ffn up to 32768, linear f16 caches, one block format for all weights): the caller then issues
+ * the separate steps. Weights, gammas and caches must outlive the stack. The launch waits for nothing on the host;
+ * every wait inside the kernel is bounded (250 ms by default), and aionhip_decoder_stack_status - a synchronising
+ * call - returns AIONHIP_EXECUTION_FAILED if a launch since the last call ran out of that time (its outputs are
+ * invalid; the stack is reset and usable again). */
+typedef struct aionhip_decoder_stack aionhip_decoder_stack;
+typedef struct aionhip_decoder_stack_layer {
+    const aionhip_weight *wq, *wk, *wv, *wo, *w_gate, *w_up, *w_down;
+    aionhip_handle norm1_gamma, norm1_beta; /* f32 [hidden]; beta 0 = none */
+    aionhip_handle norm2_gamma, norm2_beta;
+    aionhip_handle k_cache, v_cache;        /* f16 [t_cap, kv_heads, head_dim] */
+} aionhip_decoder_stack_layer;
+typedef struct aionhip_decoder_stack_desc {
+    size_t layers, hidden, heads, kv_heads, head_dim, ffn, t_cap;
+    float eps1, eps2;                        /* RMSNorm in front of q/k/v and in front of gate/up */
+    float rope_base, rope_scale, rope_proportion;
+    float attn_scale, attn_logits_soft_cap;  /* StepAttention (runtime/executable.zig:102-115) */
+    uint32_t window_left, window_right, window_chunk;
+    int rolling;                             /* must be 0: ring caches take the separate steps */
+} aionhip_decoder_stack_desc;
+int aionhip_decoder_stack_create(aionhip_ctx *ctx, const aionhip_decoder_stack_desc *desc, const aionhip_decoder_stack_layer *layers,
+                                 aionhip_decoder_stack **out);
+void aionhip_decoder_stack_destroy(aionhip_ctx *ctx, aionhip_decoder_stack *stack);
+/* x_in, x_out: f32 [hidden] (may be the same buffer); positions [1], write_index [1], kv_lengths [1]: i32, read on the device */
+int aionhip_step_decoder_stack(aionhip_ctx *ctx, aionhip_decoder_stack *stack, aionhip_handle x_in, aionhip_handle x_out,
+                               aionhip_handle positions, aionhip_handle write_index, aionhip_handle kv_lengths);
+int aionhip_decoder_stack_status(aionhip_ctx *ctx, aionhip_decoder_stack *stack, int *failed);
+/* the time a workgroup may wait for another's results before the launch gives up (tests set it to 0 to take that path) */
+int aionhip_decoder_stack_set_poll_budget(aionhip_ctx *ctx, aionhip_decoder_stack *stack, double milliseconds);
+/* diagnostics: with a buffer of 2 x layers x 10 i64 (0 = off) two workgroups (the first and the middle one) note the wall
+ * clock (100 MHz) when each of the five phases of every layer had its input and when its output was out */
+int aionhip_decoder_stack_set_stamps(aionhip_ctx *ctx, aionhip_decoder_stack *stack, aionhip_handle stamps);
+
 /* ---- programs: record a fixed step sequence once, replay it per token ----------------------
  * Session.execute(prog) (backend/backend.zig:42-44) runs aion's ExecutableProgram step list; the
  * WebGPU backend replays cached dispatch state because a decode program is identical every token
  * (backend/gpu/frame.zig:77-86). Between program_begin and program_end the aionhip_step_* calls
  * are recorded into a HIP graph instead of executed; program_execute replays it (asynchronous).
  * While recording: no h2d/d2h/free/sync, no profiling, and scratch cannot grow - run the same
- * steps once eagerly first. Per-token inputs must live in device buffers the steps read. */
+ * steps once eagerly first. Per-token inputs must live in device buffers the steps read.
+ * Lifetime: a program's launches hold the addresses of the context's work buffers (prepared
+ * activations, GEMM staging, K-split words, argmax tickets). When a later eager step needs a
+ * larger one (a longer prompt, more rows), the buffer is replaced and every program recorded
+ * before that is stale: program_execute then returns AIONHIP_INVALID_ARGUMENT without launching
+ * anything (aionhip_last_error says "stale program"), and the caller destroys it and records the
+ * steps again. aionhip_program_is_current tells the same without an error. */
 int aionhip_program_begin(aionhip_ctx *ctx);
 int aionhip_program_end(aionhip_ctx *ctx, aionhip_program **out);
 /* Leaves a recording without a program (for a caller whose step failed between begin and end): the captured work is
@@ -337,6 +385,8 @@ int aionhip_program_end(aionhip_ctx *ctx, aionhip_program **out);
 int aionhip_program_abort(aionhip_ctx *ctx);
 int aionhip_program_execute(aionhip_ctx *ctx, aionhip_program *prog);
 size_t aionhip_program_node_count(const aionhip_program *prog);
+/* 1 when the program may still run on this context, 0 when a work buffer it uses has been replaced since */
+int aionhip_program_is_current(const aionhip_ctx *ctx, const aionhip_program *prog);
 void aionhip_program_destroy(aionhip_ctx *ctx, aionhip_program *prog);
 
 /* ---- timing helpers for the roofline harness (timestamp queries of the WebGPU backend,

@@ -45,3 +45,30 @@ def rms_err(got, ref):
     ref = np.asarray(ref, dtype=np.float64)
     rms = float(np.sqrt((ref ** 2).mean())) if ref.size else 0.0
     return float(np.abs(got - ref).max() / (rms + 1e-30)) if ref.size else 0.0
+
+
+def _row_err(got, ref, norm):
+    import numpy as np
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    if ref.size == 0:
+        return 0.0
+    den = norm(ref)
+    err = np.abs(got - ref).max(axis=-1)
+    rel = np.where(den > 0, err / np.where(den > 0, den, 1.0), np.where(err > 0, np.inf, 0.0))
+    return float(rel.max())
+
+
+def row_rel_err(got, ref):
+    """Attention's gate: the max relative error of every output row (last axis = one head's values for one query) in
+    the maximum norm, max |err| / max |ref row|, worst row. An attention output is an average of values, so its size
+    shrinks with the number of visible keys; an absolute bound that fits a row seeing one key says nothing about a row
+    seeing 16384. A row whose reference is all zeros (empty window) must be all zeros."""
+    import numpy as np
+    return _row_err(got, ref, lambda r: np.abs(r).max(axis=-1))
+
+
+def row_rms_err(got, ref):
+    """The same per row against the row's rms (2.5 to 3 times smaller than its largest element): max |err| / rms(ref row)"""
+    import numpy as np
+    return _row_err(got, ref, lambda r: np.sqrt((r ** 2).mean(axis=-1)))

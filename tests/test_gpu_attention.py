@@ -1,7 +1,13 @@
 """GPU parity of the attention step against the CPU oracle (through the C ABI).
 
-Tolerances (max |err| over the output, outputs are O(1) softmax averages of N(0,1) values):
-f32 accumulate with f16 K/V: 2e-3; bf16 operands (q rounded to bf16, probabilities to bf16): 1e-2.
+Tolerances are relative and per output row (one head's values for one query: an average of values, which shrinks like
+1/sqrt(visible keys), so an absolute bound would loosen with the cache length). The gate is the row's max relative error
+in the maximum norm, max |err| / max |reference row|, worst row (conftest.row_rel_err): <= 2e-3 with f32 accumulation
+over an f16 cache, <= 1e-2 with bf16 operands. Beside it the same error against the row's rms (conftest.row_rms_err, 2.5
+to 3 times stricter) is printed and held to 1.5 times those bounds: the kernels round q and the probabilities to the
+cache's element type for the MFMA, and a float64 model of exactly that rounding and nothing else gives 1.9e-3 to 2.3e-3
+(f16) and 8e-3 to 9e-3 (bf16) for this statistic on the prompts below (it is the largest of 1e5..1e6 samples of rounding
+noise); a dropped key segment or a wrong merge weight shows as O(1) in both.
 The reference is the textbook f64 attention (orc.attention_f64); aion's blocked CPU algorithm
 (orc.attention_blocked, polynomial exp) is compared as well at the same bound.
 """
@@ -12,6 +18,7 @@ import numpy as np
 import pytest
 
 from aion_amd import backend as be
+from conftest import row_rel_err, row_rms_err
 
 pytestmark = pytest.mark.gpu
 
@@ -19,6 +26,14 @@ pytestmark = pytest.mark.gpu
 def say(*a):
     print(*a, flush=True)
     sys.stdout.flush()
+
+
+def attn_err(got, ref, tol, tag=""):
+    """asserts the worst row's max relative error under `tol` and the rms form under 1.5 * tol (see the module text)"""
+    e_max, e_rms = row_rel_err(got, ref), row_rms_err(got, ref)
+    say("  %s worst row: max|err|/max|ref| = %.2e   max|err|/rms(ref) = %.2e   (bar %.0e)" % (tag, e_max, e_rms, tol))
+    assert np.isfinite(np.asarray(got)).all() and e_max < tol and e_rms < 1.5 * tol, (tag, e_max, e_rms, tol)
+    return e_max
 
 
 def to_bf16(x):
@@ -71,11 +86,9 @@ def test_prefill_causal_gqa(gpu, orc, kind, tol, D, L, kernel):
     got = run_attention(gpu, q, k, v, 1 / math.sqrt(D), qd, kd)
     assert gpu.last_kernel() == kernel
     ref = orc.attention_f64(qf, kf, vf, 1 / math.sqrt(D))
-    err = float(np.abs(got - ref).max())
-    say("  max err", err)
-    assert err < tol
+    attn_err(got, ref, tol)
     blocked = orc.attention_blocked(qf, kf, vf, 1 / math.sqrt(D))
-    assert float(np.abs(got - blocked).max()) < tol
+    attn_err(got, blocked, tol)
 
 
 def test_prefill_head_256_stale_tail_odd_lengths_and_scales(gpu, orc):
@@ -95,9 +108,7 @@ def test_prefill_head_256_stale_tail_odd_lengths_and_scales(gpu, orc):
         got = run_attention(gpu, q, k, v, scale, qd, kd, positions=pos, kv_lengths=ends)
         assert gpu.last_kernel() == kernel
         ref = orc.attention_f64(qf, kf, vf, scale, positions=pos, kv_lengths=ends)
-        err = float(np.abs(got - ref).max())
-        say("  scale", scale, "max err", err)
-        assert np.isfinite(got).all() and err < tol
+        attn_err(got, ref, tol)
 
 
 @pytest.mark.parametrize("kind,tol", [("f16", 2e-3), ("bf16", 1e-2)])
@@ -112,9 +123,7 @@ def test_decode_split_k(gpu, orc, kind, tol, T, B):
     got = run_attention(gpu, q, k, v, 1 / 16.0, qd, kd, positions=pos, kv_lengths=end)
     assert gpu.last_kernel() == "attn_flash_split"
     ref = orc.attention_f64(qf, kf, vf, 1 / 16.0, positions=pos, kv_lengths=end)
-    err = float(np.abs(got - ref).max())
-    say("  max err", err)
-    assert err < tol
+    attn_err(got, ref, tol)
 
 
 def test_decode_ragged_lengths_and_stale_cache_tail(gpu, orc):
@@ -131,7 +140,7 @@ def test_decode_ragged_lengths_and_stale_cache_tail(gpu, orc):
     got = run_attention(gpu, q, k, v, 0.1, qd, kd, positions=pos, kv_lengths=lens)
     ref = orc.attention_f64(qf, kf, vf, 0.1, positions=pos, kv_lengths=lens)
     assert np.isfinite(got).all()
-    assert float(np.abs(got - ref).max()) < 2e-3
+    attn_err(got, ref, 2e-3)
 
 
 @pytest.mark.parametrize("window", [(100, 0, 0), (16, 0, 64), (be.UNBOUNDED, be.UNBOUNDED, 0), (5, 3, 0)])
@@ -141,13 +150,13 @@ def test_windows_prefill_and_decode(gpu, orc, window):
     (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(11, B, L, L, Hq, Hkv, D, "f16")
     got = run_attention(gpu, q, k, v, 0.125, qd, kd, window=window)
     ref = orc.attention_f64(qf, kf, vf, 0.125, window=window)
-    assert float(np.abs(got - ref).max()) < 2e-3
+    attn_err(got, ref, 2e-3)
     # one decode row with an explicit position inside the sequence
     pos = np.array([[131]], np.int32)
     end = np.array([180], np.int32)
     got1 = run_attention(gpu, q[:, :1], k, v, 0.125, qd, kd, window=window, positions=pos, kv_lengths=end)
     ref1 = orc.attention_f64(qf[:, :1], kf, vf, 0.125, window=window, positions=pos, kv_lengths=end)
-    assert float(np.abs(got1 - ref1).max()) < 2e-3
+    attn_err(got1, ref1, 2e-3)
 
 
 def test_prefill_bf16_key_segments_empty_segments_and_value_range(gpu, orc):
@@ -163,17 +172,13 @@ def test_prefill_bf16_key_segments_empty_segments_and_value_range(gpu, orc):
         got = run_attention(gpu, q, k, v, 1 / math.sqrt(D), qd, kd, window=window, positions=pos, kv_lengths=lens)
         assert gpu.last_kernel() == "attn_prefill"
         ref = orc.attention_f64(qf, kf, vf, 1 / math.sqrt(D), window=window, positions=pos, kv_lengths=lens)
-        err = float(np.abs(got - ref).max())
-        say("  max err", err)
-        assert np.isfinite(got).all() and err < 1e-2
+        attn_err(got, ref, 1e-2)
     ref = orc.attention_f64(qf, kf, vf, 1 / math.sqrt(D))
     for e in (100, -100):
         vb, vbf = to_bf16(vf * np.float32(2.0 ** e))
         got = run_attention(gpu, q, k, vb, 1 / math.sqrt(D), qd, kd)
         assert gpu.last_kernel() == "attn_prefill"
-        err = float(np.abs(got * np.float32(2.0 ** -e) - ref).max())
-        say("  values x 2^%d: max err" % e, err)
-        assert np.isfinite(got).all() and err < 1e-2
+        attn_err(got * np.float32(2.0 ** -e), ref, 1e-2)
 
 
 def test_soft_cap(gpu, orc):
@@ -183,7 +188,7 @@ def test_soft_cap(gpu, orc):
     q3 = (q * 3).astype(np.float16).astype(np.float32)
     got = run_attention(gpu, q3, k, v, 1.0, qd, kd, soft_cap=5.0)
     ref = orc.attention_f64(q3, kf, vf, 1.0, soft_cap=5.0)
-    assert float(np.abs(got - ref).max()) < 2e-3
+    attn_err(got, ref, 2e-3)
 
 
 def test_kat_uniform_softmax_sliding_window(gpu):
@@ -220,7 +225,7 @@ def test_generic_path_matches_oracle_on_odd_head_sizes(gpu, orc):
     pos = np.tile(np.arange(61, 70, dtype=np.int32), (2, 1))
     got = run_attention(gpu, q, k, v, 0.2, be.F32, be.F32, positions=pos)
     ref = orc.attention_f64(q, k, v, 0.2, positions=pos)
-    assert float(np.abs(got - ref).max()) < 1e-4
+    attn_err(got, ref, 1e-4)
 
 
 def test_empty_window_and_plain_equals_cached(gpu, orc):
@@ -255,9 +260,10 @@ def test_precise_mode_brings_f32_queries_to_f32_accuracy(gpu, orc):
         precise = run_attention(gpu, q, k, v, 1 / 16.0, qd, kd, positions=pos)
     finally:
         gpu.set_attention_precise(False)
-    e_fast, e_prec = float(np.abs(fast - ref).max()), float(np.abs(precise - ref).max())
-    say("  fast", e_fast, "precise", e_prec)
-    assert e_fast < 2e-3 and e_prec < 1e-5
+    attn_err(fast, ref, 2e-3, "fast")
+    e_prec = row_rms_err(precise, ref)
+    say("  precise: worst row max|err|/rms(row)", e_prec)
+    assert e_prec < 5e-5
 
 
 def test_prefill_config4_sizes(gpu, orc):
@@ -273,30 +279,26 @@ def test_prefill_config4_sizes(gpu, orc):
         got = run_attention(gpu, q, k, v, 1 / 16.0, qd, kd)
         assert gpu.last_kernel() == kernel
         ref = orc.attention_f64(qf, kf, vf, 1 / 16.0)
-        err = float(np.abs(got - ref).max())
-        say("  max err", err)
-        assert err < 1e-2
+        attn_err(got, ref, 1e-2)
     say("prefill config 4 L4096 properties")
     L = 4096
     (q, k, v, qd, kd), (qf, kf, vf) = make_qkv(43, 1, L, L, 8, 1, 256, "bf16")
     ones, _ = to_bf16(np.full((1, L, 1, 256), 0.75, np.float32))
     got = run_attention(gpu, q, k, ones, 1 / 16.0, qd, kd)
     assert gpu.last_kernel() == "attn_prefill"
-    assert float(np.abs(got - 0.75).max()) < 1e-2
+    assert row_rel_err(got, np.full_like(got, 0.75)) < 1e-2
     got = run_attention(gpu, q, k, v, 1 / 16.0, qd, kd)
     # one visible key: its value (the single probability is exp2 of a rounding residue, 1 to within an ulp)
     assert np.allclose(got[0, 0], np.broadcast_to(vf[0, 0, 0], (8, 256)), rtol=1e-6, atol=0)
     # the last rows against the reference on the last 16 positions only (full key range)
     ref_tail = orc.attention_f64(qf[:, L - 16:], kf, vf, 1 / 16.0, positions=np.arange(L - 16, L, dtype=np.int32).reshape(1, 16))
-    assert float(np.abs(got[:, L - 16:] - ref_tail).max()) < 1e-2
+    attn_err(got[:, L - 16:], ref_tail, 1e-2)
     # and a sample of positions over the whole range against the reference: around the 128-row workgroup tiles (8 heads x 16
     # positions each), around the middle of the key range, where a row tile's two key segments meet, and in between
     idx = np.unique(np.array([1, 15, 16, 17, 63, 64, 200, 1000, 1023, 1024, 1025, 2040, 2047, 2048, 2049, 2111, 2112, 3000, 3071, 3072,
                               4000, 4079, 4080] + list(range(777, 4096, 512))))
     ref_s = orc.attention_f64(np.ascontiguousarray(qf[:, idx]), kf, vf, 1 / 16.0, positions=idx.astype(np.int32).reshape(1, -1))
-    err = float(np.abs(got[:, idx] - ref_s).max())
-    say("  L4096 sample of", idx.size, "positions: max err", err)
-    assert err < 1e-2
+    attn_err(got[:, idx], ref_s, 1e-2)
     # just past one workgroup per CU (260 row tiles on 256 CUs): two key segments per row tile again, because the longest
     # row tile alone would take as long as two average ones
     L = 4160
@@ -306,9 +308,7 @@ def test_prefill_config4_sizes(gpu, orc):
     assert gpu.last_kernel() == "attn_prefill"
     idx = np.array([0, 1, 16, 1000, 2079, 2080, 2081, 3000, 4095, 4096, 4144, 4159])
     ref_s = orc.attention_f64(np.ascontiguousarray(qf[:, idx]), kf, vf, 1 / 16.0, positions=idx.astype(np.int32).reshape(1, -1))
-    err = float(np.abs(got[:, idx] - ref_s).max())
-    say("  L4160 sample of", idx.size, "positions: max err", err)
-    assert err < 1e-2
+    attn_err(got[:, idx], ref_s, 1e-2)
 
 
 @pytest.mark.parametrize("B,Lq,T,lens,kernel", [
@@ -329,7 +329,7 @@ def test_prefill_chunk_with_positions_over_a_longer_cache(gpu, orc, B, Lq, T, le
     kz, vz = np.nan_to_num(kf), np.nan_to_num(vf)
     ref = orc.attention_f64(qf, kz, vz, 1 / math.sqrt(D), positions=pos, kv_lengths=lens)
     assert np.isfinite(got).all()
-    assert float(np.abs(got - ref).max()) < 2e-3
+    attn_err(got, ref, 2e-3)
 
 
 # A chunk of queries over a cache at least four times its length: with enough keys the 128-row kernel (keys cut into
@@ -348,9 +348,7 @@ def test_query_chunk_over_a_long_cache(gpu, orc, kind, tol, Lq, kernel):
     assert gpu.last_kernel() == kernel
     ref = orc.attention_f64(qf, kf, vf, 1 / math.sqrt(D), positions=pos, kv_lengths=lens)
     assert np.isfinite(got).all()
-    err = float(np.abs(got - ref).max())
-    say("  max err", err)
-    assert err < tol
+    attn_err(got, ref, tol)
 
 
 def ring_of(linear, T):
@@ -393,9 +391,7 @@ def test_rolling_caches(gpu, orc, case):
     got = run_attention(gpu, q, k_ring, v_ring, 1 / math.sqrt(D), qd, kd, window=window, positions=pos, kv_lengths=ends, rolling=True)
     assert gpu.last_kernel() == kernel
     want = orc.attention_rolling_f64(qf, kr_f, vr_f, 1 / math.sqrt(D), window, pos, ends)
-    err = float(np.abs(got - want).max())
-    say("  max err", err)
-    assert np.isfinite(got).all() and err < (1e-2 if kind == "bf16" else 2e-3)
+    attn_err(got, want, (1e-2 if kind == "bf16" else 2e-3))
 
 
 @pytest.mark.parametrize("window,rolling,soft_cap", [(be.CAUSAL, False, 0.0), ((300, 0, 0), False, 0.0), ((200, 40, 64), False, 0.0),
@@ -420,4 +416,4 @@ def test_prefill_key_segments_with_windows_and_ragged_lengths(gpu, orc, window, 
     else:
         ref = orc.attention_f64(qf, kf, vf, 1 / math.sqrt(D), window=window, soft_cap=soft_cap, positions=pos, kv_lengths=ends)
     assert np.isfinite(got).all()
-    assert float(np.abs(got - ref).max()) < 2e-3
+    attn_err(got, ref, 2e-3)

@@ -78,8 +78,9 @@ def test_exact_gemm_rows_match_decode_path(gpu, orc, dtype, layout):
     w.free()
 
 
-@pytest.mark.parametrize("dtype,layout", [(be.Q8_0, be.ROWS_NK), (be.Q4_0, be.KMAJOR_KN)])
-@pytest.mark.parametrize("m,n", [(512, 4096), (2048, 14336)])
+# every (M, N) pair of config 3 (each picks its own tile and launch shape) in every weight format and layout
+@pytest.mark.parametrize("dtype,layout", CASES)
+@pytest.mark.parametrize("m,n", [(512, 4096), (512, 14336), (2048, 4096), (2048, 14336)])
 def test_config3_exact_full_size_on_row_sample(gpu, orc, dtype, layout, m, n):
     k = 4096
     say("config3 exact", dtype, m, n)
@@ -126,8 +127,8 @@ def test_bf16_gemm_ragged_shapes(gpu, orc, dtype, layout, m, n, k):
 # narrow one), the last one hanging over; (2048, 5120): 27 tiles of 192 in one round instead of two rounds of 128-row tiles.
 # (1300, 11008): 258 tiles of 256 rows would need a second round, so 473 tiles of 128 rows run in two half-time rounds.
 # Rows from every 256-row tile, all columns.
-@pytest.mark.parametrize("dtype,layout", [(be.Q8_0, be.ROWS_NK), (be.Q4_0, be.KMAJOR_KN)])
-@pytest.mark.parametrize("m,n", [(512, 4096), (2048, 14336), (2048, 9092), (2048, 13000), (2048, 5120), (1300, 11008)])
+@pytest.mark.parametrize("dtype,layout", CASES)
+@pytest.mark.parametrize("m,n", [(512, 4096), (512, 14336), (2048, 4096), (2048, 14336), (2048, 9092), (2048, 13000), (2048, 5120), (1300, 11008)])
 def test_config3_bf16_full_size_on_row_sample(gpu, orc, dtype, layout, m, n):
     k = 4096
     say("config3 bf16", dtype, m, n)

@@ -64,3 +64,44 @@ def test_large_blocks_alignment_and_foreign_handles(gpu):
     with pytest.raises(Exception):
         gpu.alloc(100, alignment=48)                 # not a power of two
     gpu.trim()
+
+
+def test_program_recorded_before_a_work_buffer_grows_is_refused(orc):
+    """A recorded program's launches address the context's work buffers. A later eager step that needs a larger one
+    replaces it; the old program must then be refused (nothing launched) instead of replaying on freed memory, and
+    recording the steps again gives a program that runs."""
+    from aion_amd import backend as be
+    from aion_amd import hip
+    g = be.HipBackend(0)                              # a context of its own: the scratch sizes are what is under test
+    try:
+        rng = np.random.default_rng(9)
+        n, k = 256, 512
+        wf = (rng.standard_normal((k, n)) * 0.05).astype(np.float32)
+        blocks = be.quantize_blocks(be.Q4_0, wf, 0)
+        w = g.upload_weight(be.Q4_0, be.KMAJOR_KN, n, k, blocks)
+        a4 = rng.standard_normal((4, k)).astype(np.float32)
+        a_buf, c_buf = g.upload(a4), g.zeros(4 * n * 4)
+        g.step_matmul(w, a_buf, 4, c_buf)             # eager once: the prepared-activation scratch gets its size for 4 rows
+        prog = g.record_program(lambda: g.step_matmul(w, a_buf, 4, c_buf))
+        assert g.program_is_current(prog)
+        g.program_execute(prog)
+        want = orc.matmul_q_packed(be.Q4_0, a4, blocks, n, threads=4)
+        assert np.abs(g.download(c_buf, np.float32, (4, n)) - want).max() <= 1e-5 * np.sqrt((want.astype(np.float64) ** 2).mean())
+        big = g.upload(rng.standard_normal((64, k)).astype(np.float32))
+        big_c = g.zeros(64 * n * 4)
+        g.step_matmul(w, big, 64, big_c)              # 64 rows: the scratch is replaced by a larger one
+        assert not g.program_is_current(prog)
+        with pytest.raises(be.AionHipError) as e:
+            g.program_execute(prog)
+        assert e.value.status == hip.INVALID_ARGUMENT and "stale program" in str(e.value)
+        g.program_destroy(prog)
+        prog = g.record_program(lambda: g.step_matmul(w, a_buf, 4, c_buf))
+        g._check(g._lib.aionhip_memset(g._ctx, c_buf.handle, 0, 0, 4 * n * 4))
+        g.program_execute(prog)
+        assert np.abs(g.download(c_buf, np.float32, (4, n)) - want).max() <= 1e-5 * np.sqrt((want.astype(np.float64) ** 2).mean())
+        g.program_destroy(prog)
+        for t in (a_buf, c_buf, big, big_c):
+            t.free()
+        w.free()
+    finally:
+        g.close()
