@@ -72,7 +72,7 @@ class Weight:
         return out
 
     def drop_bf16(self):
-        """Releases the bf16 copy the bf16 GEMM mode keeps of this weight (rebuilt on its next bf16 call)."""
+        """Releases the bf16 copy the context keeps of this weight in bf16 GEMM mode (rebuilt on its next bf16 call)."""
         if self.ptr:
             self.backend._lib.aionhip_weight_drop_bf16(self.backend._ctx, self.ptr)
 
@@ -300,6 +300,15 @@ class HipBackend:
 
     def program_execute(self, prog):
         self._check(self._lib.aionhip_program_execute(self._ctx, prog))
+
+    def set_bf16_weight_copies(self, on):
+        """bf16 GEMM mode: True (default) keeps a bf16 copy per weight, False converts the quant blocks inside the kernel."""
+        self._check(self._lib.aionhip_set_bf16_weight_copies(self._ctx, 1 if on else 0))
+
+    def bf16_copy_stats(self):
+        n, b = C.c_uint64(0), C.c_uint64(0)
+        self._check(self._lib.aionhip_bf16_copy_stats(self._ctx, C.byref(n), C.byref(b)))
+        return n.value, b.value
 
     def program_is_current(self, prog):
         """False once a work buffer the program's launches address has been replaced by a larger one: record it again."""

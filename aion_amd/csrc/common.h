@@ -9,6 +9,7 @@
 #include <cstdio>
 #include <string>
 #include <unordered_map>
+#include <utility>
 #include <vector>
 
 #include "../../include/aion_hip.h"
@@ -60,6 +61,12 @@ struct aionhip_ctx {
     uint64_t buffer_generation = 0;
     // this device's copy of the library's file-scope scratch array (ctx.hip), for the entry point that allocates nothing
     void *static_scratch = nullptr;
+    // bf16 mode of the GEMM: this context's bf16 copies of the weights it has multiplied (weight -> {copy, bytes}), built
+    // on a weight's first bf16 call, released by aionhip_weight_drop_bf16 / aionhip_weight_free / aionhip_destroy;
+    // bf16_copies_on = false: no copies, the kernel converts the quant blocks while it stages them
+    std::unordered_map<const struct aionhip_weight *, std::pair<void *, size_t>> bf16_copies;
+    size_t bf16_copy_bytes = 0;
+    bool bf16_copies_on = true;
     // true while that entry point runs: no launcher may take a path that needs scratch of its own
     bool no_scratch_paths = false;
     // attention with f32 queries: false = one MFMA pass on q rounded to the K/V element type (2e-3 class),
@@ -123,8 +130,6 @@ struct aionhip_weight {
     uint8_t *qs = nullptr;
     __half *sc = nullptr;
     size_t qs_bytes = 0, sc_bytes = 0;
-    // lazily built by the bf16 MFMA GEMM: the weight dequantized to bf16, [n / 16][k / 32][16][32] (n padded to 16 with zeros)
-    unsigned short *bf16 = nullptr;
 };
 
 int set_err(aionhip_ctx *ctx, int status, const char *fmt, ...);

@@ -209,6 +209,7 @@ void aionhip_destroy(aionhip_ctx *ctx) {
     }
     for (auto e : ctx->event_pool) (void)hipEventDestroy(e);
     for (auto &t : ctx->rope_tables) (void)hipFree(t.freq);
+    for (auto &kv : ctx->bf16_copies) (void)hipFree(kv.second.first);
     if (ctx->scratch) (void)hipFree(ctx->scratch);
     if (ctx->scratch2) (void)hipFree(ctx->scratch2);
     if (ctx->ksplit) (void)hipFree(ctx->ksplit);

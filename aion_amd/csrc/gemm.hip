@@ -11,6 +11,9 @@
 //   v_mfma_f32_32x32x16_bf16 with f32 accumulation; described at the kernel.
 #include "common.h"
 
+#include <type_traits>
+#include <utility>
+
 namespace {
 
 using u32x2 = __attribute__((ext_vector_type(2))) unsigned int;
@@ -286,10 +289,10 @@ __device__ __forceinline__ unsigned short bf16_rne(float x) {
     return (unsigned short)(u >> 16);
 }
 
-// Both bf16 operands of the MFMA kernel are private copies, laid out for its loads: 16 rows x 32 k (1 KiB) per block, blocks
-// k-major within a group of 16 rows - [rows / 16][K / 32][16][32]. One LDS-writing load of a wavefront (16 rows x 64 bytes
-// of one K step) is then 1 KiB of consecutive memory, eight whole 128-byte lines, where a row-major operand gives the L2
-// sixteen 64-byte requests, which it serves at the rate of 128-byte ones. Rows are padded to a multiple of 16 with zeros.
+// The activation operand of the MFMA kernel is a bf16 copy made per call, laid out for its loads: 16 rows x 32 k (1 KiB) per
+// block, blocks k-major within a group of 16 rows - [rows / 16][K / 32][16][32]. One LDS-writing load of a wavefront (16 rows
+// x 64 bytes of one K step) is then 1 KiB of consecutive memory, eight whole 128-byte lines, where a row-major operand gives
+// the L2 sixteen 64-byte requests, which it serves at the rate of 128-byte ones. Rows are padded to a multiple of 16 with zeros.
 __device__ __forceinline__ size_t bf16_tiled_index(size_t row, size_t k0, size_t K) {
     return (((row >> 4) * (K / G2_TILE_K) + k0 / G2_TILE_K) * 16 + (row & 15)) * G2_TILE_K + (k0 % G2_TILE_K);
 }
@@ -391,10 +394,99 @@ __device__ __forceinline__ void sched_half() {
     }
 }
 
+// The weight operand of the bf16 kernel, dequantized while it is staged (as aion's GPU GEMM does, backend/gpu/kernels/
+// matmul_q8_mx16.wgsl): thread t of the workgroup owns column n0 + t of the tile. Every four K steps it requests the next
+// four quant blocks of its row (64 bytes of q4 codes, 128 of q8, and their four f16 scales) into registers - three such
+// groups rotate: one being converted, one waiting, one in flight - and in every K step it converts one block to 32 bf16
+// values (code * f32(scale), rounded to nearest even: the bits a separate dequantization pass would give) and writes
+// them as the 64-byte row of the LDS stage two K steps ahead, in the swizzled chunk order the fragment reads expect.
+// The L2 then delivers 18 or 34 bytes per 32 weights instead of 64, and no bf16 copy of the weight exists.
+template <int BDT>
+struct WGroup {
+    static constexpr int NQ = BDT == AIONHIP_Q8_0 ? 8 : 4;      // 16-byte loads per group of four blocks
+    u32x4 q[NQ];
+    unsigned short s[4];
+};
+template <int BDT>
+struct WSource {
+    const uint8_t *row;          // this thread's weight row (codes)
+    const __half *sc;            // its block scales
+    int kb;                      // blocks per row
+    // load i of a group request (i < NQ: 16 bytes of codes, then the four scales), for callers that space the loads out
+    __device__ __forceinline__ void request_one(int group, WGroup<BDT> &g, int i) const {
+        constexpr int PER = BDT == AIONHIP_Q8_0 ? 2 : 1;
+        constexpr int NQ = WGroup<BDT>::NQ;
+        if (i < NQ) {
+            const int b = min(group * 4 + i / PER, kb - 1);
+            g.q[i] = *(const u32x4 *)(row + (size_t)b * (16 * PER) + (i % PER) * 16);
+        } else {
+            const int b = min(group * 4 + (i - NQ), kb - 1);
+            g.s[i - NQ] = __half_as_ushort(sc[b]);
+        }
+    }
+    __device__ __forceinline__ void request(int group, WGroup<BDT> &g) const {
+        constexpr int PER = BDT == AIONHIP_Q8_0 ? 2 : 1;        // 16-byte chunks per block
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int b = min(group * 4 + j, kb - 1);            // past the end: a harmless repeat into a dead stage
+#pragma unroll
+            for (int h = 0; h < PER; ++h) g.q[j * PER + h] = *(const u32x4 *)(row + (size_t)b * (16 * PER) + h * 16);
+            g.s[j] = __half_as_ushort(sc[b]);
+        }
+    }
+};
+// block j of a group -> 32 bf16 values into the 64-byte stage row `dst` of a thread whose row swizzle is `swz`
+// Conversion state of one block, advanced element by element so that the caller can put one element's three vector
+// instructions behind each MFMA: element e (0 .. 31) of block j of a group; after the eighth element of a 16-byte chunk the
+// chunk is written to the stage row.
+template <int BDT>
+struct DeqBlock {
+    float sc, off;
+    unsigned lo, hi;
+    float f[8];
+    template <int J, int E>
+    __device__ __forceinline__ void element(const WGroup<BDT> &g, unsigned char *dst, int swz) {
+        using f32x2_t = __attribute__((ext_vector_type(2))) float;
+        using bf16x2_t = __attribute__((ext_vector_type(2))) __bf16;
+        auto pk = [](float a, float b) { return __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2_t{a, b}, bf16x2_t)); };
+        constexpr int d = E / 8, i = E % 8;
+        if constexpr (E == 0 || E == 16) {
+            sc = __half2float(__ushort_as_half(g.s[J]));
+            off = (BDT == AIONHIP_Q4_0 ? -8.f : -128.f) * sc;     // (c - 8) * s = fma(c, s, -8 s): one rounding, the same value
+        }
+        if constexpr (i == 0) {
+            if constexpr (BDT == AIONHIP_Q4_0) {
+                // byte i of a word = e[8d + i] | e[8d + 4 + i] << 4
+                const unsigned w = d == 0 ? g.q[J].x : d == 1 ? g.q[J].y : d == 2 ? g.q[J].z : g.q[J].w;
+                lo = w & 0x0F0F0F0Fu;
+                hi = (w >> 4) & 0x0F0F0F0Fu;
+            } else {
+                // signed code c = u - 128 with u = c ^ 0x80
+                const u32x4 w = g.q[J * 2 + (d >> 1)];
+                lo = ((d & 1) ? w.z : w.x) ^ 0x80808080u;
+                hi = ((d & 1) ? w.w : w.y) ^ 0x80808080u;
+            }
+        }
+        f[i] = fmaf((float)(((i < 4 ? lo : hi) >> (8 * (i & 3))) & 0xFFu), sc, off);
+        if constexpr (i == 7) *(u32x4 *)(dst + ((d ^ swz) * 16)) = u32x4{pk(f[0], f[1]), pk(f[2], f[3]), pk(f[4], f[5]), pk(f[6], f[7])};
+    }
+};
+template <int I, int E, class F>
+__device__ __forceinline__ void static_for_gemm(F &&f) {
+    if constexpr (I < E) {
+        f(std::integral_constant<int, I>{});
+        static_for_gemm<I + 1, E>(f);
+    }
+}
+constexpr int vmcnt_lgkm0_imm(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4); }   // vmcnt <= n and lgkmcnt == 0
+
 // one workgroup tile: rows m0 .., columns n0 .. of C (N is the column bound of W and C as passed)
-template <int WM, int NST, int WN>
+// BDT = 0: W is a bf16 copy in the tiled layout; BDT = a block format: the weight itself (wq, wsc), dequantized while staged
+template <int WM, int NST, int WN, int BDT = 0>
 __device__ __forceinline__ void gemm_bf16_tile(unsigned char *lds2, const unsigned short *__restrict__ A, const unsigned short *__restrict__ W,
-                                               float *__restrict__ c, int M, int N, int K, size_t ldc, float alpha, float beta, int m0, int n0) {
+                                               float *__restrict__ c, int M, int N, int K, size_t ldc, float alpha, float beta, int m0, int n0,
+                                               const uint8_t *__restrict__ wq = nullptr, const __half *__restrict__ wsc = nullptr) {
+    static_assert(BDT == 0 || NST == 4, "the dequantizing form writes the stage two K steps ahead of a four-stage ring");
     constexpr int BM2 = WM * 64;
     constexpr int BN2 = WN * 64;                             // 256 columns, or 192 for the last partial round of tiles
     constexpr int A_BYTES = BM2 * G2_ROW, B_BYTES = BN2 * G2_ROW, STAGE = A_BYTES + B_BYTES;
@@ -422,7 +514,28 @@ __device__ __forceinline__ void gemm_bf16_tile(unsigned char *lds2, const unsign
 #pragma unroll
     for (int i = 0; i < NA; ++i) ga[i] = A + (size_t)min((m0 >> 4) + i * 4 + wave, a_blocks - 1) * KT * (16 * G2_BK) + in_block;
 #pragma unroll
-    for (int i = 0; i < NB; ++i) gb[i] = W + (size_t)min((n0 >> 4) + i * 4 + wave, w_blocks - 1) * KT * (16 * G2_BK) + in_block;
+    for (int i = 0; i < NB; ++i) gb[i] = BDT ? nullptr : W + (size_t)min((n0 >> 4) + i * 4 + wave, w_blocks - 1) * KT * (16 * G2_BK) + in_block;
+    (void)w_blocks;
+    // dequantizing form: this thread's weight row and its stage row
+    WSource<BDT ? BDT : AIONHIP_Q4_0> wsrc{};
+    WGroup<BDT ? BDT : AIONHIP_Q4_0> g_cur, g_nxt, g_fut;
+    const int b_row = min(tid, BN2 - 1), b_swz = (b_row >> 2) & 3;
+    if constexpr (BDT != 0) {
+        const size_t n = (size_t)min(n0 + b_row, N - 1);
+        wsrc.row = wq + n * (BDT == AIONHIP_Q8_0 ? (size_t)K : (size_t)K / 2);
+        wsrc.sc = wsc + n * (size_t)(K / 32);
+        wsrc.kb = K / 32;
+    }
+    unsigned char *const b_stage_row = lds2 + A_BYTES + b_row * G2_ROW;       // this thread's row in stage 0
+    using BT = std::integral_constant<int, BDT ? BDT : AIONHIP_Q4_0>;
+    DeqBlock<BT::value> dq;
+    auto deq_whole = [&](const WGroup<BT::value> &g, auto jc, int kt) __attribute__((always_inline)) {
+        constexpr int J = decltype(jc)::value;
+        if (tid < BN2) {
+            unsigned char *dst = b_stage_row + (kt % NST) * STAGE;
+            static_for_gemm<0, 32>([&](auto ec) __attribute__((always_inline)) { dq.template element<J, decltype(ec)::value>(g, dst, b_swz); });
+        }
+    };
 
     auto issue_loads = [&](int kt, bool a_part, bool b_part) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the builtin exists in the device pass only
@@ -432,12 +545,21 @@ __device__ __forceinline__ void gemm_bf16_tile(unsigned char *lds2, const unsign
 #pragma unroll
             for (int i = 0; i < NA; ++i)
                 __builtin_amdgcn_global_load_lds(ga[i] + k, (lds_void *)(stage + i * 64 * G2_ROW), 16, 0, 0);
-        if (b_part)
+        if (b_part && BDT == 0)
 #pragma unroll
             for (int i = 0; i < NB; ++i)
                 __builtin_amdgcn_global_load_lds(gb[i] + k, (lds_void *)(stage + A_BYTES + i * 64 * G2_ROW), 16, 0, 0);
 #endif
     };
+
+    auto issue_a_load = [&](int kt, int i) {
+#if defined(__HIP_DEVICE_COMPILE__)
+        unsigned char *stage = lds2 + (kt % NST) * STAGE + wave * 16 * G2_ROW;
+        const size_t k = (size_t)min(kt, KT - 1) * (16 * G2_BK);
+        __builtin_amdgcn_global_load_lds(ga[i] + k, (lds_void *)(stage + i * 64 * G2_ROW), 16, 0, 0);
+#endif
+    };
+    (void)issue_a_load;
 
     // fragment of sub-step ks: row (base + l31), chunk ks*2 + lh, at slot chunk ^ ((l31 >> 2) & 3)
     const int swz = (l31 >> 2) & 3;
@@ -465,13 +587,14 @@ __device__ __forceinline__ void gemm_bf16_tile(unsigned char *lds2, const unsign
     };
     constexpr int NMMA = WM * WN, NFR = WM + WN;
 
+    Frag f0, f1;
+    if constexpr (BDT == 0) {
     // issue order: A0 B0 A1 B1 .. A(NST-2) | K step 0: B(NST-2), A(NST-1) | K step 1: B(NST-1), A(NST) | ...
 #pragma unroll
     for (int i = 0; i < NST - 2; ++i) issue_loads(i, true, true);
     issue_loads(NST - 2, true, false);
     __builtin_amdgcn_s_waitcnt(vmcnt_imm((NST - 3) * NL + NA));   // stage 0 of this wavefront has landed
     __builtin_amdgcn_s_barrier();                            // ... and everybody else's
-    Frag f0, f1;
     read_frag(f0, 0, 0);
     for (int kt = 0; kt < KT; ++kt) {
         // sub-step 0 while the fragments of sub-step 1 are read
@@ -488,6 +611,67 @@ __device__ __forceinline__ void gemm_bf16_tile(unsigned char *lds2, const unsign
         issue_loads(kt + NST - 1, true, false);
         mma(f1);
         if constexpr (WM >= 2) sched_half<NMMA, NFR, NA>();
+    }
+    } else {
+    // Dequantizing form. Load order: groups 0 and 1 of the weight row, A0 A1 A2 | K step kt: (first of four: group kt/4 + 2),
+    // A(kt+3). The weight block of K step kt + 2 is converted into its stage during the first half of K step kt.
+    constexpr int NF = WGroup<BDT ? BDT : AIONHIP_Q4_0>::NQ + 4;  // loads of one group request
+    wsrc.request(0, g_cur);
+    wsrc.request(1, g_nxt);
+#pragma unroll
+    for (int i = 0; i < NST - 1; ++i) issue_loads(i, true, false);
+    deq_whole(g_cur, std::integral_constant<int, 0>{}, 0);
+    deq_whole(g_cur, std::integral_constant<int, 1>{}, 1);
+    __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm((NST - 2) * NA));  // A of stage 0 has landed, the two converted blocks are written
+    __builtin_amdgcn_s_barrier();
+    read_frag(f0, 0, 0);
+    // Half a K step: behind every MFMA one slice of everything else the half has to issue - the conversion of 16 / NMMA
+    // weight elements (the matrix pipe takes 32 cycles per MFMA, the vector pipe 4 per instruction, and a wavefront issues
+    // in order: what is to run in an MFMA's shadow has to stand behind it in the program), in the second half also one of
+    // the global loads - pinned with scheduling barriers.
+    auto half = [&](const Frag &f, int kt, auto jc, auto hc) __attribute__((always_inline)) {
+        constexpr int j = decltype(jc)::value, hf = decltype(hc)::value;
+        constexpr int J = j < 2 ? j + 2 : j - 2;                  // block of the group: 2, 3 of the current one, then 0, 1 of the next
+        const WGroup<BT::value> &g = j < 2 ? g_cur : g_nxt;
+        unsigned char *dst = b_stage_row + ((kt + 2) % NST) * STAGE;
+        constexpr int NLD = hf == 1 ? NA + (j == 0 ? NF : 0) : 0; // global loads of this half
+        static_for_gemm<0, NMMA>([&](auto ic) __attribute__((always_inline)) {
+            constexpr int i = decltype(ic)::value, mi = i / WN, ni = i % WN;
+            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, f.b[ni]), __builtin_bit_cast(bf16x8, f.a[mi]), acc[mi][ni], 0, 0, 0);
+            constexpr int e0 = hf * 16 + i * 16 / NMMA, e1 = hf * 16 + (i + 1) * 16 / NMMA;
+            if (tid < BN2) static_for_gemm<e0, e1>([&](auto ec) __attribute__((always_inline)) { dq.template element<J, decltype(ec)::value>(g, dst, b_swz); });
+            // loads: spread over the MFMAs (as many per MFMA as it takes)
+            constexpr int l0 = i * NLD / NMMA, l1 = (i + 1) * NLD / NMMA;
+            static_for_gemm<l0, l1>([&](auto lc) __attribute__((always_inline)) {
+                constexpr int li = decltype(lc)::value;
+                if constexpr (li < NA) issue_a_load(kt + NST - 1, li);
+                else wsrc.request_one(kt / 4 + 2, g_fut, li - NA);
+            });
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    auto step = [&](int kt, auto jc) __attribute__((always_inline)) {
+        constexpr int j = decltype(jc)::value;
+        read_frag(f1, kt, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        half(f0, kt, jc, std::integral_constant<int, 0>{});
+        // A of stage kt+1 landed (what was requested after it may still be in flight); the chunks converted so far are
+        // written; past this barrier nobody reads stage kt-1
+        __builtin_amdgcn_s_waitcnt(vmcnt_lgkm0_imm(j == 1 || j == 2 ? NA + NF : NA));
+        __builtin_amdgcn_s_barrier();
+        read_frag(f0, kt + 1, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        // ... and the other half of the block (written before the barrier of the next K step, behind which stage kt+2 is first read)
+        half(f1, kt, jc, std::integral_constant<int, 1>{});
+    };
+    for (int kt0 = 0; kt0 < KT; kt0 += 4) {
+        step(kt0, std::integral_constant<int, 0>{});
+        if (kt0 + 1 < KT) step(kt0 + 1, std::integral_constant<int, 1>{});
+        if (kt0 + 2 < KT) step(kt0 + 2, std::integral_constant<int, 2>{});
+        if (kt0 + 3 < KT) step(kt0 + 3, std::integral_constant<int, 3>{});
+        g_cur = g_nxt;
+        g_nxt = g_fut;
+    }
     }
     __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));                // no LDS-writing load may outlive the workgroup
 
@@ -520,23 +704,24 @@ __device__ __forceinline__ void gemm_bf16_tile(unsigned char *lds2, const unsign
     }
 }
 
-template <int WM, int NST, int WN>
-__global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const unsigned short *__restrict__ A, const unsigned short *__restrict__ W,
+template <int WM, int NST, int WN, int BDT>
+__global__ __launch_bounds__(256) void gemm_bf16_wide_kernel(const unsigned short *__restrict__ A, const uint8_t *__restrict__ wq, const __half *__restrict__ wsc,
                                                              float *__restrict__ c, int M, int N, int K, size_t ldc, float alpha,
                                                              float beta, int tiles_m, int tiles) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds2[];
     const int per_xcd = (int)gridDim.x >> 3;
     const int t = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
     if (t >= tiles) return;
-    gemm_bf16_tile<WM, NST, WN>(lds2, A, W, c, M, N, K, ldc, alpha, beta, (t % tiles_m) * (WM * 64), (t / tiles_m) * (WN * 64));
+    // (BDT = 0: wq is the weight's bf16 copy in the tiled layout)
+    gemm_bf16_tile<WM, NST, WN, BDT>(lds2, A, (const unsigned short *)wq, c, M, N, K, ldc, alpha, beta, (t % tiles_m) * (WM * 64), (t / tiles_m) * (WN * 64), wq, wsc);
 }
 
 // 256-row tiles over N = tw * 256 + (a rest covered by tn tiles of 192 columns), ONE launch: the column tiles go
 // wide, wide, narrow, narrow, ... while both kinds last. A CU's first tile is then wide on half of the CUs and narrow on the
 // other half, the CUs that finish early pick up wide tiles next, and the epilogues (64 MB of f32 stores that would otherwise
 // hit the HBM from every CU at the same moment, with the matrix pipes idle) fall into the others' main loops.
-template <int NST>
-__global__ __launch_bounds__(256) void gemm_bf16_mixed_kernel(const unsigned short *__restrict__ A, const unsigned short *__restrict__ W,
+template <int NST, int BDT>
+__global__ __launch_bounds__(256) void gemm_bf16_mixed_kernel(const unsigned short *__restrict__ A, const uint8_t *__restrict__ wq, const __half *__restrict__ wsc,
                                                               float *__restrict__ c, int M, int N, int K, size_t ldc, float alpha,
                                                               float beta, int tiles_m, int tw, int tn) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds2[];
@@ -555,8 +740,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_mixed_kernel(const unsigned sho
         wide = rest < rest_wide;
         idx = 2 * fb + (wide ? rest : rest - rest_wide);
     }
-    if (wide) gemm_bf16_tile<4, NST, 4>(lds2, A, W, c, M, N, K, ldc, alpha, beta, m0, idx * 256);
-    else gemm_bf16_tile<4, NST, 3>(lds2, A, W, c, M, N, K, ldc, alpha, beta, m0, tw * 256 + idx * 192);
+    if (wide) gemm_bf16_tile<4, NST, 4, BDT>(lds2, A, (const unsigned short *)wq, c, M, N, K, ldc, alpha, beta, m0, idx * 256, wq, wsc);
+    else gemm_bf16_tile<4, NST, 3, BDT>(lds2, A, (const unsigned short *)wq, c, M, N, K, ldc, alpha, beta, m0, tw * 256 + idx * 192, wq, wsc);
 }
 
 // Tile choice by a small cost model fitted to measurements on one MI355X (q4, K = 2048..8192, 24..2048
@@ -746,30 +931,46 @@ int launch_gemm_i8(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, Prepared
     return AIONHIP_OK;
 }
 
-int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *cw, size_t m, const float *a, size_t lda, float *c, size_t ldc, float alpha, float beta) {
-    aionhip_weight *w = const_cast<aionhip_weight *>(cw);   // the bf16 copy is a cache on the weight
+// The context's bf16 copy of a weight (tiled layout), built on first use: see aionhip_set_bf16_weight_copies.
+static int bf16_copy_of(aionhip_ctx *ctx, const aionhip_weight *w, const unsigned short **out) {
+    auto it = ctx->bf16_copies.find(w);
+    if (it != ctx->bf16_copies.end()) {
+        *out = (const unsigned short *)it->second.first;
+        return AIONHIP_OK;
+    }
+    if (ctx->capturing)
+        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "the bf16 copy of a weight cannot be built while a program is being recorded: run the steps once before recording");
+    const size_t N = w->n, K = w->k, rows_padded = (N + 15) & ~(size_t)15, bytes = rows_padded * K * 2;
+    void *p = nullptr;
+    int rc = dev_malloc(ctx, &p, bytes, "the bf16 copy of a weight");
+    if (rc) return rc;
+    const size_t threads = rows_padded * (K / 8);
+    const unsigned grid = (unsigned)((threads + 255) / 256);
+    if (w->dtype == AIONHIP_Q8_0) dequant_bf16_kernel<AIONHIP_Q8_0><<<dim3(grid), dim3(256), 0, ctx->stream>>>(w->qs, w->sc, (unsigned short *)p, N, K);
+    else dequant_bf16_kernel<AIONHIP_Q4_0><<<dim3(grid), dim3(256), 0, ctx->stream>>>(w->qs, w->sc, (unsigned short *)p, N, K);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        (void)hipFree(p);
+        return set_err(ctx, AIONHIP_EXECUTION_FAILED, "launch dequant_bf16: %s", hipGetErrorString(e));
+    }
+    ctx->bf16_copies[w] = {p, bytes};
+    ctx->bf16_copy_bytes += bytes;
+    *out = (const unsigned short *)p;
+    return AIONHIP_OK;
+}
+
+int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, const float *a, size_t lda, float *c, size_t ldc, float alpha, float beta) {
     const size_t N = w->n, K = w->k;
     if ((((uintptr_t)a) & 3) != 0) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "gemm: A must be 4-byte aligned");
-    if (!w->bf16) {
-        // The bf16 copy is built on first use and kept until aionhip_weight_drop_bf16 / aionhip_weight_free: N*K*2 bytes
-        // (about 4x a q4 weight). Not while a program is being recorded (it allocates), and the field is set only once
-        // the conversion launch has been accepted. A weight shared by several contexts must see its first bf16 call from
-        // one of them alone.
-        if (ctx->capturing)
-            return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "the bf16 copy of a weight cannot be built while a program is being recorded: run the steps once before recording");
-        void *p = nullptr;
-        const size_t rows_padded = (N + 15) & ~(size_t)15;
-        HIP_TRY(ctx, hipMalloc(&p, rows_padded * K * 2));
-        const size_t threads = rows_padded * (K / 8);
-        const unsigned grid = (unsigned)((threads + 255) / 256);
-        if (w->dtype == AIONHIP_Q8_0) dequant_bf16_kernel<AIONHIP_Q8_0><<<dim3(grid), dim3(256), 0, ctx->stream>>>(w->qs, w->sc, (unsigned short *)p, N, K);
-        else dequant_bf16_kernel<AIONHIP_Q4_0><<<dim3(grid), dim3(256), 0, ctx->stream>>>(w->qs, w->sc, (unsigned short *)p, N, K);
-        const hipError_t e = hipGetLastError();
-        if (e != hipSuccess) {
-            (void)hipFree(p);
-            return set_err(ctx, AIONHIP_EXECUTION_FAILED, "launch dequant_bf16: %s", hipGetErrorString(e));
-        }
-        w->bf16 = (unsigned short *)p;
+    // Two forms of the weight operand. With copies (the default) the kernel streams a bf16 copy of the weight that this
+    // context builds on the weight's first bf16 call and keeps: 2 bytes per weight resident, and the faster kernel
+    // (M = 2048 x N = 14336 x K = 4096, q4: 197 us). Without, the same kernel converts the quant blocks while it stages
+    // them: nothing resident, nothing allocated, 264 us - the conversion's vector instructions, the LDS writes and the
+    // scattered 16-byte requests all land in a loop that is already bound by instruction issue and power.
+    const unsigned short *wcopy = nullptr;
+    if (ctx->bf16_copies_on) {
+        const int rc0 = bf16_copy_of(ctx, w, &wcopy);
+        if (rc0) return rc0;
     }
     const size_t m_padded = (m + 15) & ~(size_t)15;
     int rc = ensure_scratch2(ctx, m_padded * K * 2);
@@ -832,30 +1033,44 @@ int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *cw, size_t m, const
         const int tm = wm == 4 ? tm4 : (wm == 2 ? tm2 : tm1);
         // 64-row tiles that still leave CUs idle (few tokens against a narrow weight): 128 columns instead of 256, twice the workgroups
         const bool half_cols = wm == 1 && (long)tm1 * tn < cus;
-        static bool attr[4] = {false, false, false, false};
-        auto launch = [&](auto kernel, int idx, int lds, const unsigned short *wp, float *cp, size_t ncols, int tiles) -> int {
-            if (!attr[idx]) {
+        // kernel variant: 0 = the bf16 copy, 1 = q4 blocks converted while staged, 2 = q8 blocks
+        const int var = wcopy ? 0 : (w->dtype == AIONHIP_Q8_0 ? 2 : 1);
+        const uint8_t *wp = wcopy ? (const uint8_t *)wcopy : w->qs;
+        static bool attr[3][5] = {};
+        auto launch = [&](auto kernel, int shape, int lds, int tiles) -> int {
+            if (!attr[var][shape]) {
                 HIP_TRY(ctx, hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-                attr[idx] = true;
+                attr[var][shape] = true;
             }
-            launch_k(ctx, kernel, dim3((unsigned)((tiles + 7) / 8 * 8)), dim3(256), lds, abf, wp, cp, (int)m, (int)ncols, (int)K, ldc, alpha, beta, tm, tiles);
+            launch_k(ctx, kernel, dim3((unsigned)((tiles + 7) / 8 * 8)), dim3(256), lds, abf, wp, w->sc, c, (int)m, (int)N, (int)K, ldc, alpha, beta, tm, tiles);
             return AIONHIP_OK;
+        };
+        auto launch_mixed = [&](auto kernel, int lds, int tiles) -> int {
+            if (!attr[var][4]) {
+                HIP_TRY(ctx, hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+                attr[var][4] = true;
+            }
+            launch_k(ctx, kernel, dim3((unsigned)((tiles + 7) / 8 * 8)), dim3(256), lds, abf, wp, w->sc, c, (int)m, (int)N, (int)K, ldc, alpha, beta,
+                     tm, tn_wide, tn_narrow);
+            return AIONHIP_OK;
+        };
+        auto with_variant = [&](auto f) -> int {
+            if (var == 0) return f(std::integral_constant<int, 0>{});
+            if (var == 1) return f(std::integral_constant<int, AIONHIP_Q4_0>{});
+            return f(std::integral_constant<int, AIONHIP_Q8_0>{});
         };
         if (tn_narrow) {
             // both kinds of tiles in one launch, interleaved (gemm_bf16_mixed_kernel)
-            static bool attr_mixed = false;
-            constexpr int lds = 4 * (256 + 256) * G2_ROW;
-            if (!attr_mixed) {
-                HIP_TRY(ctx, hipFuncSetAttribute((const void *)gemm_bf16_mixed_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-                attr_mixed = true;
-            }
-            const int tiles = tm * (tn_wide + tn_narrow);
-            launch_k(ctx, gemm_bf16_mixed_kernel<4>, dim3((unsigned)((tiles + 7) / 8 * 8)), dim3(256), lds, abf, w->bf16, c, (int)m, (int)N, (int)K, ldc, alpha, beta,
-                     tm, tn_wide, tn_narrow);
-        } else if (wm == 4) rc = launch(gemm_bf16_wide_kernel<4, 4, 4>, 0, 4 * (256 + 256) * G2_ROW, w->bf16, c, N, tm * tn_wide);
-        else if (wm == 2) rc = launch(gemm_bf16_wide_kernel<2, 4, 4>, 1, 4 * (128 + 256) * G2_ROW, w->bf16, c, N, tm * tn_wide);
-        else if (half_cols) rc = launch(gemm_bf16_wide_kernel<1, 4, 2>, 3, 4 * (64 + 128) * G2_ROW, w->bf16, c, N, tm * (int)((N + 127) / 128));
-        else rc = launch(gemm_bf16_wide_kernel<1, 4, 4>, 2, 4 * (64 + 256) * G2_ROW, w->bf16, c, N, tm * tn_wide);
+            rc = with_variant([&](auto b) { return launch_mixed(gemm_bf16_mixed_kernel<4, decltype(b)::value>, 4 * (256 + 256) * G2_ROW, tm * (tn_wide + tn_narrow)); });
+        } else if (wm == 4) {
+            rc = with_variant([&](auto b) { return launch(gemm_bf16_wide_kernel<4, 4, 4, decltype(b)::value>, 0, 4 * (256 + 256) * G2_ROW, tm * tn_wide); });
+        } else if (wm == 2) {
+            rc = with_variant([&](auto b) { return launch(gemm_bf16_wide_kernel<2, 4, 4, decltype(b)::value>, 1, 4 * (128 + 256) * G2_ROW, tm * tn_wide); });
+        } else if (half_cols) {
+            rc = with_variant([&](auto b) { return launch(gemm_bf16_wide_kernel<1, 4, 2, decltype(b)::value>, 3, 4 * (64 + 128) * G2_ROW, tm * (int)((N + 127) / 128)); });
+        } else {
+            rc = with_variant([&](auto b) { return launch(gemm_bf16_wide_kernel<1, 4, 4, decltype(b)::value>, 2, 4 * (64 + 256) * G2_ROW, tm * tn_wide); });
+        }
         if (rc) return rc;
     }
     LAUNCH_CHECK(ctx, "gemm_bf16");

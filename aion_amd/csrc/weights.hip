@@ -179,19 +179,40 @@ int aionhip_weight_upload(aionhip_ctx *ctx, int dtype, int layout, size_t n, siz
     return rc;
 }
 
-void aionhip_weight_free(aionhip_ctx *ctx, aionhip_weight *w) {
-    if (!w) return;
-    if (ctx) (void)hipStreamSynchronize(ctx->stream);
-    if (w->qs) (void)hipFree(w->qs);
-    if (w->bf16) (void)hipFree(w->bf16);
-    delete w;
+// releases this context's bf16 copy of the weight, if it holds one (the caller has waited for the stream)
+static void drop_bf16_copy(aionhip_ctx *ctx, const aionhip_weight *w) {
+    auto it = ctx->bf16_copies.find(w);
+    if (it == ctx->bf16_copies.end()) return;
+    (void)hipFree(it->second.first);
+    ctx->bf16_copy_bytes -= it->second.second;
+    ctx->bf16_copies.erase(it);
 }
 
 void aionhip_weight_drop_bf16(aionhip_ctx *ctx, aionhip_weight *w) {
-    if (!w || !w->bf16) return;
-    if (ctx) (void)hipStreamSynchronize(ctx->stream);      // launches that read the copy may still be queued
-    (void)hipFree(w->bf16);
-    w->bf16 = nullptr;
+    if (!ctx || !w || ctx->capturing || ctx->bf16_copies.find(w) == ctx->bf16_copies.end()) return;
+    (void)hipStreamSynchronize(ctx->stream);      // launches that read the copy may still be queued
+    drop_bf16_copy(ctx, w);
+}
+
+int aionhip_set_bf16_weight_copies(aionhip_ctx *ctx, int on) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    ctx->bf16_copies_on = on != 0;
+    return AIONHIP_OK;
+}
+
+int aionhip_bf16_copy_stats(aionhip_ctx *ctx, uint64_t *weights, uint64_t *bytes) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (weights) *weights = (uint64_t)ctx->bf16_copies.size();
+    if (bytes) *bytes = (uint64_t)ctx->bf16_copy_bytes;
+    return AIONHIP_OK;
+}
+
+void aionhip_weight_free(aionhip_ctx *ctx, aionhip_weight *w) {
+    if (!w) return;
+    if (ctx) (void)hipStreamSynchronize(ctx->stream);
+    if (ctx) drop_bf16_copy(ctx, w);
+    if (w->qs) (void)hipFree(w->qs);
+    delete w;
 }
 
 size_t aionhip_weight_packed_bytes(const aionhip_weight *w) {

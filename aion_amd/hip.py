@@ -63,6 +63,8 @@ _SIGS = {
     "aionhip_weight_from_device": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint64, C.POINTER(C.c_void_p)]),
     "aionhip_weight_free": (None, [C.c_void_p, C.c_void_p]),
     "aionhip_weight_drop_bf16": (None, [C.c_void_p, C.c_void_p]),
+    "aionhip_set_bf16_weight_copies": (C.c_int, [C.c_void_p, C.c_int]),
+    "aionhip_bf16_copy_stats": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "aionhip_weight_packed_bytes": (C.c_size_t, [C.c_void_p]),
     "aionhip_weight_device_bytes": (C.c_size_t, [C.c_void_p]),
     "aionhip_weight_download": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),

@@ -190,17 +190,23 @@ int aionhip_step_gate_matmul(aionhip_ctx *ctx, const aionhip_weight *b, size_t r
                              aionhip_handle c, size_t ldc, float alpha, float beta);
 
 /* How m > 8 rows are multiplied. EXACT_I8 (default): int8 activations, integer MFMA, per-block
- * f32 scaling - the same numbers as the decode path. BF16_MFMA: weights dequantized to bf16,
- * activations rounded to bf16, f32 accumulation - judged at 1e-2 instead of 2e-3; used where it is expected to
+ * f32 scaling - the same numbers as the decode path. BF16_MFMA: weights dequantized to bf16 (a copy the context
+ * keeps, or while the kernel stages them: aionhip_set_bf16_weight_copies), activations rounded to bf16, f32
+ * accumulation - judged at 1e-2 instead of 2e-3; used where it is expected to
  * be the faster kernel (from a few hundred rows on; below that the exact kernel runs, which is then both faster
  * and exact). BF16_MFMA_ALWAYS: the bf16 kernel for every m > 8, whatever the shape. */
 typedef enum aionhip_gemm_mode { AIONHIP_GEMM_EXACT_I8 = 0, AIONHIP_GEMM_BF16_MFMA = 1, AIONHIP_GEMM_BF16_MFMA_ALWAYS = 2 } aionhip_gemm_mode;
 int aionhip_set_gemm_mode(aionhip_ctx *ctx, int mode);
-/* The bf16 kernel keeps a bf16 copy of every weight it has multiplied (n rounded up to 16, times k * 2 bytes - about four times a q4_0 weight -
- * built on the first such call, never while a program is being recorded, released by aionhip_weight_free). This releases
- * the copy of one weight early (it is rebuilt on the next bf16 call); aion's derived-weight reclamation
- * (storage/derived.zig:1-17) is the counterpart. Waits for the context's stream. */
-void aionhip_weight_drop_bf16(aionhip_ctx *ctx, aionhip_weight *w);
+/* The weight operand of the bf16 kernel. on (default): the context keeps a bf16 copy of every weight it has multiplied in
+ * bf16 mode (n rounded up to 16, times k * 2 bytes - about four times a q4_0 weight), built on the weight's first such call,
+ * never while a program is being recorded, owned by the context (no other context sees it) and released by
+ * aionhip_weight_drop_bf16, aionhip_weight_free through the same context, or aionhip_destroy; aion's derived weights
+ * (storage/derived.zig:1-17) are the counterpart. off: no copies - the kernel converts the quant blocks while it stages
+ * them, as aion's GPU GEMM does (backend/gpu/kernels/matmul_q8_mx16.wgsl); nothing resident and nothing allocated, at
+ * about three quarters of the speed (measured: 264 against 197 us for 2048 x 14336 x 4096). Same results to the bit. */
+int aionhip_set_bf16_weight_copies(aionhip_ctx *ctx, int on);
+void aionhip_weight_drop_bf16(aionhip_ctx *ctx, aionhip_weight *w);       /* waits for the context's stream */
+int aionhip_bf16_copy_stats(aionhip_ctx *ctx, uint64_t *weights, uint64_t *bytes);
 /* Name of the kernel the last matmul/attention step launched (the reference's tests assert
  * which kernel ran after a parity check, backend/gpu/test_gpu_backend.zig:1116-1162). */
 const char *aionhip_last_kernel(aionhip_ctx *ctx);

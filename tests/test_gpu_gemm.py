@@ -186,6 +186,39 @@ def test_exact_gemm_k_slices(gpu, orc, dtype, layout):
     w.free(); w2.free()
 
 
+@pytest.mark.parametrize("dtype,layout", CASES)
+@pytest.mark.parametrize("m,n,k", [(2048, 14336, 4096), (512, 4096, 4096), (300, 520, 1056), (1300, 11008, 4096), (70, 200, 96)])
+def test_bf16_gemm_without_weight_copies_gives_the_same_bits(gpu, orc, dtype, layout, m, n, k):
+    """The bf16 kernel's two weight operands: the bf16 copy the context keeps of a weight, and the weight's quant blocks
+    converted while the kernel stages them (aionhip_set_bf16_weight_copies(0): nothing resident, nothing allocated).
+    Both round code * scale to bf16 once and multiply in the same order: the same bits, every tile shape (256 x 256 and
+    256 x 192 mixed, 128-row, 64-row and 64 x 128 tiles, ragged edges, a K that is not a multiple of four blocks)."""
+    say("bf16 without copies", dtype, layout, m, n, k)
+    gpu.set_gemm_mode(be.GEMM_BF16_MFMA_ALWAYS)
+    try:
+        blocks, w = make_weight(gpu, dtype, layout, n, k, seed=m + n)
+        a = bf16_round(np.random.default_rng(k).standard_normal((m, k)).astype(np.float32))
+        copies0 = gpu.bf16_copy_stats()
+        with_copy = gpu.matmul(w, a)
+        assert gpu.last_kernel() == "gemm_bf16" and gpu.bf16_copy_stats()[0] == copies0[0] + 1
+        w.drop_bf16()
+        assert gpu.bf16_copy_stats() == copies0
+        gpu.set_bf16_weight_copies(False)
+        streamed = gpu.matmul(w, a)
+        assert gpu.last_kernel() == "gemm_bf16" and gpu.bf16_copy_stats() == copies0      # no copy was built
+        assert np.array_equal(with_copy.view(np.uint32), streamed.view(np.uint32))
+        rows = np.unique(np.array([0, m // 3, m - 1]))
+        f32a = orc.matmul_q_f32a(dtype, layout == be.ROWS_NK, np.ascontiguousarray(a[rows]), blocks, n, threads=8)
+        assert rms_err(streamed[rows], f32a) < 1e-2
+        c0 = np.random.default_rng(2).standard_normal((m, n)).astype(np.float32)
+        got2 = gpu.matmul(w, a, alpha=0.5, beta=2.0, c=c0)
+        assert np.allclose(got2, 0.5 * streamed + 2.0 * c0, rtol=1e-5, atol=1e-5)
+        w.free()
+    finally:
+        gpu.set_bf16_weight_copies(True)
+        gpu.set_gemm_mode(be.GEMM_EXACT_I8)
+
+
 @pytest.mark.parametrize("ldc,c_offset", [(520, 0), (524, 0), (521, 0), (528, 3)])
 def test_bf16_gemm_alpha_beta_and_output_strides(gpu, orc, ldc, c_offset):
     """The bf16 kernel's epilogue: 16-byte stores where the output rows allow them (row pitch and base 16-byte aligned),
