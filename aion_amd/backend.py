@@ -367,6 +367,11 @@ class HipBackend:
         self._check(self._lib.aionhip_step_append_f16(self._ctx, cache.handle, src.handle, write_index.handle, b, s, t_cap, row_elems,
                                                       1 if rolling else 0))
 
+    def step_sequence_append(self, dtype, cache, new_kv, end_index, b, s, t_cap, row_elems, rolling=False):
+        """StepSequenceAppend with rows and cache of one element type, F16 or F32 (cpu/exec/sequence_append.zig:12-104)."""
+        self._check(self._lib.aionhip_step_sequence_append(self._ctx, dtype, cache.handle, new_kv.handle, end_index.handle, b, s, t_cap,
+                                                           row_elems, 1 if rolling else 0))
+
     def cache_grow(self, dst, src, outer, old_run_bytes, new_run_bytes):
         """dst [outer, new_run_bytes] <- the runs of src [outer, old_run_bytes], zero elsewhere (storage/manager/grow.zig:37-78)."""
         self._check(self._lib.aionhip_cache_grow(self._ctx, dst.handle, src.handle, outer, old_run_bytes, new_run_bytes))

@@ -289,6 +289,19 @@ __global__ void append_f16_kernel(__half *__restrict__ cache, const float *__res
     if ((size_t)t >= t_cap) return;               // never write outside the cache
     cache[(b * t_cap + (size_t)t) * row_elems + e] = __float2half_rn(src[i]);
 }
+// StepSequenceAppend as the reference states it (cpu/exec/sequence_append.zig:12-104): rows and cache of one element type
+template <typename T>
+__global__ void append_same_kernel(T *__restrict__ cache, const T *__restrict__ src, const int *__restrict__ write_index,
+                                   size_t s_len, size_t t_cap, size_t row_elems, size_t total, int rolling) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const size_t e = i % row_elems, s = (i / row_elems) % s_len, b = i / (row_elems * s_len);
+    long t = (long)write_index[b] + (long)s;
+    if (t < 0) return;
+    if (rolling) t %= (long)t_cap;
+    if ((size_t)t >= t_cap) return;
+    cache[(b * t_cap + (size_t)t) * row_elems + e] = src[i];
+}
 
 // Growth of a sequence cache along its time axis (storage/manager/grow.zig:37-78): the wider backing is zero
 // except for the `outer` preserved runs, each copied to the start of its wider slot. One pass over the new
@@ -578,6 +591,24 @@ int aionhip_step_append_f16(aionhip_ctx *ctx, aionhip_handle cache, aionhip_hand
     append_f16_kernel<<<dim3(grid_for(total, 256)), dim3(256), 0, ctx->stream>>>(dp<__half>(cache), dp<const float>(src_f32), dp<const int>(write_index),
                                                                                  s, t_cap, row_elems, total, rolling);
     LAUNCH_CHECK(ctx, "append_f16");
+    return AIONHIP_OK;
+}
+
+int aionhip_step_sequence_append(aionhip_ctx *ctx, int dtype, aionhip_handle cache, aionhip_handle new_kv, aionhip_handle end_index, size_t b,
+                                 size_t s, size_t t_cap, size_t row_elems, int rolling) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (!cache || !new_kv || !end_index) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "sequence_append: null operand");
+    if (dtype != AIONHIP_F16 && dtype != AIONHIP_F32) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "sequence_append: caches hold f16 or f32, not dtype %d", dtype);
+    if (s > t_cap) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "sequence_append: %zu new tokens exceed the cache capacity %zu", s, t_cap);
+    const size_t total = b * s * row_elems;
+    if (!total) return AIONHIP_OK;
+    if (dtype == AIONHIP_F16)
+        append_same_kernel<unsigned short><<<dim3(grid_for(total, 256)), dim3(256), 0, ctx->stream>>>(
+            dp<unsigned short>(cache), dp<const unsigned short>(new_kv), dp<const int>(end_index), s, t_cap, row_elems, total, rolling);
+    else
+        append_same_kernel<unsigned><<<dim3(grid_for(total, 256)), dim3(256), 0, ctx->stream>>>(
+            dp<unsigned>(cache), dp<const unsigned>(new_kv), dp<const int>(end_index), s, t_cap, row_elems, total, rolling);
+    LAUNCH_CHECK(ctx, "sequence_append");
     return AIONHIP_OK;
 }
 

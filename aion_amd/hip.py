@@ -106,6 +106,7 @@ _SIGS = {
     "aionhip_step_gate_gelu": (C.c_int, [C.c_void_p] + [C.c_uint64] * 3 + [C.c_size_t]),
     "aionhip_step_gather_rows": (C.c_int, [C.c_void_p, C.c_int] + [C.c_uint64] * 3 + [C.c_size_t] * 3),
     "aionhip_step_append_f16": (C.c_int, [C.c_void_p] + [C.c_uint64] * 3 + [C.c_size_t] * 4 + [C.c_int]),
+    "aionhip_step_sequence_append": (C.c_int, [C.c_void_p, C.c_int] + [C.c_uint64] * 3 + [C.c_size_t] * 4 + [C.c_int]),
     "aionhip_step_cast_f32_f16": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64, C.c_size_t]),
     "aionhip_step_headnorm_rope_append": (C.c_int, [C.c_void_p] + [C.c_uint64] * 10 + [C.c_float] + [C.c_uint64] * 4 + [C.c_size_t] * 6 +
                                           [C.c_float] * 3 + [C.c_int]),

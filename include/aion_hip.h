@@ -287,6 +287,13 @@ int aionhip_step_gather_rows(aionhip_ctx *ctx, int table_dtype, aionhip_handle o
 int aionhip_step_append_f16(aionhip_ctx *ctx, aionhip_handle cache, aionhip_handle src_f32, aionhip_handle write_index,
                             size_t b, size_t s, size_t t_cap, size_t row_elems, int rolling);
 int aionhip_step_cast_f32_f16(aionhip_ctx *ctx, aionhip_handle out_f16, aionhip_handle x_f32, size_t n);
+/* StepSequenceAppend as the step itself (runtime/executable.zig:193-206, cpu/exec/sequence_append.zig:12-104): cache
+ * [B,T,H,D] and new_kv [B,S,H,D] of the same element type `dtype` (AIONHIP_F16 or AIONHIP_F32), end_index i32 [B] on the
+ * device; rows go to token index end_index[b] .. +S (rolling = 1: to row t % T). A row that would fall outside a linear
+ * cache is not written (the reference rejects the step on the host before any write; capacity is settled before the
+ * program runs, api/loaded_model.zig:791-827). */
+int aionhip_step_sequence_append(aionhip_ctx *ctx, int dtype, aionhip_handle cache, aionhip_handle new_kv, aionhip_handle end_index,
+                                 size_t b, size_t s, size_t t_cap, size_t row_elems, int rolling);
 /* Growth of a sequence cache along its time axis with the data kept on the device
  * (storage/manager/grow.zig:37-78 growAxisOnDevice, driven by api/loaded_model.zig:791-827 and
  * storage/manager/store_view.zig:104-124): dst is the new backing [outer, new_run_bytes], src the old one

@@ -137,6 +137,30 @@ def test_kv_append_into_a_rolling_cache(gpu, orc):
     cb.free()
 
 
+@pytest.mark.parametrize("np_dtype,dtype", [(np.float16, "F16"), (np.float32, "F32")])
+def test_sequence_append_step_with_rows_of_the_cache_type(gpu, orc, np_dtype, dtype):
+    """The step as the reference states it: rows already of the cache's element type, linear and rolling."""
+    rng = np.random.default_rng(15)
+    B, T, H, D = 2, 12, 2, 32
+    for rolling in (False, True):
+        cache = np.zeros((B, T, H, D), np_dtype)
+        cb = gpu.upload(cache)
+        t0 = np.array([0, 3 if not rolling else 30], np.int32)
+        for n in (4, 1, 3) if not rolling else (5, 9, 1, 12, 7):
+            src = rng.standard_normal((B, n, H, D)).astype(np_dtype)
+            sb, wb = gpu.upload(src), gpu.upload(t0)
+            gpu.step_sequence_append(getattr(be, dtype), cb, sb, wb, B, n, T, H * D, rolling=rolling)
+            cache = orc.sequence_append(cache, src, t0, rolling=rolling)
+            assert np.array_equal(gpu.download(cb, np_dtype, cache.shape), cache)
+            t0 = t0 + n
+            sb.free(); wb.free()
+        cb.free()
+    z = gpu.zeros(64)
+    with pytest.raises(be.AionHipError):
+        gpu.step_sequence_append(be.Q8_0, z, z, z, 1, 1, 1, 1)          # caches hold f16 or f32
+    z.free()
+
+
 def test_rope_append_equals_the_separate_steps(gpu, orc):
     rng = np.random.default_rng(6)
     B, S, T, Hq, Hkv, D = 2, 3, 12, 8, 1, 64
