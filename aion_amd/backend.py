@@ -108,6 +108,13 @@ class HipBackend:
     def last_kernel(self):
         return self._lib.aionhip_last_kernel(self._ctx).decode()
 
+    def last_launch(self):
+        """The last launch a step made: {"kernel": instance name as a kernel trace prints it, "grid", "block", "lds"}."""
+        name = C.create_string_buffer(512)
+        grid, block, lds = (C.c_uint * 3)(), (C.c_uint * 3)(), C.c_size_t()
+        self._check(self._lib.aionhip_last_launch(self._ctx, name, len(name), grid, block, C.byref(lds)))
+        return {"kernel": name.value.decode(), "grid": list(grid), "block": list(block), "lds": int(lds.value)}
+
     def set_gemm_mode(self, mode):
         self._check(self._lib.aionhip_set_gemm_mode(self._ctx, mode))
 

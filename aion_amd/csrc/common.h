@@ -84,6 +84,9 @@ struct aionhip_ctx {
     // per-launch timing, off by default
     bool profiling = false;
     const char *prof_name = nullptr;   // set by ProfScope: launches made through launch_k are timed under it
+    // the last launch made through launch_k: host stub, grid and block (reports match them to a kernel trace)
+    const void *last_fn = nullptr;
+    unsigned last_grid[3] = {0, 0, 0}, last_block[3] = {0, 0, 0}, last_lds = 0;
     std::vector<ProfRecord> prof;
     std::vector<hipEvent_t> event_pool;
 };
@@ -108,6 +111,10 @@ void prof_open(aionhip_ctx *ctx, hipEvent_t *start, hipEvent_t *stop);
 // elapsed time is the kernel's duration with no barrier or launch gap in it).
 template <typename... KArgs, typename... Args>
 inline void launch_k(aionhip_ctx *ctx, void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t lds, Args... args) {
+    ctx->last_fn = (const void *)kernel;
+    ctx->last_grid[0] = grid.x, ctx->last_grid[1] = grid.y, ctx->last_grid[2] = grid.z;
+    ctx->last_block[0] = block.x, ctx->last_block[1] = block.y, ctx->last_block[2] = block.z;
+    ctx->last_lds = (unsigned)lds;
     if (ctx->profiling && ctx->prof_name) {
         hipEvent_t e0 = nullptr, e1 = nullptr;
         prof_open(ctx, &e0, &e1);

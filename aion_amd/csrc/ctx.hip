@@ -2,6 +2,9 @@
 // Backend / Session / DeviceMemory vtables (backend/backend.zig:24-107,
 // runtime/device_memory.zig:36-108).
 #include "common.h"
+
+#include <cxxabi.h>
+#include <string>
 #include <algorithm>
 
 #include <cstring>
@@ -227,6 +230,38 @@ int aionhip_sync(aionhip_ctx *ctx) {
 
 const char *aionhip_last_error(aionhip_ctx *ctx) { return ctx ? ctx->err.c_str() : "no context"; }
 const char *aionhip_last_kernel(aionhip_ctx *ctx) { return ctx ? ctx->last_kernel : ""; }
+
+int aionhip_last_launch(aionhip_ctx *ctx, char *instance, size_t instance_len, unsigned grid[3], unsigned block[3], size_t *lds_bytes) {
+    if (!ctx) return AIONHIP_INVALID_ARGUMENT;
+    if (!ctx->last_fn) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "last_launch: no kernel has been launched on this context");
+    if (instance && instance_len) {
+        // the device function's name as a kernel trace prints it: demangled, without the parameter list
+        const char *mangled = hipKernelNameRefByPtr(ctx->last_fn, ctx->stream);
+        (void)hipGetLastError();
+        int status = -1;
+        char *plain = mangled ? abi::__cxa_demangle(mangled, nullptr, nullptr, &status) : nullptr;
+        std::string name = status == 0 && plain ? plain : (mangled ? mangled : "");
+        free(plain);
+        // cut "(args...)" of the outermost call: the last '(' at template depth 0
+        int depth = 0;
+        size_t cut = std::string::npos;
+        for (size_t i = 0; i < name.size(); ++i) {
+            const char ch = name[i];
+            if (ch == '<') ++depth;
+            else if (ch == '>') --depth;
+            else if (ch == '(' && depth == 0 && name.compare(i, 21, "(anonymous namespace)") != 0) { cut = i; break; }
+        }
+        if (cut != std::string::npos) name.resize(cut);
+        if (name.rfind("void ", 0) == 0) name.erase(0, 5);
+        snprintf(instance, instance_len, "%s", name.c_str());
+    }
+    for (int i = 0; i < 3; ++i) {
+        if (grid) grid[i] = ctx->last_grid[i];
+        if (block) block[i] = ctx->last_block[i];
+    }
+    if (lds_bytes) *lds_bytes = ctx->last_lds;
+    return AIONHIP_OK;
+}
 void *aionhip_stream(aionhip_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
 
 int aionhip_set_gemm_mode(aionhip_ctx *ctx, int mode) {

@@ -46,6 +46,7 @@ _SIGS = {
     "aionhip_sync": (C.c_int, [C.c_void_p]),
     "aionhip_last_error": (C.c_char_p, [C.c_void_p]),
     "aionhip_last_kernel": (C.c_char_p, [C.c_void_p]),
+    "aionhip_last_launch": (C.c_int, [C.c_void_p, C.c_char_p, C.c_size_t, C.POINTER(C.c_uint), C.POINTER(C.c_uint), C.POINTER(C.c_size_t)]),
     "aionhip_name": (C.c_char_p, []),
     "aionhip_stream": (C.c_void_p, [C.c_void_p]),
     "aionhip_device_info": (C.c_int, [C.c_void_p, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_uint64), C.c_char_p, C.c_size_t]),

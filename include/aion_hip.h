@@ -210,6 +210,11 @@ int aionhip_bf16_copy_stats(aionhip_ctx *ctx, uint64_t *weights, uint64_t *bytes
 /* Name of the kernel the last matmul/attention step launched (the reference's tests assert
  * which kernel ran after a parity check, backend/gpu/test_gpu_backend.zig:1116-1162). */
 const char *aionhip_last_kernel(aionhip_ctx *ctx);
+/* The last launch a matmul or fused step made, for reports that are matched against a kernel trace: the kernel instance's
+ * name as a trace prints it (demangled, template arguments included, no parameter list), its grid in workgroups, its
+ * workgroup size and its dynamic LDS bytes. Any pointer may be NULL. aion's counterpart is the WebGPU backend's per-dispatch
+ * labels (backend/gpu/timestamp_profile.zig). */
+int aionhip_last_launch(aionhip_ctx *ctx, char *instance, size_t instance_len, unsigned grid[3], unsigned block[3], size_t *lds_bytes);
 
 /* ---- attention step: StepAttention (runtime/executable.zig:102-115), graph.Op.Attention
  *      (graph/graph.zig:365-393), executor cpu/exec/attention.zig:1444-1608 ------------------

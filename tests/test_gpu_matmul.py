@@ -211,6 +211,21 @@ def test_single_row_long_k(gpu, orc, dtype, layout, n, k, kernel):
     w.free()
 
 
+def test_last_launch_names_the_kernel_instance_and_its_grid(gpu, orc):
+    """What reports print beside a figure so that it can be matched to a kernel trace: the instance's name as a trace prints
+    it (template arguments included, no parameter list), the grid in workgroups, the workgroup size, the dynamic LDS bytes."""
+    n, k = 4096, 4096
+    blocks, w = make_weight(gpu, orc, be.Q4_0, be.KMAJOR_KN, n, k, seed=3)
+    gpu.matmul(w, np.ones((1, k), np.float32))
+    ll = gpu.last_launch()
+    say("last_launch", ll)
+    assert gpu.last_kernel() == "gemv_q4_fused"
+    assert "gemv_fused_kernel<" in ll["kernel"] and ll["kernel"].endswith(">") and "(" not in ll["kernel"].replace("(anonymous namespace)", "")
+    assert ll["block"] == [1024, 1, 1] and ll["grid"][1:] == [1, 1] and 1 <= ll["grid"][0] <= n // 8
+    assert ll["lds"] >= k + k // 32 * 8
+    w.free()
+
+
 def test_single_row_q4_eight_alternating_slices(gpu, orc):
     # q4 at K = 65536: eight slices over a row pitch of 32 KiB, taken in alternating order
     n, k = 24, 65536
