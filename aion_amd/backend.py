@@ -265,6 +265,10 @@ class HipBackend:
         failed = C.c_int(0)
         self._check(self._lib.aionhip_decoder_stack_status(self._ctx, stack, C.byref(failed)))
 
+    def decoder_stack_set_stamps(self, stack, buf):
+        """Time stamps of the next launches into `buf` (2 x layers x 10 counters of 8 bytes, 100 MHz), None switches them off."""
+        self._check(self._lib.aionhip_decoder_stack_set_stamps(self._ctx, stack, buf.handle if buf is not None else 0))
+
     def decoder_stack_set_poll_budget(self, stack, milliseconds):
         self._check(self._lib.aionhip_decoder_stack_set_poll_budget(self._ctx, stack, float(milliseconds)))
 

@@ -44,7 +44,7 @@ CAL_ELEMS = 1 << 26   # the counter-calibration cast: 256 MiB read, 128 MiB writ
 # counter runs of this same command scaled by what the same counters read for the calibration cast
 # (factors 1.9998 and 1.0000); the summary with the commands is profiles/gemv_q4_decode_bench_kernel_stats_and_traffic.md.
 # Counters cannot be read from inside the process, so the figures are carried here.
-MEASURED_TRAFFIC = {(4096, 4096): 9.655e6, (14336, 4096): 33.299e6, (4096, 14336): 33.879e6, (262144, 2048): 303.159e6}
+MEASURED_TRAFFIC = {(4096, 4096): 9.656e6, (14336, 4096): 33.300e6, (4096, 14336): 33.886e6, (262144, 2048): 303.150e6}
 
 
 SETTLE_MS = 80.0
@@ -93,7 +93,7 @@ def main():
     ap.add_argument("--sweep", action="store_true", help="(kept for compatibility: the sweep is part of the default run)")
     ap.add_argument("--headline-only", action="store_true", help="skip the secondary metrics (prefill GEMM, decode, sweep)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--extras", default="", help="comma list of gemm,attention,decoder")
+    ap.add_argument("--extras", default="", help="comma list of gemm,attention,decoder,decode_stack,package,package_bench_shape")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU (aion runs one program on one device, and no multi-GPU figure is asked for); "
@@ -264,6 +264,8 @@ def main():
             out["extras"]["attention"] = run_attention(gpu, be)
         if "decoder" in extras:
             out["extras"]["decoder"] = run_decoder(gpu, be, with_cpu=not args.no_cpu)
+        if "decode_stack" in extras or "decode_stack_only" in extras:
+            out["extras"]["decode_stack"] = run_decode_stack(gpu, be, compare="decode_stack" in extras)
         if "decoder_eager" in extras:
             out["extras"]["decoder_eager"] = run_decoder_eager(gpu, be)
         if "package" in extras:
@@ -339,6 +341,22 @@ def run_gemm_headline(gpu, be):
                     "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_PEAK[peak], "unit": "TFLOP/s",
                                  "frac": round(tf / MFMA_PEAK[peak], 4), "traffic": None, "peak_named": "dense " + peak + " MFMA",
                                  "counts": "every launch of the call (the sum of their durations)"}}
+    # the bf16 kernel's second weight form: no bf16 copy, the quant blocks are converted while they are staged (same bits out)
+    gpu.set_gemm_mode(be.GEMM_BF16_MFMA_ALWAYS)
+    gpu.set_bf16_weight_copies(False)
+    w.drop_bf16()
+    gpu.step_matmul(w, x, m, y)
+    settle(gpu, lambda i: gpu.step_matmul(w, x, m, y))
+    gpu.profile_start()
+    for _ in range(20):
+        gpu.step_matmul(w, x, m, y)
+    prof = gpu.profile_stop()
+    ms = sum(t for _, t in prof) / 20
+    res["bf16_mfma_blocks_converted_while_staged"] = {
+        "call_ms": round(ms, 4), "launches_per_call": len(prof) // 20, "TFLOPs": round(2.0 * m * n * k / (ms * 1e-3) / 1e12, 1),
+        "bf16_copy_bytes": int(gpu.bf16_copy_stats()[1]),
+        "note": "aionhip_set_bf16_weight_copies(ctx, 0): nothing resident beyond the q4 weight; slower than the copy form, which stays the default"}
+    gpu.set_bf16_weight_copies(True)
     gpu.set_gemm_mode(be.GEMM_EXACT_I8)
     x.free(); y.free(); w.free()
     return res
@@ -572,6 +590,56 @@ def run_decoder_eager(gpu, be, steps=8):
         tok = dec.decode_step_eager(tok)
     gpu.sync()
     return {"steps": steps, "eager_ms_per_token": round((time.perf_counter() - t) / steps * 1e3, 4)}
+
+
+def run_decode_stack(gpu, be, compare=True):
+    """Config 5's decode step as ONE cooperative launch for all 26 blocks (aionhip_step_decoder_stack) beside the replayed
+    program of the default path: ms per token of both, whether their 128 tokens agree, the launches of a step with their
+    durations, and the kernel's own time stamps (100 MHz counter, relative to the start of a block's attention) for two blocks."""
+    from aion_amd.decoder import Decoder, DecoderConfig, SyntheticWeights
+    cfg = DecoderConfig()
+    w = SyntheticWeights(cfg, 0)
+    prompt = np.random.default_rng(5).integers(0, cfg.vocab, 128).astype(np.int32)
+    res, toks = {}, {}
+    for mode in ((True, False) if compare else (True,)):     # (a kernel trace cannot follow the recording of a program)
+        dec = Decoder(gpu, cfg, w, one_launch=mode)
+        dec.prefill(prompt); dec.reset(); gpu.sync()
+        dec.begin_decode(dec.prefill(prompt)); gpu.sync()
+        dec.decode_run(64); gpu.sync()                                  # settle
+        dec.reset(); dec.begin_decode(dec.prefill(prompt)); gpu.sync()
+        t = time.perf_counter()
+        toks[mode] = list(dec.decode_run(128))
+        gpu.sync()
+        dt = time.perf_counter() - t
+        key = "one_launch" if mode else "replayed_program"
+        res[key] = {"decode_ms_per_token": round(dt / 128 * 1e3, 4), "decode_tokens_per_s": round(128 / dt, 1)}
+        if mode:
+            dec.reset(); dec.begin_decode(dec.prefill(prompt)); gpu.sync()
+            gpu.profile_start()
+            for _ in range(20):
+                dec._step_on_device()
+            agg = {}
+            for nm, ms in gpu.profile_stop():
+                agg.setdefault(nm, []).append(ms)
+            res[key]["launches_us"] = {nm: round(1e3 * sum(v) / len(v), 2) for nm, v in agg.items()}
+            st = gpu.zeros(2 * cfg.layers * 10 * 8)
+            gpu.decoder_stack_set_stamps(dec.stack, st)
+            dec._step_on_device(); gpu.sync()
+            gpu.decoder_stack_set_stamps(dec.stack, None)
+            v = gpu.download(st, np.int64, (2, cfg.layers, 10)).astype(np.float64) / 100.0      # microseconds
+            names_a = ["attention_start", "attention_end", "q_arrived", "attention_out_published", "o_in", "o_out", "ffn_in", "ffn_out", "down_in", "down_out"]
+            names_m = ["block_input_arrived", "qkv_published", "unused_2", "unused_3", "o_in", "o_out", "ffn_in", "ffn_out", "down_in", "down_out"]
+            for l in (3, 12):
+                t0 = v[0, l, 0]
+                res[key]["block_%d_us_since_attention_start" % l] = {
+                    "attention_workgroup": {nm: round(x - t0, 2) for nm, x in zip(names_a, v[0, l]) if x > 0},
+                    "a_matmul_workgroup": {nm: round(x - t0, 2) for nm, x in zip(names_m, v[1, l]) if x > 0}}
+            res[key]["block_period_us"] = [round(float(x), 2) for x in np.diff(v[0, :, 3])[:8]]
+            st.free()
+        dec.close()
+    if compare:
+        res["tokens_equal"] = toks[True] == toks[False]
+    return res
 
 
 def run_package(gpu, be):
