@@ -38,6 +38,10 @@ constexpr float PF_LAZY = 8.f;
 #define PF_PIPE_D 128      // head sizes from here on run the software-pipelined tile loop
 #endif
 using f32x16 = __attribute__((ext_vector_type(16))) float;
+// wait states between the last MFMA of a score tile and the hand-written vector read of its results (see unit 0 of the tile loop)
+constexpr int PF_SCORE_MFMA_PASSES = 8;                        // v_mfma_f32_32x32x16_{f16,bf16} on gfx950
+constexpr int PF_SCORE_WAIT = PF_SCORE_MFMA_PASSES + 4 + 2;    // required + margin
+static_assert(PF_SCORE_WAIT > 8 && PF_SCORE_WAIT <= 16, "two s_nop instructions cover 9..16 wait states");
 
 using v4s16 = __attribute__((ext_vector_type(4))) short;
 typedef __attribute__((address_space(3))) v4s16 lds_v4s16;
@@ -559,10 +563,13 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
         auto unit = [&](int u) __attribute__((always_inline)) {
             if (u < 8) {
                 // v_max3_f32 by hand: fmaxf on MFMA results first canonicalizes every input (one more instruction per score).
-                // The compiler does not see that this assembly reads MFMA results, so the wait states a vector read of
-                // them needs behind the last MFMA of S_t (ten for an 8-pass MFMA) are put here, once per tile; the
-                // other units follow behind these.
-                if (u == 0) asm volatile("s_nop 7\n\ts_nop 3" ::: "memory");
+                // The compiler does not see that this assembly reads MFMA results, so the wait states a vector read needs
+                // behind the last MFMA that wrote them are put here, once per tile; the other units follow behind these.
+                // gfx950: a VALU read of an XDL result needs passes + 4 wait states (12 for the 8-pass 32x32x16 MFMA);
+                // PF_SCORE_WAIT adds two of margin. s_nop n gives n + 1 wait states, at most 8 per instruction.
+                // This placement relies on the scheduling barriers that keep every MFMA of S_t ahead of unit 0, and the
+                // file's build flags (MFMA results in vector registers, kernel arguments preloaded) do not change it.
+                if (u == 0) asm volatile("s_nop %0\n\ts_nop %1" ::"n"(7), "n"(PF_SCORE_WAIT - 8 - 1) : "memory");
                 float t;
                 asm volatile("v_max3_f32 %0, %1, %2, %3" : "=v"(t) : "v"(mxp[u & 1]), "v"(sc[u >> 2][(4 * u) & 15]), "v"(sc[u >> 2][(4 * u + 1) & 15]));
                 asm volatile("v_max3_f32 %0, %1, %2, %3" : "=v"(mxp[u & 1]) : "v"(t), "v"(sc[u >> 2][(4 * u + 2) & 15]), "v"(sc[u >> 2][(4 * u + 3) & 15]));

@@ -339,9 +339,11 @@ __global__ void cache_grow_rolling_kernel(unsigned *__restrict__ dst, const unsi
 
 // cpu/exec/argmax.zig:56-81: strict > keeps the first maximum. ARGMAX_PARTS workgroups per row each reduce a contiguous
 // slice to (value, index); the workgroup that draws the row's last ticket then picks among the parts (ties -> the smaller
-// index, which is the first maximum) - one launch. The parts and the ticket are device-scope atomics and the ticket is
-// taken after the part's stores were acknowledged, so no device-scope fence is needed (on this GPU such a fence writes
-// back and invalidates an XCD's whole L2); the pick does not depend on which workgroup came last. Tickets return to zero.
+// index, which is the first maximum) - one launch. A part travels as ONE 64-bit word {value bits, index}, stored and loaded
+// as a single device-scope atomic, so a reader can never see the value of one store with the index of another; the ticket
+// is a device-scope read-modify-write with release (the part's word is visible before the ticket counts it) and acquire
+// (the last workgroup's loads of the parts are ordered behind its ticket) semantics. The pick does not depend on which
+// workgroup came last. Tickets return to zero.
 constexpr int ARGMAX_PARTS = 64;
 __device__ __forceinline__ void argmax_reduce_256(float &best, int &idx, float *bv, int *bi) {
     bv[threadIdx.x] = best;
@@ -362,7 +364,7 @@ __device__ __forceinline__ void argmax_reduce_256(float &best, int &idx, float *
     idx = bi[0];
     __syncthreads();
 }
-__global__ __launch_bounds__(256) void argmax_kernel(int *__restrict__ out, float *pv, int *pi, unsigned *tickets, const float *__restrict__ x, size_t n) {
+__global__ __launch_bounds__(256) void argmax_kernel(int *__restrict__ out, unsigned long long *parts, unsigned *tickets, const float *__restrict__ x, size_t n) {
     __shared__ float bv[256];
     __shared__ int bi[256];
     __shared__ int s_last;
@@ -378,18 +380,18 @@ __global__ __launch_bounds__(256) void argmax_kernel(int *__restrict__ out, floa
     }
     argmax_reduce_256(best, idx, bv, bi);
     if (threadIdx.x == 0) {
-        __hip_atomic_store(pv + row * ARGMAX_PARTS + blockIdx.x, best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(pi + row * ARGMAX_PARTS + blockIdx.x, idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
-        s_last = __hip_atomic_fetch_add(tickets + row, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ARGMAX_PARTS - 1;
+        const unsigned long long word = ((unsigned long long)__float_as_uint(best) << 32) | (unsigned)idx;
+        __hip_atomic_store(parts + row * ARGMAX_PARTS + blockIdx.x, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = __hip_atomic_fetch_add(tickets + row, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == ARGMAX_PARTS - 1;
     }
     __syncthreads();
     if (!s_last) return;
     best = -INFINITY;
     idx = 0x7FFFFFFF;
     if (threadIdx.x < ARGMAX_PARTS) {
-        best = __hip_atomic_load(pv + row * ARGMAX_PARTS + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        idx = __hip_atomic_load(pi + row * ARGMAX_PARTS + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned long long word = __hip_atomic_load(parts + row * ARGMAX_PARTS + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        best = __uint_as_float((unsigned)(word >> 32));
+        idx = (int)(unsigned)word;
     }
     argmax_reduce_256(best, idx, bv, bi);
     if (threadIdx.x == 0) {
@@ -711,9 +713,8 @@ int aionhip_step_argmax(aionhip_ctx *ctx, aionhip_handle out_i32, aionhip_handle
     if (rc) return rc;
     rc = grow_work_buffer(ctx, &ctx->tickets, &ctx->tickets_bytes, rows * sizeof(unsigned), true, "the argmax tickets");
     if (rc) return rc;
-    float *pv = (float *)ctx->scratch2;
-    int *pi = (int *)(pv + rows * ARGMAX_PARTS);
-    argmax_kernel<<<dim3(ARGMAX_PARTS, (unsigned)rows), dim3(256), 0, ctx->stream>>>(dp<int>(out_i32), pv, pi, (unsigned *)ctx->tickets, dp<const float>(x), n);
+    argmax_kernel<<<dim3(ARGMAX_PARTS, (unsigned)rows), dim3(256), 0, ctx->stream>>>(dp<int>(out_i32), (unsigned long long *)ctx->scratch2, (unsigned *)ctx->tickets,
+                                                                                     dp<const float>(x), n);
     LAUNCH_CHECK(ctx, "argmax");
     return AIONHIP_OK;
 }

@@ -137,6 +137,31 @@ def test_kv_append_into_a_rolling_cache(gpu, orc):
     cb.free()
 
 
+def test_argmax_ties_across_parts_and_repeated_launches(gpu, orc):
+    """The row is cut into 64 parts whose (value, index) words meet behind a ticket: ties that span two parts (the smaller
+    index wins whichever part's workgroup arrives last), a constant row (index 0), fewer elements than parts, negative
+    rows, and the same launch repeated (the tickets return to zero)."""
+    rng = np.random.default_rng(21)
+    for m in (262144, 64 * 5 + 3, 40, 1):
+        per = -(-m // 64)
+        rows = 6
+        x = rng.standard_normal((rows, m)).astype(np.float32)
+        if m > 64:
+            x[0, per - 1] = x[0, per] = 9.0                      # last element of part 0 and first of part 1
+            x[1, 3 * per + 1] = x[1, min(40 * per + 2, m - 2)] = x[1, min(63 * per, m - 1)] = 11.0
+            x[4, m - 1] = x[4, 0] = 12.0
+        x[2, :] = -3.5                                        # constant: the first index
+        x[3, :] = -np.abs(x[3, :]) - 1.0                      # all negative
+        x[5, m // 2] = np.inf
+        xb, idx = gpu.upload(x), gpu.alloc(rows * 4)
+        want = list(orc.argmax(x))
+        assert want == list(np.argmax(x, axis=1))
+        for _ in range(5):
+            gpu.step_argmax(idx, xb, rows, m)
+            assert list(gpu.download(idx, np.int32, (rows,))) == want, m
+        xb.free(); idx.free()
+
+
 @pytest.mark.parametrize("np_dtype,dtype", [(np.float16, "F16"), (np.float32, "F32")])
 def test_sequence_append_step_with_rows_of_the_cache_type(gpu, orc, np_dtype, dtype):
     """The step as the reference states it: rows already of the cache's element type, linear and rolling."""

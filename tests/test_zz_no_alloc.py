@@ -118,3 +118,61 @@ def test_static_entry_point_inside_a_recorded_program(gpu, orc):
         assert float(np.abs(got - ref).max()) <= 1e-5 * rms
     gpu.program_destroy(prog)
     a_buf.free(); c_buf.free(); w.free()
+
+
+def _device_free_bytes():
+    import ctypes as C
+    rt = C.CDLL("libamdhip64.so")
+    free, total = C.c_size_t(0), C.c_size_t(0)
+    assert rt.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    return free.value
+
+
+# one case per route the static entry point can take: one row with the preparation inside the kernel; one row past K = 8192
+# (separate preparation + one-row kernel); 2..8 rows (preparation + rows kernel); 5..8 rows against a wide short weight (the
+# 16-row MFMA tile); more than 8 rows (the exact GEMM, whose K slices need a buffer and are therefore off here)
+ROUTES = [("one row, fused", be.Q4_0, be.KMAJOR_KN, 1, 2100, 4096), ("one row, long K", be.Q8_0, be.ROWS_NK, 1, 520, 16416),
+          ("few rows", be.Q8_0, be.KMAJOR_KN, 3, 1030, 2048), ("few rows, 16-row tile", be.Q4_0, be.KMAJOR_KN, 6, 16390, 1024),
+          ("exact GEMM", be.Q4_0, be.KMAJOR_KN, 24, 520, 8192)]
+
+
+def test_every_route_records_on_a_fresh_context_and_allocates_nothing(orc):
+    """A context on which NO eager step ever ran (no scratch buffer has a size yet): every route of the static entry point is
+    recorded into a program - stream capture rejects an allocation, so a clean recording shows the route made none - and
+    replayed against the oracle; then the same calls eagerly, with the library's own counters and the device's free memory
+    unchanged around them."""
+    g = be.HipBackend(0)
+    try:
+        g.set_gemm_mode(be.GEMM_EXACT_I8)
+        rng = np.random.default_rng(77)
+        cases = []
+        for name, dtype, layout, m, n, k in ROUTES:
+            w = make(g, dtype, layout, n, k, seed=n + k + m)
+            a = rng.standard_normal((m, k)).astype(np.float32)
+            cases.append((name, dtype, layout, m, n, k, w, a, g.upload(a), g.zeros(m * n * 4)))
+        g.sync()
+        for name, dtype, layout, m, n, k, w, a, a_buf, c_buf in cases:
+            say("no-alloc route", name)
+            g.program_begin()
+            try:
+                g.step_matmul_static(w, a_buf, m, c_buf)
+            finally:
+                prog = g.program_end()
+            ref = orc.matmul_nt_q8(a, w.download(), n, threads=8) if layout == be.ROWS_NK else orc.matmul_q_packed(dtype, a, w.download(), n, threads=8)
+            rms = float(np.sqrt((ref.astype(np.float64) ** 2).mean()))
+            for _ in range(2):
+                g._check(g._lib.aionhip_memset(g._ctx, c_buf.handle, 0, 0, m * n * 4))
+                g.program_execute(prog)
+                got = g.download(c_buf, np.float32, (m, n))
+                assert float(np.abs(got - ref).max()) <= 1e-5 * rms, name
+            g.program_destroy(prog)
+        g.sync()
+        stats0, free0 = g.memory_stats(), _device_free_bytes()
+        for name, dtype, layout, m, n, k, w, a, a_buf, c_buf in cases:
+            g.step_matmul_static(w, a_buf, m, c_buf)
+        g.sync()
+        assert g.memory_stats() == stats0 and _device_free_bytes() == free0
+        for case in cases:
+            case[6].free(); case[8].free(); case[9].free()
+    finally:
+        g.close()
