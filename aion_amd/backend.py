@@ -179,7 +179,10 @@ class HipBackend:
         return out
 
     def upload_weight(self, dtype, layout, n, k, packed_blocks, ld_blocks=0):
-        b = np.ascontiguousarray(packed_blocks, dtype=np.uint8)
+        if dtype == F32:          # the f32 [N,K] operand of MatMulNT: the rows as they are
+            b = np.ascontiguousarray(packed_blocks, dtype=np.float32).reshape(-1).view(np.uint8)
+        else:
+            b = np.ascontiguousarray(packed_blocks, dtype=np.uint8)
         w = C.c_void_p()
         self._check(self._lib.aionhip_weight_upload(self._ctx, dtype, layout, n, k, ld_blocks, b.ctypes.data, C.byref(w)))
         return Weight(self, w, dtype, layout, n, k)

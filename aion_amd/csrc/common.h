@@ -243,6 +243,9 @@ bool gemm_bf16_pays(const aionhip_ctx *ctx, size_t m, size_t n, size_t k);
 int launch_gemm_i8_batch(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count, size_t m,
                          PreparedAct act, float alpha, float beta);
 int launch_gemm_i8_few_rows(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, PreparedAct act, float *c, size_t ldc, float alpha, float beta);
+// MatMulNT with an f32 [N,K] operand (matmul_nt_f32.hip): plain f32 arithmetic, any number of rows
+int launch_matmul_nt_f32(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, const float *a, size_t lda, float *c, size_t ldc, float alpha,
+                         float beta);
 int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, const float *a, size_t lda, float *c, size_t ldc, float alpha, float beta);
 
 // ---- wave64 cross-lane helpers -----------------------------------------------------------------

@@ -741,6 +741,7 @@ int aionhip_decoder_stack_create(aionhip_ctx *ctx, const aionhip_decoder_stack_d
             if (ws[i]->n != ns[i] || ws[i]->k != ks[i]) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "decoder stack: layer %zu: weight %d is %zu x %zu, expected %zu x %zu", l, i, ws[i]->n, ws[i]->k, ns[i], ks[i]);
             if (l == 0 && i == 0) dtype = ws[i]->dtype;
             if (ws[i]->dtype != dtype) return set_err(ctx, AIONHIP_UNSUPPORTED, "decoder stack: all weights must share one block format");
+            if (dtype != AIONHIP_Q4_0 && dtype != AIONHIP_Q8_0) return set_err(ctx, AIONHIP_UNSUPPORTED, "decoder stack: q4_0 or q8_0 weights only");
         }
         if (!s.norm1_gamma || !s.norm2_gamma || !s.k_cache || !s.v_cache) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "decoder stack: layer %zu: null gamma or cache", l);
         if ((s.norm1_gamma | s.norm1_beta | s.norm2_gamma | s.norm2_beta | s.k_cache | s.v_cache) & 15)

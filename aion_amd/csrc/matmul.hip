@@ -9,6 +9,8 @@
 // cache-append launch and the GeGLU block (two launches).
 #include "common.h"
 
+#include <cstring>
+
 #include <cmath>
 
 namespace {
@@ -32,6 +34,9 @@ int check_batch(aionhip_ctx *ctx, const char *what, size_t count, const aionhip_
     for (size_t i = 0; i < count; ++i) {
         if (!bs[i] || !c_hs[i]) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "%s: null weight or C", what);
         if (bs[i]->k != out.k || bs[i]->dtype != bs[0]->dtype) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "%s: weights must share k and dtype", what);
+        // an f32 weight is the operand of the plain MatMulNT step only: the fused and batched steps are built on block dots
+        if (bs[i]->dtype == AIONHIP_F32 && (count != 1 || strcmp(what, "matmul") != 0))
+            return set_err(ctx, AIONHIP_UNSUPPORTED, "%s: f32 weights run as single MatMulNT steps", what);
         out.ldc[i] = ldcs_in && ldcs_in[i] ? ldcs_in[i] : bs[i]->n;
         if (out.ldc[i] < bs[i]->n || (c_hs[i] & 3)) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "%s: ldc below n, or C not 4-byte aligned", what);
         out.w[i] = bs[i];
@@ -75,6 +80,7 @@ static int launch_prepared_rows(aionhip_ctx *ctx, const Batch &b, size_t m, Prep
 // to the library's file-scope device array and nothing on the way may allocate.
 int run_rows(aionhip_ctx *ctx, const Batch &b, size_t m, const float *a, size_t lda, float alpha, float beta, bool static_scratch = false) {
     if (m > 0x7FFFFFFFu) return set_err(ctx, AIONHIP_UNSUPPORTED, "matmul: m exceeds 2^31-1");
+    if (b.w[0]->dtype == AIONHIP_F32) return launch_matmul_nt_f32(ctx, b.w[0], m, a, lda, b.c[0], b.ldc[0], alpha, beta);
     if (static_scratch) {
         if (ctx->profiling) return set_err(ctx, AIONHIP_UNSUPPORTED, "matmul_static: not available while per-launch profiling is on (it creates events)");
         if (m > GEMV_MAX_M && ctx->gemm_mode != AIONHIP_GEMM_EXACT_I8)
@@ -149,8 +155,9 @@ int aionhip_step_matmul(aionhip_ctx *ctx, const aionhip_weight *b, size_t m, aio
 int aionhip_step_matmul_nt(aionhip_ctx *ctx, const aionhip_weight *b, size_t m, aionhip_handle a, size_t lda,
                            aionhip_handle c, size_t ldc, float alpha, float beta) {
     if (!ctx || !b) return AIONHIP_INVALID_ARGUMENT;
-    // StepMatMulNT: B is q8_0 [N,K] with quant_axis 1 (runtime/executable.zig:211-223)
-    if (b->layout != AIONHIP_ROWS_NK || b->dtype != AIONHIP_Q8_0) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "MatMulNT needs a q8_0 [N,K] weight (quant_axis 1)");
+    // StepMatMulNT: B is [N,K], q8_0 with quant_axis 1 or f32 (runtime/executable.zig:211-223, cpu/exec/matmul_nt.zig:100)
+    if (b->layout != AIONHIP_ROWS_NK || (b->dtype != AIONHIP_Q8_0 && b->dtype != AIONHIP_F32))
+        return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "MatMulNT needs a q8_0 (quant_axis 1) or f32 [N,K] weight");
     return run_matmul(ctx, b, m, a, lda, c, ldc, alpha, beta);
 }
 
@@ -202,6 +209,7 @@ int aionhip_step_rmsnorm_qkv_rope_append(aionhip_ctx *ctx, const aionhip_weight 
     const aionhip_weight *ws[3] = {wq, wk, wv};
     for (const aionhip_weight *w : ws)
         if (w->k != wq->k || w->dtype != wq->dtype) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "qkv_rope_append: weights must share k and dtype");
+    if (wq->dtype == AIONHIP_F32) return set_err(ctx, AIONHIP_UNSUPPORTED, "qkv_rope_append: f32 weights run as single MatMulNT steps");
     if (d == 0 || d % 8 != 0 || d > 65528 || h_q == 0 || h_kv == 0 || wq->n != h_q * d || wk->n != h_kv * d || wv->n != h_kv * d)
         return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "qkv_rope_append: weight rows must be heads x head size, head size a multiple of 8");
     // one token of one sequence, short enough K for the in-kernel prologue: anything else takes the separate steps
@@ -228,6 +236,7 @@ int aionhip_step_rmsnorm_geglu_matmul(aionhip_ctx *ctx, const aionhip_weight *w_
     if (!(eps > 0.f) || !(eps < INFINITY)) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "geglu_matmul: eps must be positive and finite");
     if (w_gate->k != w_up->k || w_gate->n != w_up->n || w_gate->dtype != w_up->dtype || w_down->k != w_gate->n)
         return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "geglu_matmul: gate and up must match, down must take their outputs");
+    if (w_gate->dtype == AIONHIP_F32 || w_down->dtype == AIONHIP_F32) return set_err(ctx, AIONHIP_UNSUPPORTED, "geglu_matmul: f32 weights run as single MatMulNT steps");
     if (c & 3) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "geglu_matmul: C not 4-byte aligned");
     if (w_gate->k > FUSED_MAX_K || w_gate->n % 32 != 0 || ((x | gamma | beta_norm) & 15))
         return set_err(ctx, AIONHIP_UNSUPPORTED, "geglu_matmul: needs k <= %zu, a hidden size that is a multiple of 32 and 16-byte aligned x/gamma/beta", FUSED_MAX_K);

@@ -99,7 +99,15 @@ int run_relay(aionhip_ctx *ctx, const aionhip_weight *w, uint8_t *packed, size_t
 }
 
 int check_weight_args(aionhip_ctx *ctx, int dtype, int layout, size_t n, size_t k, size_t ld) {
-    if (dtype != AIONHIP_Q8_0 && dtype != AIONHIP_Q4_0) return set_err(ctx, AIONHIP_UNSUPPORTED, "weight dtype %d is not q8_0/q4_0", dtype);
+    if (dtype == AIONHIP_F32) {
+        // the f32 operand of MatMulNT (runtime/executable.zig:211-223, cpu/exec/matmul_nt.zig:100): rows [N,K] as they are
+        if (layout != AIONHIP_ROWS_NK) return set_err(ctx, AIONHIP_UNSUPPORTED, "f32 weights are the [N,K] operand of MatMulNT only");
+        if (n == 0 || k == 0) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "weight shape n=%zu k=%zu", n, k);
+        if (n > 0x7FFFFFFFu || k > 0x7FFFFFFFu) return set_err(ctx, AIONHIP_UNSUPPORTED, "weight dimension exceeds 2^31-1");
+        if (ld != 0) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "ld_blocks applies to K-major quantized weights");
+        return AIONHIP_OK;
+    }
+    if (dtype != AIONHIP_Q8_0 && dtype != AIONHIP_Q4_0) return set_err(ctx, AIONHIP_UNSUPPORTED, "weight dtype %d is not q8_0 / q4_0 / f32", dtype);
     if (layout != AIONHIP_ROWS_NK && layout != AIONHIP_KMAJOR_KN) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "unknown weight layout %d", layout);
     // aion has no q4 [N,K] operand (cpu/exec/matmul.zig:233-239): MatMulNT is q8 or f32 only
     if (dtype == AIONHIP_Q4_0 && layout == AIONHIP_ROWS_NK) return set_err(ctx, AIONHIP_UNSUPPORTED, "q4_0 weights are K-major [K,N] only");
@@ -116,8 +124,8 @@ int alloc_weight(aionhip_ctx *ctx, int dtype, int layout, size_t n, size_t k, ai
     w->layout = layout;
     w->n = n;
     w->k = k;
-    w->qs_bytes = dtype == AIONHIP_Q8_0 ? n * k : n * k / 2;
-    w->sc_bytes = n * (k / QK) * sizeof(__half);
+    w->qs_bytes = dtype == AIONHIP_F32 ? n * k * sizeof(float) : (dtype == AIONHIP_Q8_0 ? n * k : n * k / 2);
+    w->sc_bytes = dtype == AIONHIP_F32 ? 0 : n * (k / QK) * sizeof(__half);
     // one allocation: quants first (16-byte aligned rows since k % 32 == 0), scales after
     const size_t qs_padded = (w->qs_bytes + 255) & ~(size_t)255;
     void *p = nullptr;
@@ -145,7 +153,12 @@ int aionhip_weight_from_device(aionhip_ctx *ctx, int dtype, int layout, size_t n
     aionhip_weight *w = nullptr;
     rc = alloc_weight(ctx, dtype, layout, n, k, &w);
     if (rc) return rc;
-    rc = run_relay<false>(ctx, w, (uint8_t *)(uintptr_t)device_blocks, ld_blocks ? ld_blocks : n);
+    if (dtype == AIONHIP_F32) {
+        const hipError_t e = hipMemcpyAsync(w->qs, (const void *)(uintptr_t)device_blocks, w->qs_bytes, hipMemcpyDeviceToDevice, ctx->stream);
+        rc = e == hipSuccess ? (int)AIONHIP_OK : set_err(ctx, AIONHIP_EXECUTION_FAILED, "f32 weight copy: %s", hipGetErrorString(e));
+    } else {
+        rc = run_relay<false>(ctx, w, (uint8_t *)(uintptr_t)device_blocks, ld_blocks ? ld_blocks : n);
+    }
     if (rc) {
         aionhip_weight_free(ctx, w);
         return rc;
@@ -163,7 +176,7 @@ int aionhip_weight_upload(aionhip_ctx *ctx, int dtype, int layout, size_t n, siz
     const size_t bb = dtype == AIONHIP_Q8_0 ? Q8_BYTES : Q4_BYTES;
     const size_t KB = k / QK;
     const size_t ld = ld_blocks ? ld_blocks : n;
-    const size_t bytes = (layout == AIONHIP_KMAJOR_KN ? ((KB - 1) * ld + n) : n * KB) * bb;
+    const size_t bytes = dtype == AIONHIP_F32 ? n * k * sizeof(float) : (layout == AIONHIP_KMAJOR_KN ? ((KB - 1) * ld + n) : n * KB) * bb;
     void *staging = nullptr;
     rc = dev_malloc(ctx, &staging, bytes, "weight upload staging");
     if (rc) return rc;
@@ -217,6 +230,7 @@ void aionhip_weight_free(aionhip_ctx *ctx, aionhip_weight *w) {
 
 size_t aionhip_weight_packed_bytes(const aionhip_weight *w) {
     if (!w) return 0;
+    if (w->dtype == AIONHIP_F32) return w->n * w->k * sizeof(float);
     return w->n * (w->k / QK) * (w->dtype == AIONHIP_Q8_0 ? Q8_BYTES : Q4_BYTES);
 }
 size_t aionhip_weight_device_bytes(const aionhip_weight *w) { return w ? w->qs_bytes + w->sc_bytes : 0; }
@@ -225,6 +239,11 @@ int aionhip_weight_download(aionhip_ctx *ctx, const aionhip_weight *w, void *hos
     if (!ctx || !w || !host_blocks) return AIONHIP_INVALID_ARGUMENT;
     const size_t want = aionhip_weight_packed_bytes(w);
     if (bytes != want) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "download: buffer is %zu bytes, packed form is %zu", bytes, want);
+    if (w->dtype == AIONHIP_F32) {           // kept as uploaded
+        hipError_t e = hipMemcpyAsync(host_blocks, w->qs, want, hipMemcpyDeviceToHost, ctx->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        return e == hipSuccess ? (int)AIONHIP_OK : set_err(ctx, AIONHIP_EXECUTION_FAILED, "weight download copy: %s", hipGetErrorString(e));
+    }
     void *staging = nullptr;
     int rc = dev_malloc(ctx, &staging, want, "weight download staging");
     if (rc) return rc;

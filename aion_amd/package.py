@@ -150,11 +150,18 @@ class PackageRunner:
                                   (t.scheme, t.quant_axis, " under a transpose" if transposed else ""))
             val = _Val("weight", w, shape, t.scheme)
         else:
-            if transposed:
-                raise Unsupported("transpose of a plain initializer")
             if _count(shape) * _ELEM[t.dtype] != t.data.size:
                 raise PackageError("InvalidFormat", "initializer payload does not match its shape")
-            val = _Val("dev", self.gpu.upload(np.asarray(t.data)), shape, t.dtype)
+            if transposed:
+                # MatMul over the transpose of a plain f32 [N,K] initializer is MatMulNT with an f32 B
+                # (graph/program/compiler.zig:337-357, cpu/exec/matmul_nt.zig:100)
+                if t.dtype != "f32" or len(shape) != 2:
+                    raise Unsupported("transpose of a plain %s initializer of rank %d" % (t.dtype, len(shape)))
+                n, k = shape
+                w = self.gpu.upload_weight(be.F32, be.ROWS_NK, n, k, np.frombuffer(np.asarray(t.data), np.float32))
+                val = _Val("weight", w, shape, "f32")
+            else:
+                val = _Val("dev", self.gpu.upload(np.asarray(t.data)), shape, t.dtype)
         self.consts[key] = val
         return val
 
@@ -207,7 +214,9 @@ class PackageRunner:
                 v = vals[vid] = _Val("dev", out, v.shape, "f32", owned=True)
             return v
 
-        def weight_of(vid):
+        def weight_of(vid, allow_f32=False):
+            """The matmul weight behind `vid`, or None. f32 weights (MatMulNT's plain operand) only where asked for: the
+            fused steps are built on block dots."""
             if vid in vals:
                 w = vals[vid]
             elif vid in producer and nodes[producer[vid]].op == "ViewTranspose2D":
@@ -220,7 +229,7 @@ class PackageRunner:
                 w = self._const(vid)
             else:
                 return None
-            return w if w.kind == "weight" else None
+            return w if w.kind == "weight" and (allow_f32 or w.dtype != "f32") else None
 
         def sole_user(vid, op=None):
             """The one node that reads `vid` (None if it has several readers or is a graph output)."""
@@ -522,12 +531,12 @@ class PackageRunner:
                 emit(g.step_rmsnorm, out, x.buf, gamma.buf, rows, cols, a["eps"], beta=beta.buf)
                 vals[n.output] = _Val("dev", out, shape, "f32", owned=True)
             elif op == "ViewTranspose2D":
-                if weight_of(n.output) is None:
-                    raise Unsupported("ViewTranspose2D of anything but a quantized weight")
+                if weight_of(n.output, allow_f32=True) is None:
+                    raise Unsupported("ViewTranspose2D of anything but a weight")
             elif op == "MatMul":
-                x, w = get(n.inputs[0]), weight_of(n.inputs[1])
+                x, w = get(n.inputs[0]), weight_of(n.inputs[1], allow_f32=True)
                 if w is None:
-                    raise Unsupported("MatMul whose right operand is not a quantized weight")
+                    raise Unsupported("MatMul whose right operand is not a weight")
                 if a["beta"] != 0.0:
                     raise Unsupported("MatMul with beta != 0 in a package")
                 m_rows, alpha = _count(x.shape[:-1]), a["alpha"]

@@ -108,8 +108,11 @@ int aionhip_quantize_device(aionhip_ctx *ctx, int dtype, size_t rows, size_t col
  *      api/gpu_device.zig:24-25, and keeps its own layout) -----------------------------------
  * Input is aion's packed blocks, exactly as the quantizer emits them: ROWS_NK -> block (n,kb)
  * at (n*K/32+kb)*block_bytes; KMAJOR_KN -> block (kb,n) at (kb*ld+n)*block_bytes (ld = row
- * stride in blocks, 0 = n; MatMulParams.ldb, backend/types.zig:225-241). Only Q8_0 may be
- * ROWS_NK. The packed bytes are consumed during the call and not referenced afterwards. */
+ * stride in blocks, 0 = n; MatMulParams.ldb, backend/types.zig:225-241). Of the block formats only Q8_0 may be
+ * ROWS_NK. dtype AIONHIP_F32 with ROWS_NK is the f32 operand of MatMulNT (runtime/executable.zig:211-223,
+ * cpu/exec/matmul_nt.zig:100): n rows of k floats, kept as they are (any k, ld_blocks 0); such a weight is accepted by
+ * aionhip_step_matmul_nt only - the batched and fused steps answer AIONHIP_UNSUPPORTED and the caller issues the separate
+ * steps. The bytes handed in are consumed during the call and not referenced afterwards. */
 int aionhip_weight_upload(aionhip_ctx *ctx, int dtype, int layout, size_t n, size_t k, size_t ld_blocks,
                           const void *host_blocks, aionhip_weight **out);
 /* same, from blocks already resident in device memory (a tensor moved by DeviceMemory.copyH2D) */
@@ -128,7 +131,8 @@ int aionhip_weight_download(aionhip_ctx *ctx, const aionhip_weight *w, void *hos
  * lda/ldc in elements (0 = k / n). Leading dims of A are folded into m by the caller
  * (cpu/exec/matmul.zig:100-163). Arithmetic follows aion's CPU kernels: A is int8-quantized
  * per (row, 32-block) (cpu/kernels/matmul_q_i8.zig:187-203), block dots are exact integers,
- * accumulation is f32. */
+ * accumulation is f32. MatMulNT with an f32 weight (cpu/kernels/matmul_nt.zig:40-126) quantizes nothing: f32 fused
+ * multiply-adds over k, f32 sums. */
 int aionhip_step_matmul(aionhip_ctx *ctx, const aionhip_weight *b, size_t m,
                         aionhip_handle a, size_t lda, aionhip_handle c, size_t ldc, float alpha, float beta);
 int aionhip_step_matmul_nt(aionhip_ctx *ctx, const aionhip_weight *b, size_t m,

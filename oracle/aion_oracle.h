@@ -23,6 +23,8 @@
  *                               causal cases, hand-computable KATs (api/test_api.zig:3256-3331,
  *                               api/test_nn.zig:799-901), split==unsplit invariant.
  *   glue (rmsnorm, rope, gate, gather, cast, append, argmax): closed forms in numpy.
+ *   matmul_nt_f32 (oracle.py, numpy; cpu/kernels/matmul_nt.zig:40-126): the float64 product within the bound K fixes,
+ *                               and bit equality on inputs whose partial sums are all exact in f32.
  */
 #ifndef AION_ORACLE_H
 #define AION_ORACLE_H

@@ -22,6 +22,13 @@ class _Quant:
         self.scheme, self.quant_axis, self.shape, self.blocks, self.transposed = scheme, quant_axis, tuple(shape), blocks, transposed
 
 
+class _PlainT:
+    """The ViewTranspose2D of a plain f32 [N,K] initializer: the right operand of a MatMulNT with an f32 B."""
+
+    def __init__(self, rows):
+        self.rows = rows
+
+
 def _initializer(pkg, vid):
     v = pkg.values[vid]
     t = pkg.tensors[v.initializer]
@@ -34,6 +41,8 @@ def _initializer(pkg, vid):
 def _matmul(x, w, alpha, attn_threads):
     m = int(np.prod(x.shape[:-1]))
     a = x.reshape(m, x.shape[-1])
+    if isinstance(w, _PlainT):                                                 # graph/program/compiler.zig:337-357: MatMulNT, f32 B
+        return orc.matmul_nt_f32(a, w.rows, alpha=alpha)
     if w.scheme == "q4_0" and w.quant_axis == 0 and not w.transposed:          # [K,N] packed along K
         return orc.matmul_q_packed(orc.Q4_0, a, w.blocks, w.shape[1], alpha=alpha, threads=attn_threads)
     if w.scheme == "q8_0" and w.quant_axis == 0 and not w.transposed:
@@ -59,8 +68,10 @@ def _eval(pkg, n, ins, a, ring, exact_attention, round_q_f16, threads):
         return orc.rmsnorm(x.reshape(-1, x.shape[-1]), gamma, a["eps"], beta=beta)
     if n.op == "ViewTranspose2D":
         w = ins[0]
+        if isinstance(w, np.ndarray) and w.dtype == np.float32 and w.ndim == 2:
+            return _PlainT(w)
         if not isinstance(w, _Quant):
-            raise ValueError("graph oracle: ViewTranspose2D of a quantized weight only")
+            raise ValueError("graph oracle: ViewTranspose2D of a weight only")
         return _Quant(w.scheme, w.quant_axis, w.shape, w.blocks, transposed=not w.transposed)
     if n.op == "MatMul":
         if a["beta"] != 0.0:
@@ -131,7 +142,7 @@ def run_graph(pkg, feeds, symbols, rolling_inputs=(), exact_attention=False, rou
         out = _eval(pkg, n, [vals[i] for i in n.inputs], n.attrs, ring, exact_attention, round_q_f16, threads)
         if n.op == "SequenceAppend" and ring:
             rolling.add(n.output)
-        vals[n.output] = out if isinstance(out, _Quant) else np.asarray(out).reshape(pkg.shape_of(n.output, symbols))
+        vals[n.output] = out if isinstance(out, (_Quant, _PlainT)) else np.asarray(out).reshape(pkg.shape_of(n.output, symbols))
     return {name: vals[vid] for name, vid in pkg.outputs}
 
 
@@ -166,7 +177,7 @@ def check_nodes(pkg, feeds, symbols, device_values, rolling_inputs=(), threads=4
             rows = sorted({0, m // 2, m - 1})
             ins = [ins[0].reshape(m, ins[0].shape[-1])[rows]] + ins[1:]
         out = _eval(pkg, n, ins, n.attrs, ring, False, False, threads)
-        if isinstance(out, _Quant):
+        if isinstance(out, (_Quant, _PlainT)):
             vals[n.output] = out
             continue
         if rows is not None:

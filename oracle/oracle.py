@@ -132,6 +132,40 @@ def matmul_nt_q8(a, b_blocks, n, alpha=1.0, beta=0.0, c=None, threads=1):
     return out
 
 
+def matmul_nt_f32(a, b, alpha=1.0, beta=0.0, c=None, lanes=8):
+    """MatMulNT with an f32 B [N,K] (cpu/kernels/matmul_nt.zig:40-126): C = alpha * A @ B^T + beta * C. The reference's order:
+    four vectors of `lanes` accumulators take k in turns (fused multiply-adds), each is reduced, the four sums are added, the
+    K tail past a multiple of 4 * lanes follows element by element; beta == 0 stores alpha * acc. numpy restatement: the
+    fused multiply-add is formed in float64 (the product of two f32 is exact there) and rounded to f32, the vector reduce is a
+    pairwise tree. Pinned by tests/test_oracle_matmul.py against the float64 product (error bound from K) and on inputs whose
+    every partial sum is exact in f32 (small integers), where any summation order gives the same bits."""
+    a, b = _f32(a), _f32(b)
+    m, k = a.shape
+    n = b.shape[0]
+    out = _c_init(m, n, c, beta)
+    step = 4 * lanes
+    k_vec = k - k % step
+    acc = np.zeros((m, n, 4, lanes), np.float32)
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    for kk in range(0, k_vec, step):
+        pa = a64[:, None, kk:kk + step].reshape(m, 1, 4, lanes)
+        pb = b64[None, :, kk:kk + step].reshape(1, n, 4, lanes)
+        acc = (pa * pb + acc.astype(np.float64)).astype(np.float32)
+    red = acc
+    while red.shape[-1] > 1:                                   # @reduce(.Add, v): pairwise
+        red = (red[..., 0::2] + red[..., 1::2]).astype(np.float32)
+    red = red[..., 0]
+    tot = ((red[..., 0] + red[..., 1]).astype(np.float32) + red[..., 2]).astype(np.float32)
+    tot = (tot + red[..., 3]).astype(np.float32)
+    for kk in range(k_vec, k):
+        tot = (tot + (a[:, None, kk] * b[None, :, kk]).astype(np.float32)).astype(np.float32)
+    al, be_ = np.float32(alpha), np.float32(beta)
+    res = (al * tot).astype(np.float32)
+    if beta != 0.0:
+        res = (res + (be_ * out).astype(np.float32)).astype(np.float32)
+    return res
+
+
 def matmul_q8_kmajor(a, b_blocks, n, alpha=1.0, beta=0.0, c=None, threads=1):
     a = _f32(a); m, k = a.shape
     b = np.ascontiguousarray(b_blocks, dtype=np.uint8)

@@ -474,3 +474,64 @@ def test_fused_prologues_at_k_up_to_8192_with_many_outputs(gpu, orc, dtype, layo
     for t in (xb, gb, c1, c2, g8, u8, c3, c4, c5):
         t.free()
     w3.free(); w4.free(); w5.free()
+
+
+# MatMulNT with an f32 B [N,K] (runtime/executable.zig:211-223; cpu/kernels/matmul_nt.zig:40-126): nothing is quantized.
+# Exact inputs (small integers: every partial sum exact in f32, so every summation order gives the same bits) must come out
+# bit-equal to the oracle; random inputs are held to the float64 product within twice the oracle's own distance from it
+# (the device sums the same terms in another order). Shapes: one row and many, K that is not a multiple of 4 (scalar loads),
+# K below a wavefront, a vocabulary-sized N, strides and alpha / beta; then what an f32 weight is refused for.
+@pytest.mark.parametrize("m,n,k", [(1, 7, 1), (1, 1000, 4096), (3, 129, 100), (8, 64, 2048), (21, 300, 515), (5, 40000, 512), (2, 5, 4099)])
+def test_matmul_nt_with_an_f32_weight(gpu, orc, m, n, k):
+    say("matmul_nt f32", m, n, k)
+    rng = np.random.default_rng(m * 7 + n + k)
+    wi = rng.integers(-8, 9, (n, k)).astype(np.float32)
+    ai = rng.integers(-8, 9, (m, k)).astype(np.float32)
+    w = gpu.upload_weight(be.F32, be.ROWS_NK, n, k, wi)
+    assert w.packed_bytes == n * k * 4 and np.array_equal(w.download().view(np.float32).reshape(n, k), wi)
+    got = gpu.matmul(w, ai)
+    assert gpu.last_kernel() == "matmul_nt_f32"
+    assert np.array_equal(got, orc.matmul_nt_f32(ai, wi)) and np.array_equal(got, (ai.astype(np.int64) @ wi.astype(np.int64).T).astype(np.float32))
+    c0 = rng.integers(-4, 5, (m, n)).astype(np.float32)
+    assert np.array_equal(gpu.matmul(w, ai, alpha=2.0, beta=-0.5, c=c0), orc.matmul_nt_f32(ai, wi, alpha=2.0, beta=-0.5, c=c0))
+    w.free()
+    wf = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+    af = rng.standard_normal((m, k)).astype(np.float32)
+    w = gpu.upload_weight(be.F32, be.ROWS_NK, n, k, wf)
+    got = gpu.matmul(w, af)
+    ref64 = af.astype(np.float64) @ wf.astype(np.float64).T
+    want = orc.matmul_nt_f32(af, wf)
+    rms = float(np.sqrt((ref64 ** 2).mean()))
+    own = float(np.abs(want - ref64).max())
+    err = float(np.abs(got - ref64).max())
+    say("   max|err| vs f64: device", err / rms, "oracle", own / rms)
+    assert err <= 2 * own + 1e-7 * rms
+    assert float(np.abs(got - want).max()) <= 1e-5 * rms
+    w.free()
+
+
+def test_an_f32_weight_is_a_matmul_nt_operand_only(gpu):
+    n, k = 64, 64
+    wf = np.ones((n, k), np.float32)
+    with pytest.raises(be.AionHipError) as e:
+        gpu.upload_weight(be.F32, be.KMAJOR_KN, n, k, wf)
+    assert e.value.status == hip.UNSUPPORTED
+    w = gpu.upload_weight(be.F32, be.ROWS_NK, n, k, wf)
+    x, g, c = gpu.upload(np.ones((1, k), np.float32)), gpu.upload(np.ones(k, np.float32)), gpu.zeros(n * 4)
+    with pytest.raises(be.AionHipError) as e:
+        gpu.step_rmsnorm_matmul([w], x, g, 1, [c], 1e-6)
+    assert e.value.status == hip.UNSUPPORTED
+    with pytest.raises(be.AionHipError) as e:
+        gpu.step_matmul_batch([w, w], x, 1, [c, c])
+    assert e.value.status == hip.UNSUPPORTED
+    gpu.step_matmul(w, x, 1, c)                      # the plain step runs
+    assert np.array_equal(gpu.download(c, np.float32, (n,)), np.full(n, k, np.float32))
+    # a strided A and C: lda / ldc in elements
+    a2 = np.arange(2 * 80, dtype=np.float32).reshape(2, 80) % 7
+    ab, cb = gpu.upload(a2), gpu.zeros(2 * 100 * 4)
+    gpu.step_matmul(w, ab, 2, cb, lda=80, ldc=100)
+    out = gpu.download(cb, np.float32, (2, 100))
+    assert np.array_equal(out[:, :n], np.repeat(a2[:, :k].sum(axis=1, keepdims=True), n, axis=1)) and not out[:, n:].any()
+    for t in (x, g, c, ab, cb):
+        t.free()
+    w.free()

@@ -96,6 +96,36 @@ def test_package_runner_refuses_what_the_backend_has_no_step_for(gpu):
         run.close()
 
 
+def test_package_with_an_f32_head_runs_as_matmul_nt(gpu, orc):
+    """MatMul over the ViewTranspose2D of a plain f32 [N,K] initializer is MatMulNT with an f32 B (graph/program/compiler.zig:
+    337-357): tokens -> f32 embedding rows -> RMSNorm -> the f32 head, for one and for several tokens, against the node-by-node
+    interpreter. Nothing on this path is quantized, so the bar is the f32 one (1e-5 of the logits' rms)."""
+    from oracle import graph_oracle
+    V, E, N = 64, 96, 200
+    rng = np.random.default_rng(31)
+    b = aion_writer.PackageBuilder()
+    seq = b.symbol("seq")
+    x = b.input("tokens", "i32", (1, seq), role="tokens", axis=1)
+    table = b.initializer("f32", (V, E), b.tensor_plain("f32", rng.standard_normal((V, E)).astype(np.float32)), "embed")
+    gamma = b.initializer("f32", (E,), b.tensor_plain("f32", (1 + 0.1 * rng.standard_normal(E)).astype(np.float32)), "gamma")
+    beta = b.initializer("f32", (E,), b.tensor_plain("f32", np.zeros(E, np.float32)), "beta")
+    head = b.initializer("f32", (N, E), b.tensor_plain("f32", (rng.standard_normal((N, E)) * 0.1).astype(np.float32)), "head")
+    h = b.rmsnorm(b.gather(table, x, (1, seq, E)), gamma, beta, 1e-6, (1, seq, E), (E,))
+    logits = b.matmul(h, b.transpose2d(head, "f32", (E, N)), (1, seq, N), alpha=0.5)
+    b.output("logits", logits)
+    pkg = aion_file.parse(b.to_bytes())
+    run = PackageRunner(gpu, pkg, capacity=8)
+    try:
+        for tokens in (np.array([5], np.int32), np.array([1, 63, 7, 7, 0], np.int32)):
+            got = run.run(tokens, want=("logits",))["logits"]
+            assert gpu.last_kernel() == "matmul_nt_f32"
+            want = graph_oracle.run_graph(pkg, {"tokens": tokens.reshape(1, -1)}, {"seq": tokens.size})["logits"]
+            rms = float(np.sqrt((want.astype(np.float64) ** 2).mean()))
+            assert got.shape == want.shape and float(np.abs(got - want).max()) <= 1e-5 * rms
+    finally:
+        run.close()
+
+
 @pytest.mark.parametrize("wdtype", [be.Q4_0, be.Q8_0])
 def test_fused_schedule_counts_steps_and_matches_the_node_by_node_one(gpu, wdtype):
     cfg = DecoderConfig(wdtype=wdtype, **SMALL)

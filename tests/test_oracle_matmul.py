@@ -191,3 +191,30 @@ def test_prepare_a_hand_computed_ties_and_special_blocks(orc):
     assert aq[4].tolist() == [127 * (-1 if t % 2 else 1) for t in range(32)]
     assert sc[0, 4] == np.float32(5e-40) / np.float32(127) and sc[0, 4] > 0
     assert sm[0].tolist() == aq.astype(np.int64).sum(axis=1).tolist()
+
+
+def test_matmul_nt_f32_restatement_against_float64_and_exact_inputs(orc):
+    """MatMulNT with an f32 B (cpu/kernels/matmul_nt.zig:40-126). Pinned two ways: (1) inputs of small integers, where every
+    product and every partial sum is an integer below 2^24 and so exact in f32 - ANY order of the additions gives the same
+    bits, so the result must equal the integer matmul, alpha / beta included (a dropped tail element, a transposed operand or
+    a wrong reduce shows); (2) random inputs against the float64 product within the worst-case bound of an f32 sum of K
+    terms, gamma_K * sum|a||b|."""
+    rng = np.random.default_rng(61)
+    for m, n, k in [(1, 7, 1), (3, 5, 31), (2, 9, 32), (4, 6, 100), (1, 3, 4099)]:
+        a = rng.integers(-8, 9, (m, k)).astype(np.float32)
+        b = rng.integers(-8, 9, (n, k)).astype(np.float32)
+        c0 = rng.integers(-4, 5, (m, n)).astype(np.float32)
+        want = a.astype(np.int64) @ b.astype(np.int64).T
+        assert np.array_equal(orc.matmul_nt_f32(a, b), want.astype(np.float32))
+        assert np.array_equal(orc.matmul_nt_f32(a, b, alpha=2.0, beta=-0.5, c=c0), (2 * want - 0.5 * c0).astype(np.float32))
+        # a different lane count is a different admissible order: same bits on exact inputs
+        assert np.array_equal(orc.matmul_nt_f32(a, b, lanes=4), want.astype(np.float32))
+    for m, n, k in [(2, 33, 64), (5, 17, 1000), (1, 8, 4096)]:
+        a = rng.standard_normal((m, k)).astype(np.float32)
+        b = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+        got = orc.matmul_nt_f32(a, b, alpha=0.75)
+        ref = 0.75 * (a.astype(np.float64) @ b.astype(np.float64).T)
+        bound = (k + 2) * 2.0 ** -24 * 0.75 * (np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64).T)
+        assert (np.abs(got - ref) <= bound).all()
+    with pytest.raises(ValueError):
+        orc.matmul_nt_f32(np.zeros((1, 4), np.float32), np.zeros((2, 4), np.float32), beta=1.0)      # beta without C
