@@ -6,9 +6,10 @@
 //   acc += f32(idot) * (a_scale * w_scale) on the VALU. Operands are staged through LDS. The per-block
 //   rescale (3 VALU ops per output element per block) is what bounds it, not the MFMA pipe.
 //
-// gemm_bf16_wide_kernel (AIONHIP_GEMM_BF16_MFMA) - weights dequantized once to bf16 [N,K] (kept
-//   per weight: 288 GB of HBM makes the 2 B/weight copy affordable), activations rounded to bf16,
-//   v_mfma_f32_32x32x16_bf16 with f32 accumulation; described at the kernel.
+// gemm_bf16_wide_kernel (AIONHIP_GEMM_BF16_MFMA) - weights as bf16, either from a copy the context builds once per
+//   weight and owns (2 B/weight; 288 GB of HBM makes it affordable) or converted from the quant blocks while they are
+//   staged (no copy; same bits, slower), activations rounded to bf16, v_mfma_f32_32x32x16_bf16 with f32 accumulation;
+//   described at the kernel.
 #include "common.h"
 
 #include <type_traits>
