@@ -333,21 +333,32 @@ __global__ void dequant_bf16_kernel(const uint8_t *__restrict__ qs, const __half
     *(u32x4 *)(out + bf16_tiled_index(n, k0, K)) = o;
 }
 
-__global__ void act_bf16_kernel(const float *__restrict__ a, size_t lda, unsigned short *__restrict__ out, size_t M, size_t K) {
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const size_t per_row = K / 8, rows = (M + 15) & ~(size_t)15;
-    if (i >= rows * per_row) return;
-    const size_t m = i / per_row, k0 = (i % per_row) * 8;
-    if (m >= M) {
-        *(u32x4 *)(out + bf16_tiled_index(m, k0, K)) = u32x4{0u, 0u, 0u, 0u};
-        return;
+// A wavefront rounds one 1 KiB block of the tiled copy - 16 rows x 32 k: lane = 4 * row + part reads 8 consecutive floats of
+// its row (the 16 rows' 128-byte lines, whole) and writes its 16 bytes of the block (1 KiB of consecutive memory); consecutive
+// wavefronts take consecutive k blocks of the same 16 rows. VEC: the rows are 16-byte aligned and the loads are two dwordx4.
+template <bool VEC>
+__global__ __launch_bounds__(256) void act_bf16_kernel(const float *__restrict__ a, size_t lda, unsigned short *__restrict__ out, size_t M, size_t K) {
+    const size_t wave = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int lane = threadIdx.x & 63, row = lane >> 2, part = lane & 3;
+    const size_t kblocks = K / G2_TILE_K, row_tiles = (M + 15) >> 4;
+    if (wave >= row_tiles * kblocks) return;
+    const size_t m = (wave / kblocks) * 16 + row, k0 = (wave % kblocks) * G2_TILE_K + part * 8;
+    u32x4 o = u32x4{0u, 0u, 0u, 0u};                       // rows past M: zeros
+    if (m < M) {
+        const float *p = a + m * lda + k0;
+        float v[8];
+        if (VEC) {
+            const f32x4 x = *(const f32x4 *)p, y = *(const f32x4 *)(p + 4);
+            v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w; v[4] = y.x; v[5] = y.y; v[6] = y.z; v[7] = y.w;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = p[i];
+        }
+        o.x = (unsigned)bf16_rne(v[0]) | ((unsigned)bf16_rne(v[1]) << 16);
+        o.y = (unsigned)bf16_rne(v[2]) | ((unsigned)bf16_rne(v[3]) << 16);
+        o.z = (unsigned)bf16_rne(v[4]) | ((unsigned)bf16_rne(v[5]) << 16);
+        o.w = (unsigned)bf16_rne(v[6]) | ((unsigned)bf16_rne(v[7]) << 16);
     }
-    const float *p = a + m * lda + k0;
-    u32x4 o;
-    o.x = (unsigned)bf16_rne(p[0]) | ((unsigned)bf16_rne(p[1]) << 16);
-    o.y = (unsigned)bf16_rne(p[2]) | ((unsigned)bf16_rne(p[3]) << 16);
-    o.z = (unsigned)bf16_rne(p[4]) | ((unsigned)bf16_rne(p[5]) << 16);
-    o.w = (unsigned)bf16_rne(p[6]) | ((unsigned)bf16_rne(p[7]) << 16);
     *(u32x4 *)(out + bf16_tiled_index(m, k0, K)) = o;
 }
 
@@ -978,9 +989,12 @@ int launch_gemm_bf16(aionhip_ctx *ctx, const aionhip_weight *w, size_t m, const 
     if (rc) return rc;
     unsigned short *abf = (unsigned short *)ctx->scratch2;
     {
-        const size_t threads = m_padded * (K / 8);
+        const size_t threads = m_padded * (K / 8);                 // = 64 lanes per (16 rows, 32 k) block
         ProfScope scope(ctx, "act_bf16");
-        launch_k(ctx, act_bf16_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, a, lda, abf, m, K);
+        if ((((uintptr_t)a) & 15) == 0 && (lda & 3) == 0)
+            launch_k(ctx, act_bf16_kernel<true>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, a, lda, abf, m, K);
+        else
+            launch_k(ctx, act_bf16_kernel<false>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, a, lda, abf, m, K);
         LAUNCH_CHECK(ctx, "act_bf16");
     }
     ProfScope scope(ctx, "gemm_bf16");
