@@ -39,6 +39,24 @@ class DecoderStackDesc(C.Structure):
                [("window_left", C.c_uint32), ("window_right", C.c_uint32), ("window_chunk", C.c_uint32), ("rolling", C.c_int)]
 
 
+MAX_RANK = 8
+
+
+class TensorRef(C.Structure):
+    """aionhip_tensor_ref: what the tensor store answers for one TensorId (address, dtype, shape)."""
+    _fields_ = [("handle", C.c_uint64), ("dtype", C.c_int32), ("rank", C.c_uint32), ("flags", C.c_uint32), ("reserved", C.c_uint32),
+                ("shape", C.c_uint64 * MAX_RANK)]
+
+
+class Step(C.Structure):
+    """aionhip_step: one step of an ExecutableProgram (runtime/executable.zig:302-345) with its operands resolved."""
+    _fields_ = [("tag", C.c_int32), ("op", C.c_int32), ("act", C.c_int32), ("broadcast", C.c_int32), ("axis", C.c_int32),
+                ("batch_dims", C.c_uint32), ("alpha", C.c_float), ("beta", C.c_float), ("eps", C.c_float), ("scale", C.c_float),
+                ("soft_cap", C.c_float), ("window_left", C.c_uint32), ("window_right", C.c_uint32), ("window_chunk", C.c_uint32),
+                ("rope_base", C.c_float), ("rope_scale", C.c_float), ("rope_proportion", C.c_float), ("to_host", C.c_int32),
+                ("out", TensorRef), ("in_", TensorRef * 5), ("host", C.c_void_p), ("host_bytes", C.c_uint64)]
+
+
 _SIGS = {
     # name: (restype, argtypes)
     "aionhip_create": (C.c_int, [C.c_int, C.c_void_p, C.POINTER(C.c_void_p)]),
@@ -98,6 +116,12 @@ _SIGS = {
     "aionhip_program_node_count": (C.c_size_t, [C.c_void_p]),
     "aionhip_program_is_current": (C.c_int, [C.c_void_p, C.c_void_p]),
     "aionhip_program_destroy": (None, [C.c_void_p, C.c_void_p]),
+    "aionhip_session_create": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p)]),
+    "aionhip_session_set_fusion": (C.c_int, [C.c_void_p, C.c_int]),
+    "aionhip_session_execute": (C.c_int, [C.c_void_p, C.POINTER(Step), C.c_size_t]),
+    "aionhip_session_stats": (C.c_int, [C.c_void_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
+    "aionhip_session_retire": (C.c_int, [C.c_void_p]),
+    "aionhip_session_destroy": (None, [C.c_void_p]),
     "aionhip_set_attention_precise": (C.c_int, [C.c_void_p, C.c_int]),
     "aionhip_set_gemm_mode": (C.c_int, [C.c_void_p, C.c_int]),
     "aionhip_step_attention": (C.c_int, [C.c_void_p, C.POINTER(Attention)]),

@@ -411,6 +411,101 @@ size_t aionhip_program_node_count(const aionhip_program *prog);
 int aionhip_program_is_current(const aionhip_ctx *ctx, const aionhip_program *prog);
 void aionhip_program_destroy(aionhip_ctx *ctx, aionhip_program *prog);
 
+/* ---- Session.execute(prog): a step list in one call (backend/backend.zig:24-52) ---------------
+ * The native twin of a Session over an ExecutableProgram's `steps` (runtime/executable.zig:302-345 Step, :378-400
+ * ExecutableProgram): the binding turns every step whose placement is this device into one aionhip_step record - the
+ * step's own attributes plus, for every TensorId, what the tensor store answers for it (runtime/tensor_store.zig:150-201:
+ * device address, dtype, shape) - and hands the array over; the dispatch by tag, the shape arithmetic, the re-laid weight
+ * cache and the launch-saving step patterns then live here instead of in every binding. `tag` is the Step union's tag in
+ * declaration order. Executed tags: MatMul, MatMulNT (b = the packed weight tensor as it lies on the device), ElemwiseBinary
+ * (f32 add/sub/mul/div with identical, scalar_b or contiguous_suffix_b broadcast; gate with gelu; i32 add), Unary, RMSNorm,
+ * Attention, ArgMax (last axis), Copy, GatherRows, Gather (axis 0, no batch dims, rank-2 table), RoPE1D, SequenceAppend,
+ * Cast (f32 -> f16), Transfer. Every other tag: AIONHIP_UNSUPPORTED before anything of the list has run (the list is checked
+ * as a whole first), as the reference's compiler keeps steps a backend's capability set lacks on the CPU
+ * (backend/backend.zig:85-107). */
+#define AIONHIP_MAX_RANK 8
+enum { AIONHIP_TENSOR_ROLLING = 1u,    /* a rolling sequence cache (storage/cache.zig:35-38) */
+       AIONHIP_TENSOR_WORKSPACE = 2u   /* lives in a planned workspace slot (graph/program/workspace.zig:1-60): nothing reads
+                                          its value after the last step of this list that does */ };
+typedef struct aionhip_tensor_ref {
+    aionhip_handle handle;             /* 0 = the step has no such operand */
+    int32_t dtype;                     /* aionhip_dtype */
+    uint32_t rank;
+    uint32_t flags;
+    uint32_t reserved;
+    uint64_t shape[AIONHIP_MAX_RANK];
+} aionhip_tensor_ref;
+enum { AIONHIP_STEP_MATMUL = 0, AIONHIP_STEP_ELEMWISE_BINARY = 1, AIONHIP_STEP_UNARY = 2, AIONHIP_STEP_RMSNORM = 8,
+       AIONHIP_STEP_ATTENTION = 9, AIONHIP_STEP_ARGMAX = 11, AIONHIP_STEP_COPY = 17, AIONHIP_STEP_GATHER_ROWS = 18,
+       AIONHIP_STEP_GATHER = 19, AIONHIP_STEP_ROPE1D = 21, AIONHIP_STEP_SEQUENCE_APPEND = 22, AIONHIP_STEP_CAST = 31,
+       AIONHIP_STEP_MATMUL_NT = 32, AIONHIP_STEP_TRANSFER = 33, AIONHIP_STEP_TAG_COUNT = 34 };
+enum { AIONHIP_BINARY_GATE = 10 };     /* ElemwiseBinaryOp.gate (backend/types.zig:92-109; ids 4..9 are the i32 comparisons) */
+/* Operands by tag (out / in[0..]):
+ *   MatMul, MatMulNT     out = c; a, b                       alpha, beta
+ *   ElemwiseBinary       out; a, b                           op (ElemwiseBinaryOp id), act (UnaryOp id of a gate), broadcast
+ *                                                            (ElementwiseBroadcastKind id: 0 identical, 1 scalar_a, 2 scalar_b,
+ *                                                            3 contiguous_suffix_a, 4 contiguous_suffix_b, 5 generic;
+ *                                                            runtime/executable.zig:28-35)
+ *   Unary                out; a                              op (UnaryOp id)
+ *   RMSNorm              out; x, gamma, beta, residual?      eps
+ *   Attention            out; q, k, v, query_positions?, kv_lengths?    scale, soft_cap, window_*
+ *   ArgMax               out; a                              axis
+ *   Copy                 out = dst; src
+ *   GatherRows           out; table, indices
+ *   Gather               out; data, indices                  axis, batch_dims
+ *   RoPE1D               out; x, positions                   rope_base, rope_scale, rope_proportion
+ *   SequenceAppend       out = cache; new_kv, end_index
+ *   Cast                 out; x                              (the target type is out.dtype)
+ *   Transfer             to_host = 1: in[0] = the device tensor, host receives; 0: out = the device tensor, host is read */
+typedef struct aionhip_step {
+    int32_t tag;
+    int32_t op, act, broadcast;
+    int32_t axis;
+    uint32_t batch_dims;
+    float alpha, beta;
+    float eps;
+    float scale, soft_cap;
+    uint32_t window_left, window_right, window_chunk;
+    float rope_base, rope_scale, rope_proportion;
+    int32_t to_host;
+    aionhip_tensor_ref out;
+    aionhip_tensor_ref in[5];
+    void *host;                        /* Transfer: the host bytes of the other side */
+    uint64_t host_bytes;
+} aionhip_step;
+
+typedef struct aionhip_session aionhip_session;
+/* Backend.createSession (backend/backend.zig:46-52). A session belongs to one context and one thread. */
+int aionhip_session_create(aionhip_ctx *ctx, aionhip_session **out);
+/* Which step patterns a session may run as one call (default: both). Results are the separate steps' to the bit either way.
+ * AIONHIP_FUSE_SIBLINGS: consecutive MatMul / MatMulNT steps reading one activation share its preparation and, up to eight
+ * rows, one launch (aionhip_step_matmul_batch); every tensor of the list is still written.
+ * AIONHIP_FUSE_WORKSPACE: a step whose output is an AIONHIP_TENSOR_WORKSPACE tensor read only by the step(s) right behind
+ * it is folded into them and that tensor is never written: RMSNorm (no residual) -> MatMul(s) (aionhip_step_rmsnorm_matmul),
+ * gate(gelu) -> MatMul (aionhip_step_gate_matmul), Cast f32 -> f16 -> SequenceAppend (aionhip_step_append_f16); and for one
+ * token of one sequence the two blocks of a decoder layer as one call each: RMSNorm -> q, k, v MatMuls -> RoPE1D on q and k ->
+ * Cast + SequenceAppend of k and of v (ten steps, aionhip_step_rmsnorm_qkv_rope_append), RMSNorm -> gate and up MatMuls ->
+ * gate(gelu) -> down MatMul (five steps, aionhip_step_rmsnorm_geglu_matmul). A MatMul (beta 0) whose workspace output is
+ * read only by an add right behind it that accumulates in place (x = x + t) writes x itself with beta 1, alone or as the
+ * last step of the patterns above: alpha * acc + x is rounded once either way. A pattern whose entry point answers
+ * AIONHIP_UNSUPPORTED for the shape runs as the next smaller pattern or as separate steps. aion folds at step level the same
+ * way (graph/opt/fuse_steps.zig:19-88). */
+enum { AIONHIP_FUSE_SIBLINGS = 1, AIONHIP_FUSE_WORKSPACE = 2 };
+int aionhip_session_set_fusion(aionhip_session *s, int mask);
+/* Session.execute (backend/backend.zig:42-44): runs the list in order on the context's stream; asynchronous unless the
+ * list holds a device-to-host Transfer, which returns when its bytes have arrived (backend/gpu/backend.zig:416-457). The
+ * first use of a MatMul / MatMulNT b builds its re-laid weight from the blocks on the device and keeps it for the session
+ * (keyed by address, dtype and shape: retire the session before a weight tensor's storage is released or reused, which is
+ * when the reference calls retireResources). May run between aionhip_program_begin and aionhip_program_end once the same list
+ * has run eagerly (weights built, scratch grown; no Transfer steps then). On failure aionhip_last_error names the step. */
+int aionhip_session_execute(aionhip_session *s, const aionhip_step *steps, size_t count);
+/* launches the last execute made (a folded pattern counts as its calls) and re-laid weights the session holds */
+int aionhip_session_stats(const aionhip_session *s, uint64_t *calls_last_execute, uint64_t *weights, uint64_t *weight_bytes);
+/* Session.retireResources (backend/backend.zig:36-38): waits for the stream and drops what may retain tensor backings -
+ * the re-laid weights and the bf16 copies the context made of them. The session stays usable. */
+int aionhip_session_retire(aionhip_session *s);
+void aionhip_session_destroy(aionhip_session *s);     /* Session.deinit; retires first */
+
 /* ---- timing helpers for the roofline harness (timestamp queries of the WebGPU backend,
  *      backend/gpu/timestamp_profile.zig, reduced to stream events) ------------------------- */
 int aionhip_event_create(aionhip_ctx *ctx, void **event);

@@ -96,3 +96,44 @@ def test_create_without_gpu_fails_loudly():
             "except be.AionHipError as e:\n    print('error', e.status)\n") % ROOT
     out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120).stdout
     assert "error" in out          # device 7 never exists on a one-GPU box or a CPU container
+
+
+def test_ctypes_structures_have_the_header_layout(tmp_path):
+    """The records a binding fills (attention parameters, tensor references, steps) as a C compiler lays them out from
+    include/aion_hip.h, field by field, against the ctypes mirrors the harness passes."""
+    import subprocess
+    mirrors = {"aionhip_attention": hip.Attention, "aionhip_tensor_ref": hip.TensorRef, "aionhip_step": hip.Step}
+    lines = []
+    for cname, mirror in mirrors.items():
+        lines.append('printf("%s size %%zu\\n", sizeof(%s));' % (cname, cname))
+        for field, _ in mirror._fields_:
+            lines.append('printf("%s %s %%zu\\n", offsetof(%s, %s));' % (cname, field, cname, field.rstrip("_")))
+    src = tmp_path / "layout.c"
+    src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "aion_hip.h"\nint main(void) {\n%s\nreturn 0; }\n' % "\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-std=c11", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split("\n")
+    seen = 0
+    for line in filter(None, out):
+        cname, field, value = line.split()
+        mirror = mirrors[cname]
+        if field == "size":
+            assert C.sizeof(mirror) == int(value), cname
+        else:
+            assert getattr(mirror, field).offset == int(value), (cname, field)
+        seen += 1
+    assert seen == sum(len(m._fields_) + 1 for m in mirrors.values())
+    # the step tags are the Step union's tags in declaration order (runtime/executable.zig:302-345)
+    from aion_amd import session as ss
+    order = ["MatMul", "ElemwiseBinary", "Unary", "Softmax", "Conv1D", "Conv2D", "MaxPool2D", "LayerNorm", "RMSNorm", "Attention", "RelPosMHA",
+             "ArgMax", "TopK", "ScatterRow", "ReduceAll", "ReduceAxis", "ConcatScalar", "Copy", "GatherRows", "Gather", "GatherND", "RoPE1D",
+             "SequenceAppend", "LSTMCellFused", "If", "Loop", "RFFT", "STFT", "ReshapeScalar", "Transpose2DScalar", "SliceNDScalar", "Cast",
+             "MatMulNT", "Transfer"]
+    header = open(os.path.join(ROOT, "include", "aion_hip.h")).read()
+    for name, const in (("MatMul", "MATMUL"), ("ElemwiseBinary", "ELEMWISE_BINARY"), ("Unary", "UNARY"), ("RMSNorm", "RMSNORM"),
+                        ("Attention", "ATTENTION"), ("ArgMax", "ARGMAX"), ("Copy", "COPY"), ("GatherRows", "GATHER_ROWS"), ("Gather", "GATHER"),
+                        ("RoPE1D", "ROPE1D"), ("SequenceAppend", "SEQUENCE_APPEND"), ("Cast", "CAST"), ("MatMulNT", "MATMUL_NT"),
+                        ("Transfer", "TRANSFER")):
+        assert getattr(ss, const) == order.index(name)
+        assert re.search(r"AIONHIP_STEP_%s = %d\b" % (const, order.index(name)), header), const
+    assert re.search(r"AIONHIP_STEP_TAG_COUNT = %d\b" % len(order), header)

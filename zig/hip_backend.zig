@@ -25,7 +25,6 @@ const BackendError = types.BackendError;
 const ExecuteProgramError = backend_mod.ExecuteProgramError;
 const TensorStore = tensor_store.TensorStore;
 const TensorId = tensor_store.TensorId;
-const TensorMeta = tensor_store.TensorMeta;
 
 fn check(rc: c_int) ExecuteProgramError!void {
     return switch (rc) {
@@ -40,9 +39,6 @@ fn check(rc: c_int) ExecuteProgramError!void {
 pub const HipBackend = struct {
     ctx: *c.aionhip_ctx,
     allocator: std.mem.Allocator,
-    /// Re-laid weights, keyed by the device handle of the packed tensor (weights are immutable
-    /// params, graph/graph.zig:55-58, so the key never goes stale while the tensor lives).
-    weights: std.AutoHashMap(u64, *c.aionhip_weight),
 
     /// This backend keeps aion's packed blocks as they are and re-lays privately.
     pub const quant_block_order: types.QuantBlockOrder = .row_major;
@@ -50,20 +46,13 @@ pub const HipBackend = struct {
     pub fn init(allocator: std.mem.Allocator, device_index: c_int) !HipBackend {
         var ctx: ?*c.aionhip_ctx = null;
         if (c.aionhip_create(device_index, null, &ctx) != c.AIONHIP_OK) return error.BackendUnavailable;
-        return .{ .ctx = ctx.?, .allocator = allocator, .weights = std.AutoHashMap(u64, *c.aionhip_weight).init(allocator) };
+        return .{ .ctx = ctx.?, .allocator = allocator };
     }
 
     /// The owner calls this; the vtable's `deinit` is a no-op like backend/gpu/backend.zig:675-678.
+    /// Sessions are destroyed first (each frees the re-laid weights it holds through this context).
     pub fn deinit(self: *HipBackend) void {
-        self.dropWeights();
-        self.weights.deinit();
         c.aionhip_destroy(self.ctx);
-    }
-
-    fn dropWeights(self: *HipBackend) void {
-        var it = self.weights.valueIterator();
-        while (it.next()) |w| c.aionhip_weight_free(self.ctx, w.*);
-        self.weights.clearRetainingCapacity();
     }
 
     // ---- Backend.VTable (backend/backend.zig:58-73)
@@ -79,8 +68,7 @@ pub const HipBackend = struct {
     fn deinitImpl(_: *anyopaque) void {}
     fn createSessionImpl(p: *anyopaque, store: TensorStore) tensor_store.StoreError!Session {
         const self: *HipBackend = @ptrCast(@alignCast(p));
-        const s = self.allocator.create(HipSession) catch return error.OutOfMemory;
-        s.* = .{ .hb = self, .host = store };
+        const s = try HipSession.create(self, store);
         return .{ .ctx = @ptrCast(s), .vtable = &HipSession.session_vtable };
     }
     const vtable = Backend.VTable{ .kind = kindImpl, .name = nameImpl, .caps = capsImpl, .deinit = deinitImpl, .createSession = createSessionImpl };
@@ -100,7 +88,6 @@ pub const HipBackend = struct {
     }
     fn dmFree(p: *anyopaque, h: dm.DeviceHandle) void {
         const self: *HipBackend = @ptrCast(@alignCast(p));
-        if (self.weights.fetchRemove(h)) |kv| c.aionhip_weight_free(self.ctx, kv.value);
         c.aionhip_free(self.ctx, h);
     }
     fn dmH2D(p: *anyopaque, h: dm.DeviceHandle, off: usize, src: []const u8) dm.DeviceError!void {
@@ -124,25 +111,58 @@ pub const HipBackend = struct {
 
     /// A session bound to one placed tensor store (backend/gpu/backend.zig:206-270). Tensors the store placed on
     /// this device answer `deviceChunk` (runtime/tensor_store.zig:150-201) with one chunk: the whole buffer.
+    /// Execution is the library's: every step becomes one `aionhip_step` record (its attributes plus, per TensorId,
+    /// address, dtype and shape) and `aionhip_session_execute` dispatches, keeps the re-laid weights and folds the
+    /// launch-saving step patterns. What stays here is what needs the store: resolving ids and host-side Transfers.
     pub const HipSession = struct {
         hb: *HipBackend,
         host: TensorStore,
+        native: *c.aionhip_session,
+        records: std.ArrayListUnmanaged(c.aionhip_step) = .{},
+
+        pub fn create(hb: *HipBackend, store: TensorStore) tensor_store.StoreError!*HipSession {
+            var native: ?*c.aionhip_session = null;
+            if (c.aionhip_session_create(hb.ctx, &native) != c.AIONHIP_OK) return error.OutOfMemory;
+            const s = hb.allocator.create(HipSession) catch {
+                c.aionhip_session_destroy(native.?);
+                return error.OutOfMemory;
+            };
+            s.* = .{ .hb = hb, .host = store, .native = native.? };
+            return s;
+        }
 
         fn execute(p: *anyopaque, prog: *const executable.ExecutableProgram) ExecuteProgramError!void {
             const s: *HipSession = @ptrCast(@alignCast(p));
             // a program carries the placement it was compiled for (backend/gpu/backend.zig:551-560)
             if (prog.target.kind != .hip) return BackendError.Unsupported;
-            for (prog.steps) |placed| try s.dispatchStep(placed.op);
+            s.records.clearRetainingCapacity();
+            for (prog.steps) |placed| {
+                switch (placed.op) {
+                    // a Transfer touches host storage under the store's access tokens: run what has gathered, then copy
+                    .Transfer => |t| {
+                        try s.flush();
+                        try s.runTransfer(t);
+                    },
+                    else => s.records.append(s.hb.allocator, try s.record(prog, placed.op)) catch return tensor_store.StoreError.OutOfMemory,
+                }
+            }
+            try s.flush();
+        }
+        fn flush(s: *HipSession) ExecuteProgramError!void {
+            if (s.records.items.len == 0) return;
+            defer s.records.clearRetainingCapacity();
+            try check(c.aionhip_session_execute(s.native, s.records.items.ptr, s.records.items.len));
         }
         /// Wait for the stream, then drop what may retain tensor backings: the re-laid weights and the
         /// bf16 copies the context made of them. Called only before storage eviction (backend.zig:36-38).
         fn retireResources(p: *anyopaque) void {
             const s: *HipSession = @ptrCast(@alignCast(p));
-            _ = c.aionhip_sync(s.hb.ctx);
-            s.hb.dropWeights();
+            _ = c.aionhip_session_retire(s.native);
         }
         fn deinitSession(p: *anyopaque) void {
             const s: *HipSession = @ptrCast(@alignCast(p));
+            c.aionhip_session_destroy(s.native);
+            s.records.deinit(s.hb.allocator);
             s.hb.allocator.destroy(s);
         }
         const session_vtable = Session.VTable{ .execute = execute, .retireResources = retireResources, .deinit = deinitSession };
@@ -151,136 +171,131 @@ pub const HipBackend = struct {
             const ref = (try s.host.deviceChunk(id, 0)) orelse return BackendError.InvalidArgument;
             return ref.handle;
         }
-        fn optAddr(s: *HipSession, id: ?TensorId) ExecuteProgramError!u64 {
-            return if (id) |t| try s.addr(t) else 0;
+
+        /// What the store answers for one tensor id, as the library wants it. A tensor in one of the program's shared
+        /// workspace slots (runtime/executable.zig:624-636) that is not a program output is dead after its last reader:
+        /// the library may then fold the step that writes it into its consumer.
+        fn tensorRef(s: *HipSession, prog: *const executable.ExecutableProgram, id: TensorId) ExecuteProgramError!c.aionhip_tensor_ref {
+            const m = try s.host.meta(id);
+            var t: c.aionhip_tensor_ref = std.mem.zeroes(c.aionhip_tensor_ref);
+            if (m.rank > c.AIONHIP_MAX_RANK) return BackendError.Unsupported;
+            t.handle = try s.addr(id);
+            t.dtype = @intFromEnum(m.dtype);
+            t.rank = m.rank;
+            for (0..m.rank) |d| t.shape[d] = m.shape[d];
+            if (s.host.sequenceCachePolicyInfo(id).kind == .rolling) t.flags |= c.AIONHIP_TENSOR_ROLLING;
+            if (inWorkspace(prog, id)) t.flags |= c.AIONHIP_TENSOR_WORKSPACE;
+            return t;
+        }
+        fn optRef(s: *HipSession, prog: *const executable.ExecutableProgram, id: ?TensorId) ExecuteProgramError!c.aionhip_tensor_ref {
+            return if (id) |t| try s.tensorRef(prog, t) else std.mem.zeroes(c.aionhip_tensor_ref);
+        }
+        fn inWorkspace(prog: *const executable.ExecutableProgram, id: TensorId) bool {
+            for (prog.outputs) |o| if (o == id) return false;
+            for (prog.workspace_slots) |slot| {
+                for (slot.members) |m| if (m == id) return true;
+            }
+            return false;
         }
 
-        // weights: re-laid at first use, straight from the packed blocks already on the device
-        fn weightFor(s: *HipSession, id: TensorId, layout: c_int) ExecuteProgramError!*c.aionhip_weight {
-            const hb = s.hb;
-            const meta = try s.host.meta(id);
-            const handle = try s.addr(id);
-            if (hb.weights.get(handle)) |w| return w;
-            const n = if (layout == c.AIONHIP_ROWS_NK) meta.shape[0] else meta.shape[1];
-            const k = if (layout == c.AIONHIP_ROWS_NK) meta.shape[1] else meta.shape[0];
-            var w: ?*c.aionhip_weight = null;
-            try check(c.aionhip_weight_from_device(hb.ctx, @intFromEnum(meta.dtype), layout, n, k, 0, handle, &w));
-            hb.weights.put(handle, w.?) catch return tensor_store.StoreError.OutOfMemory;
-            return w.?;
-        }
-
-        /// One step of a validated program (the reduced twin of backend/gpu/backend.zig:459-548): the steps of
-        /// a quantized decoder; every other tag is Unsupported and the compiler keeps it on the CPU.
-        fn dispatchStep(s: *HipSession, step: executable.Step) ExecuteProgramError!void {
-            const ctx = s.hb.ctx;
+        /// One step of a validated program as a record: `tag` is the Step union's own tag (declaration order,
+        /// runtime/executable.zig:302-345), operands by role as include/aion_hip.h lists them. Tags the device does
+        /// not run are passed on as they are: the library answers Unsupported for the list before it launches
+        /// anything, and the compiler keeps such steps on the CPU (backend/backend.zig:85-107).
+        fn record(s: *HipSession, prog: *const executable.ExecutableProgram, step: executable.Step) ExecuteProgramError!c.aionhip_step {
+            var r: c.aionhip_step = std.mem.zeroes(c.aionhip_step);
+            r.tag = @intFromEnum(std.meta.activeTag(step));
             switch (step) {
                 .MatMul => |m| {
-                    const w = try s.weightFor(m.b, c.AIONHIP_KMAJOR_KN);
-                    try check(c.aionhip_step_matmul(ctx, w, rowsOf(try s.host.meta(m.a)), try s.addr(m.a), 0, try s.addr(m.c), 0, m.alpha, m.beta));
+                    r.out = try s.tensorRef(prog, m.c);
+                    r.in[0] = try s.tensorRef(prog, m.a);
+                    r.in[1] = try s.tensorRef(prog, m.b);
+                    r.alpha = m.alpha;
+                    r.beta = m.beta;
                 },
                 .MatMulNT => |m| {
-                    const w = try s.weightFor(m.b, c.AIONHIP_ROWS_NK);
-                    try check(c.aionhip_step_matmul_nt(ctx, w, rowsOf(try s.host.meta(m.a)), try s.addr(m.a), 0, try s.addr(m.c), 0, m.alpha, m.beta));
-                },
-                .Attention => |a| {
-                    const qm = try s.host.meta(a.q);
-                    const km = try s.host.meta(a.k);
-                    const vm = try s.host.meta(a.v);
-                    var p: c.aionhip_attention = std.mem.zeroes(c.aionhip_attention);
-                    p.out = try s.addr(a.out);
-                    p.q = try s.addr(a.q);
-                    p.k = try s.addr(a.k);
-                    p.v = try s.addr(a.v);
-                    p.query_positions = try s.optAddr(a.query_positions);
-                    p.kv_lengths = try s.optAddr(a.kv_lengths);
-                    p.batch = qm.shape[0]; p.l_q = qm.shape[1]; p.h_q = qm.shape[2]; p.d_k = qm.shape[3];
-                    p.t_kv = km.shape[1]; p.h_kv = km.shape[2]; p.d_v = vm.shape[3];
-                    p.q_dtype = @intFromEnum(qm.dtype); p.kv_dtype = @intFromEnum(km.dtype);
-                    p.scale = a.scale; p.attn_logits_soft_cap = a.attn_logits_soft_cap;
-                    p.window_left = a.window.left; p.window_right = a.window.right; p.window_chunk = a.window.chunk;
-                    // a rolling sequence cache reads key t from row t % capacity (cpu/exec/attention.zig:1537-1546)
-                    p.rolling = if (s.host.sequenceCachePolicyInfo(a.k).kind == .rolling) 1 else 0;
-                    try check(c.aionhip_step_attention(ctx, &p));
-                },
-                .RMSNorm => |n| {
-                    const cols = elemCount(try s.host.meta(n.gamma));
-                    try check(c.aionhip_step_rmsnorm(ctx, try s.addr(n.out), try s.addr(n.x), try s.addr(n.gamma), try s.addr(n.beta),
-                        try s.optAddr(n.residual), elemCount(try s.host.meta(n.out)) / cols, cols, n.eps));
-                },
-                .RoPE1D => |r| {
-                    const m = try s.host.meta(r.out);
-                    try check(c.aionhip_step_rope(ctx, try s.addr(r.out), try s.addr(r.x), try s.addr(r.positions),
-                        m.shape[0], m.shape[1], m.shape[2], m.shape[3], r.base_frequency, r.scale_factor, r.rope_proportion));
-                },
-                .ArgMax => |a| {
-                    const m = try s.host.meta(a.a);
-                    if (a.axis + 1 != m.rank) return BackendError.Unsupported;
-                    const n = m.shape[m.rank - 1];
-                    try check(c.aionhip_step_argmax(ctx, try s.addr(a.out), try s.addr(a.a), elemCount(m) / n, n));
+                    r.out = try s.tensorRef(prog, m.c);
+                    r.in[0] = try s.tensorRef(prog, m.a);
+                    r.in[1] = try s.tensorRef(prog, m.b);
+                    r.alpha = m.alpha;
+                    r.beta = m.beta;
                 },
                 .ElemwiseBinary => |e| {
-                    const am = try s.host.meta(e.a);
-                    const n = elemCount(try s.host.meta(e.out));
-                    if (am.dtype == .i32) {
-                        // the decode counters (position + 1): same-shape i32 add only
-                        if (e.op != .add or e.broadcast.kind != .identical) return BackendError.Unsupported;
-                        return check(c.aionhip_step_add_i32(ctx, try s.addr(e.out), try s.addr(e.a), try s.addr(e.b), n));
-                    }
-                    if (e.op == .gate) {
-                        // gate(a, b) = act(a) * b (backend/types.zig:105-109); the device kernel is the gelu form
-                        if (e.act != .gelu or e.broadcast.kind != .identical) return BackendError.Unsupported;
-                        return check(c.aionhip_step_gate_gelu(ctx, try s.addr(e.out), try s.addr(e.a), try s.addr(e.b), n));
-                    }
-                    // add/sub/mul/div carry ElemwiseBinaryOp's own ids (backend/types.zig:92-96) across the ABI;
-                    // b may be the same shape, one element or a contiguous suffix of a's shape
-                    const op: c_int = switch (e.op) {
-                        .add, .sub, .mul, .div => @intFromEnum(e.op),
-                        else => return BackendError.Unsupported,
-                    };
-                    const nb: usize = switch (e.broadcast.kind) {
-                        .identical => n,
-                        .scalar_b => 1,
-                        .contiguous_suffix_b => elemCount(try s.host.meta(e.b)),
-                        else => return BackendError.Unsupported,
-                    };
-                    try check(c.aionhip_step_binary(ctx, op, try s.addr(e.out), try s.addr(e.a), try s.addr(e.b), n, nb));
+                    r.out = try s.tensorRef(prog, e.out);
+                    r.in[0] = try s.tensorRef(prog, e.a);
+                    r.in[1] = try s.tensorRef(prog, e.b);
+                    r.op = @intFromEnum(e.op);
+                    r.act = @intFromEnum(e.act);
+                    r.broadcast = @intFromEnum(e.broadcast.kind);
                 },
                 .Unary => |u| {
-                    // UnaryOp's ids are the ABI's (backend/types.zig:119-128); log answers AIONHIP_UNSUPPORTED
-                    try check(c.aionhip_step_unary(ctx, @intFromEnum(u.op), try s.addr(u.out), try s.addr(u.a), elemCount(try s.host.meta(u.out))));
+                    r.out = try s.tensorRef(prog, u.out);
+                    r.in[0] = try s.tensorRef(prog, u.a);
+                    r.op = @intFromEnum(u.op);
                 },
-                .Gather => |g| {
-                    // embedding lookup: rows of a [V, D] table (f32, or q8_0 blocked along D) by i32 ids
-                    const tm = try s.host.meta(g.data);
-                    if (g.axis != 0 or g.batch_dims != 0 or tm.rank != 2) return BackendError.Unsupported;
-                    try check(c.aionhip_step_gather_rows(ctx, @intFromEnum(tm.dtype), try s.addr(g.out), try s.addr(g.data), try s.addr(g.indices),
-                        elemCount(try s.host.meta(g.indices)), tm.shape[1], tm.shape[0]));
+                .RMSNorm => |n| {
+                    r.out = try s.tensorRef(prog, n.out);
+                    r.in[0] = try s.tensorRef(prog, n.x);
+                    r.in[1] = try s.tensorRef(prog, n.gamma);
+                    r.in[2] = try s.tensorRef(prog, n.beta);
+                    r.in[3] = try s.optRef(prog, n.residual);
+                    r.eps = n.eps;
                 },
-                .GatherRows => |g| {
-                    const tm = try s.host.meta(g.table);
-                    try check(c.aionhip_step_gather_rows(ctx, @intFromEnum(tm.dtype), try s.addr(g.out), try s.addr(g.table), try s.addr(g.indices),
-                        elemCount(try s.host.meta(g.indices)), tm.shape[1], tm.shape[0]));
+                .Attention => |a| {
+                    r.out = try s.tensorRef(prog, a.out);
+                    r.in[0] = try s.tensorRef(prog, a.q);
+                    r.in[1] = try s.tensorRef(prog, a.k);
+                    r.in[2] = try s.tensorRef(prog, a.v);
+                    r.in[3] = try s.optRef(prog, a.query_positions);
+                    r.in[4] = try s.optRef(prog, a.kv_lengths);
+                    r.scale = a.scale;
+                    r.soft_cap = a.attn_logits_soft_cap;
+                    r.window_left = a.window.left;
+                    r.window_right = a.window.right;
+                    r.window_chunk = a.window.chunk;
                 },
-                .Cast => |k| {
-                    const xm = try s.host.meta(k.x);
-                    if (xm.dtype != .f32 or k.to_dtype != .f16) return BackendError.Unsupported;
-                    try check(c.aionhip_step_cast_f32_f16(ctx, try s.addr(k.out), try s.addr(k.x), elemCount(xm)));
-                },
-                .SequenceAppend => |a| {
-                    // cache [B, T, H, D] and rows [B, S, H, D] of one element type (cpu/exec/sequence_append.zig:29-31)
-                    const cm = try s.host.meta(a.cache);
-                    const nm = try s.host.meta(a.new_kv);
-                    const rolling: c_int = if (s.host.sequenceCachePolicyInfo(a.cache).kind == .rolling) 1 else 0;
-                    try check(c.aionhip_step_sequence_append(ctx, @intFromEnum(cm.dtype), try s.addr(a.cache), try s.addr(a.new_kv), try s.addr(a.end_index),
-                        cm.shape[0], nm.shape[1], cm.shape[1], cm.shape[2] * cm.shape[3], rolling));
+                .ArgMax => |a| {
+                    r.out = try s.tensorRef(prog, a.out);
+                    r.in[0] = try s.tensorRef(prog, a.a);
+                    r.axis = @intCast(a.axis);
                 },
                 .Copy => |k| {
-                    const m = try s.host.meta(k.dst);
-                    try check(c.aionhip_d2d(ctx, try s.addr(k.dst), 0, try s.addr(k.src), 0, byteCount(m)));
+                    r.out = try s.tensorRef(prog, k.dst);
+                    r.in[0] = try s.tensorRef(prog, k.src);
                 },
-                .Transfer => |t| try s.runTransfer(t),
-                else => return BackendError.Unsupported,
+                .GatherRows => |g| {
+                    r.out = try s.tensorRef(prog, g.out);
+                    r.in[0] = try s.tensorRef(prog, g.table);
+                    r.in[1] = try s.tensorRef(prog, g.indices);
+                },
+                .Gather => |g| {
+                    r.out = try s.tensorRef(prog, g.out);
+                    r.in[0] = try s.tensorRef(prog, g.data);
+                    r.in[1] = try s.tensorRef(prog, g.indices);
+                    r.axis = @intCast(g.axis);
+                    r.batch_dims = @intCast(g.batch_dims);
+                },
+                .RoPE1D => |p| {
+                    r.out = try s.tensorRef(prog, p.out);
+                    r.in[0] = try s.tensorRef(prog, p.x);
+                    r.in[1] = try s.tensorRef(prog, p.positions);
+                    r.rope_base = p.base_frequency;
+                    r.rope_scale = p.scale_factor;
+                    r.rope_proportion = p.rope_proportion;
+                },
+                .SequenceAppend => |a| {
+                    r.out = try s.tensorRef(prog, a.cache);
+                    r.in[0] = try s.tensorRef(prog, a.new_kv);
+                    r.in[1] = try s.tensorRef(prog, a.end_index);
+                },
+                .Cast => |k| {
+                    r.out = try s.tensorRef(prog, k.out);
+                    r.in[0] = try s.tensorRef(prog, k.x);
+                },
+                // no operands needed: the tag alone makes the library answer Unsupported for the list
+                else => {},
             }
+            return r;
         }
 
         /// Host <-> device copy placed by the compiler (backend/gpu/backend.zig:416-457). Both copies are ordered on
@@ -306,30 +321,18 @@ pub const HipBackend = struct {
         }
     };
 
-    // Optional launch-saving pattern matches over consecutive steps of a decode program; each gives the results of
-    // the separate steps bit for bit, and a maintainer falls back to those on AIONHIP_UNSUPPORTED:
-    //   RMSNorm, MatMul x3 (q,k,v), RoPE1D x2, Cast f16 x2, SequenceAppend x2 -> aionhip_step_rmsnorm_qkv_rope_append
-    //   RMSNorm x3 (per head, q,k,v), RoPE1D x2, Cast f16 x2, SequenceAppend x2 -> aionhip_step_headnorm_rope_append
-    //   RMSNorm, MatMul x2 (gate, up), gate(gelu), MatMul (down)             -> aionhip_step_rmsnorm_geglu_matmul
-    //   RMSNorm, MatMul(s)                                                   -> aionhip_step_rmsnorm_matmul
-    //   gate(gelu), MatMul                                                   -> aionhip_step_gate_matmul
-    //   MatMul(s) sharing one A                                              -> aionhip_step_matmul_batch
-    //   Cast f32->f16 feeding only a SequenceAppend                          -> aionhip_step_append_f16
-    // A whole decode program (no If/Loop) may be recorded once between aionhip_program_begin/_end and replayed with
-    // aionhip_program_execute while aionhip_program_is_current holds (replay precedent: backend/gpu/frame.zig:77-86).
-
-    fn rowsOf(m: TensorMeta) usize {
-        var r: usize = 1;
-        for (0..m.rank - 1) |d| r *= m.shape[d];
-        return r;
-    }
-    fn elemCount(m: TensorMeta) usize {
-        var r: usize = 1;
-        for (0..m.rank) |d| r *= m.shape[d];
-        return r;
-    }
-    fn byteCount(m: TensorMeta) usize {
-        const info = m.dtype.info();
-        return elemCount(m) / info.block_elems * info.block_bytes;
-    }
+    // What aionhip_session_execute folds (each gives the separate steps' results bit for bit; AIONHIP_FUSE_* of
+    // aionhip_session_set_fusion switches them off):
+    //   RMSNorm, MatMul x3 (q,k,v), RoPE1D x2, Cast f16 x2, SequenceAppend x2, one token -> aionhip_step_rmsnorm_qkv_rope_append
+    //   RMSNorm, MatMul x2 (gate, up), gate(gelu), MatMul (down), one row              -> aionhip_step_rmsnorm_geglu_matmul
+    //   RMSNorm, MatMul(s)                                                             -> aionhip_step_rmsnorm_matmul
+    //   gate(gelu), MatMul                                                             -> aionhip_step_gate_matmul
+    //   Cast f32->f16, SequenceAppend                                                  -> aionhip_step_append_f16
+    //   MatMul(s) sharing one A                                                        -> aionhip_step_matmul_batch
+    //   MatMul, add in place (x = x + t), alone or behind the patterns above           -> the matmul with C = x, beta = 1
+    // Not folded there (a maintainer may match it here): RMSNorm x3 per head, RoPE1D x2, Cast x2, SequenceAppend x2
+    //   -> aionhip_step_headnorm_rope_append.
+    // A whole decode program (no If/Loop, no Transfer) may be recorded once between aionhip_program_begin/_end around
+    // aionhip_session_execute and replayed with aionhip_program_execute while aionhip_program_is_current holds (replay
+    // precedent: backend/gpu/frame.zig:77-86).
 };
