@@ -309,3 +309,151 @@ class Decoder:
                 t.free()
         for t in (self.embed, self.gamma, self.one, self.logits, self.token, self.history):
             t.free()
+
+
+class SessionDecoder:
+    """The same decoder the way a compiled aion program reaches a backend: one record per step of the sequence in this
+    module's header, nothing pre-fused, handed to the library's session executor (aionhip_session_execute), which folds
+    what it may. Parameters are device tensors in aion's packed form; the session re-lays them at first use. The residual
+    adds accumulate in place (x = x + o), the activations between the block's input and its output are workspace tensors.
+    Gives the tokens of `Decoder` over the same weights."""
+
+    def __init__(self, gpu, cfg, weights, fusion=None):
+        from . import session as ss
+        self.ss, self.gpu, self.cfg = ss, gpu, cfg
+        self.sess = ss.Session(gpu)
+        if fusion is not None:
+            self.sess.set_fusion(fusion)
+        self.nt = cfg.wdtype == be.Q8_0
+        self.w = {name: gpu.upload(weights.blocks(name)) for name in weight_shapes(cfg)}
+        self.embed = gpu.upload(weights.embed())
+        self.gamma = gpu.upload(np.ones(cfg.hidden, np.float32))
+        kv_bytes = cfg.max_seq * cfg.kv_dim * 2
+        self.kc = [gpu.zeros(kv_bytes) for _ in range(cfg.layers)]
+        self.vc = [gpu.zeros(kv_bytes) for _ in range(cfg.layers)]
+        self.one = gpu.upload(np.ones(1, np.int32))
+        self.logits = gpu.alloc(cfg.vocab * 4)
+        self.token = gpu.alloc(4)
+        self.state = {}
+        self.program = None
+        self.pos = 0
+
+    def _weight(self, name):
+        n, k = weight_shapes(self.cfg)[name]
+        return self.ss.tensor(self.w[name], self.cfg.wdtype, (n, k) if self.nt else (k, n))
+
+    def _program(self, s, advance=False):
+        """-> (buffers, step records) of one forward pass over `s` tokens; advance: the loop state moves on the device
+        behind it (the produced token becomes the next input, the three counters go up by one)."""
+        key = (s, advance)
+        if key in self.state:
+            return self.state[key]
+        c, g, ss = self.cfg, self.gpu, self.ss
+        f4 = 4 * s
+        b = self.state[(s, not advance)][0] if (s, not advance) in self.state else {
+            "ids": g.alloc(4 * s), "positions": g.alloc(4 * s), "write_index": g.alloc(4), "kv_len": g.alloc(4),
+            "x": g.alloc(f4 * c.hidden), "h": g.alloc(f4 * c.hidden), "o": g.alloc(f4 * c.hidden), "q": g.alloc(f4 * c.q_dim),
+            "qr": g.alloc(f4 * c.q_dim), "att": g.alloc(f4 * c.q_dim), "k": g.alloc(f4 * c.kv_dim), "kr": g.alloc(f4 * c.kv_dim),
+            "v": g.alloc(f4 * c.kv_dim), "k16": g.alloc(2 * s * c.kv_dim), "v16": g.alloc(2 * s * c.kv_dim), "gate": g.alloc(f4 * c.ffn),
+            "up": g.alloc(f4 * c.ffn), "act": g.alloc(f4 * c.ffn), "hl": g.alloc(4 * c.hidden)}
+        work = lambda nm, *shape: ss.tensor(b[nm], be.F32, shape, workspace=True)  # noqa: E731
+        x = ss.tensor(b["x"], be.F32, (1, s, c.hidden))
+        gamma = ss.tensor(self.gamma, be.F32, (c.hidden,))
+        pos, widx, kvl = (ss.tensor(b[nm], be.I32, shape) for nm, shape in (("positions", (1, s)), ("write_index", (1,)), ("kv_len", (1,))))
+        mm = (lambda p, a, w, out, **kw: p.matmul_nt(a, w, out, **kw)) if self.nt else (lambda p, a, w, out, **kw: p.matmul(a, w, out, **kw))
+        p = ss.Steps()
+        p.gather_rows(ss.tensor(self.embed, be.F32, (c.vocab, c.hidden)), ss.tensor(b["ids"], be.I32, (1, s)), x)
+        for l in range(c.layers):
+            n = "l%d." % l
+            kc = ss.tensor(self.kc[l], be.F16, (1, c.max_seq, c.kv_heads, c.head_dim))
+            vc = ss.tensor(self.vc[l], be.F16, (1, c.max_seq, c.kv_heads, c.head_dim))
+            p.rmsnorm(x, gamma, None, work("h", 1, s, c.hidden), c.eps)
+            mm(p, work("h", 1, s, c.hidden), self._weight(n + "wq"), work("q", 1, s, c.q_dim))
+            mm(p, work("h", 1, s, c.hidden), self._weight(n + "wk"), work("k", 1, s, c.kv_dim))
+            mm(p, work("h", 1, s, c.hidden), self._weight(n + "wv"), work("v", 1, s, c.kv_dim))
+            p.rope1d(work("q", 1, s, c.heads, c.head_dim), pos, work("qr", 1, s, c.heads, c.head_dim), base_frequency=c.rope_base)
+            p.rope1d(work("k", 1, s, c.kv_heads, c.head_dim), pos, work("kr", 1, s, c.kv_heads, c.head_dim), base_frequency=c.rope_base)
+            k16 = ss.tensor(b["k16"], be.F16, (1, s, c.kv_heads, c.head_dim), workspace=True)
+            v16 = ss.tensor(b["v16"], be.F16, (1, s, c.kv_heads, c.head_dim), workspace=True)
+            p.cast(work("kr", 1, s, c.kv_heads, c.head_dim), k16)
+            p.sequence_append(kc, k16, widx)
+            p.cast(work("v", 1, s, c.kv_heads, c.head_dim), v16)
+            p.sequence_append(vc, v16, widx)
+            p.attention(work("qr", 1, s, c.heads, c.head_dim), kc, vc, work("att", 1, s, c.heads, c.head_dim), 1.0 / math.sqrt(c.head_dim),
+                        query_positions=pos, kv_lengths=kvl)
+            mm(p, work("att", 1, s, c.q_dim), self._weight(n + "wo"), work("o", 1, s, c.hidden))
+            p.elemwise_binary(ss.ADD, x, work("o", 1, s, c.hidden), x)
+            p.rmsnorm(x, gamma, None, work("h", 1, s, c.hidden), c.eps)
+            mm(p, work("h", 1, s, c.hidden), self._weight(n + "wgate"), work("gate", 1, s, c.ffn))
+            mm(p, work("h", 1, s, c.hidden), self._weight(n + "wup"), work("up", 1, s, c.ffn))
+            p.elemwise_binary(ss.GATE, work("gate", 1, s, c.ffn), work("up", 1, s, c.ffn), work("act", 1, s, c.ffn), act=ss.GELU)
+            mm(p, work("act", 1, s, c.ffn), self._weight(n + "wdown"), work("o", 1, s, c.hidden))
+            p.elemwise_binary(ss.ADD, x, work("o", 1, s, c.hidden), x)
+        last = ss.tensor(b["x"], be.F32, (1, c.hidden), offset=(s - 1) * c.hidden * 4)
+        p.rmsnorm(last, gamma, None, work("hl", 1, c.hidden), c.eps)
+        mm(p, work("hl", 1, c.hidden), self._weight("lm_head"), ss.tensor(self.logits, be.F32, (1, c.vocab)))
+        p.argmax(ss.tensor(self.logits, be.F32, (1, c.vocab)), ss.tensor(self.token, be.I32, (1,)), axis=1)
+        if advance:
+            one = ss.tensor(self.one, be.I32, (1,))
+            p.copy(ss.tensor(self.token, be.I32, (1,)), ss.tensor(b["ids"], be.I32, (1,)))
+            for t in (pos, widx, kvl):
+                p.elemwise_binary(ss.ADD, t, one, t)
+        self.state[key] = (b, p, p.array())
+        return self.state[key]
+
+    def _set_state(self, b, tokens, pos):
+        g, t = self.gpu, np.ascontiguousarray(tokens, np.int32)
+        g.write(b["ids"], t)
+        g.write(b["positions"], np.arange(pos, pos + t.size, dtype=np.int32))
+        g.write(b["write_index"], np.array([pos], np.int32))
+        g.write(b["kv_len"], np.array([pos + t.size], np.int32))
+
+    def prefill(self, tokens):
+        s = len(tokens)
+        if self.pos + s > self.cfg.max_seq:
+            raise ValueError("prompt exceeds the cache capacity")
+        b, _, arr = self._program(s)
+        self._set_state(b, tokens, self.pos)
+        self.sess.execute(arr)
+        self.pos += s
+        return int(self.gpu.download(self.token, np.int32, (1,))[0])
+
+    def logits_host(self):
+        return self.gpu.download(self.logits, np.float32, (self.cfg.vocab,))
+
+    def begin_decode(self, first_token):
+        """One eager step at the current position (weights, scratch), rolled back, then the list recorded as a program."""
+        g = self.gpu
+        b, _, arr = self._program(1, advance=True)
+        if self.program is not None and not g.program_is_current(self.program):
+            g.program_destroy(self.program)
+            self.program = None
+        if self.program is None:
+            self._set_state(b, [first_token], self.pos)
+            self.sess.execute(arr)
+            g.sync()
+            self.calls_per_step = self.sess.stats()[0]
+            self.program = g.record_program(lambda: self.sess.execute(arr))
+        self._set_state(b, [first_token], self.pos)
+
+    def decode_step(self, read_token=True):
+        if self.pos + 1 > self.cfg.max_seq:
+            raise ValueError("cache capacity exhausted")
+        self.gpu.program_execute(self.program)
+        self.pos += 1
+        return int(self.gpu.download(self.token, np.int32, (1,))[0]) if read_token else None
+
+    def close(self):
+        if self.program is not None:
+            self.gpu.program_destroy(self.program)
+            self.program = None
+        self.sess.close()
+        for buf in list(self.w.values()) + [self.embed, self.gamma, self.one, self.logits, self.token] + self.kc + self.vc:
+            buf.free()
+        seen = set()
+        for b, _, _ in self.state.values():
+            for buf in b.values():
+                if id(buf) not in seen:
+                    seen.add(id(buf))
+                    buf.free()
+        self.state = {}

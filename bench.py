@@ -23,8 +23,9 @@ path, TFLOP/s against the named MFMA peak, with the tolerance class of each) and
 HBM peak), plus "sweep": config 2's q8 legs and batch 4 / 8 per shape, and "attention": config 4's longest prompt and
 largest decode shape. `--headline-only` skips the secondary object (and
 with it every stream capture: the form to run under rocprofv3, which does not survive a capture in the traced process).
-`--extras gemm,attention,decoder[,decoder_eager,package,package_bench_shape,package_bench_shape_eager]` adds the full config-3 and
-config-4 tables, the decoder with its CPU-oracle leg, and the package runner in an "extras" object.
+`--extras gemm,attention,decoder[,decoder_eager,session_decode,package,package_bench_shape,package_bench_shape_eager]` adds the full
+config-3 and config-4 tables, the decoder with its CPU-oracle leg, the decoder as an unfused step list on the library's session
+executor, and the package runner in an "extras" object.
 """
 import argparse
 import json
@@ -110,7 +111,7 @@ def main():
     ap.add_argument("--sweep", action="store_true", help="(kept for compatibility: the sweep is part of the default run)")
     ap.add_argument("--headline-only", action="store_true", help="skip the secondary metrics (prefill GEMM, decode, sweep)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--extras", default="", help="comma list of gemm,attention,decoder,decode_stack,package,package_bench_shape")
+    ap.add_argument("--extras", default="", help="comma list of gemm,attention,decoder,decode_stack,session_decode,package,package_bench_shape")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU (aion runs one program on one device, and no multi-GPU figure is asked for); "
@@ -280,6 +281,8 @@ def main():
             out["extras"]["decoder"] = run_decoder(gpu, be, with_cpu=not args.no_cpu)
         if "decode_stack" in extras or "decode_stack_only" in extras:
             out["extras"]["decode_stack"] = run_decode_stack(gpu, be, compare="decode_stack" in extras)
+        if "session_decode" in extras:
+            out["extras"]["session_decode"] = run_session_decode(gpu, be)
         if "decoder_eager" in extras:
             out["extras"]["decoder_eager"] = run_decoder_eager(gpu, be)
         if "package" in extras:
@@ -595,6 +598,43 @@ def run_decoder_eager(gpu, be, steps=8):
         tok = dec.decode_step_eager(tok)
     gpu.sync()
     return {"steps": steps, "eager_ms_per_token": round((time.perf_counter() - t) / steps * 1e3, 4)}
+
+
+def run_session_decode(gpu, be):
+    """Config 5 as a compiled program reaches a backend: one record per graph step (24 per block, nothing pre-fused), run by the
+    library's session executor (aionhip_session_execute), recorded as a program and replayed; beside the hand-routed Decoder
+    over the same weights, whose prefill logits and 128 tokens it must reproduce."""
+    from aion_amd.decoder import Decoder, DecoderConfig, SessionDecoder, SyntheticWeights
+    cfg = DecoderConfig()
+    w = SyntheticWeights(cfg, 0)
+    prompt = np.random.default_rng(5).integers(0, cfg.vocab, 128).astype(np.int32)
+    dec, ses = Decoder(gpu, cfg, w), SessionDecoder(gpu, cfg, w)
+    ta, tb = dec.prefill(prompt), ses.prefill(prompt)
+    prefill_equal = bool(np.array_equal(dec.logits_host(), ses.logits_host())) and ta == tb
+    records = len(ses._program(1, advance=True)[1].records)
+    dec.begin_decode(ta)
+    ses.begin_decode(tb)
+    want = [dec.decode_step() for _ in range(128)]
+    got = [ses.decode_step() for _ in range(128)]
+    res = {"step_records_per_token": records, "calls_per_token_after_folding": ses.calls_per_step,
+           "program_nodes": int(gpu.program_node_count(ses.program)), "prefill_logits_equal": prefill_equal, "tokens_equal": got == want}
+    for name, d in (("session", ses), ("hand_routed", dec)):
+        d.pos = 0
+        d.begin_decode(d.prefill(prompt))
+        gpu.sync()
+        t = time.perf_counter()
+        for _ in range(128):
+            d.decode_step(read_token=False)
+        gpu.sync()
+        dt = time.perf_counter() - t
+        res[name] = {"decode_ms_per_token": round(dt / 128 * 1e3, 4), "decode_tokens_per_s": round(128 / dt, 1)}
+    t = time.perf_counter()
+    ses.pos = 0
+    ses.prefill(prompt)
+    gpu.sync()
+    res["session"]["prefill_128_ms"] = round((time.perf_counter() - t) * 1e3, 3)
+    dec.close(); ses.close()
+    return res
 
 
 def run_decode_stack(gpu, be, compare=True):

@@ -141,3 +141,38 @@ def test_decode_run_without_read_back_gives_the_same_tokens(gpu, orc):
     finally:
         a.close(); b.close()
 
+
+
+@pytest.mark.parametrize("wdtype", [be.Q4_0, be.Q8_0])
+def test_the_step_list_of_the_decoder_on_the_session_executor_gives_the_same_logits(gpu, wdtype):
+    """The unfused step list (one record per graph step, in-place residual adds, workspace intermediates) run by the
+    library's session executor against the hand-routed Decoder over the same weights: prefill and every replayed decode
+    step give the same logits to the bit, and the executor folds a one-token layer into five calls."""
+    from aion_amd.decoder import SessionDecoder
+    cfg = DecoderConfig(wdtype=wdtype, **SMALL)
+    w = SyntheticWeights(cfg, 7)
+    a, b = Decoder(gpu, cfg, w), SessionDecoder(gpu, cfg, w)
+    try:
+        prompt = np.random.default_rng(4).integers(0, cfg.vocab, 11).astype(np.int32)
+        ta, tb = a.prefill(prompt), b.prefill(prompt)
+        assert np.array_equal(a.logits_host(), b.logits_host()) and ta == tb
+        a.begin_decode(ta)
+        b.begin_decode(tb)
+        # per layer: q/k/v side, attention, o + add, feed-forward + add -> 4 calls; gather, head, argmax, copy, 3 adds around them
+        assert b.calls_per_step == 4 * cfg.layers + 7
+        for step in range(6):
+            ta, tb = a.decode_step(), b.decode_step()
+            assert np.array_equal(a.logits_host(), b.logits_host()), step
+            assert ta == tb, step
+        # a second prompt on the same objects: a longer prefill may replace a work buffer, the program is recorded again
+        a.reset()
+        b.pos = 0
+        prompt = np.random.default_rng(5).integers(0, cfg.vocab, 40).astype(np.int32)
+        ta, tb = a.prefill(prompt), b.prefill(prompt)
+        assert np.array_equal(a.logits_host(), b.logits_host())
+        a.begin_decode(ta)
+        b.begin_decode(tb)
+        for step in range(3):
+            assert a.decode_step() == b.decode_step(), step
+    finally:
+        a.close(); b.close()
