@@ -8,6 +8,7 @@
 #include "common.h"
 
 #include <cstring>
+#include <initializer_list>
 #include <map>
 #include <utility>
 #include <tuple>
@@ -216,6 +217,7 @@ int aionhip_session::check(size_t i, const aionhip_step &st) {
         return AIONHIP_OK;
     }
     case AIONHIP_STEP_COPY:
+        if (bytes_of(st.out) == 0 && elems(st.out) != 0) return unsupported("Copy: an element type this device does not hold");
         if (!st.in[0].handle || !st.out.handle || bytes_of(st.in[0]) != bytes_of(st.out) || st.in[0].dtype != st.out.dtype) return bad("Copy: src and dst of one type and size");
         return AIONHIP_OK;
     case AIONHIP_STEP_GATHER:
@@ -250,6 +252,7 @@ int aionhip_session::check(size_t i, const aionhip_step &st) {
     case AIONHIP_STEP_TRANSFER: {
         const aionhip_tensor_ref &dev = st.to_host ? st.in[0] : st.out;
         if (!dev.handle || !st.host) return bad("Transfer: a device tensor and host bytes");
+        if (bytes_of(dev) == 0 && elems(dev) != 0) return unsupported("Transfer: an element type this device does not hold");
         if (st.host_bytes != bytes_of(dev)) return bad("Transfer: host bytes differ from the tensor's size");
         if (ctx->capturing) return bad("Transfer: not inside a recording");
         return AIONHIP_OK;
@@ -399,6 +402,18 @@ size_t aionhip_session::try_fused(const aionhip_step *steps, size_t count, size_
     };
     const aionhip_weight *ws[4];
     aionhip_handle cs[4];
+    // A folded call reads the pattern's first inputs while (or after) it writes the pattern's outputs, where the separate steps
+    // had finished with those inputs before the first output was written: no output may lie over such an input.
+    auto clear_of = [&](const aionhip_tensor_ref &out, std::initializer_list<const aionhip_tensor_ref *> inputs) {
+        for (const aionhip_tensor_ref *in : inputs)
+            if (in->handle && range_of(out).overlaps(range_of(*in))) return false;
+        return true;
+    };
+    auto siblings_clear_of = [&](size_t first, size_t c, std::initializer_list<const aionhip_tensor_ref *> inputs) {
+        for (size_t m = 0; m < c; ++m)
+            if (!clear_of(steps[first + m].out, inputs)) return false;
+        return true;
+    };
 
     auto dead_after = [&](const aionhip_tensor_ref &t, size_t last) { return only_read_within(steps, count, i, last, t); };
     const bool one_row = st.tag == AIONHIP_STEP_RMSNORM && !st.in[3].handle && elems(st.in[1]) == elems(st.out);
@@ -443,6 +458,8 @@ size_t aionhip_session::try_fused(const aionhip_step *steps, size_t count, size_
                  kc.shape[2] == xk.shape[2] && vc.shape[2] == xk.shape[2] && kc.shape[3] == d && vc.shape[3] == d &&
                  ((kc.flags ^ vc.flags) & AIONHIP_TENSOR_ROLLING) == 0 && app[0]->in[1].handle == app[1]->in[1].handle &&
                  !range_of(kc).overlaps(range_of(vc));
+            for (const aionhip_tensor_ref *o : {&rope[0]->out, &kc, &vc})
+                ok = ok && clear_of(*o, {&st.in[0], &st.in[1], &st.in[2], &rope[0]->in[1], &app[0]->in[1]}) && (o == &rope[0]->out || !range_of(*o).overlaps(range_of(rope[0]->out)));
             // everything between the block's input and {rotated q, the caches} lives only inside these ten steps
             ok = ok && dead_after(st.out, i + 9) && dead_after(steps[i + 1].out, i + 9) && dead_after(steps[i + 2].out, i + 9) &&
                  dead_after(steps[i + 3].out, i + 9) && dead_after(rope[1]->out, i + 9) && dead_after(cast[0]->out, i + 9) &&
@@ -466,8 +483,9 @@ size_t aionhip_session::try_fused(const aionhip_step *steps, size_t count, size_
         if (ok) {
             if (same_tensor(g.in[0], steps[i + 1].out) && same_tensor(g.in[1], steps[i + 2].out)) ig = 0;
             else if (same_tensor(g.in[0], steps[i + 2].out) && same_tensor(g.in[1], steps[i + 1].out)) ig = 1;
+            // (the output may be the block's own input x: the first of the two launches has consumed x before the second writes)
             ok = ig >= 0 && dead_after(st.out, i + 4) && dead_after(steps[i + 1].out, i + 4) && dead_after(steps[i + 2].out, i + 4) &&
-                 dead_after(g.out, i + 4);
+                 dead_after(g.out, i + 4) && clear_of(down.out, {&st.in[1], &st.in[2]});
         }
         aionhip_weight *wd = nullptr;
         if (ok && weight_for(down.in[1], down.tag == AIONHIP_STEP_MATMUL_NT ? AIONHIP_ROWS_NK : AIONHIP_KMAJOR_KN, &wd) == AIONHIP_OK) {
@@ -480,7 +498,7 @@ size_t aionhip_session::try_fused(const aionhip_step *steps, size_t count, size_
     }
     if ((fusion & AIONHIP_FUSE_WORKSPACE) && st.tag == AIONHIP_STEP_RMSNORM && !st.in[3].handle && i + 1 < count) {
         const size_t c = sibling_run(i + 1, st.out, ws, cs);
-        if (c && only_read_within(steps, count, i, i + c, st.out)) {
+        if (c && only_read_within(steps, count, i, i + c, st.out) && siblings_clear_of(i + 1, c, {&st.in[0], &st.in[1], &st.in[2]})) {
             const size_t cols = elems(st.in[1]);
             const int rc = aionhip_step_rmsnorm_matmul(ctx, c, ws, elems(st.out) / cols, st.in[0].handle, st.in[1].handle, st.in[2].handle, st.eps, cs, nullptr,
                                                        steps[i + 1].alpha, steps[i + 1].beta);
@@ -490,8 +508,9 @@ size_t aionhip_session::try_fused(const aionhip_step *steps, size_t count, size_
     if ((fusion & AIONHIP_FUSE_WORKSPACE) && st.tag == AIONHIP_STEP_ELEMWISE_BINARY && st.op == AIONHIP_BINARY_GATE && st.in[0].dtype == AIONHIP_F32 &&
         i + 1 < count) {
         const size_t c = sibling_run(i + 1, st.out, ws, cs);
-        if (c >= 1 && only_read_within(steps, count, i, i + 1, st.out)) {
-            const aionhip_handle res = residual_target(steps, count, i + 1);
+        if (c >= 1 && only_read_within(steps, count, i, i + 1, st.out) && clear_of(steps[i + 1].out, {&st.in[0], &st.in[1]})) {
+            aionhip_handle res = residual_target(steps, count, i + 1);
+            if (res && !clear_of(steps[i + 2].out, {&st.in[0], &st.in[1]})) res = 0;
             const int rc = aionhip_step_gate_matmul(ctx, ws[0], rows_of(st.out), st.in[0].handle, st.in[1].handle, res ? res : cs[0], 0, steps[i + 1].alpha,
                                                     res ? 1.f : steps[i + 1].beta);
             if (rc != AIONHIP_UNSUPPORTED) { *rc_out = wrap(i, st, rc); ++calls_last_execute; return res ? 3 : 2; }

@@ -439,3 +439,51 @@ def test_retire_drops_the_relaid_weights_and_a_list_records_as_a_program(gpu):
     _same(L.results(["logits"]), first, ["logits"])
     L.free()
     sess.close()
+
+
+def test_a_fold_is_skipped_when_an_output_lies_over_an_input_it_would_still_read(gpu):
+    """h = RMSNorm(x); x = h @ Wq (over x itself); k = h @ Wk. Step by step the norm is finished before x is overwritten; folded
+    into one launch the norm would be recomputed from an x that other workgroups are already overwriting. The executor must
+    see the overlap and keep the norm a step of its own (the two matmuls may still share a launch: they read h)."""
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((1, E)).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(E)).astype(np.float32)
+    wq = be.quantize_blocks(be.Q4_0, (rng.standard_normal((E, E)) / 16).astype(np.float32), 0)
+    wk = be.quantize_blocks(be.Q4_0, (rng.standard_normal((E, E)) / 16).astype(np.float32), 0)
+    gb, wqb, wkb = gpu.upload(g), gpu.upload(wq), gpu.upload(wk)
+    got = {}
+    sess = ss.Session(gpu)
+    for fusion in (0, ss.FUSE_SIBLINGS | ss.FUSE_WORKSPACE):
+        xb, h, k = gpu.upload(x), gpu.zeros(E * 4), gpu.zeros(E * 4)
+        f = lambda buf, ws=False: ss.tensor(buf, be.F32, (1, E), workspace=ws)  # noqa: E731
+        p = ss.Steps()
+        p.rmsnorm(f(xb), ss.tensor(gb, be.F32, (E,)), None, f(h, True), EPS)
+        p.matmul(f(h, True), ss.tensor(wqb, be.Q4_0, (E, E)), f(xb))
+        p.matmul(f(h, True), ss.tensor(wkb, be.Q4_0, (E, E)), f(k))
+        sess.set_fusion(fusion)
+        sess.execute(p)
+        assert sess.stats()[0] == (3 if fusion == 0 else 2)
+        got[fusion] = (xb.numpy(np.float32), k.numpy(np.float32), h.numpy(np.float32))
+        for buf in (xb, h, k):
+            buf.free()
+    for a, b in zip(got[0], got[3]):
+        assert np.array_equal(a, b)
+    assert got[0][2].any()                     # the norm's output was written both times
+    # the same with the gate: act(a) * b -> matmul written over a
+    a0, b0 = rng.standard_normal((1, E)).astype(np.float32), rng.standard_normal((1, E)).astype(np.float32)
+    got = {}
+    for fusion in (0, ss.FUSE_SIBLINGS | ss.FUSE_WORKSPACE):
+        ab, bb, t = gpu.upload(a0), gpu.upload(b0), gpu.zeros(E * 4)
+        p = ss.Steps()
+        p.elemwise_binary(ss.GATE, f(ab), f(bb), f(t, True), act=ss.GELU)
+        p.matmul(f(t, True), ss.tensor(wqb, be.Q4_0, (E, E)), f(ab))
+        sess.set_fusion(fusion)
+        sess.execute(p)
+        assert sess.stats()[0] == 2
+        got[fusion] = ab.numpy(np.float32)
+        for buf in (ab, bb, t):
+            buf.free()
+    assert np.array_equal(got[0], got[3])
+    sess.close()
+    for buf in (gb, wqb, wkb):
+        buf.free()
