@@ -473,6 +473,65 @@ size_t aionhip_session::try_fused(const aionhip_step *steps, size_t count, size_
             }
         }
     }
+    // Models that normalize their heads (src/bench/models.zig:455-473): RMSNorm over the head size on q, k and v -> RoPE1D on q and
+    // k -> Cast f16 + SequenceAppend of k and of v, nine steps from the first of the norms on, in any order a valid program can
+    // have them, for any batch and token count
+    if ((fusion & AIONHIP_FUSE_WORKSPACE) && st.tag == AIONHIP_STEP_RMSNORM && !st.in[3].handle && st.in[0].rank == 4 &&
+        elems(st.in[1]) == st.in[0].shape[3] && i + 8 < count) {
+        const aionhip_step *norm[3] = {nullptr, nullptr, nullptr}, *rope[2] = {nullptr, nullptr}, *cast[2] = {nullptr, nullptr}, *app[2] = {nullptr, nullptr};
+        int n_norm = 0, n_rope = 0, n_cast = 0, n_app = 0;
+        for (size_t j = i; j < i + 9; ++j) {
+            const aionhip_step &w = steps[j];
+            if (w.tag == AIONHIP_STEP_RMSNORM && n_norm < 3 && !w.in[3].handle) norm[n_norm++] = &w;
+            else if (w.tag == AIONHIP_STEP_ROPE1D && n_rope < 2) rope[n_rope++] = &w;
+            else if (w.tag == AIONHIP_STEP_CAST && n_cast < 2) cast[n_cast++] = &w;
+            else if (w.tag == AIONHIP_STEP_SEQUENCE_APPEND && n_app < 2) app[n_app++] = &w;
+            else n_norm = 9;
+        }
+        bool ok = n_norm == 3 && n_rope == 2 && n_cast == 2 && n_app == 2;
+        if (ok) {
+            // k's chain is the one whose rope output is cast; v's norm output is cast directly; q's rope output leaves the pattern
+            if (!same_tensor(cast[0]->in[0], rope[0]->out) && !same_tensor(cast[0]->in[0], rope[1]->out)) std::swap(cast[0], cast[1]);
+            if (!same_tensor(cast[0]->in[0], rope[1]->out)) std::swap(rope[0], rope[1]);      // rope[1] = k's, rope[0] = q's
+            if (!same_tensor(app[0]->in[0], cast[0]->out)) std::swap(app[0], app[1]);          // app[0] = k's, app[1] = v's
+            ok = same_tensor(cast[0]->in[0], rope[1]->out) && same_tensor(app[0]->in[0], cast[0]->out) && same_tensor(app[1]->in[0], cast[1]->out);
+        }
+        const aionhip_step *nq = nullptr, *nk = nullptr, *nv = nullptr;
+        if (ok) {
+            for (const aionhip_step *n : norm) {
+                if (same_tensor(n->out, rope[0]->in[0])) nq = n;
+                else if (same_tensor(n->out, rope[1]->in[0])) nk = n;
+                else if (same_tensor(n->out, cast[1]->in[0])) nv = n;
+            }
+            ok = nq && nk && nv;
+        }
+        if (ok) {
+            const aionhip_tensor_ref &xq = nq->in[0], &xk = nk->in[0], &xv = nv->in[0], &kc = app[0]->out, &vc = app[1]->out;
+            const size_t d = xq.shape[3];
+            ok = xq.rank == 4 && xk.rank == 4 && xv.rank == 4 && xk.shape[3] == d && xv.shape[3] == d && xk.shape[0] == xq.shape[0] &&
+                 xv.shape[0] == xq.shape[0] && xk.shape[1] == xq.shape[1] && xv.shape[1] == xq.shape[1] && xv.shape[2] == xk.shape[2] &&
+                 elems(nq->in[1]) == d && elems(nk->in[1]) == d && elems(nv->in[1]) == d && nq->eps == nk->eps && nq->eps == nv->eps &&
+                 rope[0]->in[1].handle == rope[1]->in[1].handle && rope[0]->rope_base == rope[1]->rope_base &&
+                 rope[0]->rope_scale == rope[1]->rope_scale && rope[0]->rope_proportion == rope[1]->rope_proportion &&
+                 kc.dtype == AIONHIP_F16 && vc.dtype == AIONHIP_F16 && kc.shape[0] == xq.shape[0] && vc.shape[0] == xq.shape[0] &&
+                 kc.shape[1] == vc.shape[1] && kc.shape[2] == xk.shape[2] && vc.shape[2] == xk.shape[2] && kc.shape[3] == d && vc.shape[3] == d &&
+                 ((kc.flags ^ vc.flags) & AIONHIP_TENSOR_ROLLING) == 0 && app[0]->in[1].handle == app[1]->in[1].handle &&
+                 !range_of(kc).overlaps(range_of(vc));
+            for (const aionhip_tensor_ref *o : {&rope[0]->out, &kc, &vc})
+                ok = ok && clear_of(*o, {&xq, &xk, &xv, &nq->in[1], &nq->in[2], &nk->in[1], &nk->in[2], &nv->in[1], &nv->in[2], &rope[0]->in[1], &app[0]->in[1]}) &&
+                     (o == &rope[0]->out || !range_of(*o).overlaps(range_of(rope[0]->out)));
+            ok = ok && dead_after(nq->out, i + 8) && dead_after(nk->out, i + 8) && dead_after(nv->out, i + 8) && dead_after(rope[1]->out, i + 8) &&
+                 dead_after(cast[0]->out, i + 8) && dead_after(cast[1]->out, i + 8);
+            if (ok) {
+                const int rc = aionhip_step_headnorm_rope_append(
+                    ctx, rope[0]->out.handle, xq.handle, xk.handle, xv.handle, nq->in[1].handle, nq->in[2].handle, nk->in[1].handle, nk->in[2].handle,
+                    nv->in[1].handle, nv->in[2].handle, nq->eps, kc.handle, vc.handle, rope[0]->in[1].handle, app[0]->in[1].handle, xq.shape[0],
+                    xq.shape[1], kc.shape[1], xq.shape[2], xk.shape[2], d, rope[0]->rope_base, rope[0]->rope_scale, rope[0]->rope_proportion,
+                    (kc.flags & AIONHIP_TENSOR_ROLLING) ? 1 : 0);
+                if (rc != AIONHIP_UNSUPPORTED) { *rc_out = wrap(i, st, rc); ++calls_last_execute; return 9; }
+            }
+        }
+    }
     // One row through a GeGLU feed-forward block: RMSNorm -> gate and up MatMuls -> gate(gelu) -> down MatMul
     if ((fusion & AIONHIP_FUSE_WORKSPACE) && one_row && i + 4 < count && sibling_run(i + 1, st.out, ws, cs) == 2) {
         const aionhip_step &g = steps[i + 3], &down = steps[i + 4];

@@ -487,3 +487,70 @@ def test_a_fold_is_skipped_when_an_output_lies_over_an_input_it_would_still_read
     sess.close()
     for buf in (gb, wqb, wkb):
         buf.free()
+
+
+@pytest.mark.parametrize("B,S,rolling,with_beta,order", [(1, 1, False, True, 0), (2, 3, False, False, 1), (1, 5, True, True, 2)])
+def test_head_norms_rope_and_appends_fold_into_one_call(gpu, B, S, rolling, with_beta, order):
+    """The cache side of a block whose heads are normalized (src/bench/models.zig:455-473): nine steps, one call, the
+    bits of the nine; the three chains in different step orders."""
+    Hq, Hkv, Dh, Tc = 4, 2, 64, 8
+    rng = np.random.default_rng(31 + order)
+    q = rng.standard_normal((B, S, Hq, Dh)).astype(np.float32)
+    k = rng.standard_normal((B, S, Hkv, Dh)).astype(np.float32)
+    v = rng.standard_normal((B, S, Hkv, Dh)).astype(np.float32)
+    start = 6 if rolling else 2
+    pos = np.tile(np.arange(start, start + S, dtype=np.int32), (B, 1))
+    seed = rng.standard_normal((B, Tc, Hkv, Dh)).astype(np.float16)
+    const = {nm: gpu.upload(a) for nm, a in (("q", q), ("k", k), ("v", v), ("pos", pos), ("widx", np.full(B, start, np.int32)))}
+    for nm in ("gq", "gk", "gv"):
+        const[nm] = gpu.upload((1 + 0.2 * rng.standard_normal(Dh)).astype(np.float32))
+    for nm in ("bq", "bk", "bv"):
+        const[nm] = gpu.upload((0.1 * rng.standard_normal(Dh)).astype(np.float32)) if with_beta else None
+    sess = ss.Session(gpu)
+    got = {}
+    for fusion in (0, ss.FUSE_SIBLINGS | ss.FUSE_WORKSPACE):
+        w = {nm: gpu.zeros(4 * B * S * h * Dh) for nm, h in (("nq", Hq), ("nk", Hkv), ("nv", Hkv), ("qr", Hq), ("kr", Hkv))}
+        w["k16"], w["v16"] = gpu.zeros(2 * B * S * Hkv * Dh), gpu.zeros(2 * B * S * Hkv * Dh)
+        w["kc"], w["vc"] = gpu.upload(seed), gpu.upload(seed[:, ::-1].copy())
+        f = lambda buf, h, ws=False: ss.tensor(buf, be.F32, (B, S, h, Dh), workspace=ws)  # noqa: E731
+        vec = lambda nm: ss.tensor(const[nm], be.F32, (Dh,)) if const[nm] is not None else None  # noqa: E731
+        k16 = ss.tensor(w["k16"], be.F16, (B, S, Hkv, Dh), workspace=True)
+        v16 = ss.tensor(w["v16"], be.F16, (B, S, Hkv, Dh), workspace=True)
+        kc = ss.tensor(w["kc"], be.F16, (B, Tc, Hkv, Dh), rolling=rolling)
+        vc = ss.tensor(w["vc"], be.F16, (B, Tc, Hkv, Dh), rolling=rolling)
+        posr, widx = ss.tensor(const["pos"], be.I32, (B, S)), ss.tensor(const["widx"], be.I32, (B,))
+        parts = {
+            "nq": lambda p: p.rmsnorm(f(const["q"], Hq), vec("gq"), vec("bq"), f(w["nq"], Hq, True), EPS),
+            "nk": lambda p: p.rmsnorm(f(const["k"], Hkv), vec("gk"), vec("bk"), f(w["nk"], Hkv, True), EPS),
+            "nv": lambda p: p.rmsnorm(f(const["v"], Hkv), vec("gv"), vec("bv"), f(w["nv"], Hkv, True), EPS),
+            "rq": lambda p: p.rope1d(f(w["nq"], Hq, True), posr, f(w["qr"], Hq), rope_proportion=0.5),
+            "rk": lambda p: p.rope1d(f(w["nk"], Hkv, True), posr, f(w["kr"], Hkv, True), rope_proportion=0.5),
+            "ck": lambda p: p.cast(f(w["kr"], Hkv, True), k16),
+            "cv": lambda p: p.cast(f(w["nv"], Hkv, True), v16),
+            "ak": lambda p: p.sequence_append(kc, k16, widx),
+            "av": lambda p: p.sequence_append(vc, v16, widx),
+        }
+        orders = (("nq", "nk", "nv", "rq", "rk", "ck", "ak", "cv", "av"), ("nk", "rk", "ck", "ak", "nv", "cv", "av", "nq", "rq"),
+                  ("nv", "nq", "rq", "cv", "nk", "av", "rk", "ck", "ak"))
+        p = ss.Steps()
+        for nm in orders[order]:
+            parts[nm](p)
+        # a reader of the rotated queries behind the pattern, as the attention step would be
+        p.unary(ss.RELU, f(w["qr"], Hq), f(w["nq"], Hq, True))
+        sess.set_fusion(fusion)
+        sess.execute(p)
+        assert sess.stats()[0] == (10 if fusion == 0 else 2)
+        got[fusion] = {nm: w[nm].numpy(np.float16 if nm in ("kc", "vc", "k16", "v16") else np.float32) for nm in w}
+        for buf in w.values():
+            buf.free()
+    for nm in ("qr", "kc", "vc", "nq"):
+        assert np.array_equal(got[0][nm].view(np.uint8), got[3][nm].view(np.uint8)), nm
+    assert got[0]["k16"].any() and not got[3]["k16"].any() and not got[3]["kr"].any() and not got[3]["nv"].any()
+    rows = [(start + s) % Tc if rolling else start + s for s in range(S)]
+    kc_got = got[3]["kc"].reshape(B, Tc, Hkv, Dh)
+    untouched = [t for t in range(Tc) if t not in rows]
+    assert np.array_equal(kc_got[:, untouched], seed[:, untouched]) and not np.array_equal(kc_got[:, rows], seed[:, rows])
+    sess.close()
+    for buf in const.values():
+        if buf is not None:
+            buf.free()
