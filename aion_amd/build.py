@@ -8,7 +8,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libaion_hip.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-SOURCES = ["ctx.hip", "quant.hip", "weights.hip", "gemv.hip", "gemv_fused.hip", "gemv_ksplit.hip", "gemm.hip", "matmul.hip", "matmul_nt_f32.hip", "attention.hip", "attention_prefill.hip", "decode_stack.hip", "glue.hip", "program.hip", "session.hip"]
+SOURCES = ["ctx.hip", "quant.hip", "weights.hip", "gemv.hip", "gemv_fused.hip", "gemv_ksplit.hip", "gemv_mfma.hip", "gemm.hip", "matmul.hip", "matmul_nt_f32.hip", "attention.hip", "attention_prefill.hip", "decode_stack.hip", "glue.hip", "program.hip", "session.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-result",
     # hipcc -O3 may otherwise form packed-f32 instructions, which have given wrong results on this pool

@@ -231,6 +231,11 @@ int launch_gate_gelu(aionhip_ctx *ctx, float *out, const float *a, const float *
 int rope_table(aionhip_ctx *ctx, int pairs, float freq_step, float scale_factor, const float **out);
 
 // one activation row against one weight with a long reduction axis: K cut into slices, one launch (gemv_ksplit.hip)
+// 3..8 prepared rows against a weight with very many rows, the dots on the matrix pipe (gemv_mfma.hip); launch returns -1 when
+// the shape does not suit the kernel after all
+bool gemv_mfma_applies(const aionhip_weight *const *ws, int count, int m);
+int launch_gemv_mfma(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *const *cs, const size_t *ldcs, int count, int m, PreparedAct act,
+                     float alpha, float beta);
 bool gemv_ksplit_applies(const aionhip_ctx *ctx, const aionhip_weight *w, const float *x);
 int launch_gemv_ksplit(aionhip_ctx *ctx, const aionhip_weight *w, float *c, const float *x, float alpha, float beta);
 int launch_gemv(aionhip_ctx *ctx, const aionhip_weight *w, int m, PreparedAct act, float *c, size_t ldc, float alpha, float beta);

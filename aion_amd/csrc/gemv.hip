@@ -418,6 +418,16 @@ int launch_gemv_batch(aionhip_ctx *ctx, const aionhip_weight *const *ws, float *
                       PreparedAct act, float alpha, float beta) {
     if (m < 1 || m > 8) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "gemv: m=%d outside 1..8", m);
     if (count < 1 || count > 4) return set_err(ctx, AIONHIP_INVALID_ARGUMENT, "gemv: %d weights in one launch (1..4)", count);
+    if (gemv_mfma_applies(ws, count, m)) {
+        const char *mname = ws[0]->dtype == AIONHIP_Q8_0 ? "gemv_q8_mfma" : "gemv_q4_mfma";
+        ProfScope scope(ctx, mname);
+        const int rc = launch_gemv_mfma(ctx, ws, cs, ldcs, count, m, act, alpha, beta);
+        if (rc == AIONHIP_OK) {
+            LAUNCH_CHECK(ctx, mname);
+            return AIONHIP_OK;
+        }
+        if (rc != -1) return rc;
+    }
     const char *name = ws[0]->dtype == AIONHIP_Q8_0 ? "gemv_q8" : "gemv_q4";
     ProfScope scope(ctx, name);
     // 5..8 rows against a wide, short weight (a logits head at batch 8): the 16-row MFMA tile of the LDS-staged int8

@@ -72,3 +72,15 @@ def row_rms_err(got, ref):
     """The same per row against the row's rms (2.5 to 3 times smaller than its largest element): max |err| / rms(ref row)"""
     import numpy as np
     return _row_err(got, ref, lambda r: np.sqrt((r ** 2).mean(axis=-1)))
+
+
+def rows_kernel(q8, m, n, k):
+    """The kernel 2..8 activation rows against an [n, k] weight run on (what aionhip_last_kernel reports): the matrix-pipe GEMV for
+    many weight rows and a K of 2048..4096 in whole 256-code stages (q4: from 14336 rows at 5..8 activation rows, from 65536 at
+    3..4; q8: from 65536 rows up to 300 M weights), the exact GEMM's 16-row tile for 5..8 rows over a K past 4096, else the
+    vector-ALU rows kernel."""
+    tag = "q8" if q8 else "q4"
+    if 3 <= m <= 8 and 2048 <= k <= 4096 and k % 256 == 0:
+        if (not q8 and n >= (14336 if m >= 5 else 65536)) or (q8 and n >= 65536 and n * k <= 300_000_000):
+            return "gemv_%s_mfma" % tag
+    return ("gemm_i8_" if m >= 5 and k > 4096 else "gemv_") + tag

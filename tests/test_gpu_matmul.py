@@ -12,7 +12,7 @@ import pytest
 
 from aion_amd import backend as be
 from aion_amd import hip
-from conftest import norm_err, rms_err
+from conftest import norm_err, rms_err, rows_kernel
 
 pytestmark = pytest.mark.gpu
 TOL = 2e-3      # elementwise, floored
@@ -239,6 +239,34 @@ def test_single_row_q4_eight_alternating_slices(gpu, orc):
     w.free()
 
 
+# Sibling weights at 3..8 rows whose rows together reach the matrix-pipe GEMV's range (gate / up of a feed-forward block, a short
+# prompt): one launch walks the tiles of all weights; ragged column counts, a sibling far smaller than the others, alpha / beta.
+@pytest.mark.parametrize("dtype,m,ns,k", [(be.Q4_0, 6, (8200, 8192), 2048), (be.Q4_0, 5, (14000, 40, 1000), 4096), (be.Q4_0, 3, (40000, 30000), 2304),
+                                          (be.Q8_0, 4, (33000, 33000), 2048)])
+def test_sibling_weights_share_a_matrix_pipe_gemv_launch(gpu, orc, dtype, m, ns, k):
+    say("sibling gemv mfma", dtype, m, ns, k)
+    layout = be.ROWS_NK if dtype == be.Q8_0 else be.KMAJOR_KN
+    made = [make_weight(gpu, orc, dtype, layout, n, k, seed=n + 3 * i, std=0.1) for i, n in enumerate(ns)]
+    rng = np.random.default_rng(m + k)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    c0 = [rng.standard_normal((m, n)).astype(np.float32) for n in ns]
+    a_buf = gpu.upload(a)
+    for alpha, beta in ((1.0, 0.0), (-0.5, 1.5)):
+        c_bufs = [gpu.upload(c) for c in c0]
+        gpu.profile_start()
+        gpu.step_matmul_batch([w for _b, w in made], a_buf, m, c_bufs, alpha=alpha, beta=beta)
+        names = [nm for nm, _ms in gpu.profile_stop()]
+        assert names.count("gemv_%s_mfma" % ("q8" if dtype == be.Q8_0 else "q4")) == 1 and len(names) == 2, names   # + the preparation
+        for (blocks, _w), cb, c, n in zip(made, c_bufs, c0, ns):
+            got = gpu.download(cb, np.float32, (m, n))
+            want = oracle_matmul(orc, dtype, layout, a, blocks, n, alpha=alpha, beta=beta, c=c)
+            assert norm_err(got, want) < TOL and rms_err(got, want) < RMS_TOL, (n, alpha)
+            cb.free()
+    a_buf.free()
+    for _b, w in made:
+        w.free()
+
+
 # Sibling weights over one activation (q/k/v, gate/up) with more than eight rows: one launch of the exact GEMM whose
 # column tiles are dealt out to the weights in order. Column counts that do not fill a tile, one to four weights,
 # row counts around the tile heights, alpha/beta on pre-filled outputs - each output against the oracle.
@@ -307,11 +335,13 @@ def test_exact_gemm_shapes_and_edges(gpu, orc, dtype, layout, m, n, k):
 # not a multiple of the rows a wavefront works on, K of one LDS pass, K that needs most of a CU's LDS (16384 at 4 rows) and K
 # long enough to run as several K-range launches (32768 at 3 rows), alpha/beta on a pre-filled C. Three shapes (5..8 rows, at
 # least 16384 columns, K up to 4096) run on the 16-row tile of the LDS-staged MFMA kernel instead: ragged N, K of one and of
-# many steps. Five to eight rows over a K past 4096 take the exact GEMM (its 16-row tile is far ahead there).
+# many steps. Five to eight rows over a K past 4096 take the exact GEMM (its 16-row tile is far ahead there). Many weight rows
+# over a K of 2048 ... 4096 take the matrix-pipe GEMV (gemv_mfma_kernel; conftest.rows_kernel states where): one wavefront per
+# 16-row tile and two sharing a tile's K (14400 rows), ragged N, K of 8 / 9 / 16 stages, 3 ... 8 rows, both weight types.
 @pytest.mark.parametrize("dtype,layout", CASES)
 @pytest.mark.parametrize("m,n,k", [(2, 70, 96), (3, 1001, 1056), (5, 333, 2048), (8, 1030, 14336), (7, 4100, 7200), (4, 9000, 512),
                                    (5, 16390, 256), (8, 20001, 2048), (6, 16384, 4096), (4, 1030, 16384), (3, 300, 32768),
-                                   (5, 70, 4128), (8, 14336, 8192)])
+                                   (5, 70, 4128), (8, 14336, 8192), (5, 14400, 4096), (3, 65600, 2048), (8, 65539, 2304), (4, 14336, 4096)])
 def test_decode_gemv_two_to_eight_rows(gpu, orc, dtype, layout, m, n, k):
     say("gemv rows", dtype, layout, m, n, k)
     blocks, w = make_weight(gpu, orc, dtype, layout, n, k, seed=m * 31 + n + k, std=0.05)
@@ -319,7 +349,7 @@ def test_decode_gemv_two_to_eight_rows(gpu, orc, dtype, layout, m, n, k):
     a = rng.standard_normal((m, k)).astype(np.float32)
     c0 = rng.standard_normal((m, n)).astype(np.float32)
     got = gpu.matmul(w, a)
-    assert gpu.last_kernel() == ("gemm_i8_" if m >= 5 and k > 4096 else "gemv_") + ("q8" if dtype == be.Q8_0 else "q4")
+    assert gpu.last_kernel() == rows_kernel(dtype == be.Q8_0, m, n, k)
     want = oracle_matmul(orc, dtype, layout, a, blocks, n)
     assert norm_err(got, want) < TOL and rms_err(got, want) < RMS_TOL
     got2 = gpu.matmul(w, a, alpha=-1.5, beta=0.25, c=c0)

@@ -133,7 +133,7 @@ def _device_free_bytes():
 # 16-row MFMA tile); more than 8 rows (the exact GEMM, whose K slices need a buffer and are therefore off here)
 ROUTES = [("one row, fused", be.Q4_0, be.KMAJOR_KN, 1, 2100, 4096), ("one row, long K", be.Q8_0, be.ROWS_NK, 1, 520, 16416),
           ("few rows", be.Q8_0, be.KMAJOR_KN, 3, 1030, 2048), ("few rows, 16-row tile", be.Q4_0, be.KMAJOR_KN, 6, 16390, 1024),
-          ("exact GEMM", be.Q4_0, be.KMAJOR_KN, 24, 520, 8192)]
+          ("few rows, matrix pipe", be.Q4_0, be.KMAJOR_KN, 5, 14400, 2048), ("exact GEMM", be.Q4_0, be.KMAJOR_KN, 24, 520, 8192)]
 
 
 def test_every_route_records_on_a_fresh_context_and_allocates_nothing(orc):
