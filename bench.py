@@ -111,7 +111,7 @@ def main():
     ap.add_argument("--sweep", action="store_true", help="(kept for compatibility: the sweep is part of the default run)")
     ap.add_argument("--headline-only", action="store_true", help="skip the secondary metrics (prefill GEMM, decode, sweep)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--extras", default="", help="comma list of gemm,attention,decoder,decode_stack,session_decode,package,package_bench_shape")
+    ap.add_argument("--extras", default="", help="comma list of sweep,gemm,attention,decoder,decode_stack,session_decode,package,package_bench_shape")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU (aion runs one program on one device, and no multi-GPU figure is asked for); "
@@ -273,6 +273,8 @@ def main():
                             "sweep": run_sweep(gpu, be, host_blocks), "attention": run_attention_headline(gpu, be)}
     if extras:
         out["extras"] = {}
+        if "sweep" in extras:          # the sweep of the default run on its own (for a kernel trace: --headline-only --extras sweep)
+            out["extras"]["sweep"] = run_sweep(gpu, be, host_blocks)
         if "gemm" in extras:
             out["extras"]["prefill_gemm"] = run_gemm(gpu, be)
         if "attention" in extras:
