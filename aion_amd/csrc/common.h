@@ -172,6 +172,7 @@ size_t prepared_act_bytes(size_t m, size_t k);
 PreparedAct prepared_act_carve(void *base, size_t m, size_t k);
 int launch_prepare_act(aionhip_ctx *ctx, const float *a, size_t lda, size_t m, size_t k, PreparedAct out);
 int launch_prepare_gate(aionhip_ctx *ctx, const float *gate, const float *up, size_t m, size_t k, PreparedAct out);
+int launch_prepare_rmsnorm(aionhip_ctx *ctx, const float *x, const float *gamma, const float *beta, float eps, size_t m, size_t k, PreparedAct out);
 
 // ---- matmul back ends --------------------------------------------------------------------------
 // Up to four weights that multiply the SAME activation rows (q/k/v, gate/up) run as one launch:

@@ -184,7 +184,21 @@ int aionhip_step_rmsnorm_matmul(aionhip_ctx *ctx, size_t count, const aionhip_we
     const float *xp = (const float *)(uintptr_t)x, *gp = (const float *)(uintptr_t)gamma, *bp = (const float *)(uintptr_t)beta_norm;
     if (rows == 1 && fused_row_pays(b) && ((x | gamma | beta_norm) & 15) == 0)
         return launch_gemv_fused(ctx, b.w, b.c, b.ldc, (int)b.count, PRO_RMSNORM, FusedIn{xp, nullptr, gp, bp, eps}, alpha, beta);
-    // several rows: the norm runs as its own kernel into scratch, then the ordinary routing
+    // Two rows and more on the exact kernels: the norm and the int8 preparation in one launch (the bits of the norm step followed
+    // by the preparation launch), then the GEMV or GEMM on the prepared rows. One row keeps the route below (a long K is cut
+    // into slices that prepare their own part), and so does a call that the bf16 kernel takes (it wants the f32 rows).
+    bool bf16_route = rows > GEMV_MAX_M && ctx->gemm_mode != AIONHIP_GEMM_EXACT_I8;
+    if (bf16_route && ctx->gemm_mode == AIONHIP_GEMM_BF16_MFMA)
+        for (size_t i = 0; i < b.count; ++i) bf16_route = bf16_route && gemm_bf16_pays(ctx, rows, b.w[i]->n, b.k);
+    if (rows >= 2 && rows <= 0x7FFFFFFFu && !bf16_route && ((x | gamma | beta_norm) & 15) == 0) {
+        rc = ensure_scratch(ctx, prepared_act_bytes(rows, b.k));
+        if (rc) return rc;
+        PreparedAct act = prepared_act_carve(ctx->scratch, rows, b.k);
+        rc = launch_prepare_rmsnorm(ctx, xp, gp, bp, eps, rows, b.k, act);
+        if (rc) return rc;
+        return launch_prepared_rows(ctx, b, rows, act, alpha, beta);
+    }
+    // otherwise the norm runs as its own kernel into scratch, then the ordinary routing
     const size_t act_bytes = (prepared_act_bytes(rows, b.k) + 255) & ~(size_t)255;
     rc = ensure_scratch(ctx, act_bytes + rows * b.k * sizeof(float));
     if (rc) return rc;

@@ -112,6 +112,70 @@ __global__ void quantize_rank2_kernel(const float *__restrict__ src, uint8_t *__
 
 // Activation preparation (aion matmul_q_i8.zig:187-203): 8 lanes share one 32-element block.
 // GATE: the activation is gelu_tanh(a) * up (aion cpu/exec/elementwise.zig:25-37), not written out.
+// RMSNorm + int8 preparation, one workgroup per row of k columns (k a multiple of 32; x, gamma, beta 16-byte aligned). The sum
+// of squares runs in the norm kernels' order (thread c of 256 adds x[c]^2, x[c + 256]^2, ...; then block_sum_256) and a value
+// is rounded as they round it ((x * inv) * gamma + beta), so the codes, scales and code sums are those of the norm step followed
+// by the preparation launch. SHORT: rows of up to 2048 columns, every load requested before the reduction (one memory round
+// trip); otherwise two passes over the row.
+template <bool SHORT>
+__global__ __launch_bounds__(256) void rmsnorm_prepare_kernel(const float *__restrict__ x, const float *__restrict__ gamma, const float *__restrict__ beta,
+                                                              size_t cols, float eps, int *__restrict__ aq, float *__restrict__ a_scale,
+                                                              int *__restrict__ a_sum) {
+    __shared__ float red[4];
+    const size_t row = blockIdx.x;
+    const float *xr = x + row * cols;
+    const size_t chunks = cols >> 2, kb_per_row = cols / QK;
+    const int tid = threadIdx.x;
+    auto emit = [&](size_t c4, bool live, f32x4 xv, f32x4 gv, f32x4 bv, float inv) {
+        const float y0 = (xv.x * inv) * gv.x + (beta ? bv.x : 0.f), y1 = (xv.y * inv) * gv.y + (beta ? bv.y : 0.f);
+        const float y2 = (xv.z * inv) * gv.z + (beta ? bv.z : 0.f), y3 = (xv.w * inv) * gv.w + (beta ? bv.w : 0.f);
+        int word, sm;
+        float scale;
+        prepare_act_block8(y0, y1, y2, y3, word, scale, sm);         // (all eight lanes of a block take part: chunks is a multiple of 8)
+        if (live) {
+            aq[row * chunks + c4] = word;
+            if ((c4 & 7) == 0) {
+                a_scale[row * kb_per_row + (c4 >> 3)] = scale;
+                a_sum[row * kb_per_row + (c4 >> 3)] = sm;
+            }
+        }
+    };
+    const f32x4 *x4 = (const f32x4 *)xr, *g4 = (const f32x4 *)gamma, *b4 = (const f32x4 *)(beta ? beta : gamma);
+    if (SHORT) {
+        float sv[8];
+        f32x4 xc[2], gc[2], bc[2];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) sv[j] = xr[min((size_t)tid + 256 * j, cols - 1)];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const size_t c4 = min((size_t)tid + 256 * i, chunks - 1);
+            xc[i] = x4[c4];
+            gc[i] = g4[c4];
+            bc[i] = b4[c4];
+        }
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            if ((size_t)tid + 256 * j < cols) ss += sv[j] * sv[j];
+        ss = block_sum_256(ss, red);
+        const float inv = 1.f / sqrtf(ss * (1.f / (float)cols) + eps);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const size_t c4 = (size_t)tid + 256 * i;
+            if (256 * (size_t)i < chunks) emit(c4, c4 < chunks, xc[i], gc[i], bc[i], inv);      // (uniform per workgroup)
+        }
+    } else {
+        float ss = 0.f;
+        for (size_t c = tid; c < cols; c += 256) ss += xr[c] * xr[c];
+        ss = block_sum_256(ss, red);
+        const float inv = 1.f / sqrtf(ss * (1.f / (float)cols) + eps);
+        for (size_t base = 0; base < chunks; base += 256) {
+            const size_t c4 = base + tid, cc = min(c4, chunks - 1);
+            emit(c4, c4 < chunks, x4[cc], g4[cc], b4[cc], inv);
+        }
+    }
+}
+
 template <bool GATE>
 __global__ __launch_bounds__(256) void prepare_act_kernel(const float *__restrict__ a, const float *__restrict__ up, size_t lda, size_t m, size_t k,
                                                           int *__restrict__ aq, float *__restrict__ a_scale, int *__restrict__ a_sum) {
@@ -175,6 +239,17 @@ int launch_prepare_gate(aionhip_ctx *ctx, const float *gate, const float *up, si
     ProfScope scope(ctx, "prepare_gate");
     launch_k(ctx, prepare_act_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, gate, up, k, m, k, (int *)out.q, out.scale, out.sum);
     LAUNCH_CHECK(ctx, "prepare_gate");
+    return AIONHIP_OK;
+}
+
+// StepRMSNorm (cpu/exec/layernorm.zig:54-155) followed by the int8 preparation of its rows, as one launch: what the norm step
+// and the preparation launch give, to the bit, without the normalized rows' trip through memory.
+int launch_prepare_rmsnorm(aionhip_ctx *ctx, const float *x, const float *gamma, const float *beta, float eps, size_t m, size_t k, PreparedAct out) {
+    if (!m || !k) return AIONHIP_OK;
+    ProfScope scope(ctx, "prepare_rmsnorm");
+    if (k <= 2048) launch_k(ctx, rmsnorm_prepare_kernel<true>, dim3((unsigned)m), dim3(256), 0, x, gamma, beta, k, eps, (int *)out.q, out.scale, out.sum);
+    else launch_k(ctx, rmsnorm_prepare_kernel<false>, dim3((unsigned)m), dim3(256), 0, x, gamma, beta, k, eps, (int *)out.q, out.scale, out.sum);
+    LAUNCH_CHECK(ctx, "prepare_rmsnorm");
     return AIONHIP_OK;
 }
 

@@ -183,7 +183,7 @@ int aionhip_step_rmsnorm_geglu_matmul(aionhip_ctx *ctx, const aionhip_weight *w_
                                       aionhip_handle c, float alpha, float beta);
 /* StepRMSNorm feeding MatMul steps, and the fused gate feeding a MatMul step, as one call each:
  * the normalised (or gated) activation is not written out; for one row it is built inside the GEMV
- * kernel. Same arithmetic as aionhip_step_rmsnorm / aionhip_step_gate_gelu followed by the matmul
+ * kernel, for more rows on the exact kernels the norm (or gate) and the int8 preparation are one launch. Same arithmetic as aionhip_step_rmsnorm / aionhip_step_gate_gelu followed by the matmul
  * step(s). aion fuses at step level the same way (RMSNorm.residual, ElemwiseBinary.gate:
  * graph/opt/fuse_steps.zig:19-88); these two go one step further because a decode step on this
  * GPU is bound by launch count, not bandwidth. */

@@ -407,6 +407,35 @@ def test_single_row_fused_kernel_equals_prepared_path(gpu, orc, dtype, layout):
         w.free()
 
 
+# Two rows and more on the exact kernels take the norm and the int8 preparation as one launch: rows of up to 2048 columns
+# (everything requested before the reduction) and longer ones (two passes), column counts that leave the last 256-thread pass
+# partly empty, with and without the norm's beta, 2..8 rows (GEMV) and more (GEMM) - the bits of the norm step followed by the
+# matmul step, and one launch fewer.
+@pytest.mark.parametrize("k", [96, 1056, 2048, 2080, 4096, 8224])
+@pytest.mark.parametrize("rows,with_beta", [(2, False), (5, True), (9, True), (70, False)])
+def test_rmsnorm_and_preparation_in_one_launch_give_the_bits_of_the_two_steps(gpu, orc, k, rows, with_beta):
+    say("rmsnorm + prepare", k, rows, with_beta)
+    rng = np.random.default_rng(k + rows)
+    n = 72
+    _b, w = make_weight(gpu, orc, be.Q4_0, be.KMAJOR_KN, n, k, seed=k)
+    x = (rng.standard_normal((rows, k)) * (1 + rng.random((rows, 1)) * 5)).astype(np.float32)
+    gamma = (1 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    beta = (0.1 * rng.standard_normal(k)).astype(np.float32)
+    xb, gb, bb = gpu.upload(x), gpu.upload(gamma), (gpu.upload(beta) if with_beta else None)
+    c1, c2, hb = gpu.alloc(rows * n * 4), gpu.alloc(rows * n * 4), gpu.alloc(rows * k * 4)
+    gpu.set_gemm_mode(be.GEMM_EXACT_I8)
+    gpu.profile_start()
+    gpu.step_rmsnorm_matmul([w], xb, gb, rows, [c1], 1e-6, beta_norm=bb)
+    names = [nm for nm, _ in gpu.profile_stop()]
+    assert names[0] == "prepare_rmsnorm" and "prepare_act" not in names, names
+    gpu.step_rmsnorm(hb, xb, gb, rows, k, 1e-6, beta=bb)
+    gpu.step_matmul(w, hb, rows, c2)
+    assert np.array_equal(gpu.download(c1, np.float32, (rows, n)), gpu.download(c2, np.float32, (rows, n)))
+    for t in (xb, gb, c1, c2, hb) + ((bb,) if bb is not None else ()):
+        t.free()
+    w.free()
+
+
 @pytest.mark.parametrize("dtype,layout", CASES)
 @pytest.mark.parametrize("rows", [1, 3, 6, 40])
 def test_rmsnorm_matmul_and_gate_matmul_match_the_separate_steps(gpu, orc, dtype, layout, rows):
