@@ -344,6 +344,9 @@ def test_a_list_is_checked_as_a_whole_before_anything_runs(gpu):
         assert e.value.status == hip.INVALID_ARGUMENT
     assert np.array_equal(out.numpy(np.float32), np.full(64, 7.0, np.float32))
     sess.execute(ss.Steps())          # an empty list is a program with nothing to do
+    with pytest.raises(be.AionHipError) as e:
+        sess.set_fusion(8)
+    assert e.value.status == hip.INVALID_ARGUMENT
     sess.close()
     xb.free()
     out.free()

@@ -137,3 +137,14 @@ def test_ctypes_structures_have_the_header_layout(tmp_path):
         assert getattr(ss, const) == order.index(name)
         assert re.search(r"AIONHIP_STEP_%s = %d\b" % (const, order.index(name)), header), const
     assert re.search(r"AIONHIP_STEP_TAG_COUNT = %d\b" % len(order), header)
+
+
+def test_session_entry_points_reject_null_handles_without_a_gpu():
+    lib = hip.load_library()
+    p = C.c_void_p()
+    assert lib.aionhip_session_create(None, C.byref(p)) == hip.INVALID_ARGUMENT
+    assert lib.aionhip_session_execute(None, None, 0) == hip.INVALID_ARGUMENT
+    assert lib.aionhip_session_set_fusion(None, 3) == hip.INVALID_ARGUMENT
+    assert lib.aionhip_session_retire(None) == hip.INVALID_ARGUMENT
+    assert lib.aionhip_session_stats(None, None, None, None) == hip.INVALID_ARGUMENT
+    lib.aionhip_session_destroy(None)          # a no-op
