@@ -124,9 +124,9 @@ struct aionhip_session {
     int check(size_t i, const aionhip_step &st);
     int check_list(const aionhip_step *steps, size_t count);
     int run_one(size_t i, const aionhip_step &st);
-    // value written by step i into `t`: true when every step that reads it lies in [i + 1, last] (nothing before its next
-    // overwrite, and - the tensor being a workspace tensor - nothing after the list)
-    bool only_read_within(const aionhip_step *steps, size_t count, size_t i, size_t last, const aionhip_tensor_ref &t) const;
+    // the value a pattern ending at step `last` would leave unwritten in `t`: true when no step behind `last` reads it before it
+    // is overwritten in full (and - the tensor being a workspace tensor - nothing reads it after the list)
+    bool only_read_within(const aionhip_step *steps, size_t count, size_t last, const aionhip_tensor_ref &t) const;
     size_t try_fused(const aionhip_step *steps, size_t count, size_t i, int *rc);
     // steps[j]: a MatMul with beta 0 into a workspace tensor T that only the step right behind it reads, that step being an
     // add that accumulates in place (X = X + T or X = T + X). The matmul may then write X itself with beta 1: alpha * acc + X
@@ -348,7 +348,7 @@ int aionhip_session::run_one(size_t i, const aionhip_step &st) {
     return wrap(i, st, rc);
 }
 
-bool aionhip_session::only_read_within(const aionhip_step *steps, size_t count, size_t i, size_t last, const aionhip_tensor_ref &t) const {
+bool aionhip_session::only_read_within(const aionhip_step *steps, size_t count, size_t last, const aionhip_tensor_ref &t) const {
     if (!(t.flags & AIONHIP_TENSOR_WORKSPACE)) return false;
     const Range r = range_of(t);
     for (size_t j = last + 1; j < count; ++j) {
@@ -371,7 +371,7 @@ aionhip_handle aionhip_session::residual_target(const aionhip_step *steps, size_
     const aionhip_tensor_ref *x = same_tensor(add.in[1], t) ? &add.in[0] : same_tensor(add.in[0], t) ? &add.in[1] : nullptr;
     if (!x || !same_tensor(add.out, *x)) return 0;
     if (range_of(*x).overlaps(range_of(t)) || range_of(*x).overlaps(range_of(mm.in[0])) || range_of(*x).overlaps(range_of(mm.in[1]))) return 0;
-    if (!only_read_within(steps, count, j, j + 1, t)) return 0;
+    if (!only_read_within(steps, count, j + 1, t)) return 0;
     return x->handle;
 }
 
@@ -415,7 +415,7 @@ size_t aionhip_session::try_fused(const aionhip_step *steps, size_t count, size_
         return true;
     };
 
-    auto dead_after = [&](const aionhip_tensor_ref &t, size_t last) { return only_read_within(steps, count, i, last, t); };
+    auto dead_after = [&](const aionhip_tensor_ref &t, size_t last) { return only_read_within(steps, count, last, t); };
     const bool one_row = st.tag == AIONHIP_STEP_RMSNORM && !st.in[3].handle && elems(st.in[1]) == elems(st.out);
 
     // One token of one sequence, the input side of an attention block: RMSNorm -> the q, k, v MatMuls -> RoPE1D on q and k ->
@@ -557,7 +557,7 @@ size_t aionhip_session::try_fused(const aionhip_step *steps, size_t count, size_
     }
     if ((fusion & AIONHIP_FUSE_WORKSPACE) && st.tag == AIONHIP_STEP_RMSNORM && !st.in[3].handle && i + 1 < count) {
         const size_t c = sibling_run(i + 1, st.out, ws, cs);
-        if (c && only_read_within(steps, count, i, i + c, st.out) && siblings_clear_of(i + 1, c, {&st.in[0], &st.in[1], &st.in[2]})) {
+        if (c && only_read_within(steps, count, i + c, st.out) && siblings_clear_of(i + 1, c, {&st.in[0], &st.in[1], &st.in[2]})) {
             const size_t cols = elems(st.in[1]);
             const int rc = aionhip_step_rmsnorm_matmul(ctx, c, ws, elems(st.out) / cols, st.in[0].handle, st.in[1].handle, st.in[2].handle, st.eps, cs, nullptr,
                                                        steps[i + 1].alpha, steps[i + 1].beta);
@@ -567,7 +567,7 @@ size_t aionhip_session::try_fused(const aionhip_step *steps, size_t count, size_
     if ((fusion & AIONHIP_FUSE_WORKSPACE) && st.tag == AIONHIP_STEP_ELEMWISE_BINARY && st.op == AIONHIP_BINARY_GATE && st.in[0].dtype == AIONHIP_F32 &&
         i + 1 < count) {
         const size_t c = sibling_run(i + 1, st.out, ws, cs);
-        if (c >= 1 && only_read_within(steps, count, i, i + 1, st.out) && clear_of(steps[i + 1].out, {&st.in[0], &st.in[1]})) {
+        if (c >= 1 && only_read_within(steps, count, i + 1, st.out) && clear_of(steps[i + 1].out, {&st.in[0], &st.in[1]})) {
             aionhip_handle res = residual_target(steps, count, i + 1);
             if (res && !clear_of(steps[i + 2].out, {&st.in[0], &st.in[1]})) res = 0;
             const int rc = aionhip_step_gate_matmul(ctx, ws[0], rows_of(st.out), st.in[0].handle, st.in[1].handle, res ? res : cs[0], 0, steps[i + 1].alpha,
@@ -578,7 +578,7 @@ size_t aionhip_session::try_fused(const aionhip_step *steps, size_t count, size_
     if ((fusion & AIONHIP_FUSE_WORKSPACE) && st.tag == AIONHIP_STEP_CAST && i + 1 < count) {
         const aionhip_step &ap = steps[i + 1];
         if (ap.tag == AIONHIP_STEP_SEQUENCE_APPEND && ap.out.dtype == AIONHIP_F16 && same_tensor(ap.in[0], st.out) &&
-            !range_of(ap.out).overlaps(range_of(st.in[0])) && only_read_within(steps, count, i, i + 1, st.out)) {
+            !range_of(ap.out).overlaps(range_of(st.in[0])) && only_read_within(steps, count, i + 1, st.out)) {
             const aionhip_tensor_ref &cache = ap.out, &nk = ap.in[0];
             const int rc = aionhip_step_append_f16(ctx, cache.handle, st.in[0].handle, ap.in[1].handle, cache.shape[0], nk.shape[1], cache.shape[1],
                                                    cache.shape[2] * cache.shape[3], (cache.flags & AIONHIP_TENSOR_ROLLING) ? 1 : 0);
