@@ -341,7 +341,7 @@ def test_exact_gemm_shapes_and_edges(gpu, orc, dtype, layout, m, n, k):
 @pytest.mark.parametrize("dtype,layout", CASES)
 @pytest.mark.parametrize("m,n,k", [(2, 70, 96), (3, 1001, 1056), (5, 333, 2048), (8, 1030, 14336), (7, 4100, 7200), (4, 9000, 512),
                                    (5, 16390, 256), (8, 20001, 2048), (6, 16384, 4096), (4, 1030, 16384), (3, 300, 32768),
-                                   (5, 70, 4128), (8, 14336, 8192), (5, 14400, 4096), (3, 65600, 2048), (8, 65539, 2304), (4, 14336, 4096)])
+                                   (5, 70, 4128), (8, 14336, 8192), (5, 14400, 4096), (3, 65600, 2048), (8, 65539, 2304), (4, 14336, 4096), (6, 65552, 4096)])
 def test_decode_gemv_two_to_eight_rows(gpu, orc, dtype, layout, m, n, k):
     say("gemv rows", dtype, layout, m, n, k)
     blocks, w = make_weight(gpu, orc, dtype, layout, n, k, seed=m * 31 + n + k, std=0.05)
