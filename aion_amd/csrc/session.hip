@@ -7,6 +7,7 @@
 // nothing done.
 #include "common.h"
 
+#include <cmath>
 #include <cstring>
 #include <initializer_list>
 #include <map>
@@ -159,6 +160,8 @@ int aionhip_session::check(size_t i, const aionhip_step &st) {
         if (a.shape[a.rank - 1] != k || c.shape[c.rank - 1] != n || rows_of(a) != rows_of(c)) return bad("MatMul: operand shapes do not agree");
         if (nt ? (b.dtype != AIONHIP_Q8_0 && b.dtype != AIONHIP_F32) : (b.dtype != AIONHIP_Q8_0 && b.dtype != AIONHIP_Q4_0))
             return unsupported(nt ? "MatMulNT: b is q8_0 or f32" : "MatMul: b is q4_0 or q8_0 (an f32 [K,N] operand stays on the CPU)");
+        if (b.dtype != AIONHIP_F32 && k % 32 != 0) return bad("MatMul: the quantized axis is a whole number of 32-element blocks");
+        if (!n || !k) return bad("MatMul: empty weight");
         return AIONHIP_OK;
     }
     case AIONHIP_STEP_ELEMWISE_BINARY: {
@@ -194,6 +197,7 @@ int aionhip_session::check(size_t i, const aionhip_step &st) {
         if (cols == 0 || x.rank < 1 || x.shape[x.rank - 1] != cols || elems(x) != elems(st.out)) return bad("RMSNorm: gamma spans x's last axis");
         if (be.handle && (!is_f32(be) || elems(be) != cols)) return bad("RMSNorm: beta like gamma");
         if (res.handle && (!is_f32(res) || elems(res) != elems(x))) return bad("RMSNorm: residual like x");
+        if (!(st.eps > 0.f) || !(st.eps < INFINITY)) return bad("RMSNorm: eps positive and finite");
         return AIONHIP_OK;
     }
     case AIONHIP_STEP_ATTENTION: {
@@ -207,6 +211,9 @@ int aionhip_session::check(size_t i, const aionhip_step &st) {
             return bad("Attention: out is [B, L, Hq, Dv]");
         if (st.in[3].handle && (!is_i32(st.in[3]) || elems(st.in[3]) != q.shape[0] * q.shape[1])) return bad("Attention: query_positions i32 [B, L]");
         if (st.in[4].handle && (!is_i32(st.in[4]) || elems(st.in[4]) != q.shape[0])) return bad("Attention: kv_lengths i32 [B]");
+        for (const aionhip_tensor_ref *t : {&q, &k})
+            if (t->dtype != AIONHIP_F32 && t->dtype != AIONHIP_F16 && t->dtype != AIONHIP_BF16) return unsupported("Attention: f32, f16 or bf16 operands");
+        if (k.shape[2] == 0 || q.shape[2] % k.shape[2] != 0) return bad("Attention: query heads are a multiple of the kv heads");
         return AIONHIP_OK;
     }
     case AIONHIP_STEP_ARGMAX: {
@@ -228,12 +235,17 @@ int aionhip_session::check(size_t i, const aionhip_step &st) {
         if (!t.handle || t.rank != 2) return unsupported("Gather: a rank-2 table");
         if (t.dtype != AIONHIP_F32 && t.dtype != AIONHIP_Q8_0) return unsupported("Gather: an f32 or q8_0 table");
         if (!is_i32(ids) || !is_f32(st.out) || elems(st.out) != elems(ids) * t.shape[1]) return bad("Gather: i32 indices, f32 out [indices..., D]");
+        if (t.dtype == AIONHIP_Q8_0 && t.shape[1] % 32 != 0) return bad("Gather: a q8_0 row is a whole number of 32-element blocks");
         return AIONHIP_OK;
     }
     case AIONHIP_STEP_ROPE1D: {
         const aionhip_tensor_ref &x = st.in[0], &pos = st.in[1];
         if (!is_f32(x) || !is_f32(st.out) || x.rank != 4 || elems(x) != elems(st.out)) return bad("RoPE1D: f32 [B, T, H, D] in and out");
         if (!is_i32(pos) || elems(pos) != x.shape[0] * x.shape[1]) return bad("RoPE1D: positions i32 [B, T]");
+        if (x.shape[3] % 2 != 0 || x.shape[3] > 65534 || x.shape[2] > 65535) return bad("RoPE1D: an even head size");
+        if (!(st.rope_base > 0.f) || !(st.rope_base < INFINITY) || !(st.rope_scale > 0.f) || !(st.rope_scale < INFINITY) ||
+            !(st.rope_proportion >= 0.f && st.rope_proportion <= 1.f))
+            return bad("RoPE1D: base and scale positive and finite, proportion in [0, 1]");
         return AIONHIP_OK;
     }
     case AIONHIP_STEP_SEQUENCE_APPEND: {

@@ -336,13 +336,23 @@ def test_a_list_is_checked_as_a_whole_before_anything_runs(gpu):
                 lambda q: q.matmul(ss.tensor(xb, be.F32, (1, 64)), ss.tensor(xb, be.Q4_0, (32, 64)), ss.tensor(out, be.F32, (1, 64))),
                 lambda q: q.rmsnorm(ss.tensor(xb, be.F32, (2, 32)), f(out, 16), None, ss.tensor(out, be.F32, (2, 32)), EPS),
                 lambda q: q.copy(f(xb), f(out, 32)),
-                lambda q: q.transfer_to_host(f(xb), np.zeros(8, np.float32))):
+                lambda q: q.transfer_to_host(f(xb), np.zeros(8, np.float32)),
+                # limits of the entry points behind the tags, found before the first launch as well
+                lambda q: q.matmul(ss.tensor(xb, be.F32, (1, 48)), ss.tensor(xb, be.Q4_0, (48, 32)), ss.tensor(out, be.F32, (1, 32))),
+                lambda q: q.rmsnorm(ss.tensor(xb, be.F32, (2, 32)), f(out, 32), None, ss.tensor(out, be.F32, (2, 32)), 0.0),
+                lambda q: q.rope1d(ss.tensor(xb, be.F32, (1, 1, 4, 3)), ss.tensor(xb, be.I32, (1, 1)), ss.tensor(out, be.F32, (1, 1, 4, 3))),
+                lambda q: q.rope1d(ss.tensor(xb, be.F32, (1, 1, 2, 8)), ss.tensor(xb, be.I32, (1, 1)), ss.tensor(out, be.F32, (1, 1, 2, 8)),
+                                   rope_proportion=1.5),
+                lambda q: q.gather(ss.tensor(xb, be.Q8_0, (4, 16)), ss.tensor(xb, be.I32, (2,)), f(out, 32)),
+                lambda q: q.attention(ss.tensor(xb, be.F32, (1, 1, 3, 8)), ss.tensor(xb, be.F16, (1, 2, 2, 8)), ss.tensor(xb, be.F16, (1, 2, 2, 8)),
+                                      ss.tensor(out, be.F32, (1, 1, 3, 8)), 0.1)):
         q = ss.Steps()
+        q.unary(ss.RELU, f(xb), f(out))          # a valid step in front: it may not have run when the list is refused
         bad(q)
         with pytest.raises(be.AionHipError) as e:
             sess.execute(q)
-        assert e.value.status == hip.INVALID_ARGUMENT
-    assert np.array_equal(out.numpy(np.float32), np.full(64, 7.0, np.float32))
+        assert e.value.status == hip.INVALID_ARGUMENT and "step 1" in str(e.value)
+        assert np.array_equal(out.numpy(np.float32), np.full(64, 7.0, np.float32))
     sess.execute(ss.Steps())          # an empty list is a program with nothing to do
     with pytest.raises(be.AionHipError) as e:
         sess.set_fusion(8)
