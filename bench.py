@@ -603,7 +603,7 @@ def run_decoder_eager(gpu, be, steps=8):
 
 
 def run_session_decode(gpu, be):
-    """Config 5 as a compiled program reaches a backend: one record per graph step (24 per block, nothing pre-fused), run by the
+    """Config 5 as a compiled program reaches a backend: one record per graph step (19 per block, nothing pre-fused), run by the
     library's session executor (aionhip_session_execute), recorded as a program and replayed; beside the hand-routed Decoder
     over the same weights, whose prefill logits and 128 tokens it must reproduce."""
     from aion_amd.decoder import Decoder, DecoderConfig, SessionDecoder, SyntheticWeights

@@ -134,3 +134,28 @@ def test_config5_full_size_node_by_node_prompt_and_decode_steps(gpu, orc):
         assert fused.step_count(1) <= 6 * cfg.layers + 6 and plain.step_count(1) > 15 * cfg.layers
     finally:
         plain.close(); fused.close(); dec.close()
+
+
+def test_config5_full_size_step_list_on_the_session_executor_equals_the_decoder(gpu):
+    """The config-5 decode program as a compiled aion program hands it to a backend - 502 step records for one token, nothing
+    pre-fused - run by the library's session executor, against the hand-routed Decoder over the same weights: the 128-token
+    prompt's logits (262144 values) and every replayed decode step's logits are the same to the bit, and the executor folds a
+    block into four calls."""
+    from aion_amd.decoder import SessionDecoder
+    cfg = DecoderConfig()
+    weights = SyntheticWeights(cfg, 0)
+    dec, ses = Decoder(gpu, cfg, weights), SessionDecoder(gpu, cfg, weights)
+    try:
+        prompt = np.random.default_rng(5).integers(0, cfg.vocab, 128).astype(np.int32)
+        ta, tb = dec.prefill(prompt), ses.prefill(prompt)
+        assert np.array_equal(dec.logits_host(), ses.logits_host()) and ta == tb
+        dec.begin_decode(ta)
+        ses.begin_decode(tb)
+        assert len(ses._program(1, advance=True)[1].records) == 19 * cfg.layers + 8
+        assert ses.calls_per_step == 4 * cfg.layers + 7
+        for step in range(6):
+            ta, tb = dec.decode_step(), ses.decode_step()
+            assert np.array_equal(dec.logits_host(), ses.logits_host()), step
+            assert ta == tb, step
+    finally:
+        dec.close(); ses.close()
