@@ -467,8 +467,10 @@ def run_sweep(gpu, be, q4_blocks):
                 # five to eight rows over a K past 4096 run on the exact GEMM's 16-row tile, everything else on a GEMV kernel
                 ms = time_kernel(gpu, ws, x, y, m, (kname, "gemm_i8_" + kname[-2:]) if m >= 5 and k > 4096 else kname)
                 by = algorithmic_bytes(bb, n, k, m)
+                ll = gpu.last_launch()
                 res["%s %dx%d b%d" % ("q4" if dtype == be.Q4_0 else "q8", n, k, m)] = {
-                    "kernels": gpu.last_kernel(), "kernel_us": round(ms * 1e3, 2), "GBps": round(by / (ms * 1e-3) / 1e9, 1),
+                    "kernels": gpu.last_kernel(), "launched": "%s grid %s x %d" % (ll["kernel"].replace("(anonymous namespace)::", ""), ll["grid"], ll["block"][0]),
+                    "kernel_us": round(ms * 1e3, 2), "GBps": round(by / (ms * 1e-3) / 1e9, 1),
                     "frac_hbm_peak": round(by / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 3)}
                 x.free(); y.free()
             for w in ws:
