@@ -475,7 +475,8 @@ typedef struct aionhip_step {
 } aionhip_step;
 
 typedef struct aionhip_session aionhip_session;
-/* Backend.createSession (backend/backend.zig:46-52). A session belongs to one context and one thread. */
+/* Backend.createSession (backend/backend.zig:46-52). A session belongs to one context and one thread, and is destroyed before
+ * its context (it frees its re-laid weights through it). */
 int aionhip_session_create(aionhip_ctx *ctx, aionhip_session **out);
 /* Which step patterns a session may run as one call (default: both). Results are the separate steps' to the bit either way.
  * AIONHIP_FUSE_SIBLINGS: consecutive MatMul / MatMulNT steps reading one activation share its preparation and, up to eight
