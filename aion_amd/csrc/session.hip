@@ -141,6 +141,49 @@ bool is_f32(const aionhip_tensor_ref &t) { return t.handle && t.dtype == AIONHIP
 bool is_i32(const aionhip_tensor_ref &t) { return t.handle && t.dtype == AIONHIP_I32; }
 bool is_matmul_tag(int tag) { return tag == AIONHIP_STEP_MATMUL || tag == AIONHIP_STEP_MATMUL_NT; }
 
+// The cache side of an attention block among consecutive steps: RoPE1D on q and k, Cast f16 + SequenceAppend of k and of v,
+// with or without an RMSNorm over the head size in front of each of q, k and v - in whatever order a valid program has them.
+struct KvTail {
+    const aionhip_step *norm[3] = {nullptr, nullptr, nullptr};      // sorted: q's, k's, v's
+    const aionhip_step *rope[2] = {nullptr, nullptr};               // q's, k's
+    const aionhip_step *cast[2] = {nullptr, nullptr};               // k's, v's
+    const aionhip_step *app[2] = {nullptr, nullptr};                // k's, v's
+};
+// steps [lo, hi) are exactly `norms` head norms (0 or 3), two ropes, two casts and two appends wired as above
+bool sort_kv_tail(const aionhip_step *steps, size_t lo, size_t hi, int norms, KvTail &t) {
+    int n_norm = 0, n_rope = 0, n_cast = 0, n_app = 0;
+    const aionhip_step *norm[3] = {nullptr, nullptr, nullptr};
+    for (size_t j = lo; j < hi; ++j) {
+        const aionhip_step &w = steps[j];
+        if (w.tag == AIONHIP_STEP_RMSNORM && n_norm < norms && !w.in[3].handle) norm[n_norm++] = &w;
+        else if (w.tag == AIONHIP_STEP_ROPE1D && n_rope < 2) t.rope[n_rope++] = &w;
+        else if (w.tag == AIONHIP_STEP_CAST && n_cast < 2) t.cast[n_cast++] = &w;
+        else if (w.tag == AIONHIP_STEP_SEQUENCE_APPEND && n_app < 2) t.app[n_app++] = &w;
+        else return false;
+    }
+    if (n_norm != norms || n_rope != 2 || n_cast != 2 || n_app != 2) return false;
+    // the cast that reads a rope's output is k's; that rope is k's, the other one q's, whose output leaves the pattern
+    if (!same_tensor(t.cast[0]->in[0], t.rope[0]->out) && !same_tensor(t.cast[0]->in[0], t.rope[1]->out)) std::swap(t.cast[0], t.cast[1]);
+    if (!same_tensor(t.cast[0]->in[0], t.rope[1]->out)) std::swap(t.rope[0], t.rope[1]);
+    if (!same_tensor(t.app[0]->in[0], t.cast[0]->out)) std::swap(t.app[0], t.app[1]);
+    if (!same_tensor(t.cast[0]->in[0], t.rope[1]->out) || !same_tensor(t.app[0]->in[0], t.cast[0]->out) || !same_tensor(t.app[1]->in[0], t.cast[1]->out))
+        return false;
+    if (same_tensor(t.cast[1]->in[0], t.rope[0]->out)) return false;          // v's cast reads no rope
+    for (const aionhip_step *n : norm) {
+        if (!n) continue;
+        if (same_tensor(n->out, t.rope[0]->in[0])) t.norm[0] = n;
+        else if (same_tensor(n->out, t.rope[1]->in[0])) t.norm[1] = n;
+        else if (same_tensor(n->out, t.cast[1]->in[0])) t.norm[2] = n;
+    }
+    if (norms && (!t.norm[0] || !t.norm[1] || !t.norm[2])) return false;
+    // one positions tensor and one set of RoPE parameters, one write index, f16 caches of one policy that do not overlap
+    const aionhip_tensor_ref &kc = t.app[0]->out, &vc = t.app[1]->out;
+    return t.rope[0]->in[1].handle == t.rope[1]->in[1].handle && t.rope[0]->rope_base == t.rope[1]->rope_base &&
+           t.rope[0]->rope_scale == t.rope[1]->rope_scale && t.rope[0]->rope_proportion == t.rope[1]->rope_proportion &&
+           t.app[0]->in[1].handle == t.app[1]->in[1].handle && kc.dtype == AIONHIP_F16 && vc.dtype == AIONHIP_F16 &&
+           kc.shape[1] == vc.shape[1] && ((kc.flags ^ vc.flags) & AIONHIP_TENSOR_ROLLING) == 0 && !range_of(kc).overlaps(range_of(vc));
+}
+
 }  // namespace
 
 int aionhip_session::check(size_t i, const aionhip_step &st) {
@@ -430,57 +473,42 @@ size_t aionhip_session::try_fused(const aionhip_step *steps, size_t count, size_
     auto dead_after = [&](const aionhip_tensor_ref &t, size_t last) { return only_read_within(steps, count, last, t); };
     const bool one_row = st.tag == AIONHIP_STEP_RMSNORM && !st.in[3].handle && elems(st.in[1]) == elems(st.out);
 
+    // outputs of a folded cache side (rotated q, the two caches) clear of everything the fold reads, and of each other
+    auto tail_outputs_clear = [&](const KvTail &t, std::initializer_list<const aionhip_tensor_ref *> inputs) {
+        const aionhip_tensor_ref &qo = t.rope[0]->out, &kc = t.app[0]->out, &vc = t.app[1]->out;
+        for (const aionhip_tensor_ref *o : {&qo, &kc, &vc})
+            if (!clear_of(*o, inputs) || !clear_of(*o, {&t.rope[0]->in[1], &t.app[0]->in[1]})) return false;
+        return !range_of(kc).overlaps(range_of(qo)) && !range_of(vc).overlaps(range_of(qo));
+    };
+
     // One token of one sequence, the input side of an attention block: RMSNorm -> the q, k, v MatMuls -> RoPE1D on q and k ->
     // Cast f16 + SequenceAppend of k and of v (the six steps behind the matmuls in any order a valid program can have them)
-    if ((fusion & AIONHIP_FUSE_WORKSPACE) && one_row && i + 9 < count && sibling_run(i + 1, st.out, ws, cs) == 3) {
-        const aionhip_step *rope[2] = {nullptr, nullptr}, *cast[2] = {nullptr, nullptr}, *app[2] = {nullptr, nullptr};
-        int n_rope = 0, n_cast = 0, n_app = 0;
-        for (size_t j = i + 4; j < i + 10; ++j) {
-            const aionhip_step &w = steps[j];
-            if (w.tag == AIONHIP_STEP_ROPE1D && n_rope < 2) rope[n_rope++] = &w;
-            else if (w.tag == AIONHIP_STEP_CAST && n_cast < 2) cast[n_cast++] = &w;
-            else if (w.tag == AIONHIP_STEP_SEQUENCE_APPEND && n_app < 2) app[n_app++] = &w;
-            else n_rope = 9;
-        }
-        bool ok = n_rope == 2 && n_cast == 2 && n_app == 2 && steps[i + 1].alpha == 1.f && steps[i + 1].beta == 0.f;
-        if (ok) {
-            // the cast that reads a rope's output is k's; that rope is k's, the other one q's
-            if (!same_tensor(cast[0]->in[0], rope[0]->out) && !same_tensor(cast[0]->in[0], rope[1]->out)) std::swap(cast[0], cast[1]);
-            if (!same_tensor(cast[0]->in[0], rope[1]->out)) std::swap(rope[0], rope[1]);      // rope[1] = k's, rope[0] = q's
-            if (!same_tensor(app[0]->in[0], cast[0]->out)) std::swap(app[0], app[1]);          // app[0] = k's, app[1] = v's
-            ok = same_tensor(cast[0]->in[0], rope[1]->out) && same_tensor(app[0]->in[0], cast[0]->out) && same_tensor(app[1]->in[0], cast[1]->out);
-        }
-        int iq = -1, ik = -1, iv = -1;
-        if (ok) {
+    if ((fusion & AIONHIP_FUSE_WORKSPACE) && one_row && i + 9 < count && sibling_run(i + 1, st.out, ws, cs) == 3 &&
+        steps[i + 1].alpha == 1.f && steps[i + 1].beta == 0.f) {
+        KvTail t;
+        if (sort_kv_tail(steps, i + 4, i + 10, 0, t)) {
+            int iq = -1, ik = -1, iv = -1;
             for (int m = 0; m < 3; ++m) {
                 const aionhip_tensor_ref &o = steps[i + 1 + m].out;
-                if (same_tensor(o, rope[0]->in[0])) iq = m;
-                else if (same_tensor(o, rope[1]->in[0])) ik = m;
-                else if (same_tensor(o, cast[1]->in[0])) iv = m;
+                if (same_tensor(o, t.rope[0]->in[0])) iq = m;
+                else if (same_tensor(o, t.rope[1]->in[0])) ik = m;
+                else if (same_tensor(o, t.cast[1]->in[0])) iv = m;
             }
-            ok = iq >= 0 && ik >= 0 && iv >= 0;
-        }
-        if (ok) {
-            const aionhip_tensor_ref &xq = rope[0]->in[0], &xk = rope[1]->in[0], &kc = app[0]->out, &vc = app[1]->out;
+            const aionhip_tensor_ref &xq = t.rope[0]->in[0], &xk = t.rope[1]->in[0], &kc = t.app[0]->out, &vc = t.app[1]->out;
             const size_t d = xq.shape[3];
-            ok = xq.shape[0] == 1 && xq.shape[1] == 1 && xk.shape[0] == 1 && xk.shape[1] == 1 && xk.shape[3] == d && d % 8 == 0 &&
-                 rope[0]->in[1].handle == rope[1]->in[1].handle && rope[0]->rope_base == rope[1]->rope_base &&
-                 rope[0]->rope_scale == rope[1]->rope_scale && rope[0]->rope_proportion == rope[1]->rope_proportion &&
-                 kc.dtype == AIONHIP_F16 && vc.dtype == AIONHIP_F16 && kc.shape[0] == 1 && vc.shape[0] == 1 && kc.shape[1] == vc.shape[1] &&
-                 kc.shape[2] == xk.shape[2] && vc.shape[2] == xk.shape[2] && kc.shape[3] == d && vc.shape[3] == d &&
-                 ((kc.flags ^ vc.flags) & AIONHIP_TENSOR_ROLLING) == 0 && app[0]->in[1].handle == app[1]->in[1].handle &&
-                 !range_of(kc).overlaps(range_of(vc));
-            for (const aionhip_tensor_ref *o : {&rope[0]->out, &kc, &vc})
-                ok = ok && clear_of(*o, {&st.in[0], &st.in[1], &st.in[2], &rope[0]->in[1], &app[0]->in[1]}) && (o == &rope[0]->out || !range_of(*o).overlaps(range_of(rope[0]->out)));
+            bool ok = iq >= 0 && ik >= 0 && iv >= 0 && xq.shape[0] == 1 && xq.shape[1] == 1 && xk.shape[0] == 1 && xk.shape[1] == 1 &&
+                      xk.shape[3] == d && d % 8 == 0 && kc.shape[0] == 1 && vc.shape[0] == 1 && kc.shape[2] == xk.shape[2] &&
+                      vc.shape[2] == xk.shape[2] && kc.shape[3] == d && vc.shape[3] == d &&
+                      tail_outputs_clear(t, {&st.in[0], &st.in[1], &st.in[2]});
             // everything between the block's input and {rotated q, the caches} lives only inside these ten steps
             ok = ok && dead_after(st.out, i + 9) && dead_after(steps[i + 1].out, i + 9) && dead_after(steps[i + 2].out, i + 9) &&
-                 dead_after(steps[i + 3].out, i + 9) && dead_after(rope[1]->out, i + 9) && dead_after(cast[0]->out, i + 9) &&
-                 dead_after(cast[1]->out, i + 9);
+                 dead_after(steps[i + 3].out, i + 9) && dead_after(t.rope[1]->out, i + 9) && dead_after(t.cast[0]->out, i + 9) &&
+                 dead_after(t.cast[1]->out, i + 9);
             if (ok) {
                 const int rc = aionhip_step_rmsnorm_qkv_rope_append(
-                    ctx, ws[iq], ws[ik], ws[iv], st.in[0].handle, st.in[1].handle, st.in[2].handle, st.eps, rope[0]->out.handle, kc.handle, vc.handle,
-                    rope[0]->in[1].handle, app[0]->in[1].handle, kc.shape[1], xq.shape[2], xk.shape[2], d, rope[0]->rope_base, rope[0]->rope_scale,
-                    rope[0]->rope_proportion, (kc.flags & AIONHIP_TENSOR_ROLLING) ? 1 : 0);
+                    ctx, ws[iq], ws[ik], ws[iv], st.in[0].handle, st.in[1].handle, st.in[2].handle, st.eps, t.rope[0]->out.handle, kc.handle, vc.handle,
+                    t.rope[0]->in[1].handle, t.app[0]->in[1].handle, kc.shape[1], xq.shape[2], xk.shape[2], d, t.rope[0]->rope_base,
+                    t.rope[0]->rope_scale, t.rope[0]->rope_proportion, (kc.flags & AIONHIP_TENSOR_ROLLING) ? 1 : 0);
                 if (rc != AIONHIP_UNSUPPORTED) { *rc_out = wrap(i, st, rc); ++calls_last_execute; return 10; }
             }
         }
@@ -490,57 +518,48 @@ size_t aionhip_session::try_fused(const aionhip_step *steps, size_t count, size_
     // have them, for any batch and token count
     if ((fusion & AIONHIP_FUSE_WORKSPACE) && st.tag == AIONHIP_STEP_RMSNORM && !st.in[3].handle && st.in[0].rank == 4 &&
         elems(st.in[1]) == st.in[0].shape[3] && i + 8 < count) {
-        const aionhip_step *norm[3] = {nullptr, nullptr, nullptr}, *rope[2] = {nullptr, nullptr}, *cast[2] = {nullptr, nullptr}, *app[2] = {nullptr, nullptr};
-        int n_norm = 0, n_rope = 0, n_cast = 0, n_app = 0;
-        for (size_t j = i; j < i + 9; ++j) {
-            const aionhip_step &w = steps[j];
-            if (w.tag == AIONHIP_STEP_RMSNORM && n_norm < 3 && !w.in[3].handle) norm[n_norm++] = &w;
-            else if (w.tag == AIONHIP_STEP_ROPE1D && n_rope < 2) rope[n_rope++] = &w;
-            else if (w.tag == AIONHIP_STEP_CAST && n_cast < 2) cast[n_cast++] = &w;
-            else if (w.tag == AIONHIP_STEP_SEQUENCE_APPEND && n_app < 2) app[n_app++] = &w;
-            else n_norm = 9;
-        }
-        bool ok = n_norm == 3 && n_rope == 2 && n_cast == 2 && n_app == 2;
-        if (ok) {
-            // k's chain is the one whose rope output is cast; v's norm output is cast directly; q's rope output leaves the pattern
-            if (!same_tensor(cast[0]->in[0], rope[0]->out) && !same_tensor(cast[0]->in[0], rope[1]->out)) std::swap(cast[0], cast[1]);
-            if (!same_tensor(cast[0]->in[0], rope[1]->out)) std::swap(rope[0], rope[1]);      // rope[1] = k's, rope[0] = q's
-            if (!same_tensor(app[0]->in[0], cast[0]->out)) std::swap(app[0], app[1]);          // app[0] = k's, app[1] = v's
-            ok = same_tensor(cast[0]->in[0], rope[1]->out) && same_tensor(app[0]->in[0], cast[0]->out) && same_tensor(app[1]->in[0], cast[1]->out);
-        }
-        const aionhip_step *nq = nullptr, *nk = nullptr, *nv = nullptr;
-        if (ok) {
-            for (const aionhip_step *n : norm) {
-                if (same_tensor(n->out, rope[0]->in[0])) nq = n;
-                else if (same_tensor(n->out, rope[1]->in[0])) nk = n;
-                else if (same_tensor(n->out, cast[1]->in[0])) nv = n;
-            }
-            ok = nq && nk && nv;
-        }
-        if (ok) {
-            const aionhip_tensor_ref &xq = nq->in[0], &xk = nk->in[0], &xv = nv->in[0], &kc = app[0]->out, &vc = app[1]->out;
+        KvTail t;
+        if (sort_kv_tail(steps, i, i + 9, 3, t)) {
+            const aionhip_step *nq = t.norm[0], *nk = t.norm[1], *nv = t.norm[2];
+            const aionhip_tensor_ref &xq = nq->in[0], &xk = nk->in[0], &xv = nv->in[0], &kc = t.app[0]->out, &vc = t.app[1]->out;
             const size_t d = xq.shape[3];
-            ok = xq.rank == 4 && xk.rank == 4 && xv.rank == 4 && xk.shape[3] == d && xv.shape[3] == d && xk.shape[0] == xq.shape[0] &&
-                 xv.shape[0] == xq.shape[0] && xk.shape[1] == xq.shape[1] && xv.shape[1] == xq.shape[1] && xv.shape[2] == xk.shape[2] &&
-                 elems(nq->in[1]) == d && elems(nk->in[1]) == d && elems(nv->in[1]) == d && nq->eps == nk->eps && nq->eps == nv->eps &&
-                 rope[0]->in[1].handle == rope[1]->in[1].handle && rope[0]->rope_base == rope[1]->rope_base &&
-                 rope[0]->rope_scale == rope[1]->rope_scale && rope[0]->rope_proportion == rope[1]->rope_proportion &&
-                 kc.dtype == AIONHIP_F16 && vc.dtype == AIONHIP_F16 && kc.shape[0] == xq.shape[0] && vc.shape[0] == xq.shape[0] &&
-                 kc.shape[1] == vc.shape[1] && kc.shape[2] == xk.shape[2] && vc.shape[2] == xk.shape[2] && kc.shape[3] == d && vc.shape[3] == d &&
-                 ((kc.flags ^ vc.flags) & AIONHIP_TENSOR_ROLLING) == 0 && app[0]->in[1].handle == app[1]->in[1].handle &&
-                 !range_of(kc).overlaps(range_of(vc));
-            for (const aionhip_tensor_ref *o : {&rope[0]->out, &kc, &vc})
-                ok = ok && clear_of(*o, {&xq, &xk, &xv, &nq->in[1], &nq->in[2], &nk->in[1], &nk->in[2], &nv->in[1], &nv->in[2], &rope[0]->in[1], &app[0]->in[1]}) &&
-                     (o == &rope[0]->out || !range_of(*o).overlaps(range_of(rope[0]->out)));
-            ok = ok && dead_after(nq->out, i + 8) && dead_after(nk->out, i + 8) && dead_after(nv->out, i + 8) && dead_after(rope[1]->out, i + 8) &&
-                 dead_after(cast[0]->out, i + 8) && dead_after(cast[1]->out, i + 8);
+            bool ok = xq.rank == 4 && xk.rank == 4 && xv.rank == 4 && xk.shape[3] == d && xv.shape[3] == d && xk.shape[0] == xq.shape[0] &&
+                      xv.shape[0] == xq.shape[0] && xk.shape[1] == xq.shape[1] && xv.shape[1] == xq.shape[1] && xv.shape[2] == xk.shape[2] &&
+                      elems(nq->in[1]) == d && elems(nk->in[1]) == d && elems(nv->in[1]) == d && nq->eps == nk->eps && nq->eps == nv->eps &&
+                      kc.shape[0] == xq.shape[0] && vc.shape[0] == xq.shape[0] && kc.shape[2] == xk.shape[2] && vc.shape[2] == xk.shape[2] &&
+                      kc.shape[3] == d && vc.shape[3] == d &&
+                      tail_outputs_clear(t, {&xq, &xk, &xv, &nq->in[1], &nq->in[2], &nk->in[1], &nk->in[2], &nv->in[1], &nv->in[2]});
+            ok = ok && dead_after(nq->out, i + 8) && dead_after(nk->out, i + 8) && dead_after(nv->out, i + 8) && dead_after(t.rope[1]->out, i + 8) &&
+                 dead_after(t.cast[0]->out, i + 8) && dead_after(t.cast[1]->out, i + 8);
             if (ok) {
                 const int rc = aionhip_step_headnorm_rope_append(
-                    ctx, rope[0]->out.handle, xq.handle, xk.handle, xv.handle, nq->in[1].handle, nq->in[2].handle, nk->in[1].handle, nk->in[2].handle,
-                    nv->in[1].handle, nv->in[2].handle, nq->eps, kc.handle, vc.handle, rope[0]->in[1].handle, app[0]->in[1].handle, xq.shape[0],
-                    xq.shape[1], kc.shape[1], xq.shape[2], xk.shape[2], d, rope[0]->rope_base, rope[0]->rope_scale, rope[0]->rope_proportion,
+                    ctx, t.rope[0]->out.handle, xq.handle, xk.handle, xv.handle, nq->in[1].handle, nq->in[2].handle, nk->in[1].handle, nk->in[2].handle,
+                    nv->in[1].handle, nv->in[2].handle, nq->eps, kc.handle, vc.handle, t.rope[0]->in[1].handle, t.app[0]->in[1].handle, xq.shape[0],
+                    xq.shape[1], kc.shape[1], xq.shape[2], xk.shape[2], d, t.rope[0]->rope_base, t.rope[0]->rope_scale, t.rope[0]->rope_proportion,
                     (kc.flags & AIONHIP_TENSOR_ROLLING) ? 1 : 0);
                 if (rc != AIONHIP_UNSUPPORTED) { *rc_out = wrap(i, st, rc); ++calls_last_execute; return 9; }
+            }
+        }
+    }
+    // The cache side without head norms, for any batch and token count (a prompt, several sequences): RoPE1D on q and k -> Cast f16
+    // + SequenceAppend of k and of v, six steps from the first of the ropes on, linear caches
+    if ((fusion & AIONHIP_FUSE_WORKSPACE) && st.tag == AIONHIP_STEP_ROPE1D && i + 5 < count) {
+        KvTail t;
+        if (sort_kv_tail(steps, i, i + 6, 0, t)) {
+            const aionhip_tensor_ref &xq = t.rope[0]->in[0], &xk = t.rope[1]->in[0], &xv = t.cast[1]->in[0], &kc = t.app[0]->out, &vc = t.app[1]->out;
+            const size_t d = xq.shape[3];
+            bool ok = xv.rank == 4 && xk.shape[3] == d && xv.shape[3] == d && xk.shape[0] == xq.shape[0] && xv.shape[0] == xq.shape[0] &&
+                      xk.shape[1] == xq.shape[1] && xv.shape[1] == xq.shape[1] && xv.shape[2] == xk.shape[2] && is_f32(xv) &&
+                      kc.shape[0] == xq.shape[0] && vc.shape[0] == xq.shape[0] && kc.shape[2] == xk.shape[2] && vc.shape[2] == xk.shape[2] &&
+                      kc.shape[3] == d && vc.shape[3] == d && !(kc.flags & AIONHIP_TENSOR_ROLLING) && xq.shape[1] <= kc.shape[1] &&
+                      tail_outputs_clear(t, {&xq, &xk, &xv});
+            ok = ok && dead_after(t.rope[1]->out, i + 5) && dead_after(t.cast[0]->out, i + 5) && dead_after(t.cast[1]->out, i + 5);
+            if (ok) {
+                const int rc = aionhip_step_rope_append(ctx, t.rope[0]->out.handle, xq.handle, xk.handle, xv.handle, kc.handle, vc.handle,
+                                                        t.rope[0]->in[1].handle, t.app[0]->in[1].handle, xq.shape[0], xq.shape[1], kc.shape[1],
+                                                        xq.shape[2], xk.shape[2], d, t.rope[0]->rope_base, t.rope[0]->rope_scale,
+                                                        t.rope[0]->rope_proportion);
+                if (rc != AIONHIP_UNSUPPORTED) { *rc_out = wrap(i, st, rc); ++calls_last_execute; return 6; }
             }
         }
     }

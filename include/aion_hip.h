@@ -488,7 +488,8 @@ int aionhip_session_create(aionhip_ctx *ctx, aionhip_session **out);
  * Cast + SequenceAppend of k and of v (ten steps, aionhip_step_rmsnorm_qkv_rope_append), RMSNorm -> gate and up MatMuls ->
  * gate(gelu) -> down MatMul (five steps, aionhip_step_rmsnorm_geglu_matmul); and for any batch and token count the cache
  * side of a block that normalizes its heads: RMSNorm over the head size on q, k, v -> RoPE1D on q and k -> Cast +
- * SequenceAppend of k and of v (nine steps, aionhip_step_headnorm_rope_append). A MatMul (beta 0) whose workspace output is
+ * SequenceAppend of k and of v (nine steps, aionhip_step_headnorm_rope_append), and the same without the norms over linear
+ * caches (six steps, aionhip_step_rope_append). A MatMul (beta 0) whose workspace output is
  * read only by an add right behind it that accumulates in place (x = x + t) writes x itself with beta 1, alone or as the
  * last step of the patterns above: alpha * acc + x is rounded once either way. A pattern whose entry point answers
  * AIONHIP_UNSUPPORTED for the shape runs as the next smaller pattern or as separate steps. aion folds at step level the same

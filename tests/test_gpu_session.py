@@ -224,7 +224,11 @@ def test_a_decoder_layer_as_a_step_list_equals_the_steps_issued_one_by_one(gpu, 
     lean = Layer(gpu, S, past, rolling)
     for order in (False, True):
         sess.execute(lean.steps(lean=True, casts_first=order))
-        assert sess.stats()[0] == (calls_plain - 9 - 4 if S == 1 else (calls_plain - 8 if not order else calls_plain - 6))
+        # more rows: norm + q/k/v (4 steps, 1 call), the six rope / cast / append steps in either order (1 call), norm + gate / up
+        # (3 steps, 1 call), gate + down (2 steps, 1 call)
+        # (a rolling cache has no one-call form of the six: there the cast + append pairs fold where they stand side by side)
+        tail = 5 if not rolling else (0 if order else 2)
+        assert sess.stats()[0] == (calls_plain - 9 - 4 if S == 1 else calls_plain - 3 - tail - 2 - 1)
         got = lean.results(every)
         if S == 1:
             folded = ("q", "k", "v", "kr", "gt", "upj")      # o and dn feed adds that write elsewhere: still written
@@ -232,7 +236,10 @@ def test_a_decoder_layer_as_a_step_list_equals_the_steps_issued_one_by_one(gpu, 
             for n in list(Layer.WORKSPACE) + list(folded):
                 assert not got[n].any(), n
         else:
-            _same(got, want, [n for n in Layer.KEPT if n not in ("widx", "len")])
+            gone = ["kr", "k16", "v16"] if not rolling else ([] if order else ["k16", "v16"])
+            _same(got, want, [n for n in Layer.KEPT if n not in ["widx", "len"] + gone])
+            for n in ["h", "h2", "gg"] + gone:
+                assert not got[n].any(), n
         # the second pass appends the same rows at the same place: put the counters back
         gpu.write(lean.bufs["widx"], np.array([past], np.int32))
         gpu.write(lean.bufs["len"], np.array([past + S], np.int32))
@@ -246,9 +253,9 @@ def test_a_decoder_layer_as_a_step_list_equals_the_steps_issued_one_by_one(gpu, 
     ref.free()
     acc = Layer(gpu, S, past, rolling, inplace=True)
     sess.execute(acc.steps(lean=True))
-    assert sess.stats()[0] == (calls_plain - 15 if S == 1 else calls_plain - 10)
+    assert sess.stats()[0] == (calls_plain - 15 if S == 1 else (calls_plain - 13 if not rolling else calls_plain - 10))
     got = acc.results(every)
-    folded = ("o", "dn") + (("q", "k", "v", "kr", "gt", "upj") if S == 1 else ())
+    folded = ("o", "dn") + (("q", "k", "v", "kr", "gt", "upj") if S == 1 else (("kr",) if not rolling else ()))
     _same(got, want_inplace, [n for n in Layer.KEPT if n not in folded])
     for n in list(Layer.WORKSPACE) + list(folded):
         assert not got[n].any(), n

@@ -331,6 +331,7 @@ pub const HipBackend = struct {
     //   MatMul(s) sharing one A                                                        -> aionhip_step_matmul_batch
     //   MatMul, add in place (x = x + t), alone or behind the patterns above           -> the matmul with C = x, beta = 1
     //   RMSNorm x3 per head (q,k,v), RoPE1D x2, Cast f16 x2, SequenceAppend x2         -> aionhip_step_headnorm_rope_append
+    //   RoPE1D x2, Cast f16 x2, SequenceAppend x2 (linear caches)                      -> aionhip_step_rope_append
     // A whole decode program (no If/Loop, no Transfer) may be recorded once between aionhip_program_begin/_end around
     // aionhip_session_execute and replayed with aionhip_program_execute while aionhip_program_is_current holds (replay
     // precedent: backend/gpu/frame.zig:77-86).
